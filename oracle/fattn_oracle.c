@@ -1,0 +1,454 @@
+/*
+ * CPU oracle for GGML_OP_FLASH_ATTN_EXT - see fattn_oracle.h for what is pinned
+ * and what is recalled.  Test infrastructure only; never linked into the product.
+ */
+#include "fattn_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+#if defined(__F16C__)
+#include <immintrin.h>
+#endif
+
+/* ------------------------------------------------------------------ fp16 -- */
+
+/* IEEE-754 binary32 -> binary16, round-to-nearest-even, overflow to inf, NaN kept
+ * quiet.  This is what ggml's GGML_FP32_TO_FP16 computes on every platform and what
+ * the reference's ggml_cast(F32 -> F16) of the mask relies on (src/core/fastconformer.h:918,
+ * src/crispasr.cpp:3141). */
+static uint16_t fp32_to_fp16_soft(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    const uint32_t absx = x & 0x7fffffffu;
+    if (absx >= 0x7f800000u) {                         /* inf / nan */
+        return (uint16_t)(sign | (absx > 0x7f800000u ? 0x7e00u : 0x7c00u));
+    }
+    if (absx >= 0x477ff000u) {                         /* >= 65520 rounds to inf */
+        return (uint16_t)(sign | 0x7c00u);
+    }
+    if (absx < 0x33000001u) {                          /* <= 2^-25 rounds to zero */
+        return (uint16_t)sign;
+    }
+    int32_t  e = (int32_t)(absx >> 23) - 127;          /* unbiased exponent */
+    uint32_t m = (absx & 0x007fffffu) | 0x00800000u;   /* 24-bit significand */
+    uint32_t shift;
+    uint32_t base;
+    if (e < -14) {                                     /* subnormal half */
+        shift = (uint32_t)(13 + (-14 - e));
+        base  = 0;
+    } else {
+        shift = 13;
+        base  = (uint32_t)(e + 15) << 10;
+        m &= 0x007fffffu;
+    }
+    uint32_t q    = m >> shift;
+    uint32_t rem  = m & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) {
+        q++;                                           /* carries into the exponent correctly */
+    }
+    return (uint16_t)(sign | (base + q));
+}
+
+static float fp16_to_fp32_soft(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    const uint32_t e    = (h >> 10) & 0x1fu;
+    const uint32_t m    = h & 0x3ffu;
+    uint32_t x;
+    if (e == 0) {
+        if (m == 0) {
+            x = sign;
+        } else {                                       /* subnormal: m * 2^-24 */
+            float f = (float)m * 5.9604644775390625e-08f;
+            memcpy(&x, &f, 4);
+            x |= sign;
+        }
+    } else if (e == 31) {
+        x = sign | 0x7f800000u | (m << 13);
+    } else {
+        x = sign | ((e + 112u) << 23) | (m << 13);
+    }
+    float f;
+    memcpy(&f, &x, 4);
+    return f;
+}
+
+uint16_t ora_fp32_to_fp16(float f) { return fp32_to_fp16_soft(f); }
+float    ora_fp16_to_fp32(uint16_t h) { return fp16_to_fp32_soft(h); }
+
+/* fast paths used inside the hot loops; the tests check them against the soft ones */
+static inline float h2f(uint16_t h) {
+#if defined(__F16C__)
+    return _cvtsh_ss(h);
+#else
+    return fp16_to_fp32_soft(h);
+#endif
+}
+static inline uint16_t f2h(float f) {
+#if defined(__F16C__)
+    return _cvtss_sh(f, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC);
+#else
+    return fp32_to_fp16_soft(f);
+#endif
+}
+
+void ora_fp32_to_fp16_row(const float * x, uint16_t * y, int64_t n) {
+    for (int64_t i = 0; i < n; i++) y[i] = f2h(x[i]);
+}
+void ora_fp16_to_fp32_row(const uint16_t * x, float * y, int64_t n) {
+    for (int64_t i = 0; i < n; i++) y[i] = h2f(x[i]);
+}
+
+/* ------------------------------------------------------------------ Q8_0 -- */
+
+/* Block of 32: d = amax/127 kept in f32 for the division, stored as fp16;
+ * q = round(x * (1/d)) with the unrounded f32 d
+ * (tools/upstream-prs/09-metal-q8_0-bit-match.md:24-31; "block-32" layout
+ * src/core/attention.h:79-83).  ggml-cpu's SIMD quantisers round to nearest even,
+ * its scalar quantize_row_q8_0_ref rounds half away from zero: both selectable. */
+void ora_quantize_row_q8_0(const float * x, ora_block_q8_0 * y, int64_t n, int rounding) {
+    const int64_t nb = n / ORA_QK8_0;
+    for (int64_t i = 0; i < nb; i++) {
+        float amax = 0.0f;
+        for (int j = 0; j < ORA_QK8_0; j++) {
+            const float a = fabsf(x[i * ORA_QK8_0 + j]);
+            if (a > amax) amax = a;
+        }
+        const float d  = amax / 127.0f;
+        const float id = d != 0.0f ? 1.0f / d : 0.0f;
+        y[i].d = fp32_to_fp16_soft(d);
+        for (int j = 0; j < ORA_QK8_0; j++) {
+            const float x0 = x[i * ORA_QK8_0 + j] * id;
+            y[i].qs[j] = (int8_t)(rounding == ORA_ROUND_HALF_AWAY ? roundf(x0) : nearbyintf(x0));
+        }
+    }
+}
+
+/* x = q * d  (f32 product of the exact int8 and the exact fp16 scale) */
+void ora_dequantize_row_q8_0(const ora_block_q8_0 * x, float * y, int64_t n) {
+    const int64_t nb = n / ORA_QK8_0;
+    for (int64_t i = 0; i < nb; i++) {
+        const float d = fp16_to_fp32_soft(x[i].d);
+        for (int j = 0; j < ORA_QK8_0; j++) y[i * ORA_QK8_0 + j] = (float)x[i].qs[j] * d;
+    }
+}
+
+/* ------------------------------------------------------------------- RNG -- */
+
+static inline uint64_t splitmix64_at(uint64_t seed, uint64_t idx) {
+    uint64_t z = seed * 0xD1342543DE82EF95ull + (idx + 1) * 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+void ora_randn(uint64_t seed, int64_t n, float * out) {
+    const double two_pi = 6.283185307179586476925286766559;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) {
+        const uint64_t a  = splitmix64_at(seed, 2 * (uint64_t)i);
+        const uint64_t b  = splitmix64_at(seed, 2 * (uint64_t)i + 1);
+        const double   u1 = ((double)(a >> 11) + 1.0) * (1.0 / 9007199254740992.0); /* (0,1] */
+        const double   u2 = (double)(b >> 11) * (1.0 / 9007199254740992.0);         /* [0,1) */
+        out[i] = (float)(sqrt(-2.0 * log(u1)) * cos(two_pi * u2));
+    }
+}
+
+int64_t ora_randint(uint64_t seed, int64_t i, int64_t lo, int64_t hi) {
+    const uint64_t span = (uint64_t)(hi - lo + 1);
+    return lo + (int64_t)(splitmix64_at(seed ^ 0xA5A5A5A5A5A5A5A5ull, (uint64_t)i) % span);
+}
+
+int ora_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+/* ------------------------------------------------------- flash_attn_ext -- */
+
+static inline const char * row_ptr(const ora_tensor * t, int64_t i1, int64_t i2, int64_t i3) {
+    return (const char *)t->data + i1 * t->nb[1] + i2 * t->nb[2] + i3 * t->nb[3];
+}
+
+static int type_ok(int t) { return t == ORA_TYPE_F32 || t == ORA_TYPE_F16 || t == ORA_TYPE_Q8_0; }
+
+/* one K or V row -> f32 (exact for every storage type) */
+static void row_to_f32(const char * p, int type, int64_t n, float * out) {
+    if (type == ORA_TYPE_F32) {
+        memcpy(out, p, (size_t)n * 4);
+    } else if (type == ORA_TYPE_F16) {
+        const uint16_t * h = (const uint16_t *)p;
+        for (int64_t i = 0; i < n; i++) out[i] = h2f(h[i]);
+    } else {
+        ora_dequantize_row_q8_0((const ora_block_q8_0 *)p, out, n);
+    }
+}
+
+/* ALiBi slope of head h; 1 when max_bias == 0.  Every call site of the reference
+ * passes max_bias = 0 (e.g. src/crispasr.cpp:2821, src/core/attention.h:992).
+ * Formula recalled from ggml: PARITY UNPINNED. */
+static float alibi_slope(float max_bias, int64_t h, int64_t n_head) {
+    if (max_bias <= 0.0f) return 1.0f;
+    const uint32_t n_head_log2 = 1u << (uint32_t)floor(log2((double)n_head));
+    const float m0 = powf(2.0f, -(max_bias) / n_head_log2);
+    const float m1 = powf(2.0f, -(max_bias / 2.0f) / n_head_log2);
+    return h < (int64_t)n_head_log2 ? powf(m0, (float)(h + 1)) : powf(m1, (float)(2 * (h - n_head_log2) + 1));
+}
+
+typedef struct {
+    const ora_tensor *q, *k, *v, *mask;
+    float * dst;
+    float   scale, max_bias, softcap;
+    int64_t D, DV, Nq, Hq, B, Nkv, Hkv, Bk;
+} fa_args;
+
+/* fp64 two-pass softmax(scale*q.k [softcap] + slope*mask) . V, exact dequantisation.
+ * Math and operand roles: src/core/fastconformer.h:883-885 (mask is added after the
+ * scale), src/core/attention.h:923-933 (consecutive q heads share a kv head),
+ * src/crispasr.cpp:3485-3487 (-inf mask entries are excluded keys),
+ * src/crispasr.cpp:2823 + src/core/attention.h:1000 (output is [DV, Hq, Nq, B]). */
+static void fa_row_exact(const fa_args * a, int64_t iq1, int64_t iq2, int64_t iq3,
+                         double * s, float * tmp, double * acc) {
+    const int64_t ik2 = iq2 / (a->Hq / a->Hkv);
+    const int64_t ik3 = iq3 / (a->B / a->Bk);
+    const float * qrow = (const float *)row_ptr(a->q, iq1, iq2, iq3);
+    const uint16_t * mrow = NULL;
+    if (a->mask) {
+        mrow = (const uint16_t *)row_ptr(a->mask, iq1, iq2 % a->mask->ne[2], iq3 % a->mask->ne[3]);
+    }
+    const double slope = alibi_slope(a->max_bias, iq2, a->Hq);
+    double smax = -INFINITY;
+    for (int64_t j = 0; j < a->Nkv; j++) {
+        double mv = 0.0;
+        if (mrow) {
+            mv = slope * (double)fp16_to_fp32_soft(mrow[j]);
+            if (mv == -INFINITY) { s[j] = -INFINITY; continue; }
+        }
+        row_to_f32(row_ptr(a->k, j, ik2, ik3), a->k->type, a->D, tmp);
+        double dot = 0.0;
+        for (int64_t d = 0; d < a->D; d++) dot += (double)qrow[d] * (double)tmp[d];
+        double sc = dot * (double)a->scale;
+        if (a->softcap != 0.0f) sc = (double)a->softcap * tanh(sc / (double)a->softcap);
+        sc += mv;
+        s[j] = sc;
+        if (sc > smax) smax = sc;
+    }
+    for (int64_t d = 0; d < a->DV; d++) acc[d] = 0.0;
+    double sum = 0.0;
+    if (smax > -INFINITY) {
+        for (int64_t j = 0; j < a->Nkv; j++) {
+            if (s[j] == -INFINITY) continue;
+            const double p = exp(s[j] - smax);
+            sum += p;
+            row_to_f32(row_ptr(a->v, j, ik2, ik3), a->v->type, a->DV, tmp);
+            for (int64_t d = 0; d < a->DV; d++) acc[d] += p * (double)tmp[d];
+        }
+    }
+    float * out = a->dst + ((iq3 * a->Nq + iq1) * a->Hq + iq2) * a->DV;
+    const double inv = sum > 0.0 ? 1.0 / sum : 0.0;
+    for (int64_t d = 0; d < a->DV; d++) out[d] = (float)(acc[d] * inv);
+}
+
+/* f32 online softmax in key order, the way ggml-cpu walks one query row
+ * (recurrence as in src/core/cpu_attention.h:53-83).  RECALLED details, PARITY UNPINNED:
+ * the Q row is converted to K's vec_dot_type (F32 for F32/F16 K in the fork -
+ * tools/upstream-prs/01-cpu-f16-saturation.md:17-23 - and Q8_0 for Q8_0 K), and the
+ * P.V accumulator is fp16 when V is F16. */
+static void fa_row_ggml_like(const fa_args * a, int64_t iq1, int64_t iq2, int64_t iq3,
+                             float * tmp, float * acc32, uint16_t * acc16, ora_block_q8_0 * qq) {
+    const int64_t ik2 = iq2 / (a->Hq / a->Hkv);
+    const int64_t ik3 = iq3 / (a->B / a->Bk);
+    const float * qrow = (const float *)row_ptr(a->q, iq1, iq2, iq3);
+    const uint16_t * mrow = NULL;
+    if (a->mask) {
+        mrow = (const uint16_t *)row_ptr(a->mask, iq1, iq2 % a->mask->ne[2], iq3 % a->mask->ne[3]);
+    }
+    const float slope = alibi_slope(a->max_bias, iq2, a->Hq);
+    float scale = a->scale;
+    if (a->softcap != 0.0f) scale /= a->softcap;
+
+    const int     ktype  = a->k->type;
+    const int     vtype  = a->v->type;
+    const int64_t D      = a->D;
+    const int64_t DV     = a->DV;
+    const int     v_f16  = vtype == ORA_TYPE_F16;
+
+    if (ktype == ORA_TYPE_Q8_0) ora_quantize_row_q8_0(qrow, qq, D, ORA_ROUND_NEAREST_EVEN);
+
+    float S = 0.0f;
+    float M = -INFINITY;
+    if (v_f16) memset(acc16, 0, (size_t)DV * 2); else memset(acc32, 0, (size_t)DV * 4);
+
+    for (int64_t j = 0; j < a->Nkv; j++) {
+        const float mv = mrow ? slope * h2f(mrow[j]) : 0.0f;
+        if (mv == -INFINITY) continue;
+
+        const char * kp = row_ptr(a->k, j, ik2, ik3);
+        float s = 0.0f;
+        if (ktype == ORA_TYPE_F32) {
+            const float * kf = (const float *)kp;
+#pragma omp simd reduction(+ : s)
+            for (int64_t d = 0; d < D; d++) s += kf[d] * qrow[d];
+        } else if (ktype == ORA_TYPE_F16) {
+            const uint16_t * kh = (const uint16_t *)kp;
+#if defined(__F16C__) && defined(__AVX2__) && defined(__FMA__)
+            __m256 vs = _mm256_setzero_ps();
+            int64_t d = 0;
+            for (; d + 8 <= D; d += 8) {
+                const __m256 kf = _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(kh + d)));
+                vs = _mm256_fmadd_ps(kf, _mm256_loadu_ps(qrow + d), vs);
+            }
+            __m128 lo = _mm_add_ps(_mm256_castps256_ps128(vs), _mm256_extractf128_ps(vs, 1));
+            lo = _mm_add_ps(lo, _mm_movehl_ps(lo, lo));
+            lo = _mm_add_ss(lo, _mm_movehdup_ps(lo));
+            s = _mm_cvtss_f32(lo);
+            for (; d < D; d++) s += h2f(kh[d]) * qrow[d];
+#else
+            for (int64_t d = 0; d < D; d++) s += h2f(kh[d]) * qrow[d];
+#endif
+        } else {
+            const ora_block_q8_0 * kb = (const ora_block_q8_0 *)kp;
+            for (int64_t ib = 0; ib < D / ORA_QK8_0; ib++) {
+                int sumi = 0;
+                for (int e = 0; e < ORA_QK8_0; e++) sumi += (int)kb[ib].qs[e] * (int)qq[ib].qs[e];
+                s += (float)sumi * (h2f(kb[ib].d) * h2f(qq[ib].d));
+            }
+        }
+        s *= scale;
+        if (a->softcap != 0.0f) s = a->softcap * tanhf(s);
+        s += mv;
+
+        const float Mold = M;
+        float ms = 1.0f, vs = 1.0f;
+        const char * vp = row_ptr(a->v, j, ik2, ik3);
+        if (v_f16) {
+            const uint16_t * vh = (const uint16_t *)vp;
+            if (s > M) {
+                M  = s;
+                ms = expf(Mold - M);
+                for (int64_t d = 0; d < DV; d++) acc16[d] = f2h(h2f(acc16[d]) * ms);
+            } else {
+                vs = expf(s - M);
+            }
+            for (int64_t d = 0; d < DV; d++) acc16[d] = f2h(h2f(acc16[d]) + h2f(vh[d]) * vs);
+        } else {
+            if (s > M) {
+                M  = s;
+                ms = expf(Mold - M);
+                for (int64_t d = 0; d < DV; d++) acc32[d] *= ms;
+            } else {
+                vs = expf(s - M);
+            }
+            const float * vf;
+            if (vtype == ORA_TYPE_F32) {
+                vf = (const float *)vp;
+            } else {
+                ora_dequantize_row_q8_0((const ora_block_q8_0 *)vp, tmp, DV);
+                vf = tmp;
+            }
+            for (int64_t d = 0; d < DV; d++) acc32[d] += vf[d] * vs;
+        }
+        S = S * ms + vs;
+    }
+    if (v_f16) {
+        for (int64_t d = 0; d < DV; d++) acc32[d] = h2f(acc16[d]);
+    }
+    const float S_inv = S == 0.0f ? 0.0f : 1.0f / S;
+    float * out = a->dst + ((iq3 * a->Nq + iq1) * a->Hq + iq2) * a->DV;
+    for (int64_t d = 0; d < DV; d++) out[d] = acc32[d] * S_inv;
+}
+
+int ora_flash_attn_ext(const ora_tensor * q, const ora_tensor * k, const ora_tensor * v,
+                       const ora_tensor * mask, float * dst,
+                       float scale, float max_bias, float logit_softcap,
+                       int mode, int n_threads) {
+    if (!q || !k || !v || !dst) return -1;
+    if (mask && !mask->data) mask = NULL;
+    if (q->type != ORA_TYPE_F32 || !type_ok(k->type) || !type_ok(v->type)) return -2;
+    if (mask && mask->type != ORA_TYPE_F16) return -2;
+
+    fa_args a;
+    a.q = q; a.k = k; a.v = v; a.mask = mask; a.dst = dst;
+    a.scale = scale; a.max_bias = max_bias; a.softcap = logit_softcap;
+    a.D = q->ne[0]; a.Nq = q->ne[1]; a.Hq = q->ne[2]; a.B = q->ne[3];
+    a.DV = v->ne[0]; a.Nkv = k->ne[1]; a.Hkv = k->ne[2]; a.Bk = k->ne[3];
+
+    /* contract of the constructor (ggml_flash_attn_ext), as the call sites use it */
+    if (k->ne[0] != a.D || v->ne[1] != a.Nkv || v->ne[2] != a.Hkv || v->ne[3] != a.Bk) return -3;
+    if (a.Hkv <= 0 || a.Bk <= 0 || a.Hq % a.Hkv != 0 || a.B % a.Bk != 0) return -3;
+    if ((k->type == ORA_TYPE_Q8_0 && a.D % ORA_QK8_0) || (v->type == ORA_TYPE_Q8_0 && a.DV % ORA_QK8_0)) return -3;
+    if (mask) {
+        if (mask->ne[0] < a.Nkv || mask->ne[1] < a.Nq) return -4;
+        if (a.Hq % mask->ne[2] != 0 || a.B % mask->ne[3] != 0) return -4;
+        if (mask->nb[0] != 2) return -4;
+    }
+    if (max_bias > 0.0f && !mask) return -5;
+    if (q->nb[0] != 4) return -6;
+
+    const int64_t n_rows = a.Nq * a.Hq * a.B;
+    int nt = n_threads > 0 ? n_threads : 1;
+#ifndef _OPENMP
+    nt = 1;
+#endif
+
+#pragma omp parallel num_threads(nt)
+    {
+        const int64_t Dm = a.D > a.DV ? a.D : a.DV;
+        double *        s     = mode == ORA_MODE_EXACT ? (double *)malloc((size_t)(a.Nkv > 0 ? a.Nkv : 1) * 8) : NULL;
+        double *        acc   = (double *)malloc((size_t)Dm * 8);
+        float *         tmp   = (float *)malloc((size_t)Dm * 4);
+        float *         acc32 = (float *)malloc((size_t)Dm * 4);
+        uint16_t *      acc16 = (uint16_t *)malloc((size_t)Dm * 2);
+        ora_block_q8_0 * qq   = (ora_block_q8_0 *)malloc(sizeof(ora_block_q8_0) * (size_t)(a.D / ORA_QK8_0 + 1));
+#pragma omp for schedule(dynamic, 16)
+        for (int64_t ir = 0; ir < n_rows; ir++) {
+            const int64_t iq3 = ir / (a.Hq * a.Nq);
+            const int64_t iq2 = (ir - iq3 * a.Hq * a.Nq) / a.Nq;
+            const int64_t iq1 = ir - iq3 * a.Hq * a.Nq - iq2 * a.Nq;
+            if (mode == ORA_MODE_EXACT) {
+                fa_row_exact(&a, iq1, iq2, iq3, s, tmp, acc);
+            } else {
+                fa_row_ggml_like(&a, iq1, iq2, iq3, tmp, acc32, acc16, qq);
+            }
+        }
+        free(s); free(acc); free(tmp); free(acc32); free(acc16); free(qq);
+    }
+    return 0;
+}
+
+/* --------------------------------------------------------- KV-cache write -- */
+
+/* ggml_cpy of an F32 tensor into a view of the KV cache (src/crispasr.cpp:2810-2811,
+ * 3185-3203; src/core/attention.h:342-378, 850-867).  Element (i0,i1,i2,i3) of src goes
+ * to the same index of dst; for Q8_0 a dst row is ne0/32 consecutive blocks. */
+int ora_cpy_f32(const ora_tensor * src, void * dst_data, int32_t dst_type, const int64_t dst_nb[4],
+                int rounding) {
+    if (!src || src->type != ORA_TYPE_F32 || !type_ok(dst_type)) return -2;
+    if (dst_type == ORA_TYPE_Q8_0 && src->ne[0] % ORA_QK8_0) return -3;
+    const int64_t n0 = src->ne[0];
+    float * tmp = (float *)malloc((size_t)(n0 > 0 ? n0 : 1) * 4);
+    for (int64_t i3 = 0; i3 < src->ne[3]; i3++)
+    for (int64_t i2 = 0; i2 < src->ne[2]; i2++)
+    for (int64_t i1 = 0; i1 < src->ne[1]; i1++) {
+        const char * sp = (const char *)src->data + i1 * src->nb[1] + i2 * src->nb[2] + i3 * src->nb[3];
+        char *       dp = (char *)dst_data + i1 * dst_nb[1] + i2 * dst_nb[2] + i3 * dst_nb[3];
+        for (int64_t i0 = 0; i0 < n0; i0++) tmp[i0] = *(const float *)(sp + i0 * src->nb[0]);
+        if (dst_type == ORA_TYPE_F32) {
+            for (int64_t i0 = 0; i0 < n0; i0++) *(float *)(dp + i0 * dst_nb[0]) = tmp[i0];
+        } else if (dst_type == ORA_TYPE_F16) {
+            for (int64_t i0 = 0; i0 < n0; i0++) *(uint16_t *)(dp + i0 * dst_nb[0]) = fp32_to_fp16_soft(tmp[i0]);
+        } else {
+            ora_quantize_row_q8_0(tmp, (ora_block_q8_0 *)dp, n0, rounding);
+        }
+    }
+    free(tmp);
+    return 0;
+}

@@ -1,0 +1,94 @@
+/*
+ * CPU oracle for GGML_OP_FLASH_ATTN_EXT and the KV-cache copies around it.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing under oracle/ is part of the shipped
+ * library: it is the checker that the parity tests, the smoke run and the
+ * benchmark's cpu_baseline leg compare the HIP kernels against.
+ *
+ * The arithmetic restated here lives in a third-party dependency of the
+ * reference that is absent from its tree: ggml (CrispStrobe/ggml, branch
+ * sync/upstream-v0.17, commit a0f7289d = ggml v0.17.0 + fork patches; pin named
+ * in tools/upstream-prs/SYNC-v0.17-CONFLICTS.md:3-7,197).  The restatement is
+ * anchored on the reference's own call sites and notes, cited per function.
+ *
+ * Parity status of each function:
+ *   ora_fp32_to_fp16 / ora_fp16_to_fp32 : pinned (IEEE-754 binary16, RNE; checked
+ *       exhaustively against numpy.float16).
+ *   ora_quantize_row_q8_0 / ora_dequantize_row_q8_0 : pinned by the reference's
+ *       description of the format (tools/upstream-prs/09-metal-q8_0-bit-match.md:24-31),
+ *       known-answer blocks and the round-trip bound of
+ *       tests/test-kv-quant-roundtrip.cpp:193.
+ *   ora_flash_attn_ext, mode ORA_MODE_EXACT : pinned by the mathematics (fp64
+ *       textbook softmax(scale*QK^T + mask)V written independently in numpy, closed
+ *       forms, brute force) and by the layouts the call sites fix.
+ *   ora_flash_attn_ext, mode ORA_MODE_GGML_LIKE (f32 online softmax, Q row
+ *       quantised to Q8_0 for Q8_0 K, f16 accumulator for F16 V), and the
+ *       max_bias (ALiBi) slope formula : PARITY UNPINNED - recalled
+ *       behaviour of ggml-cpu that no file, test or fixture of the reference
+ *       holds.  logit_softcap is pinned by its closed form only.
+ */
+#ifndef FATTN_ORACLE_H
+#define FATTN_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ggml type ids of the types this path meets */
+enum { ORA_TYPE_F32 = 0, ORA_TYPE_F16 = 1, ORA_TYPE_Q8_0 = 8 };
+
+enum { ORA_MODE_EXACT = 0, ORA_MODE_GGML_LIKE = 1 };
+
+/* rounding of x/d in the Q8_0 quantiser */
+enum { ORA_ROUND_NEAREST_EVEN = 0, ORA_ROUND_HALF_AWAY = 1 };
+
+#define ORA_QK8_0 32
+
+typedef struct {
+    uint16_t d;               /* fp16 scale */
+    int8_t   qs[ORA_QK8_0];   /* quants */
+} ora_block_q8_0;             /* 34 bytes, no padding */
+
+/* a ggml tensor view: ne = elements per dim, nb = byte strides, dim 0 fastest */
+typedef struct {
+    const void * data;
+    int32_t      type;
+    int64_t      ne[4];
+    int64_t      nb[4];
+} ora_tensor;
+
+uint16_t ora_fp32_to_fp16(float f);
+float    ora_fp16_to_fp32(uint16_t h);
+void     ora_fp32_to_fp16_row(const float * x, uint16_t * y, int64_t n);
+void     ora_fp16_to_fp32_row(const uint16_t * x, float * y, int64_t n);
+
+void ora_quantize_row_q8_0(const float * x, ora_block_q8_0 * y, int64_t n, int rounding);
+void ora_dequantize_row_q8_0(const ora_block_q8_0 * x, float * y, int64_t n);
+
+/* deterministic N(0,1): splitmix64 counter -> Box-Muller in fp64 -> float.
+ * element i of stream `seed` depends only on (seed, i). */
+void ora_randn(uint64_t seed, int64_t n, float * out);
+/* uniform integer in [lo, hi] for element i of stream seed */
+int64_t ora_randint(uint64_t seed, int64_t i, int64_t lo, int64_t hi);
+
+/* dst: contiguous f32 [DV, Hq, Nq, B].  mask may be NULL (or mask->data NULL).
+ * returns 0, or a negative code when the shapes break the op's contract. */
+int ora_flash_attn_ext(const ora_tensor * q, const ora_tensor * k, const ora_tensor * v,
+                       const ora_tensor * mask, float * dst,
+                       float scale, float max_bias, float logit_softcap,
+                       int mode, int n_threads);
+
+/* KV-cache writes (ggml_cpy F32 -> F16/F32/Q8_0 into a strided view whose rows
+ * are contiguous): src and dst have equal ne, src is F32. */
+int ora_cpy_f32(const ora_tensor * src, void * dst_data, int32_t dst_type, const int64_t dst_nb[4],
+                int rounding);
+
+int ora_max_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
