@@ -1,0 +1,495 @@
+// extern "C" entry points of libmi355x_fattn.so: validation, kernel choice, scratch, launches.
+#include "fattn_common.h"
+
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <mutex>
+#include <vector>
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int status, const char * fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int hip_fail(hipError_t e, const char * what) {
+    return fail(MI355X_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                                   \
+    do {                                                \
+        hipError_t e_ = (expr);                         \
+        if (e_ != hipSuccess) return hip_fail(e_, #expr); \
+    } while (0)
+
+size_t type_size(int t) {
+    switch (t) {
+        case MI355X_TYPE_F32:  return 4;
+        case MI355X_TYPE_F16:  return 2;
+        case MI355X_TYPE_Q8_0: return FATTN_Q8_0_BYTES;
+        default:               return 0;
+    }
+}
+int64_t block_size(int t) { return t == MI355X_TYPE_Q8_0 ? FATTN_QK8_0 : 1; }
+
+bool is_contiguous(const mi355x_tensor * t) {
+    const size_t ts = type_size(t->type);
+    if (!ts) return false;
+    size_t nb = ts;
+    if (t->nb[0] != nb) return false;
+    nb *= (size_t)(t->ne[0] / block_size(t->type));
+    for (int i = 1; i < 4; i++) {
+        if (t->ne[i] != 1 && t->nb[i] != nb) return false;
+        nb *= (size_t)t->ne[i];
+    }
+    return true;
+}
+
+struct DeviceCache {
+    int  cus = 0;
+    bool init = false;
+};
+DeviceCache g_dev[64];
+std::mutex  g_mu;
+
+int device_cus() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_dev[dev].init) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        g_dev[dev].cus  = cus;
+        g_dev[dev].init = true;
+    }
+    return g_dev[dev].cus;
+}
+
+// Library-owned scratch for the split-KV partials: one growing allocation per device.
+// Outgrown blocks stay allocated until the process ends, so launches still in flight on
+// other streams keep valid memory.
+struct Scratch {
+    void * ptr  = nullptr;
+    size_t size = 0;
+};
+Scratch g_scratch[64];
+
+int get_scratch(size_t bytes, void ** out) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return fail(MI355X_ERR_HIP, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lk(g_mu);
+    Scratch & s = g_scratch[dev];
+    if (s.size < bytes) {
+        size_t want = s.size ? s.size : (size_t)(8u << 20);
+        while (want < bytes) want *= 2;
+        void * p = nullptr;
+        HIP_TRY(hipMalloc(&p, want));
+        s.ptr  = p;          // the previous block is deliberately kept alive
+        s.size = want;
+    }
+    *out = s.ptr;
+    return MI355X_OK;
+}
+
+// a mask argument with no extent is the same as no mask
+bool has_mask(const mi355x_tensor * mask) { return mask && mask->ne[0] > 0; }
+
+struct Plan {
+    int     kernel;
+    int     n_splits;
+    int     keys_per_split;
+    size_t  workspace;
+};
+
+int check(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+          const mi355x_tensor * mask, const mi355x_tensor * dst, const mi355x_fattn_params * p) {
+    if (!q || !k || !v || !p) return fail(MI355X_ERR_INVALID, "null argument");
+    if (q->type != MI355X_TYPE_F32) return fail(MI355X_ERR_UNSUPPORTED, "q must be F32 (type %d)", q->type);
+    if (!type_size(k->type)) return fail(MI355X_ERR_UNSUPPORTED, "K type %d not covered", k->type);
+    if (k->type != v->type) return fail(MI355X_ERR_UNSUPPORTED, "K and V types differ (%d, %d)", k->type, v->type);
+
+    const int64_t D = q->ne[0], Nq = q->ne[1], Hq = q->ne[2], B = q->ne[3];
+    const int64_t Nkv = k->ne[1], Hkv = k->ne[2], Bk = k->ne[3];
+    if (k->ne[0] != D) return fail(MI355X_ERR_INVALID, "k.ne0 %lld != q.ne0 %lld", (long long)k->ne[0], (long long)D);
+    if (v->ne[1] != Nkv || v->ne[2] != Hkv || v->ne[3] != Bk) return fail(MI355X_ERR_INVALID, "k and v shapes differ");
+    if (Hkv <= 0 || Bk <= 0 || Hq % Hkv || B % Bk) return fail(MI355X_ERR_INVALID, "q heads/batch not a multiple of kv heads/batch");
+    if (v->ne[0] != D) return fail(MI355X_ERR_UNSUPPORTED, "DV %lld != DK %lld", (long long)v->ne[0], (long long)D);
+    if (D <= 0 || D % 8 || D > 256) return fail(MI355X_ERR_UNSUPPORTED, "head size %lld (need a multiple of 8, <= 256)", (long long)D);
+    if (k->type == MI355X_TYPE_Q8_0 && D % FATTN_QK8_0) return fail(MI355X_ERR_INVALID, "Q8_0 rows need D %% 32 == 0");
+    if (Nq < 0 || Nkv < 0 || Hq <= 0 || B <= 0) return fail(MI355X_ERR_INVALID, "negative or zero extent");
+    if (q->nb[0] != 4) return fail(MI355X_ERR_UNSUPPORTED, "q rows must be contiguous (nb0 = %zu)", q->nb[0]);
+    if (k->nb[0] != type_size(k->type) || v->nb[0] != type_size(v->type))
+        return fail(MI355X_ERR_UNSUPPORTED, "k/v rows must be contiguous");
+    const size_t al = k->type == MI355X_TYPE_F32 ? 4 : 2;
+    for (int i = 1; i < 4; i++) {
+        if (q->nb[i] % 4 || k->nb[i] % al || v->nb[i] % al) return fail(MI355X_ERR_UNSUPPORTED, "misaligned strides");
+    }
+    if (((uintptr_t)q->data % 4) || ((uintptr_t)k->data % al) || ((uintptr_t)v->data % al))
+        return fail(MI355X_ERR_UNSUPPORTED, "misaligned data pointers");
+    if (has_mask(mask)) {
+        if (mask->type != MI355X_TYPE_F16) return fail(MI355X_ERR_UNSUPPORTED, "mask must be F16 (type %d)", mask->type);
+        if (mask->nb[0] != 2) return fail(MI355X_ERR_INVALID, "mask rows must be contiguous");
+        if (mask->ne[0] < Nkv || mask->ne[1] < Nq) return fail(MI355X_ERR_INVALID, "mask smaller than [Nkv, Nq]");
+        if (mask->ne[2] <= 0 || mask->ne[3] <= 0 || Hq % mask->ne[2] || B % mask->ne[3])
+            return fail(MI355X_ERR_INVALID, "mask broadcast extents do not divide q's");
+        for (int i = 1; i < 4; i++) if (mask->nb[i] % 2) return fail(MI355X_ERR_UNSUPPORTED, "misaligned mask strides");
+    } else if (p->max_bias > 0.0f) {
+        return fail(MI355X_ERR_INVALID, "max_bias > 0 needs a mask");
+    }
+    if (dst) {
+        if (dst->type != MI355X_TYPE_F32) return fail(MI355X_ERR_INVALID, "dst must be F32");
+        if (dst->ne[0] != D || dst->ne[1] != Hq || dst->ne[2] != Nq || dst->ne[3] != B)
+            return fail(MI355X_ERR_INVALID, "dst must be [DV, Hq, Nq, B]");
+        if (!is_contiguous(dst)) return fail(MI355X_ERR_UNSUPPORTED, "dst must be contiguous");
+    }
+    if (Nq * Hq * B > (int64_t)1 << 26 || Nkv > (int64_t)1 << 30) return fail(MI355X_ERR_UNSUPPORTED, "problem too large");
+    if (p->prec != 0 && p->prec != 10) return fail(MI355X_ERR_INVALID, "unknown prec %d", p->prec);
+    return MI355X_OK;
+}
+
+void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+               const mi355x_tensor * mask, float * dst, const mi355x_fattn_params * p) {
+    memset(&a, 0, sizeof(a));
+    a.q = (const char *)q->data; a.k = (const char *)k->data; a.v = (const char *)v->data;
+    a.mask = has_mask(mask) ? (const char *)mask->data : nullptr;
+    a.dst = dst;
+    a.D = (int)q->ne[0]; a.Nq = (int)q->ne[1]; a.Hq = (int)q->ne[2]; a.B = (int)q->ne[3];
+    a.Nkv = (int)k->ne[1]; a.Hkv = (int)k->ne[2]; a.Bk = (int)k->ne[3];
+    a.gqa = a.Hq / a.Hkv; a.bq = a.B / a.Bk;
+    a.nbq1 = q->nb[1]; a.nbq2 = q->nb[2]; a.nbq3 = q->nb[3];
+    a.nbk1 = k->nb[1]; a.nbk2 = k->nb[2]; a.nbk3 = k->nb[3];
+    a.nbv1 = v->nb[1]; a.nbv2 = v->nb[2]; a.nbv3 = v->nb[3];
+    a.Hm = 1; a.Bm = 1;
+    bool al16 = !((uintptr_t)q->data % 16) && !((uintptr_t)k->data % 16) && !((uintptr_t)v->data % 16);
+    for (int i = 1; i < 4; i++) al16 = al16 && !(q->nb[i] % 16) && !(k->nb[i] % 16) && !(v->nb[i] % 16);
+    if (a.mask) {
+        a.Hm = (int)mask->ne[2]; a.Bm = (int)mask->ne[3];
+        a.nbm1 = mask->nb[1]; a.nbm2 = mask->nb[2]; a.nbm3 = mask->nb[3];
+        al16 = al16 && !((uintptr_t)mask->data % 16);
+        for (int i = 1; i < 4; i++) al16 = al16 && !(mask->nb[i] % 16);
+    }
+    a.aligned16 = al16 ? 1 : 0;
+    a.softcap = p->logit_softcap;
+    a.scale   = p->logit_softcap != 0.0f ? p->scale / p->logit_softcap : p->scale;
+    a.max_bias = p->max_bias;
+    // ALiBi slope bases, as ggml derives them from the head count
+    const uint32_t n2 = 1u << (uint32_t)floorf(log2f((float)a.Hq));
+    a.n_head_log2 = (int)n2;
+    a.m0 = powf(2.0f, -(p->max_bias) / n2);
+    a.m1 = powf(2.0f, -(p->max_bias / 2.0f) / n2);
+    a.n_splits = 1;
+    a.keys_per_split = a.Nkv;
+}
+
+void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Plan & plan) {
+    int kernel = p->kernel;
+    if (kernel == MI355X_FATTN_AUTO) {
+        kernel = (a.Nq >= 16 && fattn_mma_supported(a, ktype)) ? MI355X_FATTN_MMA : MI355X_FATTN_VEC;
+    }
+    plan.kernel = kernel;
+    plan.n_splits = 1;
+    plan.keys_per_split = a.Nkv;
+    plan.workspace = 0;
+    if (kernel == MI355X_FATTN_VEC) {
+        const int64_t rows = (int64_t)a.Nq * a.Hq * a.B;
+        int ns = p->n_splits;
+        if (ns <= 0) {
+            // enough workgroups to fill the chip, but at least 128 keys per split
+            const int64_t target = (int64_t)device_cus() * 4;
+            ns = (int)((target + rows - 1) / (rows > 0 ? rows : 1));
+            const int max_by_keys = (a.Nkv + 127) / 128;
+            if (ns > max_by_keys) ns = max_by_keys;
+        }
+        if (ns > a.Nkv) ns = a.Nkv;
+        if (ns < 1) ns = 1;
+        if (ns > 256) ns = 256;
+        int kps = (a.Nkv + ns - 1) / ns;
+        if (kps < 1) kps = 1;
+        ns = a.Nkv > 0 ? (a.Nkv + kps - 1) / kps : 1;
+        plan.n_splits = ns;
+        plan.keys_per_split = a.Nkv > 0 ? kps : 0;
+        if (ns > 1) plan.workspace = (size_t)rows * ns * (a.D + 2) * sizeof(float);
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi355x_api_version(void) { return MI355X_FATTN_API_VERSION; }
+
+const char * mi355x_status_string(int status) {
+    switch (status) {
+        case MI355X_OK:              return "ok";
+        case MI355X_ERR_UNSUPPORTED: return "unsupported";
+        case MI355X_ERR_INVALID:     return "invalid argument";
+        case MI355X_ERR_HIP:         return "HIP runtime error";
+        case MI355X_ERR_NO_DEVICE:   return "no device";
+        case MI355X_ERR_WORKSPACE:   return "workspace too small";
+        default:                     return "unknown status";
+    }
+}
+
+const char * mi355x_last_error(void) { return g_err; }
+
+int mi355x_device_count(int * count) {
+    if (!count) return fail(MI355X_ERR_INVALID, "null argument");
+    int n = 0;
+    const hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) {
+        *count = 0;
+        (void)hipGetLastError();
+        return fail(MI355X_ERR_NO_DEVICE, "hipGetDeviceCount: %s", hipGetErrorString(e));
+    }
+    *count = n;
+    return MI355X_OK;
+}
+
+int mi355x_device_get_info(int device, mi355x_device_info * info) {
+    if (!info) return fail(MI355X_ERR_INVALID, "null argument");
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device));
+    memset(info, 0, sizeof(*info));
+    snprintf(info->name, sizeof(info->name), "%s", prop.name);
+    snprintf(info->arch, sizeof(info->arch), "%s", prop.gcnArchName);
+    info->compute_units       = prop.multiProcessorCount;
+    info->clock_khz           = prop.clockRate;
+    info->memory_clock_khz    = prop.memoryClockRate;
+    info->memory_bus_bits     = prop.memoryBusWidth;
+    info->total_memory        = prop.totalGlobalMem;
+    info->lds_bytes_per_block = (int32_t)prop.sharedMemPerBlock;
+    info->wavefront_size      = prop.warpSize;
+    int cur = 0;
+    HIP_TRY(hipGetDevice(&cur));
+    HIP_TRY(hipSetDevice(device));
+    size_t fr = 0, tot = 0;
+    const hipError_t e = hipMemGetInfo(&fr, &tot);
+    (void)hipSetDevice(cur);
+    if (e != hipSuccess) return hip_fail(e, "hipMemGetInfo");
+    info->free_memory = fr;
+    return MI355X_OK;
+}
+
+int mi355x_set_device(int device) {
+    HIP_TRY(hipSetDevice(device));
+    return MI355X_OK;
+}
+
+int mi355x_stream_synchronize(void * stream) {
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return MI355X_OK;
+}
+
+int mi355x_fattn_supports(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                          const mi355x_tensor * mask, const mi355x_tensor * dst,
+                          const mi355x_fattn_params * params) {
+    return check(q, k, v, mask, dst, params);
+}
+
+int mi355x_fattn_plan(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                      const mi355x_tensor * mask, const mi355x_fattn_params * params,
+                      int32_t * kernel, int32_t * n_splits) {
+    const int rc = check(q, k, v, mask, nullptr, params);
+    if (rc) return rc;
+    FattnArgs a;
+    fill_args(a, q, k, v, mask, nullptr, params);
+    Plan plan;
+    make_plan(a, k->type, params, plan);
+    if (kernel) *kernel = plan.kernel;
+    if (n_splits) *n_splits = plan.n_splits;
+    return MI355X_OK;
+}
+
+int mi355x_fattn_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                                const mi355x_tensor * mask, const mi355x_fattn_params * params,
+                                size_t * bytes) {
+    if (!bytes) return fail(MI355X_ERR_INVALID, "null argument");
+    const int rc = check(q, k, v, mask, nullptr, params);
+    if (rc) return rc;
+    FattnArgs a;
+    fill_args(a, q, k, v, mask, nullptr, params);
+    Plan plan;
+    make_plan(a, k->type, params, plan);
+    *bytes = plan.workspace;
+    return MI355X_OK;
+}
+
+int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                          const mi355x_tensor * mask, const mi355x_tensor * dst,
+                          const mi355x_fattn_params * params, void * stream) {
+    if (!dst) return fail(MI355X_ERR_INVALID, "null dst");
+    int rc = check(q, k, v, mask, dst, params);
+    if (rc) return rc;
+    if (q->ne[1] != 0 && (!q->data || !k->data || !v->data || !dst->data || (has_mask(mask) && !mask->data)))
+        return fail(MI355X_ERR_INVALID, "null data pointer");
+    FattnArgs a;
+    fill_args(a, q, k, v, mask, (float *)dst->data, params);
+    if ((int64_t)a.Nq * a.Hq * a.B == 0) return MI355X_OK;
+
+    Plan plan;
+    make_plan(a, k->type, params, plan);
+    hipStream_t st = (hipStream_t)stream;
+
+    if (plan.kernel == MI355X_FATTN_MMA) {
+        if (!fattn_mma_supported(a, k->type)) return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the MFMA kernel");
+        const int e = fattn_mma_launch(a, k->type, st);
+        if (e) return hip_fail((hipError_t)e, "fattn_mma launch");
+        return MI355X_OK;
+    }
+    if (plan.kernel != MI355X_FATTN_VEC) return fail(MI355X_ERR_UNSUPPORTED, "kernel %d not available", plan.kernel);
+
+    a.n_splits = plan.n_splits;
+    a.keys_per_split = plan.keys_per_split;
+    if (plan.n_splits > 1) {
+        void * ws = params->workspace;
+        if (ws) {
+            if (params->workspace_size < plan.workspace)
+                return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, plan.workspace);
+        } else {
+            rc = get_scratch(plan.workspace, &ws);
+            if (rc) return rc;
+        }
+        const size_t rows = (size_t)a.Nq * a.Hq * a.B;
+        a.part_acc = (float *)ws;
+        a.part_ml  = a.part_acc + rows * plan.n_splits * a.D;
+    }
+    int e = fattn_vec_launch(a, k->type, st);
+    if (e) return hip_fail((hipError_t)e, "fattn_vec launch");
+    if (plan.n_splits > 1) {
+        e = fattn_merge_launch(a, st);
+        if (e) return hip_fail((hipError_t)e, "fattn_merge launch");
+    }
+    return MI355X_OK;
+}
+
+// ---- copies ------------------------------------------------------------------------------
+
+static int cpy_check(const mi355x_tensor * src, const mi355x_tensor * dst) {
+    if (!src || !dst) return fail(MI355X_ERR_INVALID, "null argument");
+    const int s = src->type, d = dst->type;
+    const bool ok = (s == MI355X_TYPE_F32 && (d == MI355X_TYPE_F32 || d == MI355X_TYPE_F16 || d == MI355X_TYPE_Q8_0)) ||
+                    (s == MI355X_TYPE_F16 && (d == MI355X_TYPE_F16 || d == MI355X_TYPE_F32)) ||
+                    (s == MI355X_TYPE_Q8_0 && (d == MI355X_TYPE_F32 || d == MI355X_TYPE_Q8_0));
+    if (!ok) return fail(MI355X_ERR_UNSUPPORTED, "copy %d -> %d not covered", s, d);
+    int64_t ns = 1, nd = 1;
+    for (int i = 0; i < 4; i++) { ns *= src->ne[i]; nd *= dst->ne[i]; }
+    if (ns != nd) return fail(MI355X_ERR_INVALID, "element counts differ (%lld vs %lld)", (long long)ns, (long long)nd);
+    if (dst->nb[0] != type_size(d)) return fail(MI355X_ERR_UNSUPPORTED, "dst rows must be contiguous");
+    if (s == MI355X_TYPE_Q8_0 && src->nb[0] != FATTN_Q8_0_BYTES) return fail(MI355X_ERR_UNSUPPORTED, "src blocks must be contiguous");
+    if (s == MI355X_TYPE_Q8_0 || d == MI355X_TYPE_Q8_0) {
+        if (src->ne[0] % FATTN_QK8_0 || dst->ne[0] % FATTN_QK8_0)
+            return fail(MI355X_ERR_INVALID, "Q8_0 copies need ne0 %% 32 == 0 on both sides");
+    }
+    return MI355X_OK;
+}
+
+int mi355x_cpy_supports(const mi355x_tensor * src, const mi355x_tensor * dst) { return cpy_check(src, dst); }
+
+int mi355x_cpy(const mi355x_tensor * src, const mi355x_tensor * dst, void * stream) {
+    const int rc = cpy_check(src, dst);
+    if (rc) return rc;
+    CpyArgs a;
+    memset(&a, 0, sizeof(a));
+    a.src = (const char *)src->data;
+    a.dst = (char *)dst->data;
+    int64_t n = 1;
+    for (int i = 0; i < 4; i++) {
+        a.sne[i] = src->ne[i]; a.dne[i] = dst->ne[i];
+        a.snb[i] = (int64_t)src->nb[i]; a.dnb[i] = (int64_t)dst->nb[i];
+        n *= src->ne[i];
+    }
+    const bool blocks = src->type == MI355X_TYPE_Q8_0 || dst->type == MI355X_TYPE_Q8_0;
+    a.n = blocks ? n / FATTN_QK8_0 : n;
+    if (a.n == 0) return MI355X_OK;
+    if (!a.src || !a.dst) return fail(MI355X_ERR_INVALID, "null data pointer");
+    if (a.n > ((int64_t)1 << 38)) return fail(MI355X_ERR_UNSUPPORTED, "copy too large");
+    const int e = cpy_launch(a, src->type, dst->type, (hipStream_t)stream);
+    if (e) return hip_fail((hipError_t)e, "cpy launch");
+    return MI355X_OK;
+}
+
+int mi355x_set_rows(const mi355x_tensor * src, const void * idx, int32_t idx_type,
+                    const int64_t idx_ne[3], const size_t idx_nb[3],
+                    const mi355x_tensor * dst, void * stream) {
+    if (!src || !dst || !idx_ne || !idx_nb) return fail(MI355X_ERR_INVALID, "null argument");
+    if (src->type != MI355X_TYPE_F32) return fail(MI355X_ERR_UNSUPPORTED, "set_rows source must be F32");
+    if (!type_size(dst->type)) return fail(MI355X_ERR_UNSUPPORTED, "set_rows destination type %d", dst->type);
+    if (idx_type != 64 && idx_type != 32) return fail(MI355X_ERR_INVALID, "index type must be 32 or 64");
+    if (src->ne[0] != dst->ne[0] || src->ne[2] != dst->ne[2] || src->ne[3] != dst->ne[3])
+        return fail(MI355X_ERR_INVALID, "set_rows shapes do not match");
+    if (idx_ne[0] != src->ne[1] || idx_ne[1] <= 0 || idx_ne[2] <= 0 || src->ne[2] % idx_ne[1] || src->ne[3] % idx_ne[2])
+        return fail(MI355X_ERR_INVALID, "set_rows index shape does not match");
+    if (dst->nb[0] != type_size(dst->type)) return fail(MI355X_ERR_UNSUPPORTED, "dst rows must be contiguous");
+    if (dst->type == MI355X_TYPE_Q8_0 && src->ne[0] % FATTN_QK8_0) return fail(MI355X_ERR_INVALID, "Q8_0 rows need ne0 %% 32 == 0");
+    CpyArgs a;
+    memset(&a, 0, sizeof(a));
+    a.src = (const char *)src->data;
+    a.dst = (char *)dst->data;
+    a.idx = (const char *)idx;
+    a.idx_is_i64 = idx_type == 64;
+    int64_t n = 1;
+    for (int i = 0; i < 4; i++) {
+        a.sne[i] = src->ne[i]; a.dne[i] = dst->ne[i];
+        a.snb[i] = (int64_t)src->nb[i]; a.dnb[i] = (int64_t)dst->nb[i];
+        n *= src->ne[i];
+    }
+    for (int i = 0; i < 3; i++) { a.ine[i] = idx_ne[i]; a.inb[i] = (int64_t)idx_nb[i]; }
+    a.n = dst->type == MI355X_TYPE_Q8_0 ? n / FATTN_QK8_0 : n;
+    if (a.n == 0) return MI355X_OK;
+    if (!a.src || !a.dst || !a.idx) return fail(MI355X_ERR_INVALID, "null data pointer");
+    const int e = set_rows_launch(a, dst->type, (hipStream_t)stream);
+    if (e) return hip_fail((hipError_t)e, "set_rows launch");
+    return MI355X_OK;
+}
+
+// ---- buffers -----------------------------------------------------------------------------
+
+int mi355x_buffer_alloc(size_t size, void ** ptr) {
+    if (!ptr) return fail(MI355X_ERR_INVALID, "null argument");
+    *ptr = nullptr;
+    HIP_TRY(hipMalloc(ptr, size ? size : 1));
+    return MI355X_OK;
+}
+
+int mi355x_buffer_free(void * ptr) {
+    if (ptr) HIP_TRY(hipFree(ptr));
+    return MI355X_OK;
+}
+
+int mi355x_buffer_memset(void * ptr, int value, size_t size, void * stream) {
+    if (size == 0) return MI355X_OK;
+    HIP_TRY(hipMemsetAsync(ptr, value, size, (hipStream_t)stream));
+    return MI355X_OK;
+}
+
+int mi355x_buffer_set(void * dst, const void * host_src, size_t size, void * stream) {
+    if (size == 0) return MI355X_OK;
+    HIP_TRY(hipMemcpyAsync(dst, host_src, size, hipMemcpyHostToDevice, (hipStream_t)stream));
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return MI355X_OK;
+}
+
+int mi355x_buffer_get(void * host_dst, const void * src, size_t size, void * stream) {
+    if (size == 0) return MI355X_OK;
+    HIP_TRY(hipMemcpyAsync(host_dst, src, size, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    return MI355X_OK;
+}
+
+int mi355x_buffer_copy(void * dst, const void * src, size_t size, void * stream) {
+    if (size == 0) return MI355X_OK;
+    HIP_TRY(hipMemcpyAsync(dst, src, size, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+    return MI355X_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,149 @@
+// GGML_OP_CPY / CONT / DUP / SET_ROWS with the destination in device memory: the KV-cache
+// writes that feed FLASH_ATTN_EXT (src/crispasr.cpp:2810-2811, 3185-3203, 2956-2973;
+// src/core/attention.h:342-378) and the dequantising reads (src/core/attention.h:917-920).
+// HBM-bound byte work: one element (or one Q8_0 block of 32) per lane, coalesced along
+// dimension 0.  Source and destination may have different shapes with equal element
+// counts (the reference copies a [n_state, n_ctx] tensor into a 1-D cache view).
+#include "fattn_common.h"
+
+namespace {
+
+// byte offset of unit i, where a unit is `unit0` elements along dimension 0 and one step of
+// nb[0] covers `per_nb0` elements (32 for a Q8_0 tensor, 1 otherwise)
+__device__ __forceinline__ int64_t offset_of(int64_t i, const int64_t (&ne)[4], const int64_t (&nb)[4],
+                                             int64_t unit0, int64_t per_nb0 = 1) {
+    const int64_t n0 = ne[0] / unit0;
+    const int64_t i0 = i % n0;  i /= n0;
+    const int64_t i1 = i % ne[1]; i /= ne[1];
+    const int64_t i2 = i % ne[2];
+    const int64_t i3 = i / ne[2];
+    return i0 * (unit0 / per_nb0) * nb[0] + i1 * nb[1] + i2 * nb[2] + i3 * nb[3];
+}
+
+template <typename TS, typename TD>
+__global__ void __launch_bounds__(256) cpy_scalar_kernel(const CpyArgs a) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= a.n) return;
+    const TS x = *(const TS *)(a.src + offset_of(i, a.sne, a.snb, 1));
+    *(TD *)(a.dst + offset_of(i, a.dne, a.dnb, 1)) = (TD)x;     // f32 -> f16 is round-to-nearest-even
+}
+
+// quantise one block of 32 held one element per lane (32 consecutive lanes):
+// d = amax/127 (f32), q = rne(x * (1/d)), d stored as fp16
+// (called by every lane of the wave: the reduction runs before any divergence)
+__device__ __forceinline__ void quantize_block_store(float x, char * blk, int e, bool ok) {
+    const float amax = group_max<32>(fabsf(x));
+    const float d    = amax / 127.0f;
+    const float id   = d != 0.0f ? 1.0f / d : 0.0f;
+    const int   qi   = (int)rintf(x * id);
+    if (ok) {
+        ((int8_t *)(blk + 2))[e] = (int8_t)qi;
+        if (e == 0) *(_Float16 *)blk = (_Float16)d;
+    }
+}
+
+// F32 -> Q8_0; one block per 32 lanes
+__global__ void __launch_bounds__(256) cpy_f32_q8_0_kernel(const CpyArgs a) {
+    const int64_t blk = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+    const int     e   = threadIdx.x & 31;
+    const bool    ok  = blk < a.n;
+    const int64_t bc  = ok ? blk : 0;                       // keep all lanes in the reduction
+    const char *  sp  = a.src + offset_of(bc, a.sne, a.snb, FATTN_QK8_0) + e * a.snb[0];
+    const float   x   = ok ? *(const float *)sp : 0.0f;
+    char * dp = a.dst + offset_of(bc, a.dne, a.dnb, FATTN_QK8_0, FATTN_QK8_0);
+    quantize_block_store(x, dp, e, ok);
+}
+
+// Q8_0 -> F32; one block per 32 lanes
+__global__ void __launch_bounds__(256) cpy_q8_0_f32_kernel(const CpyArgs a) {
+    const int64_t blk = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+    const int     e   = threadIdx.x & 31;
+    if (blk >= a.n) return;
+    const char * sp = a.src + offset_of(blk, a.sne, a.snb, FATTN_QK8_0, FATTN_QK8_0);
+    const float  d  = h2f_bits(*(const uint16_t *)sp);
+    const float  x  = (float)((const int8_t *)(sp + 2))[e] * d;
+    char * dp = a.dst + offset_of(blk, a.dne, a.dnb, FATTN_QK8_0) + e * a.dnb[0];
+    *(float *)dp = x;
+}
+
+// Q8_0 -> Q8_0: move 34-byte blocks as 17 halfwords
+__global__ void __launch_bounds__(256) cpy_q8_0_q8_0_kernel(const CpyArgs a) {
+    const int64_t t   = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t blk = t / 17;
+    const int     w   = (int)(t % 17);
+    if (blk >= a.n) return;
+    const uint16_t * sp = (const uint16_t *)(a.src + offset_of(blk, a.sne, a.snb, FATTN_QK8_0, FATTN_QK8_0));
+    uint16_t *       dp = (uint16_t *)(a.dst + offset_of(blk, a.dne, a.dnb, FATTN_QK8_0, FATTN_QK8_0));
+    dp[w] = sp[w];
+}
+
+// SET_ROWS: dst[:, idx[i1, i2 % ine1, i3 % ine2], i2, i3] = convert(src[:, i1, i2, i3]), src F32
+template <int DTYPE>
+__global__ void __launch_bounds__(256) set_rows_kernel(const CpyArgs a) {
+    // one unit = 32 elements of a source row (Q8_0) or 1 element (F16/F32)
+    constexpr int UNIT = DTYPE == MI355X_TYPE_Q8_0 ? FATTN_QK8_0 : 1;
+    int64_t u;
+    int     e = 0;
+    if (UNIT == 1) {
+        u = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    } else {
+        u = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
+        e = threadIdx.x & 31;
+    }
+    const bool ok = u < a.n;
+    int64_t    r  = ok ? u : 0;
+    const int64_t n0 = a.sne[0] / UNIT;
+    const int64_t i0 = r % n0;      r /= n0;
+    const int64_t i1 = r % a.sne[1]; r /= a.sne[1];
+    const int64_t i2 = r % a.sne[2];
+    const int64_t i3 = r / a.sne[2];
+    const char * ip = a.idx + i1 * a.inb[0] + (i2 % a.ine[1]) * a.inb[1] + (i3 % a.ine[2]) * a.inb[2];
+    const int64_t drow = a.idx_is_i64 ? *(const int64_t *)ip : (int64_t)*(const int32_t *)ip;
+    const char * sp = a.src + (i0 * UNIT + e) * a.snb[0] + i1 * a.snb[1] + i2 * a.snb[2] + i3 * a.snb[3];
+    const float  x  = ok ? *(const float *)sp : 0.0f;
+    char * dp = a.dst + i0 * a.dnb[0] + drow * a.dnb[1] + i2 * a.dnb[2] + i3 * a.dnb[3];
+    if (DTYPE == MI355X_TYPE_Q8_0) {
+        quantize_block_store(x, dp, e, ok);
+    } else if (ok) {
+        if (DTYPE == MI355X_TYPE_F16) *(_Float16 *)dp = (_Float16)x;
+        else                          *(float *)dp = x;
+    }
+}
+
+}  // namespace
+
+int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream) {
+    if (a.n == 0) return 0;
+    const unsigned g256 = (unsigned)((a.n + 255) / 256);
+    const unsigned g8   = (unsigned)((a.n + 7) / 8);
+    if (stype == MI355X_TYPE_F32 && dtype == MI355X_TYPE_F32)
+        hipLaunchKernelGGL((cpy_scalar_kernel<float, float>), dim3(g256), dim3(256), 0, stream, a);
+    else if (stype == MI355X_TYPE_F32 && dtype == MI355X_TYPE_F16)
+        hipLaunchKernelGGL((cpy_scalar_kernel<float, _Float16>), dim3(g256), dim3(256), 0, stream, a);
+    else if (stype == MI355X_TYPE_F16 && dtype == MI355X_TYPE_F16)
+        hipLaunchKernelGGL((cpy_scalar_kernel<_Float16, _Float16>), dim3(g256), dim3(256), 0, stream, a);
+    else if (stype == MI355X_TYPE_F16 && dtype == MI355X_TYPE_F32)
+        hipLaunchKernelGGL((cpy_scalar_kernel<_Float16, float>), dim3(g256), dim3(256), 0, stream, a);
+    else if (stype == MI355X_TYPE_F32 && dtype == MI355X_TYPE_Q8_0)
+        hipLaunchKernelGGL(cpy_f32_q8_0_kernel, dim3(g8), dim3(256), 0, stream, a);
+    else if (stype == MI355X_TYPE_Q8_0 && dtype == MI355X_TYPE_F32)
+        hipLaunchKernelGGL(cpy_q8_0_f32_kernel, dim3(g8), dim3(256), 0, stream, a);
+    else if (stype == MI355X_TYPE_Q8_0 && dtype == MI355X_TYPE_Q8_0)
+        hipLaunchKernelGGL(cpy_q8_0_q8_0_kernel, dim3((unsigned)((a.n * 17 + 255) / 256)), dim3(256), 0, stream, a);
+    else
+        return (int)hipErrorInvalidValue;
+    return (int)hipGetLastError();
+}
+
+int set_rows_launch(const CpyArgs & a, int dtype, hipStream_t stream) {
+    if (a.n == 0) return 0;
+    if (dtype == MI355X_TYPE_Q8_0)
+        hipLaunchKernelGGL((set_rows_kernel<MI355X_TYPE_Q8_0>), dim3((unsigned)((a.n + 7) / 8)), dim3(256), 0, stream, a);
+    else if (dtype == MI355X_TYPE_F16)
+        hipLaunchKernelGGL((set_rows_kernel<MI355X_TYPE_F16>), dim3((unsigned)((a.n + 255) / 256)), dim3(256), 0, stream, a);
+    else if (dtype == MI355X_TYPE_F32)
+        hipLaunchKernelGGL((set_rows_kernel<MI355X_TYPE_F32>), dim3((unsigned)((a.n + 255) / 256)), dim3(256), 0, stream, a);
+    else
+        return (int)hipErrorInvalidValue;
+    return (int)hipGetLastError();
+}

@@ -1,0 +1,106 @@
+// Shared between the gfx950 attention kernels and their launchers (internal).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mi355x_fattn.h"
+
+#define FATTN_QK8_0 32
+#define FATTN_Q8_0_BYTES 34
+
+// Everything a kernel needs about one FLASH_ATTN_EXT node, by value.
+struct FattnArgs {
+    const char * q;      // F32  [D, Nq, Hq, B]
+    const char * k;      // K/V storage type [D, Nkv, Hkv, Bk]
+    const char * v;
+    const char * mask;   // F16 [>=Nkv, >=Nq, Hm, Bm] or nullptr
+    float *      dst;    // F32 [D, Hq, Nq, B] contiguous
+
+    int32_t D, Nq, Hq, B, Nkv, Hkv, Bk;
+    int32_t gqa;         // Hq / Hkv
+    int32_t bq;          // B / Bk
+    int32_t Hm, Bm;      // mask broadcast extents
+
+    int64_t nbq1, nbq2, nbq3;
+    int64_t nbk1, nbk2, nbk3;
+    int64_t nbv1, nbv2, nbv3;
+    int64_t nbm1, nbm2, nbm3;
+
+    float scale;         // already divided by logit_softcap when that is non-zero
+    float softcap;
+    float max_bias, m0, m1;
+    int32_t n_head_log2;
+
+    int32_t aligned16;   // q/k/v/mask bases and strides are all multiples of 16 bytes
+
+    // split-KV
+    int32_t n_splits;
+    int32_t keys_per_split;
+    float * part_acc;    // [rows, n_splits, D]  unnormalised accumulators
+    float * part_ml;     // [rows, n_splits, 2]  running max, running sum
+};
+
+static __device__ __forceinline__ float fattn_slope(const FattnArgs & a, int h) {
+    if (a.max_bias <= 0.0f) return 1.0f;
+    return h < a.n_head_log2 ? powf(a.m0, (float)(h + 1)) : powf(a.m1, (float)(2 * (h - a.n_head_log2) + 1));
+}
+
+static __device__ __forceinline__ float h2f_bits(uint16_t h) {
+    return (float)__builtin_bit_cast(_Float16, h);
+}
+
+// ---- DPP wavefront reductions -------------------------------------------------------
+// Butterfly sums over aligned groups of lanes; every lane of a group ends with the total.
+template <int CTRL>
+static __device__ __forceinline__ float dpp_mov(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+
+static __device__ __forceinline__ float xor_shuffle(float x, int mask) {
+    return __shfl_xor(x, mask, 64);
+}
+
+template <int GROUP>
+static __device__ __forceinline__ float group_sum(float x) {
+    static_assert(GROUP == 4 || GROUP == 8 || GROUP == 16 || GROUP == 32 || GROUP == 64, "group size");
+    x += dpp_mov<0xB1>(x);                        // quad_perm [1,0,3,2]
+    x += dpp_mov<0x4E>(x);                        // quad_perm [2,3,0,1]
+    if (GROUP >= 8)  x += dpp_mov<0x141>(x);      // row_half_mirror: pairs the two quads of 8 lanes
+    if (GROUP >= 16) x += dpp_mov<0x140>(x);      // row_mirror: pairs the two halves of a row of 16
+    if (GROUP >= 32) x += xor_shuffle(x, 16);
+    if (GROUP >= 64) x += xor_shuffle(x, 32);
+    return x;
+}
+
+template <int GROUP>
+static __device__ __forceinline__ float group_max(float x) {
+    x = fmaxf(x, dpp_mov<0xB1>(x));
+    x = fmaxf(x, dpp_mov<0x4E>(x));
+    if (GROUP >= 8)  x = fmaxf(x, dpp_mov<0x141>(x));
+    if (GROUP >= 16) x = fmaxf(x, dpp_mov<0x140>(x));
+    if (GROUP >= 32) x = fmaxf(x, xor_shuffle(x, 16));
+    if (GROUP >= 64) x = fmaxf(x, xor_shuffle(x, 32));
+    return x;
+}
+
+// One CPY / SET_ROWS node.
+struct CpyArgs {
+    const char * src;
+    char *       dst;
+    int64_t sne[4], dne[4];
+    int64_t snb[4], dnb[4];
+    int64_t n;                 // elements (or blocks of 32 when a side is Q8_0)
+    // SET_ROWS only
+    const char * idx;
+    int32_t idx_is_i64;
+    int64_t ine[3], inb[3];
+};
+
+// Launchers implemented next to their kernels; all return hipError_t as int.
+int fattn_vec_launch(const FattnArgs & a, int ktype, hipStream_t stream);
+int fattn_merge_launch(const FattnArgs & a, hipStream_t stream);
+int fattn_mma_launch(const FattnArgs & a, int ktype, hipStream_t stream);
+bool fattn_mma_supported(const FattnArgs & a, int ktype);
+int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream);
+int set_rows_launch(const CpyArgs & a, int dtype, hipStream_t stream);

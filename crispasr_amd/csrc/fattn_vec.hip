@@ -1,0 +1,285 @@
+// Split-KV vector attention kernel for gfx950 (wave64) and the merge of its partials.
+//
+// One workgroup (4 waves) owns one query row (query, head, batch) and one KV split.
+// A row of K or V is spread over LPR lanes, 8 elements (one 128-bit load for f16) per
+// lane, so a wave reads 64/LPR whole rows per load instruction - contiguous 128- or
+// 256-byte segments.  Each group of LPR lanes keeps its own online-softmax state
+// (m, l, acc[8] per lane) over the keys it visits; the dot products are reduced across
+// the group with DPP butterflies.  Groups are merged with cross-lane shuffles, waves
+// through LDS, and splits by fattn_merge_kernel.
+//
+// Semantics follow GGML_OP_FLASH_ATTN_EXT as the reference's call sites use it
+// (src/crispasr.cpp:3208-3222, 3269-3282; src/core/attention.h:992; src/canary.cpp:966-972):
+// s = scale*<q,k> [soft-capped] + slope*mask, -inf mask entries exclude a key, GQA by
+// h / (Hq/Hkv), mask broadcast by h % Hm and b % Bm, output [D, Hq, Nq, B].
+#include "fattn_common.h"
+
+namespace {
+
+constexpr int VEC_WAVES   = 4;
+constexpr int VEC_THREADS = VEC_WAVES * 64;
+constexpr int VEC_UNROLL  = 4;
+
+// 8 consecutive elements of a K/V row starting at element d0, as f32 (exact for all types)
+template <int TYPE>
+__device__ __forceinline__ void load8(const char * row, int d0, bool aligned16, float (&out)[8]) {
+    if (TYPE == MI355X_TYPE_F16) {
+        const char * p = row + (size_t)d0 * 2;
+        if (aligned16) {
+            const uint4 u = *(const uint4 *)p;
+            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                out[2 * i]     = h2f_bits((uint16_t)(w[i] & 0xffffu));
+                out[2 * i + 1] = h2f_bits((uint16_t)(w[i] >> 16));
+            }
+        } else {
+            const uint16_t * h = (const uint16_t *)p;
+#pragma unroll
+            for (int i = 0; i < 8; i++) out[i] = h2f_bits(h[i]);
+        }
+    } else if (TYPE == MI355X_TYPE_F32) {
+        const char * p = row + (size_t)d0 * 4;
+        if (aligned16) {
+            const float4 a = *(const float4 *)p;
+            const float4 b = *(const float4 *)(p + 16);
+            out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
+            out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
+        } else {
+            const float * f = (const float *)p;
+#pragma unroll
+            for (int i = 0; i < 8; i++) out[i] = f[i];
+        }
+    } else {  // Q8_0: block = fp16 d + 32 int8; blocks are only 2-byte aligned
+        const char * blk = row + (size_t)(d0 / FATTN_QK8_0) * FATTN_Q8_0_BYTES;
+        const float  d   = h2f_bits(*(const uint16_t *)blk);
+        const uint16_t * qs = (const uint16_t *)(blk + 2 + (d0 % FATTN_QK8_0));
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint16_t w = qs[i];
+            out[2 * i]     = (float)(int8_t)(w & 0xff) * d;
+            out[2 * i + 1] = (float)(int8_t)(w >> 8) * d;
+        }
+    }
+}
+
+struct Partial {
+    float m, l;
+    float acc[8];
+};
+
+__device__ __forceinline__ void merge_partial(Partial & a, const Partial & b) {
+    const float mn = fmaxf(a.m, b.m);
+    // a state that has seen no key has m = -inf and l = 0: its factor must be 0, not NaN
+    const float fa = a.m == -INFINITY ? 0.0f : __expf(a.m - mn);
+    const float fb = b.m == -INFINITY ? 0.0f : __expf(b.m - mn);
+    a.l = a.l * fa + b.l * fb;
+#pragma unroll
+    for (int e = 0; e < 8; e++) a.acc[e] = a.acc[e] * fa + b.acc[e] * fb;
+    a.m = mn;
+}
+
+template <int TYPE, int LPR>
+__global__ void __launch_bounds__(VEC_THREADS) fattn_vec_kernel(const FattnArgs a) {
+    constexpr int G = 64 / LPR;                 // key rows per wave per load
+    const int tid  = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int grp  = lane / LPR;
+    const int lig  = lane % LPR;                // lane in group
+    const int d0   = lig * 8;
+    const bool dvalid = d0 < a.D;               // D is a multiple of 8
+    const int d0c  = dvalid ? d0 : 0;
+
+    // blockIdx.x = row * n_splits + split, row = (b*Nq + iq1)*Hq + h  (the dst row order)
+    const int split = blockIdx.x % a.n_splits;
+    const int row   = blockIdx.x / a.n_splits;
+    const int h     = row % a.Hq;
+    const int iq1   = (row / a.Hq) % a.Nq;
+    const int b     = row / (a.Hq * a.Nq);
+    const int hk    = h / a.gqa;
+    const int bk    = b / a.bq;
+
+    const int k_begin = split * a.keys_per_split;
+    const int k_end   = min(a.Nkv, k_begin + a.keys_per_split);
+
+    float q[8];
+    {
+        const float * qrow = (const float *)(a.q + iq1 * a.nbq1 + h * a.nbq2 + b * a.nbq3);
+#pragma unroll
+        for (int e = 0; e < 8; e++) q[e] = dvalid ? qrow[d0 + e] : 0.0f;
+    }
+    const char * kbase = a.k + hk * a.nbk2 + bk * a.nbk3;
+    const char * vbase = a.v + hk * a.nbv2 + bk * a.nbv3;
+    const uint16_t * mrow = a.mask
+        ? (const uint16_t *)(a.mask + iq1 * a.nbm1 + (h % a.Hm) * a.nbm2 + (b % a.Bm) * a.nbm3)
+        : nullptr;
+    const float slope = fattn_slope(a, h);
+    const bool  al    = a.aligned16 != 0;
+
+    Partial st;
+    st.m = -INFINITY;
+    st.l = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) st.acc[e] = 0.0f;
+
+    // every lane runs the same trip count so that the DPP reductions see full groups
+    const int stride = VEC_WAVES * G * VEC_UNROLL;
+    for (int j0 = k_begin; j0 < k_end; j0 += stride) {
+        float kf[VEC_UNROLL][8];
+        float vf[VEC_UNROLL][8];
+        float s[VEC_UNROLL];
+        int   jj[VEC_UNROLL];
+#pragma unroll
+        for (int u = 0; u < VEC_UNROLL; u++) {
+            jj[u] = j0 + (u * VEC_WAVES + wave) * G + grp;
+            const int jc = min(jj[u], k_end - 1);
+            load8<TYPE>(kbase + (size_t)jc * a.nbk1, d0c, al, kf[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < VEC_UNROLL; u++) {
+            const int jc = min(jj[u], k_end - 1);
+            load8<TYPE>(vbase + (size_t)jc * a.nbv1, d0c, al, vf[u]);
+        }
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < VEC_UNROLL; u++) {
+            float dot = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) dot = fmaf(q[e], kf[u][e], dot);
+            dot = group_sum<LPR>(dot);
+            float sc = dot * a.scale;
+            if (a.softcap != 0.0f) sc = a.softcap * tanhf(sc);
+            if (mrow) {
+                const int jc = min(jj[u], k_end - 1);
+                sc += slope * h2f_bits(mrow[jc]);
+            }
+            if (jj[u] >= k_end) sc = -INFINITY;
+            s[u] = sc;
+            mloc = fmaxf(mloc, sc);
+        }
+        if (mloc > st.m) {                       // uniform within a group
+            const float alpha = __expf(st.m - mloc);   // exp(-inf) = 0 on the first hit
+            st.l *= alpha;
+#pragma unroll
+            for (int e = 0; e < 8; e++) st.acc[e] *= alpha;
+            st.m = mloc;
+        }
+        if (st.m > -INFINITY) {
+#pragma unroll
+            for (int u = 0; u < VEC_UNROLL; u++) {
+                const float p = __expf(s[u] - st.m);   // 0 for excluded keys
+                st.l += p;
+#pragma unroll
+                for (int e = 0; e < 8; e++) st.acc[e] = fmaf(p, vf[u][e], st.acc[e]);
+            }
+        }
+    }
+
+    // merge the G groups of this wave (lanes with equal lig)
+#pragma unroll
+    for (int off = LPR; off < 64; off <<= 1) {
+        Partial o;
+        o.m = xor_shuffle(st.m, off);
+        o.l = xor_shuffle(st.l, off);
+#pragma unroll
+        for (int e = 0; e < 8; e++) o.acc[e] = xor_shuffle(st.acc[e], off);
+        merge_partial(st, o);
+    }
+
+    // merge the waves through LDS
+    __shared__ float sh[VEC_WAVES][LPR][10];
+    if (lane < LPR) {
+        sh[wave][lane][0] = st.m;
+        sh[wave][lane][1] = st.l;
+#pragma unroll
+        for (int e = 0; e < 8; e++) sh[wave][lane][2 + e] = st.acc[e];
+    }
+    __syncthreads();
+    if (wave == 0 && lane < LPR) {
+#pragma unroll
+        for (int w = 1; w < VEC_WAVES; w++) {
+            Partial o;
+            o.m = sh[w][lane][0];
+            o.l = sh[w][lane][1];
+#pragma unroll
+            for (int e = 0; e < 8; e++) o.acc[e] = sh[w][lane][2 + e];
+            merge_partial(st, o);
+        }
+        if (dvalid) {
+            if (a.n_splits == 1) {
+                const float inv = st.l > 0.0f ? 1.0f / st.l : 0.0f;
+                float * out = a.dst + (size_t)row * a.D + d0;
+#pragma unroll
+                for (int e = 0; e < 8; e++) out[e] = st.acc[e] * inv;
+            } else {
+                float * pa = a.part_acc + ((size_t)row * a.n_splits + split) * a.D + d0;
+#pragma unroll
+                for (int e = 0; e < 8; e++) pa[e] = st.acc[e];
+                if (lane == 0) {
+                    float * pm = a.part_ml + ((size_t)row * a.n_splits + split) * 2;
+                    pm[0] = st.m;
+                    pm[1] = st.l;
+                }
+            }
+        }
+    }
+}
+
+// out[row] = sum_s acc_s * exp(m_s - M) / sum_s l_s * exp(m_s - M)
+__global__ void __launch_bounds__(256) fattn_merge_kernel(const FattnArgs a, int rows) {
+    const int rows_per_block = 256 / 64;
+    const int row = blockIdx.x * rows_per_block + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int lane = threadIdx.x & 63;
+    const float * pm = a.part_ml + (size_t)row * a.n_splits * 2;
+    float M = -INFINITY;
+    for (int s = 0; s < a.n_splits; s++) M = fmaxf(M, pm[2 * s]);
+    float L = 0.0f;
+    for (int s = 0; s < a.n_splits; s++) {
+        const float m = pm[2 * s];
+        L += m == -INFINITY ? 0.0f : pm[2 * s + 1] * __expf(m - M);
+    }
+    const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+    for (int d = lane; d < a.D; d += 64) {
+        float acc = 0.0f;
+        for (int s = 0; s < a.n_splits; s++) {
+            const float m = pm[2 * s];
+            if (m != -INFINITY) {
+                acc += a.part_acc[((size_t)row * a.n_splits + s) * a.D + d] * __expf(m - M);
+            }
+        }
+        a.dst[(size_t)row * a.D + d] = acc * inv;
+    }
+}
+
+template <int TYPE>
+int launch_typed(const FattnArgs & a, hipStream_t stream) {
+    const int64_t rows = (int64_t)a.Nq * a.Hq * a.B;
+    const dim3 grid((unsigned)(rows * a.n_splits));
+    const dim3 block(VEC_THREADS);
+    const int  lanes = (a.D + 7) / 8;
+    if (lanes <= 4)       hipLaunchKernelGGL((fattn_vec_kernel<TYPE, 4>),  grid, block, 0, stream, a);
+    else if (lanes <= 8)  hipLaunchKernelGGL((fattn_vec_kernel<TYPE, 8>),  grid, block, 0, stream, a);
+    else if (lanes <= 16) hipLaunchKernelGGL((fattn_vec_kernel<TYPE, 16>), grid, block, 0, stream, a);
+    else                  hipLaunchKernelGGL((fattn_vec_kernel<TYPE, 32>), grid, block, 0, stream, a);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+int fattn_vec_launch(const FattnArgs & a, int ktype, hipStream_t stream) {
+    switch (ktype) {
+        case MI355X_TYPE_F16:  return launch_typed<MI355X_TYPE_F16>(a, stream);
+        case MI355X_TYPE_F32:  return launch_typed<MI355X_TYPE_F32>(a, stream);
+        case MI355X_TYPE_Q8_0: return launch_typed<MI355X_TYPE_Q8_0>(a, stream);
+        default:               return (int)hipErrorInvalidValue;
+    }
+}
+
+int fattn_merge_launch(const FattnArgs & a, hipStream_t stream) {
+    const int rows = a.Nq * a.Hq * a.B;
+    const dim3 grid((unsigned)((rows + 3) / 4));
+    hipLaunchKernelGGL(fattn_merge_kernel, grid, dim3(256), 0, stream, a, rows);
+    return (int)hipGetLastError();
+}

@@ -1,0 +1,309 @@
+"""Host-side mirror of the ggml operator interface for the attention path.
+
+``Tensor`` carries what a ``ggml_tensor`` carries for this path - type, ``ne`` (elements
+per dimension, dimension 0 fastest), ``nb`` (byte strides), a byte offset into a device
+buffer - and ``flash_attn_ext`` / ``cpy`` / ``set_rows`` take the same arguments, with the
+same meaning and the same contract checks, as ``ggml_flash_attn_ext`` (call sites:
+src/crispasr.cpp:2821, 3220, 3280; src/core/attention.h:992; src/core/fastconformer.h:924-934),
+``ggml_cpy`` (src/crispasr.cpp:2810-2811) and ``ggml_set_rows`` (src/core/attention.h:366-376)
+in the reference.  All arithmetic happens in libmi355x_fattn.so; torch only owns the device
+memory and the stream.  There is no CPU fallback: without the built library every op raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional, Sequence
+
+import numpy as np
+import torch
+
+F32, F16, Q8_0 = 0, 1, 8
+QK8_0 = 32
+TYPE_SIZE = {F32: 4, F16: 2, Q8_0: 34}
+BLOCK_SIZE = {F32: 1, F16: 1, Q8_0: QK8_0}
+
+KERNEL_AUTO, KERNEL_VEC, KERNEL_MMA, KERNEL_DECODE_MMA = 0, 1, 2, 3
+PREC_DEFAULT, PREC_F32 = 0, 10
+
+OK, ERR_UNSUPPORTED, ERR_INVALID, ERR_HIP, ERR_NO_DEVICE, ERR_WORKSPACE = range(6)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmi355x_fattn.so")
+
+
+class Mi355xError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"mi355x status {status}: {message}")
+        self.status = status
+
+
+class UnsupportedError(Mi355xError):
+    """The op is valid but outside the kernels' coverage (a backend would route it to CPU)."""
+
+
+class InvalidError(Mi355xError, ValueError):
+    """The arguments break the op's contract (ggml would assert)."""
+
+
+class CTensor(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("type", ctypes.c_int32),
+                ("ne", ctypes.c_int64 * 4), ("nb", ctypes.c_size_t * 4)]
+
+
+class CParams(ctypes.Structure):
+    _fields_ = [("scale", ctypes.c_float), ("max_bias", ctypes.c_float), ("logit_softcap", ctypes.c_float),
+                ("prec", ctypes.c_int32), ("kernel", ctypes.c_int32), ("n_splits", ctypes.c_int32),
+                ("workspace", ctypes.c_void_p), ("workspace_size", ctypes.c_size_t)]
+
+
+class CDeviceInfo(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char * 128), ("arch", ctypes.c_char * 32),
+                ("compute_units", ctypes.c_int32), ("clock_khz", ctypes.c_int32),
+                ("memory_clock_khz", ctypes.c_int32), ("memory_bus_bits", ctypes.c_int32),
+                ("total_memory", ctypes.c_uint64), ("free_memory", ctypes.c_uint64),
+                ("lds_bytes_per_block", ctypes.c_int32), ("wavefront_size", ctypes.c_int32)]
+
+
+# every symbol include/mi355x_fattn.h declares
+EXPORTS = [
+    "mi355x_api_version", "mi355x_status_string", "mi355x_last_error",
+    "mi355x_device_count", "mi355x_device_get_info", "mi355x_set_device", "mi355x_stream_synchronize",
+    "mi355x_fattn_supports", "mi355x_flash_attn_ext", "mi355x_fattn_workspace_size", "mi355x_fattn_plan",
+    "mi355x_cpy_supports", "mi355x_cpy", "mi355x_set_rows",
+    "mi355x_buffer_alloc", "mi355x_buffer_free", "mi355x_buffer_memset", "mi355x_buffer_set",
+    "mi355x_buffer_get", "mi355x_buffer_copy",
+]
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """The C-ABI library; raises when it has not been built (no fallback exists)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+                "(hipcc, --offload-arch=gfx950). There is no CPU fallback for this path.")
+        L = ctypes.CDLL(LIB_PATH)
+        PT, PP = ctypes.POINTER(CTensor), ctypes.POINTER(CParams)
+        L.mi355x_api_version.restype = ctypes.c_int
+        L.mi355x_status_string.restype = ctypes.c_char_p
+        L.mi355x_status_string.argtypes = [ctypes.c_int]
+        L.mi355x_last_error.restype = ctypes.c_char_p
+        L.mi355x_device_count.argtypes = [ctypes.POINTER(ctypes.c_int)]
+        L.mi355x_device_get_info.argtypes = [ctypes.c_int, ctypes.POINTER(CDeviceInfo)]
+        L.mi355x_set_device.argtypes = [ctypes.c_int]
+        L.mi355x_stream_synchronize.argtypes = [ctypes.c_void_p]
+        L.mi355x_fattn_supports.argtypes = [PT, PT, PT, PT, PT, PP]
+        L.mi355x_flash_attn_ext.argtypes = [PT, PT, PT, PT, PT, PP, ctypes.c_void_p]
+        L.mi355x_fattn_workspace_size.argtypes = [PT, PT, PT, PT, PP, ctypes.POINTER(ctypes.c_size_t)]
+        L.mi355x_fattn_plan.argtypes = [PT, PT, PT, PT, PP, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]
+        L.mi355x_cpy_supports.argtypes = [PT, PT]
+        L.mi355x_cpy.argtypes = [PT, PT, ctypes.c_void_p]
+        L.mi355x_set_rows.argtypes = [PT, ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_int64),
+                                      ctypes.POINTER(ctypes.c_size_t), PT, ctypes.c_void_p]
+        L.mi355x_buffer_alloc.argtypes = [ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]
+        L.mi355x_buffer_free.argtypes = [ctypes.c_void_p]
+        L.mi355x_buffer_memset.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p]
+        L.mi355x_buffer_set.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        L.mi355x_buffer_get.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        L.mi355x_buffer_copy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        for name in EXPORTS:
+            fn = getattr(L, name)
+            if name not in ("mi355x_status_string", "mi355x_last_error"):
+                fn.restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+def _check(status: int) -> None:
+    if status == OK:
+        return
+    msg = lib().mi355x_last_error().decode(errors="replace")
+    if status == ERR_UNSUPPORTED:
+        raise UnsupportedError(status, msg)
+    if status == ERR_INVALID:
+        raise InvalidError(status, msg)
+    raise Mi355xError(status, msg)
+
+
+def row_size(type_: int, ne0: int) -> int:
+    """ggml_row_size"""
+    return TYPE_SIZE[type_] * (ne0 // BLOCK_SIZE[type_])
+
+
+def contiguous_nb(type_: int, ne: Sequence[int]) -> tuple:
+    nb1 = row_size(type_, ne[0])
+    return (TYPE_SIZE[type_], nb1, nb1 * ne[1], nb1 * ne[1] * ne[2])
+
+
+class Tensor:
+    """A ggml tensor (or view) living in a device buffer."""
+
+    def __init__(self, buf: Optional[torch.Tensor], type_: int, ne: Sequence[int],
+                 nb: Optional[Sequence[int]] = None, offset: int = 0):
+        self.buf = buf                      # 1-D uint8 device tensor, or None (planning only)
+        self.type = int(type_)
+        self.ne = tuple(int(x) for x in ne) + (1,) * (4 - len(ne))
+        self.nb = tuple(int(x) for x in (nb if nb is not None else contiguous_nb(self.type, self.ne)))
+        self.offset = int(offset)
+        if buf is not None:
+            assert buf.dtype == torch.uint8 and buf.dim() == 1 and buf.is_contiguous()
+
+    # -- construction ---------------------------------------------------------------------
+    @staticmethod
+    def empty(type_: int, ne: Sequence[int], device="cuda") -> "Tensor":
+        """ggml_new_tensor + allocation in a device buffer"""
+        ne4 = tuple(int(x) for x in ne) + (1,) * (4 - len(ne))
+        nbytes = row_size(type_, ne4[0]) * ne4[1] * ne4[2] * ne4[3]
+        return Tensor(torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device), type_, ne4)
+
+    @staticmethod
+    def from_host(raw: np.ndarray, type_: int, ne, nb=None, offset: int = 0, device="cuda") -> "Tensor":
+        """ggml_backend_tensor_set of a whole buffer; the view (ne, nb, offset) is kept as is"""
+        raw = np.ascontiguousarray(raw).view(np.uint8).reshape(-1)
+        buf = torch.from_numpy(raw.copy()).to(device)
+        if buf.numel() == 0:
+            buf = torch.zeros(1, dtype=torch.uint8, device=device)
+        return Tensor(buf, type_, ne, nb, offset)
+
+    def view(self, ne, nb, offset: int = 0, type_: Optional[int] = None) -> "Tensor":
+        """ggml_view_{1,2,3,4}d: same buffer, new extents/strides, offset relative to this view"""
+        return Tensor(self.buf, self.type if type_ is None else type_, ne, nb, self.offset + offset)
+
+    # -- access -----------------------------------------------------------------------------
+    def span(self) -> int:
+        if any(n == 0 for n in self.ne):
+            return 0
+        last = (self.ne[0] // BLOCK_SIZE[self.type] - 1) * self.nb[0]
+        last += sum((self.ne[i] - 1) * self.nb[i] for i in (1, 2, 3))
+        return last + TYPE_SIZE[self.type]
+
+    def data_ptr(self) -> int:
+        if self.buf is None:
+            return 0
+        if self.offset + self.span() > self.buf.numel():
+            raise InvalidError(ERR_INVALID, "tensor view exceeds its buffer")
+        return self.buf.data_ptr() + self.offset
+
+    def c(self) -> CTensor:
+        t = CTensor()
+        t.data = self.data_ptr()
+        t.type = self.type
+        t.ne = (ctypes.c_int64 * 4)(*self.ne)
+        t.nb = (ctypes.c_size_t * 4)(*self.nb)
+        return t
+
+    def to_host(self) -> np.ndarray:
+        """ggml_backend_tensor_get of the whole underlying buffer (uint8)"""
+        return self.buf.cpu().numpy()
+
+    def numpy_f32(self) -> np.ndarray:
+        """contiguous F32 tensor -> numpy [ne3, ne2, ne1, ne0]"""
+        assert self.type == F32 and self.nb == contiguous_nb(F32, self.ne)
+        n = self.ne[0] * self.ne[1] * self.ne[2] * self.ne[3]
+        raw = self.buf[self.offset:self.offset + 4 * n].cpu().numpy()
+        return raw.view(np.float32).reshape(self.ne[3], self.ne[2], self.ne[1], self.ne[0]).copy()
+
+
+def _stream_handle(stream) -> int:
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return int(stream.cuda_stream)
+
+
+def _params(scale, max_bias, logit_softcap, prec, kernel, n_splits, workspace) -> CParams:
+    p = CParams()
+    p.scale, p.max_bias, p.logit_softcap = float(scale), float(max_bias), float(logit_softcap)
+    p.prec, p.kernel, p.n_splits = int(prec), int(kernel), int(n_splits)
+    if workspace is not None:
+        p.workspace = workspace.data_ptr()
+        p.workspace_size = workspace.numel() * workspace.element_size()
+    else:
+        p.workspace, p.workspace_size = None, 0
+    return p
+
+
+def _opt(t: Optional[Tensor]):
+    return ctypes.byref(t.c()) if t is not None else None
+
+
+def flash_attn_supports(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor] = None, scale: float = 1.0,
+                        max_bias: float = 0.0, logit_softcap: float = 0.0, prec: int = PREC_DEFAULT) -> int:
+    """What the backend's supports_op asks: OK, ERR_UNSUPPORTED or ERR_INVALID.  Touches no device."""
+    p = _params(scale, max_bias, logit_softcap, prec, KERNEL_AUTO, 0, None)
+    cq, ck, cv = q.c(), k.c(), v.c()
+    cm = mask.c() if mask is not None else None
+    return lib().mi355x_fattn_supports(ctypes.byref(cq), ctypes.byref(ck), ctypes.byref(cv),
+                                       ctypes.byref(cm) if cm is not None else None, None, ctypes.byref(p))
+
+
+def flash_attn_plan(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor] = None, scale: float = 1.0,
+                    max_bias: float = 0.0, logit_softcap: float = 0.0, kernel: int = KERNEL_AUTO,
+                    n_splits: int = 0):
+    p = _params(scale, max_bias, logit_softcap, PREC_DEFAULT, kernel, n_splits, None)
+    cq, ck, cv = q.c(), k.c(), v.c()
+    cm = mask.c() if mask is not None else None
+    kern, ns = ctypes.c_int32(0), ctypes.c_int32(0)
+    _check(lib().mi355x_fattn_plan(ctypes.byref(cq), ctypes.byref(ck), ctypes.byref(cv),
+                                   ctypes.byref(cm) if cm is not None else None, ctypes.byref(p),
+                                   ctypes.byref(kern), ctypes.byref(ns)))
+    return kern.value, ns.value
+
+
+def flash_attn_ext(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor], scale: float,
+                   max_bias: float = 0.0, logit_softcap: float = 0.0, *, prec: int = PREC_DEFAULT,
+                   kernel: int = KERNEL_AUTO, n_splits: int = 0, out: Optional[Tensor] = None,
+                   workspace: Optional[torch.Tensor] = None, stream=None) -> Tensor:
+    """ggml_flash_attn_ext(ctx, q, k, v, mask, scale, max_bias, logit_softcap) computed on the GPU.
+
+    Returns the F32 result tensor with ne = [DV, Hq, Nq, B] (what the reference's callers
+    immediately reshape_2d to [DV*Hq, Nq])."""
+    if out is None:
+        out = Tensor.empty(F32, (v.ne[0], q.ne[2], q.ne[1], q.ne[3]), device=q.buf.device)
+    p = _params(scale, max_bias, logit_softcap, prec, kernel, n_splits, workspace)
+    cq, ck, cv, co = q.c(), k.c(), v.c(), out.c()
+    cm = mask.c() if mask is not None else None
+    with torch.cuda.device(q.buf.device):
+        _check(lib().mi355x_flash_attn_ext(ctypes.byref(cq), ctypes.byref(ck), ctypes.byref(cv),
+                                           ctypes.byref(cm) if cm is not None else None, ctypes.byref(co),
+                                           ctypes.byref(p), _stream_handle(stream)))
+    return out
+
+
+def cpy(src: Tensor, dst: Tensor, stream=None) -> Tensor:
+    """ggml_cpy(ctx, src, dst): convert src's elements into dst's type and layout"""
+    cs, cd = src.c(), dst.c()
+    with torch.cuda.device(dst.buf.device):
+        _check(lib().mi355x_cpy(ctypes.byref(cs), ctypes.byref(cd), _stream_handle(stream)))
+    return dst
+
+
+def set_rows(dst: Tensor, src: Tensor, idx: torch.Tensor, stream=None) -> Tensor:
+    """ggml_set_rows(ctx, dst, src, idx): dst[:, idx[i], ...] = src[:, i, ...]; idx int64/int32 device tensor
+    of shape [n_rows] (or [I2, I1, n_rows] in numpy order, broadcast over dims 2 and 3)"""
+    assert idx.dtype in (torch.int64, torch.int32) and idx.is_contiguous()
+    shape = (1,) * (3 - idx.dim()) + tuple(idx.shape)
+    ine = (ctypes.c_int64 * 3)(shape[2], shape[1], shape[0])
+    es = idx.element_size()
+    inb = (ctypes.c_size_t * 3)(es, es * shape[2], es * shape[2] * shape[1])
+    cs, cd = src.c(), dst.c()
+    with torch.cuda.device(dst.buf.device):
+        _check(lib().mi355x_set_rows(ctypes.byref(cs), idx.data_ptr(), 64 if idx.dtype == torch.int64 else 32,
+                                     ine, inb, ctypes.byref(cd), _stream_handle(stream)))
+    return dst
+
+
+def device_info(device: int = 0) -> dict:
+    info = CDeviceInfo()
+    _check(lib().mi355x_device_get_info(device, ctypes.byref(info)))
+    return {f: (getattr(info, f).decode() if isinstance(getattr(info, f), bytes) else getattr(info, f))
+            for f, _ in CDeviceInfo._fields_}
+
+
+def device_count() -> int:
+    n = ctypes.c_int(0)
+    lib().mi355x_device_count(ctypes.byref(n))
+    return n.value

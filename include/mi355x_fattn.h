@@ -1,0 +1,178 @@
+/*
+ * mi355x_fattn.h - C ABI of the MI355X (gfx950) attention library.
+ *
+ * This is the launcher layer a ggml backend ("ggml-mi355x") binds for
+ * GGML_OP_FLASH_ATTN_EXT and for the tensor copies that op needs.  Plain pointers,
+ * sizes and scalars only: no ggml, HIP or torch types cross this boundary.  All data
+ * pointers are device pointers (hipMalloc / hipMallocManaged / hipHostMalloc-mapped
+ * memory the GPU can address); `stream` is a hipStream_t passed as void* (NULL = the
+ * default stream).  Calls are asynchronous on `stream` unless stated otherwise.
+ *
+ * Every entry point returns an mi355x_status; on a non-zero status
+ * mi355x_last_error() holds a message for the calling thread.
+ *
+ * Reference interfaces replaced (paths relative to the CrispASR tree):
+ *   - the op node built by ggml_flash_attn_ext(ctx, q, k, v, mask, scale, max_bias,
+ *     logit_softcap) at src/crispasr.cpp:2821, :3220, :3280, src/core/attention.h:992,
+ *     src/core/fastconformer.h:924-934, src/core/cross_attn.h:119-153, src/canary.cpp:966-972
+ *     and executed by whichever backend ggml_backend_sched assigned
+ *     (src/crispasr.cpp:256-280 -> ggml_backend_sched_graph_compute);
+ *   - the KV-cache writes ggml_cpy(F32 -> cache view) at src/crispasr.cpp:2810-2811,
+ *     3185-3203, 2956-2973 and src/core/attention.h:342-378;
+ *   - the buffer vtable a backend fills (member order pinned by the reference's own
+ *     initialiser, src/core/gguf_loader.cpp:332-344): memset_tensor / set_tensor /
+ *     get_tensor / cpy_tensor / clear.
+ */
+#ifndef MI355X_FATTN_H
+#define MI355X_FATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355X_FATTN_API_VERSION 1
+
+/* ggml type ids of the storage types this path meets */
+enum mi355x_type {
+    MI355X_TYPE_F32  = 0,
+    MI355X_TYPE_F16  = 1,
+    MI355X_TYPE_Q8_0 = 8   /* blocks of 32: fp16 scale d + 32 x int8, 34 bytes, x = q*d */
+};
+
+enum mi355x_status {
+    MI355X_OK              = 0,
+    MI355X_ERR_UNSUPPORTED = 1,   /* valid op, but outside what these kernels cover: route to CPU */
+    MI355X_ERR_INVALID     = 2,   /* breaks the op's contract (ggml would assert) */
+    MI355X_ERR_HIP         = 3,   /* a HIP runtime call failed */
+    MI355X_ERR_NO_DEVICE   = 4,
+    MI355X_ERR_WORKSPACE   = 5    /* caller-provided workspace too small */
+};
+
+/* The fields of ggml_tensor the kernels read: data, type, ne (elements per dimension,
+ * dimension 0 fastest), nb (byte strides; nb[0] is the element - or block - size). */
+typedef struct mi355x_tensor {
+    void *  data;
+    int32_t type;
+    int64_t ne[4];
+    size_t  nb[4];
+} mi355x_tensor;
+
+enum mi355x_fattn_kernel {
+    MI355X_FATTN_AUTO       = 0,
+    MI355X_FATTN_VEC        = 1,  /* split-KV vector kernel: any supported shape */
+    MI355X_FATTN_MMA        = 2,  /* f16 MFMA tile kernel: prefill / encoder shapes */
+    MI355X_FATTN_DECODE_MMA = 3   /* split-KV MFMA kernel: few query rows per KV head */
+};
+
+/* op_params of the node (scale, max_bias, logit_softcap as f32, prec as i32) plus
+ * launch overrides used by the tests and the benchmark. */
+typedef struct mi355x_fattn_params {
+    float   scale;
+    float   max_bias;
+    float   logit_softcap;
+    int32_t prec;            /* GGML_PREC_DEFAULT = 0, GGML_PREC_F32 = 10; accumulation is f32 either way */
+    int32_t kernel;          /* mi355x_fattn_kernel */
+    int32_t n_splits;        /* 0 = choose; forces the KV split count of the split-KV kernels */
+    void *  workspace;       /* NULL = library-owned scratch (grown with hipMalloc when needed) */
+    size_t  workspace_size;
+} mi355x_fattn_params;
+
+typedef struct mi355x_device_info {
+    char     name[128];
+    char     arch[32];           /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+    int32_t  compute_units;
+    int32_t  clock_khz;
+    int32_t  memory_clock_khz;
+    int32_t  memory_bus_bits;
+    uint64_t total_memory;
+    uint64_t free_memory;
+    int32_t  lds_bytes_per_block;
+    int32_t  wavefront_size;
+} mi355x_device_info;
+
+/* ---- library / device ---------------------------------------------------------------- */
+
+int          mi355x_api_version(void);
+const char * mi355x_status_string(int status);
+const char * mi355x_last_error(void);
+
+/* ggml_backend_reg_i::get_device_count / ggml_backend_device_i::get_props, get_memory */
+int mi355x_device_count(int * count);
+int mi355x_device_get_info(int device, mi355x_device_info * info);
+int mi355x_set_device(int device);
+/* ggml_backend_i::synchronize */
+int mi355x_stream_synchronize(void * stream);
+
+/* ---- GGML_OP_FLASH_ATTN_EXT ------------------------------------------------------------ */
+
+/*
+ * dst[DV, Hq, Nq, B] (f32, contiguous) = softmax(scale * q.k^T [soft-capped] + slope(h) * mask) . v
+ *
+ *   q    F32  [D,  Nq,  Hq,  B ]   any strides with nb[0] == 4
+ *   k    F16 | F32 | Q8_0 [D,  Nkv, Hkv, Bk]   rows contiguous (nb[0] == type size)
+ *   v    same type as k   [DV, Nkv, Hkv, Bk]   DV == D
+ *   mask NULL, or F16 [>=Nkv, >=Nq, Hm, Bm], rows contiguous; head h reads h % Hm,
+ *        batch b reads b % Bm; -inf entries exclude the key
+ *   Hq % Hkv == 0 (query head h reads KV head h / (Hq/Hkv)), B % Bk == 0.
+ *   A row whose keys are all excluded (or Nkv == 0) yields zeros.
+ *   Excluded keys still have to hold finite K/V values (they are multiplied by 0).
+ *
+ * mi355x_fattn_supports is the predicate the backend's supports_op mirrors: it returns
+ * MI355X_OK, MI355X_ERR_UNSUPPORTED or MI355X_ERR_INVALID without touching the device.
+ * Data pointers may be NULL there (graph planning happens before allocation).
+ */
+int mi355x_fattn_supports(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                          const mi355x_tensor * mask, const mi355x_tensor * dst,
+                          const mi355x_fattn_params * params);
+
+int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                          const mi355x_tensor * mask, const mi355x_tensor * dst,
+                          const mi355x_fattn_params * params, void * stream);
+
+/* bytes of scratch the call above would use with these shapes (0 when none) */
+int mi355x_fattn_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                                const mi355x_tensor * mask, const mi355x_fattn_params * params,
+                                size_t * bytes);
+
+/* which kernel and split count AUTO resolves to (for logs, tests and the benchmark) */
+int mi355x_fattn_plan(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                      const mi355x_tensor * mask, const mi355x_fattn_params * params,
+                      int32_t * kernel, int32_t * n_splits);
+
+/* ---- GGML_OP_CPY / CONT / DUP with the destination in a device buffer --------------------- */
+
+/*
+ * dst[i] = convert(src[i]) for tensors of equal ne.  Supported: F32 -> F32 | F16 | Q8_0,
+ * F16 -> F16 | F32, Q8_0 -> F32 | Q8_0.  F32 -> F16 rounds to nearest even; F32 -> Q8_0
+ * uses d = amax/127, q = round-to-nearest-even(x * (1/d)) per block of 32 along
+ * dimension 0.  src may have any strides; dst rows (dimension 0) must be contiguous.
+ */
+int mi355x_cpy_supports(const mi355x_tensor * src, const mi355x_tensor * dst);
+int mi355x_cpy(const mi355x_tensor * src, const mi355x_tensor * dst, void * stream);
+
+/*
+ * GGML_OP_SET_ROWS, the write into a quantised KV cache (src/core/attention.h:366-376):
+ * dst[:, idx[i1, i2 % I1, i3 % I2], i2, i3] = convert(src[:, i1, i2, i3]).
+ * src F32 [n0, n_rows, n2, n3]; idx I64 (idx_type 64) or I32 (idx_type 32) with
+ * ne = {n_rows, I1, I2} and byte strides idx_nb; dst F32 | F16 | Q8_0 [n0, rows, n2, n3].
+ */
+int mi355x_set_rows(const mi355x_tensor * src, const void * idx, int32_t idx_type,
+                    const int64_t idx_ne[3], const size_t idx_nb[3],
+                    const mi355x_tensor * dst, void * stream);
+
+/* ---- buffer vtable helpers (ggml_backend_buffer_i / ggml_backend_buffer_type_i) ------------ */
+
+int mi355x_buffer_alloc(size_t size, void ** ptr);                 /* alloc_buffer (256-byte aligned) */
+int mi355x_buffer_free(void * ptr);                                /* free_buffer */
+int mi355x_buffer_memset(void * ptr, int value, size_t size, void * stream);         /* memset_tensor / clear */
+int mi355x_buffer_set(void * dst, const void * host_src, size_t size, void * stream);   /* set_tensor  (sync) */
+int mi355x_buffer_get(void * host_dst, const void * src, size_t size, void * stream);   /* get_tensor  (sync) */
+int mi355x_buffer_copy(void * dst, const void * src, size_t size, void * stream);      /* cpy_tensor D2D */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355X_FATTN_H */

@@ -1,0 +1,101 @@
+"""GPU parity: the HIP kernels, called through the C-ABI, against the CPU oracle (exact mode)
+on the same seeded inputs.  Tolerance as stated for this path: max-abs 2e-3, rel-L2 1e-3."""
+import numpy as np
+import pytest
+
+import crispasr_amd as ca
+import oracle as ora
+from cases import make_case, to_f32
+from crispasr_amd import ggml
+from gpu_util import assert_parity, run_gpu, run_oracle, upload
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    dict(seed=1, D=64, Nq=37, Nkv=53, Hq=4),
+    dict(seed=2, D=64, Nq=5, Nkv=130, Hq=3, q_layout="thd", kv_layout="thd"),
+    dict(seed=3, D=128, Nq=9, Nkv=77, Hq=8, Hkv=2, ktype=ora.Q8_0),
+    dict(seed=4, D=128, Nq=1, Nkv=200, Hq=8, Hkv=2, B=2, ktype=ora.Q8_0, kv_layout="gap"),
+    dict(seed=5, D=64, Nq=1, Nkv=64, Hq=4, B=3, mask="random_inf_batched"),
+    dict(seed=6, D=64, Nq=16, Nkv=48, Hq=2, mask="causal"),
+    dict(seed=7, D=128, Nq=12, Nkv=12, Hq=4, B=2, mask="bias_perhead", ktype=ora.F32),
+    dict(seed=8, D=128, Nq=20, Nkv=20, Hq=2, B=3, mask="bias_perhead_pad", lengths=[20, 11, 15]),
+    dict(seed=9, D=64, Nq=6, Nkv=40, Hq=4, B=4, Bk=2, ktype=ora.F16, mask="bias"),
+    dict(seed=10, D=64, Nq=6, Nkv=40, Hq=4, softcap=5.0, scale=0.9),
+    dict(seed=11, D=64, Nq=6, Nkv=40, Hq=8, mask="bias", max_bias=8.0),
+    dict(seed=12, D=64, Nq=6, Nkv=40, Hq=6, mask="bias", max_bias=4.0),
+    dict(seed=13, D=64, Nq=9, Nkv=31, Hq=2, mask="all_masked_rows"),
+    dict(seed=14, D=64, Nq=8, Nkv=30, Hq=2, kv_pad_rows=6, kv_layout="thd"),
+    dict(seed=15, D=80, Nq=3, Nkv=17, Hq=2, ktype=ora.F16),
+    dict(seed=16, D=32, Nq=4, Nkv=9, Hq=2, ktype=ora.Q8_0, mask="random_inf"),
+    dict(seed=17, D=256, Nq=2, Nkv=70, Hq=2, ktype=ora.F16),
+    dict(seed=18, D=64, Nq=3, Nkv=1000, Hq=2, ktype=ora.F32, kv_layout="gap"),
+    dict(seed=19, D=128, Nq=2, Nkv=513, Hq=4, Hkv=1, ktype=ora.F16, kv_layout="gap", mask="random_inf"),
+]
+
+
+@pytest.mark.parametrize("n_splits", [1, 0, 3])
+@pytest.mark.parametrize("spec", SHAPES, ids=lambda s: "seed%d" % s["seed"])
+def test_vec_kernel_matches_oracle(spec, n_splits):
+    case = make_case(**spec)
+    print("case", spec, "n_splits", n_splits, flush=True)
+    ref = run_oracle(case)
+    got = run_gpu(case, kernel=ggml.KERNEL_VEC, n_splits=n_splits)
+    assert_parity(got, ref, str(spec))
+
+
+def test_vec_one_hot_mask_is_exact_and_all_masked_rows_are_zero():
+    """Mask indexing is bit-exact: a one-hot mask row must return that V row unchanged."""
+    Nq, Nkv = 6, 300
+    case = make_case(seed=31, D=64, Nq=Nq, Nkv=Nkv, Hq=3, B=2, ktype=ora.Q8_0)
+    m = np.full((2, 1, Nq, Nkv), -np.inf, np.float32)
+    pick = {(0, 0): 3, (0, 1): 0, (0, 2): 299, (0, 3): 128, (1, 0): 255, (1, 1): 256, (1, 2): 77, (1, 4): 1}
+    for (b, i), j in pick.items():
+        m[b, 0, i, j] = 0.0
+    case["mask"] = ora.from_f32(m, ora.F16)
+    v = to_f32(case["v"])                       # exact dequantisation, [B, H, Nkv, D]
+    for ns in (1, 4):
+        print("one-hot n_splits", ns, flush=True)
+        got = run_gpu(case, kernel=ggml.KERNEL_VEC, n_splits=ns)
+        for b in range(2):
+            for i in range(Nq):
+                for h in range(3):
+                    if (b, i) in pick:
+                        assert np.array_equal(got[b, i, h], v[b, h, pick[(b, i)]]), (b, i, h)
+                    else:
+                        assert not got[b, i, h].any()
+
+
+def test_empty_inputs():
+    case = make_case(seed=32, D=64, Nq=2, Nkv=0, Hq=2)
+    got = run_gpu(case, kernel=ggml.KERNEL_VEC)
+    assert got.shape == (1, 2, 2, 64) and not got.any()
+    case = make_case(seed=33, D=64, Nq=0, Nkv=5, Hq=2)
+    got = run_gpu(case)
+    assert got.shape == (1, 0, 2, 64)
+
+
+def test_invalid_arguments_raise_and_leave_the_device_usable():
+    case = make_case(seed=34, D=64, Nq=2, Nkv=8, Hq=4, Hkv=2)
+    q, k, v = upload(case["q"]), upload(case["k"]), upload(case["v"])
+    bad_out = ca.Tensor.empty(ca.F32, (64, 2, 4, 1))            # [DV, Nq, Hq] instead of [DV, Hq, Nq]
+    with pytest.raises(ggml.InvalidError):
+        ca.flash_attn_ext(q, k, v, None, 1.0, out=bad_out)
+    with pytest.raises(ggml.InvalidError):
+        ca.flash_attn_ext(q, k, v, None, 1.0, max_bias=1.0)
+    with pytest.raises(ggml.Mi355xError):                        # caller workspace too small
+        import torch
+        big = make_case(seed=35, D=64, Nq=1, Nkv=4096, Hq=2)
+        ca.flash_attn_ext(upload(big["q"]), upload(big["k"]), upload(big["v"]), None, 0.125,
+                          kernel=ggml.KERNEL_VEC, n_splits=8,
+                          workspace=torch.empty(16, dtype=torch.uint8, device="cuda"))
+    got = run_gpu(case)
+    assert_parity(got, run_oracle(case), "after errors")
+
+
+def test_device_info_reports_a_gfx950():
+    info = ggml.device_info(0)
+    print(info, flush=True)
+    assert ggml.device_count() >= 1
+    assert info["arch"].startswith("gfx950")
+    assert info["wavefront_size"] == 64 and info["compute_units"] >= 64

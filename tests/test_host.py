@@ -1,0 +1,101 @@
+"""CPU-side checks of the drop-in boundary: the C-ABI library loads, exports every symbol the
+header declares, and its supports/plan predicates (which touch no device) answer like the
+op's contract says.  No compute call is made here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import crispasr_amd as ca
+from crispasr_amd import ggml
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "mi355x_fattn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355x_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = ggml.lib()
+    names = _declared_symbols()
+    assert len(names) >= 18
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in include/mi355x_fattn.h but not exported"
+    assert sorted(ggml.EXPORTS) == names
+    assert L.mi355x_api_version() == 1
+    assert L.mi355x_status_string(0) == b"ok"
+
+
+def _t(type_, ne, nb=None):
+    return ca.Tensor(None, type_, ne, nb)
+
+
+def test_supports_accepts_the_reference_call_shapes():
+    # Whisper encoder: strided [token][head][dim] views, K/V padded to 1536 (src/crispasr.cpp:2806-2821)
+    H, n_state = 20, 1280
+    q = _t(ca.F32, (64, 1500, H, 1), (4, 4 * n_state, 256, 4 * n_state * 1500))
+    k = _t(ca.F16, (64, 1536, H, 1), (2, 2 * n_state, 128, 2 * n_state * 1536))
+    assert ggml.flash_attn_supports(q, k, k, None, 0.125) == ggml.OK
+    # Whisper decoder self-attn with an F16 mask [n_kv, n_tok]
+    q = _t(ca.F32, (64, 5, H, 1), (4, 4 * n_state, 256, 4 * n_state * 5))
+    k = _t(ca.F16, (64, 224, H, 1), (2, 2 * n_state, 128, 2 * n_state * 224))
+    m = _t(ca.F16, (224, 5, 1, 1))
+    assert ggml.flash_attn_supports(q, k, k, m, 1.0) == ggml.OK
+    # Canary decoder: quantised cache view straight into the op (src/canary.cpp:966-972)
+    q = _t(ca.F32, (128, 1, 8, 1))
+    k = _t(ca.Q8_0, (128, 300, 8, 1), (34, 136, 136 * 1024, 136 * 1024 * 8))
+    assert ggml.flash_attn_supports(q, k, k, None, 128 ** -0.5) == ggml.OK
+    # FastConformer: F32 K/V strided into a fused QKV buffer, per-head F16 mask [T,T,H]
+    T, d = 750, 1024
+    q = _t(ca.F32, (128, T, 8, 1), (4, 3 * d * 4, 128 * 4, 3 * d * 4 * T))
+    m = _t(ca.F16, (T, T, 8, 1))
+    assert ggml.flash_attn_supports(q, q, q, m, 128 ** -0.5) == ggml.OK
+    # GQA, native
+    q = _t(ca.F32, (128, 407, 32, 1))
+    k = _t(ca.Q8_0, (128, 407, 8, 1))
+    m = _t(ca.F16, (407, 407, 1, 1))
+    assert ggml.flash_attn_supports(q, k, k, m, 128 ** -0.5) == ggml.OK
+
+
+def test_supports_rejects_contract_violations_and_uncovered_ops():
+    q = _t(ca.F32, (64, 4, 8, 1))
+    k = _t(ca.F16, (64, 16, 8, 1))
+    assert ggml.flash_attn_supports(q, _t(ca.F16, (128, 16, 8, 1)), k, None) == ggml.ERR_INVALID        # D mismatch
+    assert ggml.flash_attn_supports(q, _t(ca.F16, (64, 16, 3, 1)), _t(ca.F16, (64, 16, 3, 1)), None) == ggml.ERR_INVALID
+    assert ggml.flash_attn_supports(q, k, _t(ca.F16, (64, 17, 8, 1)), None) == ggml.ERR_INVALID          # Nkv mismatch
+    assert ggml.flash_attn_supports(q, k, k, None, max_bias=1.0) == ggml.ERR_INVALID                     # needs a mask
+    assert ggml.flash_attn_supports(q, k, k, _t(ca.F16, (8, 4, 1, 1))) == ggml.ERR_INVALID               # mask too narrow
+    assert ggml.flash_attn_supports(q, k, k, _t(ca.F16, (16, 4, 3, 1))) == ggml.ERR_INVALID              # 8 % 3
+    # valid for ggml, outside these kernels: goes to the CPU backend
+    assert ggml.flash_attn_supports(q, k, _t(ca.F32, (64, 16, 8, 1)), None) == ggml.ERR_UNSUPPORTED      # mixed K/V types
+    assert ggml.flash_attn_supports(_t(ca.F16, (64, 4, 8, 1)), k, k, None) == ggml.ERR_UNSUPPORTED       # q not F32
+    assert ggml.flash_attn_supports(q, _t(2, (64, 16, 8, 1), (18, 36, 576, 4608)), _t(2, (64, 16, 8, 1), (18, 36, 576, 4608)), None) == ggml.ERR_UNSUPPORTED  # Q4_0
+    assert ggml.flash_attn_supports(q, k, k, _t(ca.F32, (16, 4, 1, 1))) == ggml.ERR_UNSUPPORTED          # F32 mask
+    q72 = _t(ca.F32, (36, 4, 8, 1))
+    assert ggml.flash_attn_supports(q72, _t(ca.F16, (36, 16, 8, 1)), _t(ca.F16, (36, 16, 8, 1)), None) == ggml.ERR_UNSUPPORTED
+    assert ggml.flash_attn_supports(q, k, _t(ca.F16, (32, 16, 8, 1)), None) == ggml.ERR_UNSUPPORTED      # DV != DK
+    assert ggml.lib().mi355x_last_error() != b""
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(ggml, "_lib", None)
+    monkeypatch.setattr(ggml, "LIB_PATH", "/nonexistent/libmi355x_fattn.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ggml.lib()
+
+
+def test_cpy_supports_matrix():
+    L = ggml.lib()
+    def ok(s, d, ne_s=(64, 4, 2, 1), ne_d=None):
+        a, b = _t(s, ne_s).c(), _t(d, ne_d or ne_s).c()
+        return L.mi355x_cpy_supports(ctypes.byref(a), ctypes.byref(b))
+    assert ok(ca.F32, ca.F16) == ok(ca.F32, ca.Q8_0) == ok(ca.F32, ca.F32) == ggml.OK
+    assert ok(ca.F16, ca.F32) == ok(ca.Q8_0, ca.F32) == ok(ca.Q8_0, ca.Q8_0) == ggml.OK
+    assert ok(ca.F16, ca.Q8_0) == ggml.ERR_UNSUPPORTED
+    assert ok(ca.F32, ca.F16, (64, 4, 2, 1), (512, 1, 1, 1)) == ggml.OK          # reshape with equal counts
+    assert ok(ca.F32, ca.F16, (64, 4, 2, 1), (64, 5, 2, 1)) == ggml.ERR_INVALID
+    assert ok(ca.F32, ca.Q8_0, (48, 4, 2, 1)) == ggml.ERR_INVALID
