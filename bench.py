@@ -1,0 +1,285 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+A step is one pass of GGML_OP_FLASH_ATTN_EXT over the Whisper large-v3 encoder's 32 layers for
+a batch of 4 thirty-second windows (20 heads x 64, 1500 x 1500 non-causal, Q f32 / K,V f16,
+scale 1/8): 32 launches of the f16-MFMA tile kernel on distinct per-layer buffers that are
+resident in HBM before the timed region starts.  Prints ONE JSON line.
+
+Extra keys beside the contract's: `roofline` (dominant kernel against the f16 dense MFMA peak),
+`cpu_baseline` (the CPU oracle's ggml-like mode on a bounded sample, host cores of this box),
+`parity` (the timed configuration checked against the oracle on a sample of rows) and
+`decode` (the HBM-bound decode shapes, GB/s against 8 TB/s).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+PEAK_F16_TFLOPS = 2500.0     # MI355X dense f16 MFMA
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def attn_flops(D, Nq, Nkv, Hq, B):
+    return 4.0 * Nq * Nkv * D * Hq * B
+
+
+def make_layer(ca, ora, seed, D, N, H, B, kv_type):
+    """One layer's Q/K/V in the layout the Whisper runtime passes: [token][head][dim] memory viewed
+    as ne [D, N, H, B] (src/crispasr.cpp:2806-2819)."""
+    import numpy as np
+    q = ora.randn(seed * 10 + 1, (B, N, H, D))
+    k = ora.randn(seed * 10 + 2, (B, N, H, D))
+    v = ora.randn(seed * 10 + 3, (B, N, H, D))
+    n_state = H * D
+
+    def view(x, t):
+        ts = ora.TYPE_SIZE[t]
+        raw = x.view(np.uint8).reshape(-1) if t == ora.F32 else ora.fp32_to_fp16(x).view(np.uint8).reshape(-1)
+        nb = (ts, ts * n_state, ts * D, ts * n_state * N)
+        return ora.Tensor(raw, t, (D, N, H, B), nb)
+
+    host = {"q": view(q, ora.F32), "k": view(k, kv_type), "v": view(v, kv_type)}
+    dev = {n: ca.Tensor.from_host(t.buf, t.type, t.ne, t.nb, t.offset) for n, t in host.items()}
+    return host, dev
+
+
+def check_parity_sample(ca, ora, host, dev_out, scale, n_rows=48):
+    """Oracle (exact mode) on a sample of query rows of the timed configuration."""
+    import numpy as np
+    from cases import errors
+    D, N, H, B = host["q"].ne
+    rng = np.random.default_rng(0)
+    rows = sorted(set(int(x) for x in rng.integers(0, N, n_rows)) | {0, N - 1})
+    q = host["q"]
+    qa = q.buf.view(np.float32).reshape(B, N, H, D)
+    qs = np.ascontiguousarray(qa[:, rows])                                   # [B, R, H, D]
+    ts = 4
+    qsub = ora.Tensor(qs.view(np.uint8).reshape(-1), ora.F32, (D, len(rows), H, B),
+                      (ts, ts * H * D, ts * D, ts * H * D * len(rows)))
+    ref = ora.flash_attn_ext(qsub, host["k"], host["v"], None, scale, mode=ora.MODE_EXACT)   # [B, R, H, D]
+    got = dev_out.numpy_f32()[:, rows]
+    return errors(got, ref)
+
+
+def bench_encoder(args, ca, ora, torch):
+    D, N, H, B, L = 64, 1500, 20, 4, 32
+    scale = 0.125
+    t0 = time.time()
+    layers = []
+    host0 = None
+    for l in range(L):
+        host, dev = make_layer(ca, ora, 100 + l, D, N, H, B, ora.F16)
+        if l == 0:
+            host0 = host
+        dev["out"] = ca.Tensor.empty(ca.F32, (D, H, N, B))
+        layers.append(dev)
+    torch.cuda.synchronize()
+    log(f"[bench] generated and uploaded {L} layers in {time.time() - t0:.1f}s")
+
+    def step():
+        for dev in layers:
+            ca.flash_attn_ext(dev["q"], dev["k"], dev["v"], None, scale, out=dev["out"],
+                              kernel=ca.ggml.KERNEL_MMA)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        ev[s][0].record(stream)
+        step()
+        ev[s][1].record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ev_ms = [a.elapsed_time(b) for a, b in ev]
+    ms_per_step = wall * 1e3 / args.steps
+    flops_layer = attn_flops(D, N, N, H, B)
+    value = flops_layer * L / (ms_per_step * 1e-3) / 1e12
+    kernel_ms = sum(ev_ms) / (args.steps * L)            # HIP events on the launch stream
+    achieved = flops_layer / (kernel_ms * 1e-3) / 1e12
+
+    max_abs, rel = check_parity_sample(ca, ora, host0, layers[0]["out"], scale)
+    log(f"[bench] encoder: {ms_per_step:.3f} ms/step, {value:.1f} TFLOP/s, kernel {kernel_ms * 1e3:.1f} us/launch, "
+        f"parity max_abs={max_abs:.2e} rel_l2={rel:.2e}")
+    from cases import MAX_ABS_TOL, REL_L2_TOL
+    parity_ok = max_abs <= MAX_ABS_TOL and rel <= REL_L2_TOL
+
+    res = {
+        "value": value, "ms_per_step": ms_per_step,
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_F16_TFLOPS, "traffic": None,
+                     "kernel": "fattn_mma_kernel<64,2,F16>", "us_per_launch": kernel_ms * 1e3,
+                     "flops_per_launch": flops_layer},
+        "parity": {"max_abs": max_abs, "rel_l2": rel, "ok": bool(parity_ok), "rows_checked": 50,
+                   "oracle": "oracle/fattn_oracle.c exact mode"},
+    }
+    return res, host0
+
+
+def cpu_baseline(args, ora, host0):
+    """The oracle's ggml-like mode (f32 online softmax, f16 accumulator, threads over query rows) on a
+    bounded sample of the same workload: layer 0, window 0, all 20 heads."""
+    import numpy as np
+    D, N, H, B = host0["q"].ne
+
+    def one_window(t):
+        return ora.Tensor(t.buf, t.type, (D, N, H, 1), t.nb, t.offset)
+
+    q, k, v = one_window(host0["q"]), one_window(host0["k"]), one_window(host0["v"])
+    threads = min(ora.max_threads(), 16)
+    times = []
+    budget = time.time() + 25.0
+    for i in range(5):
+        t0 = time.perf_counter()
+        ora.flash_attn_ext(q, k, v, None, 0.125, mode=ora.MODE_GGML_LIKE, n_threads=threads)
+        times.append(time.perf_counter() - t0)
+        if time.time() > budget:
+            break
+    med = float(np.median(times))
+    tflops = attn_flops(D, N, N, H, 1) / med / 1e12
+    log(f"[bench] cpu baseline: {med * 1e3:.1f} ms per (layer, window) on {threads} threads = {tflops * 1e3:.1f} GFLOP/s")
+    return {"value": tflops, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"1 of 32 layers x 1 of 4 windows (20 heads, 1500x1500), median of {len(times)} runs, "
+                      f"oracle ggml-like mode (restatement of ggml-cpu; real ggml is absent)"}
+
+
+def bench_decode(args, ca, ora, torch):
+    """HBM-bound decode shapes: per-call GB/s over all layers of a step with distinct per-layer
+    buffers (cache-cold: the rotating working set exceeds the 256 MB Infinity Cache)."""
+    import numpy as np
+    out = {}
+
+    def run(name, layers, scale, bytes_per_layer, reps):
+        def step():
+            for dev in layers:
+                ca.flash_attn_ext(dev["q"], dev["k"], dev["v"], dev.get("mask"), scale, out=dev["out"])
+        for _ in range(3):
+            step()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (reps * len(layers))
+        gbs = bytes_per_layer / (us * 1e-6) / 1e9
+        kern, ns = ca.ggml.flash_attn_plan(layers[0]["q"], layers[0]["k"], layers[0]["v"], layers[0].get("mask"), scale)
+        out[name] = {"us_per_call": us, "GB/s": gbs, "frac_of_hbm_peak": gbs / PEAK_HBM_GBS,
+                     "bytes_per_call": bytes_per_layer, "layers_rotated": len(layers), "kernel": kern, "n_splits": ns}
+        log(f"[bench] decode {name}: {us:.2f} us/call, {gbs:.0f} GB/s ({100 * gbs / PEAK_HBM_GBS:.1f}% of HBM peak), "
+            f"kernel {kern}, splits {ns}")
+
+    # Whisper large-v3 cross-attention, beam 5: 5 queries vs one shared 1500-entry f16 K/V, 20 heads x 64
+    D, H, Nkv, NL = 64, 20, 1500, 64
+    layers = []
+    for l in range(NL):
+        k = torch.randn(Nkv * H * D, device="cuda").half().view(torch.uint8)
+        v = torch.randn(Nkv * H * D, device="cuda").half().view(torch.uint8)
+        q = torch.randn(5 * H * D, device="cuda").view(torch.uint8)
+        nbk = (2, 2 * H * D, 2 * D, 2 * H * D * Nkv)
+        layers.append({"q": ca.Tensor(q, ca.F32, (D, 5, H, 1), (4, 4 * H * D, 4 * D, 4 * H * D * 5)),
+                       "k": ca.Tensor(k, ca.F16, (D, Nkv, H, 1), nbk), "v": ca.Tensor(v, ca.F16, (D, Nkv, H, 1), nbk),
+                       "out": ca.Tensor.empty(ca.F32, (D, H, 5, 1))})
+    bytes_ = 2 * Nkv * H * D * 2 + 2 * 5 * H * D * 4
+    run("whisper_cross_beam5_f16", layers, 64 ** -0.25, bytes_, 20)
+
+    # Voxtral-style LLM decode: 32 q heads / 8 kv heads, D 128, Q8_0 cache of 663 entries
+    D, Hq, Hkv, Lk, NL = 128, 32, 8, 663, 60
+    layers = []
+    rs = 136
+    for l in range(NL):
+        kf = ora.randn(900 + l, (Hkv * Lk * D,))
+        raw = ora.quantize_q8_0(kf)
+        k = torch.from_numpy(raw).cuda()
+        v = torch.from_numpy(ora.quantize_q8_0(kf[::-1].copy())).cuda()
+        q = torch.randn(Hq * D, device="cuda").view(torch.uint8)
+        nbk = (34, rs, rs * Lk, rs * Lk * Hkv)
+        layers.append({"q": ca.Tensor(q, ca.F32, (D, 1, Hq, 1)),
+                       "k": ca.Tensor(k, ca.Q8_0, (D, Lk, Hkv, 1), nbk), "v": ca.Tensor(v, ca.Q8_0, (D, Lk, Hkv, 1), nbk),
+                       "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 1))})
+    bytes_ = 2 * Lk * Hkv * rs + 2 * Hq * D * 4
+    run("voxtral_decode_q8_0_gqa4", layers, 128 ** -0.5, bytes_, 20)
+
+    # saturating variant: the same Q8_0 decode with 64 independent sequences (ne3) per call
+    Bs = 64
+    kf = ora.randn(990, (Bs * Hkv * Lk * D,))
+    k = torch.from_numpy(ora.quantize_q8_0(kf)).cuda()
+    v = torch.from_numpy(ora.quantize_q8_0(kf[::-1].copy())).cuda()
+    layers = []
+    for l in range(8):
+        q = torch.randn(Bs * Hq * D, device="cuda").view(torch.uint8)
+        nbk = (34, rs, rs * Lk, rs * Lk * Hkv)
+        layers.append({"q": ca.Tensor(q, ca.F32, (D, 1, Hq, Bs)),
+                       "k": ca.Tensor(k.clone(), ca.Q8_0, (D, Lk, Hkv, Bs), nbk),
+                       "v": ca.Tensor(v.clone(), ca.Q8_0, (D, Lk, Hkv, Bs), nbk),
+                       "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, Bs))})
+    bytes_ = Bs * (2 * Lk * Hkv * rs + 2 * Hq * D * 4)
+    run("voxtral_decode_q8_0_gqa4_x64seq", layers, 128 ** -0.5, bytes_, 20)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU form in this build (heads and windows "
+              "are independent, so it would shard without collectives). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import crispasr_amd as ca
+    import oracle as ora
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    ca.ggml.lib()
+    info = ca.ggml.device_info(0)
+    log(f"[bench] device {info['name']} {info['arch']} CUs={info['compute_units']} clock={info['clock_khz']} kHz; "
+        f"roofline constants: f16 dense MFMA {PEAK_F16_TFLOPS} TFLOP/s, HBM {PEAK_HBM_GBS} GB/s")
+
+    enc, host0 = bench_encoder(args, ca, ora, torch)
+    line = {
+        "metric": "attn TFLOP/s (encoder) + decode-attn HBM GB/s, % of MI355X roofline, 1 GPU",
+        "value": enc["value"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": enc["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "Whisper large-v3 encoder self-attention: 32 layers x (20 heads, head_dim 64, "
+                               "1500x1500 non-causal), batch of 4 windows, Q f32 / K,V f16, scale 1/8; "
+                               "N(0,1) per-layer seeded; FLOPs = 4*Nq*Nkv*D*H*B per layer",
+                   "layers": 32, "heads": 20, "head_dim": 64, "n_q": 1500, "n_kv": 1500, "batch": 4},
+        "roofline": enc["roofline"], "parity": enc["parity"],
+        "device": {"name": info["name"], "arch": info["arch"], "cus": info["compute_units"], "clock_khz": info["clock_khz"]},
+    }
+    if not args.no_decode:
+        line["decode"] = bench_decode(args, ca, ora, torch)
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(args, ora, host0)
+    if not enc["parity"]["ok"]:
+        line["value"] = None
+        line["error"] = "parity check failed: timing withheld"
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -170,13 +170,20 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
     a.nbk1 = k->nb[1]; a.nbk2 = k->nb[2]; a.nbk3 = k->nb[3];
     a.nbv1 = v->nb[1]; a.nbv2 = v->nb[2]; a.nbv3 = v->nb[3];
     a.Hm = 1; a.Bm = 1;
-    bool al16 = !((uintptr_t)q->data % 16) && !((uintptr_t)k->data % 16) && !((uintptr_t)v->data % 16);
-    for (int i = 1; i < 4; i++) al16 = al16 && !(q->nb[i] % 16) && !(k->nb[i] % 16) && !(v->nb[i] % 16);
+    bool q16 = !((uintptr_t)q->data % 16);
+    bool kv16 = !((uintptr_t)k->data % 16) && !((uintptr_t)v->data % 16);
+    for (int i = 1; i < 4; i++) {
+        q16  = q16 && !(q->nb[i] % 16);
+        kv16 = kv16 && !(k->nb[i] % 16) && !(v->nb[i] % 16);
+    }
+    a.q_aligned16 = q16 ? 1 : 0;
+    const bool al16 = q16 && kv16;
     if (a.mask) {
         a.Hm = (int)mask->ne[2]; a.Bm = (int)mask->ne[3];
         a.nbm1 = mask->nb[1]; a.nbm2 = mask->nb[2]; a.nbm3 = mask->nb[3];
-        al16 = al16 && !((uintptr_t)mask->data % 16);
-        for (int i = 1; i < 4; i++) al16 = al16 && !(mask->nb[i] % 16);
+        bool m8 = !((uintptr_t)mask->data % 8);
+        for (int i = 1; i < 4; i++) m8 = m8 && !(mask->nb[i] % 8);
+        a.mask_al8 = m8 ? 1 : 0;
     }
     a.aligned16 = al16 ? 1 : 0;
     a.softcap = p->logit_softcap;

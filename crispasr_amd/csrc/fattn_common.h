@@ -32,7 +32,9 @@ struct FattnArgs {
     float max_bias, m0, m1;
     int32_t n_head_log2;
 
-    int32_t aligned16;   // q/k/v/mask bases and strides are all multiples of 16 bytes
+    int32_t aligned16;   // q, k and v bases and strides are all multiples of 16 bytes
+    int32_t q_aligned16; // q alone
+    int32_t mask_al8;    // mask base and strides are multiples of 8 bytes
 
     // split-KV
     int32_t n_splits;

@@ -1,3 +1,397 @@
+// f16-MFMA tile kernel for prefill / encoder attention on gfx950 (CDNA4, wave64).
+//
+// A workgroup of 4 waves owns 4*32*NQB consecutive queries of one (head, batch) and walks
+// the keys in tiles of 64.  Both products run on v_mfma_f32_32x32x16_f16 in the transposed
+// form, so that a lane keeps one query column for the whole kernel:
+//
+//   S^T[key, query] = K[key, :] . Q[query, :]^T        A = K tile (LDS),   B = Q (registers)
+//   O^T[d,   query] = V[:, d]^T . P^T[:, query]        A = V^T (LDS),      B = P (registers)
+//
+// With the 32x32 accumulator layout lane l holds query l%32 and keys {8g + 4(l/32) + r},
+// which is exactly the B-operand layout the second product needs (after choosing the order
+// of its reduction index), so the probabilities never leave registers and the online softmax
+// needs one cross-lane exchange (lane l <-> l+32) per tile for the running maximum.
+//
+// K and V tiles are staged through LDS in their natural [key][d] layout (converted to f16
+// when the cache is F32 or Q8_0), double-buffered, with the next tile's global loads in
+// flight during the current tile's MFMAs.  K rows are padded to a pitch of 16 mod 128 bytes
+// so the 128-bit operand reads of 8 consecutive lanes fall into distinct banks.  V^T
+// operands are produced by ds_read_b64_tr_b16 (LDS transpose read): 16 lanes present four
+// 32-byte row segments of four keys and each lane receives the four keys' values of its own
+// d - V's pitch is 64 mod 128 bytes so that those four segments tile the banks.
+//
+// Softmax runs in base 2: scale*log2(e) is folded into Q when it is converted to f16.
 #include "fattn_common.h"
-bool fattn_mma_supported(const FattnArgs &, int) { return false; }
-int fattn_mma_launch(const FattnArgs &, int, hipStream_t) { return (int)hipErrorNotSupported; }
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float    float16v __attribute__((ext_vector_type(16)));
+typedef short    short4v __attribute__((ext_vector_type(4)));
+
+constexpr int   MMA_WAVES   = 4;
+constexpr int   MMA_THREADS = MMA_WAVES * 64;
+constexpr int   BC          = 64;                 // keys per tile
+constexpr float LOG2E       = 1.4426950408889634f;
+
+template <int D> struct Pitch {
+    static constexpr int K = D + 8;               // halves: (2D + 16) bytes = 16 mod 128
+    static constexpr int V = D + 32;              // halves: (2D + 64) bytes = 64 mod 128
+};
+
+// raw global data of one 8-element chunk of a K or V row, converted to f16 when written to LDS
+struct Raw {
+    uint4 a, b;
+};
+
+template <int TYPE>
+__device__ __forceinline__ Raw load_chunk(const char * row, int c, bool valid) {
+    Raw r;
+    r.a = make_uint4(0, 0, 0, 0);
+    r.b = make_uint4(0, 0, 0, 0);
+    if (!valid) return r;
+    if (TYPE == MI355X_TYPE_F16) {
+        r.a = *(const uint4 *)(row + c * 16);
+    } else if (TYPE == MI355X_TYPE_F32) {
+        r.a = *(const uint4 *)(row + c * 32);
+        r.b = *(const uint4 *)(row + c * 32 + 16);
+    } else {
+        const char * blk = row + (c >> 2) * FATTN_Q8_0_BYTES;
+        const uint16_t * qs = (const uint16_t *)(blk + 2 + (c & 3) * 8);
+        r.a.x = (uint32_t)qs[0] | ((uint32_t)qs[1] << 16);
+        r.a.y = (uint32_t)qs[2] | ((uint32_t)qs[3] << 16);
+        r.a.z = *(const uint16_t *)blk;
+    }
+    return r;
+}
+
+template <int TYPE>
+__device__ __forceinline__ half8 to_half8(const Raw & r) {
+    half8 h;
+    if (TYPE == MI355X_TYPE_F16) {
+        h = __builtin_bit_cast(half8, r.a);
+    } else if (TYPE == MI355X_TYPE_F32) {
+        const float f[8] = {__uint_as_float(r.a.x), __uint_as_float(r.a.y), __uint_as_float(r.a.z), __uint_as_float(r.a.w),
+                            __uint_as_float(r.b.x), __uint_as_float(r.b.y), __uint_as_float(r.b.z), __uint_as_float(r.b.w)};
+#pragma unroll
+        for (int e = 0; e < 8; e++) h[e] = (_Float16)f[e];
+    } else {
+        const float d = h2f_bits((uint16_t)r.a.z);
+        const uint32_t w[2] = {r.a.x, r.a.y};
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int8_t q = (int8_t)((w[e >> 2] >> (8 * (e & 3))) & 0xff);
+            h[e] = (_Float16)((float)q * d);       // exact q*d, then one rounding to f16
+        }
+    }
+    return h;
+}
+
+template <int D, int NQB, int TYPE>
+__global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnArgs a, const int n_qtiles) {
+    constexpr int KS   = D / 16;                   // reduction steps of Q.K^T
+    constexpr int DB   = D / 32;                   // 32-wide blocks of the output's d
+    constexpr int CH   = D / 8;                    // 8-element chunks per row
+    constexpr int RPP  = MMA_THREADS / CH;         // rows staged per pass
+    constexpr int NP   = BC / RPP;                 // passes per tile
+    constexpr int PK   = Pitch<D>::K;
+    constexpr int PV   = Pitch<D>::V;
+    constexpr int BMW  = 32 * NQB;                 // queries per wave
+    constexpr int BMG  = BMW * MMA_WAVES;          // queries per workgroup
+
+    extern __shared__ __attribute__((aligned(16))) _Float16 lds_raw[];
+    _Float16 (*k_lds)[BC * PK] = (_Float16 (*)[BC * PK])lds_raw;
+    _Float16 (*v_lds)[BC * PV] = (_Float16 (*)[BC * PV])(lds_raw + 2 * BC * PK);
+
+    const int tid  = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int l32  = lane & 31;
+    const int hh   = lane >> 5;                    // which half of the wave
+
+    // Workgroups are handed to the 8 XCDs round-robin; renumber them so that the query tiles
+    // of one (head, batch) - which share K/V - sit on one XCD and hit its L2.
+    int bid = blockIdx.x;
+    {
+        const int nb = gridDim.x;
+        const int per = nb / 8;
+        if (bid < per * 8) bid = (bid % 8) * per + bid / 8;
+    }
+    const int qt = bid % n_qtiles;
+    const int h  = (bid / n_qtiles) % a.Hq;
+    const int b  = bid / (n_qtiles * a.Hq);
+    const int hk = h / a.gqa;
+    const int bk = b / a.bq;
+
+    const int q0 = qt * BMG + wave * BMW;          // first query of this wave
+
+    // ---- Q -> f16 B operands, scaled so that the MFMA result is already in log2 units ----
+    const float qscale = a.softcap != 0.0f ? a.scale : a.scale * LOG2E;   // a.scale is scale/softcap when capped
+    half8 qreg[NQB][KS];
+#pragma unroll
+    for (int qb = 0; qb < NQB; qb++) {
+        const int qi = min(q0 + qb * 32 + l32, a.Nq - 1);
+        const float * qrow = (const float *)(a.q + (int64_t)qi * a.nbq1 + (int64_t)h * a.nbq2 + (int64_t)b * a.nbq3);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const float4 x0 = *(const float4 *)(qrow + ks * 16 + hh * 8);
+            const float4 x1 = *(const float4 *)(qrow + ks * 16 + hh * 8 + 4);
+            half8 v;
+            v[0] = (_Float16)(x0.x * qscale); v[1] = (_Float16)(x0.y * qscale);
+            v[2] = (_Float16)(x0.z * qscale); v[3] = (_Float16)(x0.w * qscale);
+            v[4] = (_Float16)(x1.x * qscale); v[5] = (_Float16)(x1.y * qscale);
+            v[6] = (_Float16)(x1.z * qscale); v[7] = (_Float16)(x1.w * qscale);
+            qreg[qb][ks] = v;
+        }
+    }
+
+    const char * kbase = a.k + (int64_t)hk * a.nbk2 + (int64_t)bk * a.nbk3;
+    const char * vbase = a.v + (int64_t)hk * a.nbv2 + (int64_t)bk * a.nbv3;
+    const float  mslope = fattn_slope(a, h) * LOG2E;
+    const char * mbase = a.mask ? a.mask + (int64_t)(h % a.Hm) * a.nbm2 + (int64_t)(b % a.Bm) * a.nbm3 : nullptr;
+
+    // staging assignment: chunk c of rows r0 + p*RPP
+    const int sc = tid % CH;
+    const int sr = tid / CH;
+
+    Raw kraw[NP], vraw[NP];
+    auto load_tile = [&](int j0) {
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            const int  key = j0 + sr + p * RPP;
+            const bool ok  = key < a.Nkv;
+            kraw[p] = load_chunk<TYPE>(kbase + (int64_t)key * a.nbk1, sc, ok);
+            vraw[p] = load_chunk<TYPE>(vbase + (int64_t)key * a.nbv1, sc, ok);
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            const int row = sr + p * RPP;
+            *(half8 *)&k_lds[buf][row * PK + sc * 8] = to_half8<TYPE>(kraw[p]);
+            *(half8 *)&v_lds[buf][row * PV + sc * 8] = to_half8<TYPE>(vraw[p]);
+        }
+    };
+
+    float16v oacc[NQB][DB];
+    float    m_run[NQB], l_run[NQB];
+#pragma unroll
+    for (int qb = 0; qb < NQB; qb++) {
+        m_run[qb] = -INFINITY;
+        l_run[qb] = 0.0f;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[qb][db][r] = 0.0f;
+    }
+
+    const int n_tiles = (a.Nkv + BC - 1) / BC;
+    if (n_tiles > 0) {
+        load_tile(0);
+        store_tile(0);
+    }
+    __syncthreads();
+
+    for (int t = 0; t < n_tiles; t++) {
+        const int  j0   = t * BC;
+        const int  buf  = t & 1;
+        const bool more = t + 1 < n_tiles;
+        if (more) load_tile(j0 + BC);
+
+        // ---- S^T = K . Q^T --------------------------------------------------------------
+        float16v s[2][NQB];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int qb = 0; qb < NQB; qb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) s[kb][qb][r] = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                const half8 ka = *(const half8 *)&k_lds[buf][(kb * 32 + l32) * PK + ks * 16 + hh * 8];
+#pragma unroll
+                for (int qb = 0; qb < NQB; qb++)
+                    s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[qb][ks], s[kb][qb], 0, 0, 0);
+            }
+        }
+
+        // ---- soft cap, mask, key tail ------------------------------------------------------
+        if (a.softcap != 0.0f) {
+            const float c2 = a.softcap * LOG2E;
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int qb = 0; qb < NQB; qb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) s[kb][qb][r] = c2 * tanhf(s[kb][qb][r]);
+        }
+        const bool tail = j0 + BC > a.Nkv;
+        if (mbase) {
+#pragma unroll
+            for (int qb = 0; qb < NQB; qb++) {
+                const int qi = min(q0 + qb * 32 + l32, a.Nq - 1);
+                const uint16_t * mrow = (const uint16_t *)(mbase + (int64_t)qi * a.nbm1);
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const int key = j0 + kb * 32 + g * 8 + hh * 4;
+                        uint16_t mv[4];
+                        if (!tail && a.mask_al8) {
+                            const uint2 u = *(const uint2 *)(mrow + key);
+                            mv[0] = (uint16_t)(u.x & 0xffff); mv[1] = (uint16_t)(u.x >> 16);
+                            mv[2] = (uint16_t)(u.y & 0xffff); mv[3] = (uint16_t)(u.y >> 16);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++) mv[e] = key + e < a.Nkv ? mrow[key + e] : (uint16_t)0;
+                        }
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            s[kb][qb][g * 4 + e] = fmaf(mslope, h2f_bits(mv[e]), s[kb][qb][g * 4 + e]);
+                    }
+            }
+        }
+        if (tail) {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int key = j0 + kb * 32 + (r >> 2) * 8 + hh * 4 + (r & 3);
+                    if (key >= a.Nkv) {
+#pragma unroll
+                        for (int qb = 0; qb < NQB; qb++) s[kb][qb][r] = -INFINITY;
+                    }
+                }
+        }
+
+        // ---- online softmax (base 2) and P in f16 -----------------------------------------------
+        half8 preg[NQB][4];
+#pragma unroll
+        for (int qb = 0; qb < NQB; qb++) {
+            float mloc = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, s[kb][qb][r]);
+            mloc = fmaxf(mloc, xor_shuffle(mloc, 32));
+            const float m_new = fmaxf(m_run[qb], mloc);
+            const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_use);
+            float lsum = 0.0f;
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const float p = __builtin_amdgcn_exp2f(s[kb][qb][r] - m_use);
+                    lsum += p;
+                    preg[qb][kb * 2 + (r >> 3)][r & 7] = (_Float16)p;
+                }
+            l_run[qb] = l_run[qb] * alpha + lsum;
+            m_run[qb] = m_new;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[qb][db][r] *= alpha;
+        }
+
+        // ---- O^T += V^T . P^T ----------------------------------------------------------------------
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                // transpose read: lane i of a 16-lane block addresses 4 halves of key (i/4) at d0 + 4*(i%4)
+                const int i16 = lane & 15;
+                const int d0  = db * 32 + ((lane >> 4) & 1) * 16;
+                const int kr  = kk * 16 + hh * 4 + (i16 >> 2);
+                const _Float16 * p0 = &v_lds[buf][kr * PV + d0 + (i16 & 3) * 4];
+                const _Float16 * p1 = p0 + 8 * PV;
+                const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p0);
+                const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p1);
+                half8 va;
+                const half4 lo4 = __builtin_bit_cast(half4, lo);
+                const half4 hi4 = __builtin_bit_cast(half4, hi);
+                va[0] = lo4[0]; va[1] = lo4[1]; va[2] = lo4[2]; va[3] = lo4[3];
+                va[4] = hi4[0]; va[5] = hi4[1]; va[6] = hi4[2]; va[7] = hi4[3];
+#pragma unroll
+                for (int qb = 0; qb < NQB; qb++)
+                    oacc[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, preg[qb][kk], oacc[qb][db], 0, 0, 0);
+            }
+        }
+
+        if (more) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- normalise and write dst[D, Hq, Nq, B] -------------------------------------------------------
+#pragma unroll
+    for (int qb = 0; qb < NQB; qb++) {
+        const float ltot = l_run[qb] + xor_shuffle(l_run[qb], 32);
+        const float inv  = ltot > 0.0f ? 1.0f / ltot : 0.0f;
+        const int   qi   = q0 + qb * 32 + l32;
+        if (qi < a.Nq) {
+            float * out = a.dst + (((int64_t)b * a.Nq + qi) * a.Hq + h) * D;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    float4 o;
+                    o.x = oacc[qb][db][g * 4 + 0] * inv;
+                    o.y = oacc[qb][db][g * 4 + 1] * inv;
+                    o.z = oacc[qb][db][g * 4 + 2] * inv;
+                    o.w = oacc[qb][db][g * 4 + 3] * inv;
+                    *(float4 *)(out + db * 32 + g * 8 + hh * 4) = o;
+                }
+        }
+    }
+}
+
+template <int D, int NQB, int TYPE>
+int launch(const FattnArgs & a, hipStream_t stream) {
+    const int bmg = 32 * NQB * MMA_WAVES;
+    const int n_qtiles = (a.Nq + bmg - 1) / bmg;
+    const dim3 grid((unsigned)(n_qtiles * a.Hq * a.B));
+    const size_t lds = (size_t)2 * BC * (Pitch<D>::K + Pitch<D>::V) * sizeof(_Float16);
+    static bool attr_set = false;     // per instantiation; the attribute only matters above 64 KiB
+    if (!attr_set && lds > 64 * 1024) {
+        const hipError_t e = hipFuncSetAttribute((const void *)fattn_mma_kernel<D, NQB, TYPE>,
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
+    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, TYPE>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
+    return (int)hipGetLastError();
+}
+
+template <int TYPE>
+int launch_type(const FattnArgs & a, hipStream_t stream) {
+    // two query blocks per wave halve the LDS operand traffic per MFMA; one block keeps more
+    // workgroups in flight when there are few queries
+    const int64_t wg2 = (int64_t)((a.Nq + 255) / 256) * a.Hq * a.B;
+    const bool two = wg2 >= 128;
+    if (a.D == 64)  return two ? launch<64, 2, TYPE>(a, stream) : launch<64, 1, TYPE>(a, stream);
+    if (a.D == 128) return launch<128, 1, TYPE>(a, stream);
+    return (int)hipErrorInvalidValue;
+}
+
+}  // namespace
+
+bool fattn_mma_supported(const FattnArgs & a, int ktype) {
+    if (a.D != 64 && a.D != 128) return false;
+    if (a.Nq < 1 || a.Nkv < 1) return false;
+    if (ktype != MI355X_TYPE_Q8_0 && !a.aligned16) return false;   // 128-bit K/V loads
+    if (ktype == MI355X_TYPE_Q8_0 && !a.q_aligned16) return false;
+    return ktype == MI355X_TYPE_F16 || ktype == MI355X_TYPE_F32 || ktype == MI355X_TYPE_Q8_0;
+}
+
+int fattn_mma_launch(const FattnArgs & a, int ktype, hipStream_t stream) {
+    switch (ktype) {
+        case MI355X_TYPE_F16:  return launch_type<MI355X_TYPE_F16>(a, stream);
+        case MI355X_TYPE_F32:  return launch_type<MI355X_TYPE_F32>(a, stream);
+        case MI355X_TYPE_Q8_0: return launch_type<MI355X_TYPE_Q8_0>(a, stream);
+        default:               return (int)hipErrorInvalidValue;
+    }
+}

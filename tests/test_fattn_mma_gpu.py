@@ -1,0 +1,77 @@
+"""GPU parity of the f16-MFMA tile kernel (prefill / encoder shapes) against the CPU oracle."""
+import numpy as np
+import pytest
+
+import oracle as ora
+from cases import make_case, to_f32
+from crispasr_amd import ggml
+from gpu_util import assert_parity, run_gpu, run_oracle
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    dict(seed=101, D=64, Nq=37, Nkv=53, Hq=4),
+    dict(seed=102, D=64, Nq=256, Nkv=256, Hq=2),
+    dict(seed=103, D=64, Nq=300, Nkv=333, Hq=3, B=2, q_layout="thd", kv_layout="thd"),
+    dict(seed=104, D=64, Nq=130, Nkv=200, Hq=2, kv_pad_rows=56, kv_layout="thd"),          # Whisper zero-pad rows
+    dict(seed=105, D=128, Nq=150, Nkv=190, Hq=8, Hkv=2),
+    dict(seed=106, D=128, Nq=77, Nkv=407, Hq=8, Hkv=2, ktype=ora.Q8_0, mask="causal"),
+    dict(seed=107, D=64, Nq=100, Nkv=100, Hq=4, mask="causal"),
+    dict(seed=108, D=128, Nq=90, Nkv=90, Hq=4, B=2, mask="bias_perhead", ktype=ora.F32),
+    dict(seed=109, D=128, Nq=75, Nkv=75, Hq=2, B=3, mask="bias_perhead_pad", lengths=[75, 40, 61]),
+    dict(seed=110, D=64, Nq=64, Nkv=128, Hq=4, B=4, Bk=2, mask="bias"),
+    dict(seed=111, D=64, Nq=70, Nkv=129, Hq=4, softcap=5.0, scale=0.9),
+    dict(seed=112, D=64, Nq=66, Nkv=140, Hq=8, mask="bias", max_bias=8.0),
+    dict(seed=113, D=64, Nq=99, Nkv=131, Hq=2, mask="all_masked_rows"),
+    dict(seed=114, D=64, Nq=50, Nkv=500, Hq=2, mask="random_inf", kv_layout="gap"),
+    dict(seed=115, D=128, Nq=33, Nkv=64, Hq=2, ktype=ora.F32, kv_layout="gap", q_layout="thd"),
+    dict(seed=116, D=64, Nq=1, Nkv=70, Hq=2),
+    dict(seed=117, D=64, Nq=1500, Nkv=1500, Hq=2, scale=0.125),                              # Whisper base geometry, 2 heads
+    dict(seed=118, D=64, Nq=512, Nkv=640, Hq=8, B=4, scale=0.125),                           # enough workgroups for 2 query blocks per wave
+]
+
+
+@pytest.mark.parametrize("spec", SHAPES, ids=lambda s: "seed%d" % s["seed"])
+def test_mma_kernel_matches_oracle(spec):
+    case = make_case(**spec)
+    print("case", spec, flush=True)
+    ref = run_oracle(case)
+    got = run_gpu(case, kernel=ggml.KERNEL_MMA)
+    err = assert_parity(got, ref, str(spec))
+    print("max_abs %.3e rel_l2 %.3e" % err, flush=True)
+
+
+def test_mma_one_hot_mask_returns_the_v_row():
+    """Mask/causal indexing: a one-hot row must return exactly f16(V row) (f32 V is rounded once to
+    f16 when staged; an f16 cache is returned bit-exactly)."""
+    Nq, Nkv = 70, 200
+    case = make_case(seed=121, D=64, Nq=Nq, Nkv=Nkv, Hq=2, B=2)
+    m = np.full((2, 1, Nq, Nkv), -np.inf, np.float32)
+    rng = np.random.default_rng(5)
+    pick = rng.integers(0, Nkv, size=(2, Nq))
+    pick[0, 0], pick[0, 1], pick[1, 0], pick[1, 69] = 0, 199, 63, 64
+    for b in range(2):
+        for i in range(Nq):
+            if i % 7 != 3:
+                m[b, 0, i, pick[b, i]] = 0.0
+    case["mask"] = ora.from_f32(m, ora.F16)
+    v = to_f32(case["v"])
+    got = run_gpu(case, kernel=ggml.KERNEL_MMA)
+    for b in range(2):
+        for i in range(Nq):
+            for h in range(2):
+                if i % 7 != 3:
+                    assert np.array_equal(got[b, i, h], v[b, h, pick[b, i]]), (b, i, h)
+                else:
+                    assert not got[b, i, h].any()
+
+
+def test_auto_picks_the_tile_kernel_for_prefill_and_the_vector_kernel_for_decode():
+    from gpu_util import upload
+    pre = make_case(seed=122, D=64, Nq=200, Nkv=200, Hq=4)
+    dec = make_case(seed=123, D=64, Nq=1, Nkv=200, Hq=4)
+    odd = make_case(seed=124, D=80, Nq=200, Nkv=200, Hq=4)
+    for case, want in ((pre, ggml.KERNEL_MMA), (dec, ggml.KERNEL_VEC), (odd, ggml.KERNEL_VEC)):
+        kern, _ = ggml.flash_attn_plan(upload(case["q"]), upload(case["k"]), upload(case["v"]), None, case["scale"])
+        assert kern == want
+        assert_parity(run_gpu(case), run_oracle(case), "auto")
