@@ -23,6 +23,8 @@
 // Softmax runs in base 2: scale*log2(e) is folded into Q when it is converted to f16.
 #include "fattn_common.h"
 
+#include <type_traits>
+
 namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -30,6 +32,7 @@ typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float    float16v __attribute__((ext_vector_type(16)));
 typedef short    short4v __attribute__((ext_vector_type(4)));
+typedef unsigned uint2v __attribute__((ext_vector_type(2)));
 
 constexpr int   MMA_WAVES   = 4;
 constexpr int   MMA_THREADS = MMA_WAVES * 64;
@@ -89,7 +92,29 @@ __device__ __forceinline__ half8 to_half8(const Raw & r) {
     return h;
 }
 
-template <int D, int NQB, int TYPE>
+// max / sum of a value held by lane l and lane l^32.  Only used off the hot path (reference
+// raises, epilogue), so the LDS-crossbar shuffle is good enough.
+__device__ __forceinline__ float max_xor32(float x) { return fmaxf(x, xor_shuffle(x, 32)); }
+__device__ __forceinline__ float sum_xor32(float x) { return x + xor_shuffle(x, 32); }
+
+// branch-free tanh: 1 - 2/(2^(2x*log2e) + 1); exact limits at +-inf
+__device__ __forceinline__ float fast_tanh(float x) {
+    const float e = __builtin_amdgcn_exp2f(x * (2.0f * LOG2E));
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+
+// Running softmax state of one 32-query block, per lane (= per query, mirrored in lane l^32).
+// Scores are kept relative to `m`, a reference that trails the true running maximum by at
+// most RESCALE_SLACK (in log2 units): it is folded into the accumulator's initial value, so
+// the common tile needs no subtraction and no rescale of O.
+struct RowState {
+    float m;        // reference subtracted from the scores (finite)
+    float l;        // sum of p over this lane's keys
+    bool  have;     // a finite score has been seen
+};
+constexpr float RESCALE_SLACK = 8.0f;
+
+template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP>
 __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnArgs a, const int n_qtiles) {
     constexpr int KS   = D / 16;                   // reduction steps of Q.K^T
     constexpr int DB   = D / 32;                   // 32-wide blocks of the output's d
@@ -128,7 +153,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     const int q0 = qt * BMG + wave * BMW;          // first query of this wave
 
     // ---- Q -> f16 B operands, scaled so that the MFMA result is already in log2 units ----
-    const float qscale = a.softcap != 0.0f ? a.scale : a.scale * LOG2E;   // a.scale is scale/softcap when capped
+    const float qscale = SOFTCAP ? a.scale : a.scale * LOG2E;   // a.scale is scale/softcap when capped
     half8 qreg[NQB][KS];
 #pragma unroll
     for (int qb = 0; qb < NQB; qb++) {
@@ -149,10 +174,17 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
 
     const char * kbase = a.k + (int64_t)hk * a.nbk2 + (int64_t)bk * a.nbk3;
     const char * vbase = a.v + (int64_t)hk * a.nbv2 + (int64_t)bk * a.nbv3;
-    const float  mslope = fattn_slope(a, h) * LOG2E;
-    const char * mbase = a.mask ? a.mask + (int64_t)(h % a.Hm) * a.nbm2 + (int64_t)(b % a.Bm) * a.nbm3 : nullptr;
+    const float  mslope = MASK ? fattn_slope(a, h) * LOG2E : 0.0f;
+    const uint16_t * mrow[NQB];
+#pragma unroll
+    for (int qb = 0; qb < NQB; qb++) {
+        const int qi = min(q0 + qb * 32 + l32, a.Nq - 1);
+        mrow[qb] = MASK ? (const uint16_t *)(a.mask + (int64_t)(h % a.Hm) * a.nbm2 + (int64_t)(b % a.Bm) * a.nbm3 +
+                                             (int64_t)qi * a.nbm1)
+                        : nullptr;
+    }
 
-    // staging assignment: chunk c of rows r0 + p*RPP
+    // staging assignment: chunk sc of rows sr + p*RPP
     const int sc = tid % CH;
     const int sr = tid / CH;
 
@@ -176,160 +208,200 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     };
 
     float16v oacc[NQB][DB];
-    float    m_run[NQB], l_run[NQB];
+    RowState st[NQB];
 #pragma unroll
     for (int qb = 0; qb < NQB; qb++) {
-        m_run[qb] = -INFINITY;
-        l_run[qb] = 0.0f;
+        st[qb].m = 0.0f;
+        st[qb].l = 0.0f;
+        st[qb].have = false;
 #pragma unroll
         for (int db = 0; db < DB; db++)
 #pragma unroll
             for (int r = 0; r < 16; r++) oacc[qb][db][r] = 0.0f;
     }
 
-    const int n_tiles = (a.Nkv + BC - 1) / BC;
-    if (n_tiles > 0) {
-        load_tile(0);
-        store_tile(0);
-    }
-    __syncthreads();
+    // One tile of 64 keys.  TAIL: the tile runs past Nkv (keys beyond it are excluded).
+    auto tile = [&](const int j0, const int buf, auto tail_tag) {
+        constexpr bool TAIL = decltype(tail_tag)::value;
 
-    for (int t = 0; t < n_tiles; t++) {
-        const int  j0   = t * BC;
-        const int  buf  = t & 1;
-        const bool more = t + 1 < n_tiles;
-        if (more) load_tile(j0 + BC);
-
-        // ---- S^T = K . Q^T --------------------------------------------------------------
-        float16v s[2][NQB];
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++)
+        // additive mask values of this lane's 32 (key, query) pairs per query block, fetched early
+        uint2 mraw[NQB][2][4];
+        if (MASK) {
 #pragma unroll
             for (int qb = 0; qb < NQB; qb++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) s[kb][qb][r] = 0.0f;
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                const half8 ka = *(const half8 *)&k_lds[buf][(kb * 32 + l32) * PK + ks * 16 + hh * 8];
-#pragma unroll
-                for (int qb = 0; qb < NQB; qb++)
-                    s[kb][qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[qb][ks], s[kb][qb], 0, 0, 0);
-            }
-        }
-
-        // ---- soft cap, mask, key tail ------------------------------------------------------
-        if (a.softcap != 0.0f) {
-            const float c2 = a.softcap * LOG2E;
-#pragma unroll
-            for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                for (int qb = 0; qb < NQB; qb++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) s[kb][qb][r] = c2 * tanhf(s[kb][qb][r]);
-        }
-        const bool tail = j0 + BC > a.Nkv;
-        if (mbase) {
-#pragma unroll
-            for (int qb = 0; qb < NQB; qb++) {
-                const int qi = min(q0 + qb * 32 + l32, a.Nq - 1);
-                const uint16_t * mrow = (const uint16_t *)(mbase + (int64_t)qi * a.nbm1);
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
                         const int key = j0 + kb * 32 + g * 8 + hh * 4;
-                        uint16_t mv[4];
-                        if (!tail && a.mask_al8) {
-                            const uint2 u = *(const uint2 *)(mrow + key);
-                            mv[0] = (uint16_t)(u.x & 0xffff); mv[1] = (uint16_t)(u.x >> 16);
-                            mv[2] = (uint16_t)(u.y & 0xffff); mv[3] = (uint16_t)(u.y >> 16);
+                        if (!TAIL && a.mask_al8) {
+                            mraw[qb][kb][g] = *(const uint2 *)(mrow[qb] + key);
                         } else {
+                            uint16_t mv[4];
 #pragma unroll
-                            for (int e = 0; e < 4; e++) mv[e] = key + e < a.Nkv ? mrow[key + e] : (uint16_t)0;
+                            for (int e = 0; e < 4; e++) mv[e] = (!TAIL || key + e < a.Nkv) ? mrow[qb][key + e] : (uint16_t)0;
+                            mraw[qb][kb][g].x = (uint32_t)mv[0] | ((uint32_t)mv[1] << 16);
+                            mraw[qb][kb][g].y = (uint32_t)mv[2] | ((uint32_t)mv[3] << 16);
                         }
+                    }
+        }
+
+        // the tile is consumed in two blocks of 32 keys to keep the score registers few
 #pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            s[kb][qb][g * 4 + e] = fmaf(mslope, h2f_bits(mv[e]), s[kb][qb][g * 4 + e]);
+        for (int kb = 0; kb < 2; kb++) {
+            // ---- S^T = K . Q^T - m  (the reference m enters as the accumulator's initial value) ----
+            float16v s[NQB];
+#pragma unroll
+            for (int qb = 0; qb < NQB; qb++) {
+                const float init = (MASK || SOFTCAP) ? 0.0f : -st[qb].m;
+#pragma unroll
+                for (int r = 0; r < 16; r++) s[qb][r] = init;
+            }
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                const half8 ka = *(const half8 *)&k_lds[buf][(kb * 32 + l32) * PK + ks * 16 + hh * 8];
+#pragma unroll
+                for (int qb = 0; qb < NQB; qb++)
+                    s[qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[qb][ks], s[qb], 0, 0, 0);
+            }
+
+            // ---- soft cap, mask (these paths subtract m explicitly), key tail -----------------------
+            if (SOFTCAP) {
+                const float c2 = a.softcap * LOG2E;
+#pragma unroll
+                for (int qb = 0; qb < NQB; qb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) s[qb][r] = c2 * fast_tanh(s[qb][r]);
+            }
+            if (MASK) {
+#pragma unroll
+                for (int qb = 0; qb < NQB; qb++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const uint32_t w[2] = {mraw[qb][kb][g].x, mraw[qb][kb][g].y};
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const float mv = h2f_bits((uint16_t)(w[e >> 1] >> (16 * (e & 1))));
+                            s[qb][g * 4 + e] = fmaf(mslope, mv, s[qb][g * 4 + e]);
+                        }
                     }
             }
-        }
-        if (tail) {
+            if (MASK || SOFTCAP) {
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+                for (int qb = 0; qb < NQB; qb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) s[qb][r] -= st[qb].m;
+            }
+            if (TAIL) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int key = j0 + kb * 32 + (r >> 2) * 8 + hh * 4 + (r & 3);
                     if (key >= a.Nkv) {
 #pragma unroll
-                        for (int qb = 0; qb < NQB; qb++) s[kb][qb][r] = -INFINITY;
+                        for (int qb = 0; qb < NQB; qb++) s[qb][r] = -INFINITY;
                     }
                 }
-        }
+            }
 
-        // ---- online softmax (base 2) and P in f16 -----------------------------------------------
-        half8 preg[NQB][4];
+            // ---- keep the reference within RESCALE_SLACK of the running maximum --------------------------
+            float tmax[NQB];
+            bool  raise = false;
 #pragma unroll
-        for (int qb = 0; qb < NQB; qb++) {
-            float mloc = -INFINITY;
+            for (int qb = 0; qb < NQB; qb++) {
+                float mx = s[qb][0];
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+                for (int r = 1; r < 16; r++) mx = fmaxf(mx, s[qb][r]);
+                tmax[qb] = mx;
+                raise = raise || (mx > RESCALE_SLACK) || (!st[qb].have && mx > -INFINITY);
+            }
+            if (__builtin_amdgcn_ballot_w64(raise) != 0) {       // wave-uniform: rare after the first block
 #pragma unroll
-                for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, s[kb][qb][r]);
-            mloc = fmaxf(mloc, xor_shuffle(mloc, 32));
-            const float m_new = fmaxf(m_run[qb], mloc);
-            const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-            const float alpha = __builtin_amdgcn_exp2f(m_run[qb] - m_use);
-            float lsum = 0.0f;
+                for (int qb = 0; qb < NQB; qb++) {
+                    const float tm = max_xor32(tmax[qb]);        // both halves of a query must agree
+                    float delta = 0.0f;
+                    if (tm > -INFINITY) {
+                        delta = st[qb].have ? fmaxf(tm, 0.0f) : tm;
+                        st[qb].have = true;
+                    }
+                    const float f = __builtin_amdgcn_exp2f(-delta);
+                    st[qb].m += delta;
+                    st[qb].l *= f;
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+                    for (int db = 0; db < DB; db++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const float p = __builtin_amdgcn_exp2f(s[kb][qb][r] - m_use);
-                    lsum += p;
-                    preg[qb][kb * 2 + (r >> 3)][r & 7] = (_Float16)p;
+                        for (int r = 0; r < 16; r++) oacc[qb][db][r] *= f;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) s[qb][r] -= delta;
                 }
-            l_run[qb] = l_run[qb] * alpha + lsum;
-            m_run[qb] = m_new;
-#pragma unroll
-            for (int db = 0; db < DB; db++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) oacc[qb][db][r] *= alpha;
-        }
+            }
 
-        // ---- O^T += V^T . P^T ----------------------------------------------------------------------
+            // ---- P = 2^s in f16; the row sum is taken over the rounded values the MFMA will use -----------
+            half8 preg[NQB][2];
+            const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
+            for (int qb = 0; qb < NQB; qb++) {
+                float lsum = 0.0f;
 #pragma unroll
-            for (int db = 0; db < DB; db++) {
-                // transpose read: lane i of a 16-lane block addresses 4 halves of key (i/4) at d0 + 4*(i%4)
-                const int i16 = lane & 15;
-                const int d0  = db * 32 + ((lane >> 4) & 1) * 16;
-                const int kr  = kk * 16 + hh * 4 + (i16 >> 2);
-                const _Float16 * p0 = &v_lds[buf][kr * PV + d0 + (i16 & 3) * 4];
-                const _Float16 * p1 = p0 + 8 * PV;
-                const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p0);
-                const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p1);
-                half8 va;
-                const half4 lo4 = __builtin_bit_cast(half4, lo);
-                const half4 hi4 = __builtin_bit_cast(half4, hi);
-                va[0] = lo4[0]; va[1] = lo4[1]; va[2] = lo4[2]; va[3] = lo4[3];
-                va[4] = hi4[0]; va[5] = hi4[1]; va[6] = hi4[2]; va[7] = hi4[3];
+                for (int r = 0; r < 16; r += 2) {
+                    half2v p2;
+                    p2[0] = (_Float16)__builtin_amdgcn_exp2f(s[qb][r]);
+                    p2[1] = (_Float16)__builtin_amdgcn_exp2f(s[qb][r + 1]);
+                    lsum = __builtin_amdgcn_fdot2(p2, ones, lsum, false);
+                    preg[qb][r >> 3][r & 7]       = p2[0];
+                    preg[qb][r >> 3][(r & 7) + 1] = p2[1];
+                }
+                st[qb].l += lsum;
+            }
+
+            // ---- O^T += V^T . P^T ------------------------------------------------------------------------------
 #pragma unroll
-                for (int qb = 0; qb < NQB; qb++)
-                    oacc[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, preg[qb][kk], oacc[qb][db], 0, 0, 0);
+            for (int k2 = 0; k2 < 2; k2++) {
+                const int kk = kb * 2 + k2;
+#pragma unroll
+                for (int db = 0; db < DB; db++) {
+                    // transpose read: lane i of a 16-lane block addresses 4 halves of key (i/4) at d0 + 4*(i%4)
+                    const int i16 = lane & 15;
+                    const int d0  = db * 32 + ((lane >> 4) & 1) * 16;
+                    const int kr  = kk * 16 + hh * 4 + (i16 >> 2);
+                    const _Float16 * p0 = &v_lds[buf][kr * PV + d0 + (i16 & 3) * 4];
+                    const _Float16 * p1 = p0 + 8 * PV;
+                    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p0);
+                    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p1);
+                    half8 va;
+                    const half4 lo4 = __builtin_bit_cast(half4, lo);
+                    const half4 hi4 = __builtin_bit_cast(half4, hi);
+                    va[0] = lo4[0]; va[1] = lo4[1]; va[2] = lo4[2]; va[3] = lo4[3];
+                    va[4] = hi4[0]; va[5] = hi4[1]; va[6] = hi4[2]; va[7] = hi4[3];
+#pragma unroll
+                    for (int qb = 0; qb < NQB; qb++)
+                        oacc[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, preg[qb][k2], oacc[qb][db], 0, 0, 0);
+                }
             }
         }
+    };
 
+    const int n_tiles = (a.Nkv + BC - 1) / BC;
+    const int n_full  = a.Nkv / BC;
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+
+    // full tiles: the steady-state loop carries no tail handling at all
+    for (int t = 0; t < n_full; t++) {
+        const int  buf  = t & 1;
+        const bool more = t + 1 < n_tiles;
+        if (more) load_tile((t + 1) * BC);
+        tile(t * BC, buf, std::false_type{});
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
+    // at most one partial tile, already staged by the last iteration above (or the prologue)
+    if (n_full < n_tiles) tile(n_full * BC, n_full & 1, std::true_type{});
 
     // ---- normalise and write dst[D, Hq, Nq, B] -------------------------------------------------------
 #pragma unroll
     for (int qb = 0; qb < NQB; qb++) {
-        const float ltot = l_run[qb] + xor_shuffle(l_run[qb], 32);
+        const float ltot = sum_xor32(st[qb].l);
         const float inv  = ltot > 0.0f ? 1.0f / ltot : 0.0f;
         const int   qi   = q0 + qb * 32 + l32;
         if (qi < a.Nq) {
@@ -349,7 +421,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     }
 }
 
-template <int D, int NQB, int TYPE>
+template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP>
 int launch(const FattnArgs & a, hipStream_t stream) {
     const int bmg = 32 * NQB * MMA_WAVES;
     const int n_qtiles = (a.Nq + bmg - 1) / bmg;
@@ -357,13 +429,20 @@ int launch(const FattnArgs & a, hipStream_t stream) {
     const size_t lds = (size_t)2 * BC * (Pitch<D>::K + Pitch<D>::V) * sizeof(_Float16);
     static bool attr_set = false;     // per instantiation; the attribute only matters above 64 KiB
     if (!attr_set && lds > 64 * 1024) {
-        const hipError_t e = hipFuncSetAttribute((const void *)fattn_mma_kernel<D, NQB, TYPE>,
+        const hipError_t e = hipFuncSetAttribute((const void *)fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
         attr_set = true;
     }
-    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, TYPE>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
+    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
     return (int)hipGetLastError();
+}
+
+template <int D, int NQB, int TYPE>
+int launch_flags(const FattnArgs & a, hipStream_t stream) {
+    const bool mask = a.mask != nullptr;
+    if (a.softcap != 0.0f) return mask ? launch<D, NQB, TYPE, true, true>(a, stream) : launch<D, NQB, TYPE, false, true>(a, stream);
+    return mask ? launch<D, NQB, TYPE, true, false>(a, stream) : launch<D, NQB, TYPE, false, false>(a, stream);
 }
 
 template <int TYPE>
@@ -372,8 +451,8 @@ int launch_type(const FattnArgs & a, hipStream_t stream) {
     // workgroups in flight when there are few queries
     const int64_t wg2 = (int64_t)((a.Nq + 255) / 256) * a.Hq * a.B;
     const bool two = wg2 >= 128;
-    if (a.D == 64)  return two ? launch<64, 2, TYPE>(a, stream) : launch<64, 1, TYPE>(a, stream);
-    if (a.D == 128) return launch<128, 1, TYPE>(a, stream);
+    if (a.D == 64)  return two ? launch_flags<64, 2, TYPE>(a, stream) : launch_flags<64, 1, TYPE>(a, stream);
+    if (a.D == 128) return launch_flags<128, 1, TYPE>(a, stream);
     return (int)hipErrorInvalidValue;
 }
 
