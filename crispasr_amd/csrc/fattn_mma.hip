@@ -23,6 +23,8 @@
 // Softmax runs in base 2: scale*log2(e) is folded into Q when it is converted to f16.
 #include "fattn_common.h"
 
+#include <stdio.h>
+#include <stdlib.h>
 #include <type_traits>
 
 namespace {
@@ -104,15 +106,16 @@ __device__ __forceinline__ float fast_tanh(float x) {
 }
 
 // Running softmax state of one 32-query block, per lane (= per query, mirrored in lane l^32).
-// Scores are kept relative to `m`, a reference that trails the true running maximum by at
-// most RESCALE_SLACK (in log2 units): it is folded into the accumulator's initial value, so
-// the common tile needs no subtraction and no rescale of O.
+// Scores are kept relative to `m`, a reference that may trail the true running maximum by up
+// to 13 (in log2 units, see SUM_LIMIT): it enters the Q.K^T MFMA as its C operand, so the
+// common block needs no subtraction, no maximum and no rescale of O.
 struct RowState {
     float m;        // reference subtracted from the scores (finite)
     float l;        // sum of p over this lane's keys
     bool  have;     // a finite score has been seen
 };
-constexpr float RESCALE_SLACK = 8.0f;
+// a block of 16 probabilities summing to more than this means the reference is > 9 behind
+constexpr float SUM_LIMIT = 8192.0f;
 
 template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP>
 __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnArgs a, const int n_qtiles) {
@@ -208,12 +211,15 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     };
 
     float16v oacc[NQB][DB];
+    float16v negm[NQB];            // -m in all 16 slots: the C operand of the first Q.K^T MFMA
     RowState st[NQB];
 #pragma unroll
     for (int qb = 0; qb < NQB; qb++) {
         st[qb].m = 0.0f;
         st[qb].l = 0.0f;
         st[qb].have = false;
+#pragma unroll
+        for (int r = 0; r < 16; r++) negm[qb][r] = 0.0f;
 #pragma unroll
         for (int db = 0; db < DB; db++)
 #pragma unroll
@@ -246,24 +252,58 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                     }
         }
 
+        // K operands of a 32-key block: KS 128-bit reads per lane
+        auto load_k = [&](int kb, half8 (&ka)[KS]) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++)
+                ka[ks] = *(const half8 *)&k_lds[buf][(kb * 32 + l32) * PK + ks * 16 + hh * 8];
+        };
+        // V^T operands of a 32-key block by transpose reads: lane i of a 16-lane block addresses
+        // 4 halves of key (i/4) at d0 + 4*(i%4) and receives 4 keys' values of d0 + i
+        auto load_v = [&](int kb, half8 (&va)[2][DB]) {
+            const int i16 = lane & 15;
+#pragma unroll
+            for (int k2 = 0; k2 < 2; k2++)
+#pragma unroll
+                for (int db = 0; db < DB; db++) {
+                    const int d0 = db * 32 + ((lane >> 4) & 1) * 16;
+                    const int kr = (kb * 2 + k2) * 16 + hh * 4 + (i16 >> 2);
+                    const _Float16 * p0 = &v_lds[buf][kr * PV + d0 + (i16 & 3) * 4];
+                    const _Float16 * p1 = p0 + 8 * PV;
+                    const half4 lo = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p0));
+                    const half4 hi = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p1));
+                    va[k2][db] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+        };
+
+        // with few reduction steps the next block's K operands are requested a block ahead
+        constexpr bool K_AHEAD = KS <= 4;
+        half8 ka[K_AHEAD ? 2 : 1][KS];
+        load_k(0, ka[0]);
+
         // the tile is consumed in two blocks of 32 keys to keep the score registers few
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
-            // ---- S^T = K . Q^T - m  (the reference m enters as the accumulator's initial value) ----
+            // ---- S^T = K . Q^T - m  (the reference m enters as the C operand of the first MFMA) ----
             float16v s[NQB];
 #pragma unroll
             for (int qb = 0; qb < NQB; qb++) {
-                const float init = (MASK || SOFTCAP) ? 0.0f : -st[qb].m;
+                if (MASK || SOFTCAP) {
 #pragma unroll
-                for (int r = 0; r < 16; r++) s[qb][r] = init;
+                    for (int r = 0; r < 16; r++) s[qb][r] = 0.0f;
+                } else {
+                    s[qb] = negm[qb];
+                }
             }
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                const half8 ka = *(const half8 *)&k_lds[buf][(kb * 32 + l32) * PK + ks * 16 + hh * 8];
+            for (int ks = 0; ks < KS; ks++)
 #pragma unroll
                 for (int qb = 0; qb < NQB; qb++)
-                    s[qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qreg[qb][ks], s[qb], 0, 0, 0);
-            }
+                    s[qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[K_AHEAD ? kb : 0][ks], qreg[qb][ks], s[qb], 0, 0, 0);
+            // operands needed next are requested now, so their LDS latency hides behind the softmax
+            half8 va[2][DB];
+            load_v(kb, va);
+            if (kb == 0) load_k(1, ka[K_AHEAD ? 1 : 0]);
 
             // ---- soft cap, mask (these paths subtract m explicitly), key tail -----------------------
             if (SOFTCAP) {
@@ -303,21 +343,38 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                 }
             }
 
-            // ---- keep the reference within RESCALE_SLACK of the running maximum --------------------------
-            float tmax[NQB];
-            bool  raise = false;
+            // ---- P = 2^s in f16; the row sum is taken over the rounded values the MFMA will use -----------
+            // No maximum is computed on this path: a reference that has fallen too far behind shows up
+            // as a large (or infinite) block sum, and only then is the block redone with a new reference.
+            half8 preg[NQB][2];
+            float lsum[NQB];
+            const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+            auto exp_block = [&](int qb) {
+                float acc = 0.0f;
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) {
+                    half2v p2;
+                    p2[0] = (_Float16)__builtin_amdgcn_exp2f(s[qb][r]);
+                    p2[1] = (_Float16)__builtin_amdgcn_exp2f(s[qb][r + 1]);
+                    acc = __builtin_amdgcn_fdot2(p2, ones, acc, false);
+                    preg[qb][r >> 3][r & 7]       = p2[0];
+                    preg[qb][r >> 3][(r & 7) + 1] = p2[1];
+                }
+                lsum[qb] = acc;
+            };
+            bool redo = false;
 #pragma unroll
             for (int qb = 0; qb < NQB; qb++) {
-                float mx = s[qb][0];
-#pragma unroll
-                for (int r = 1; r < 16; r++) mx = fmaxf(mx, s[qb][r]);
-                tmax[qb] = mx;
-                raise = raise || (mx > RESCALE_SLACK) || (!st[qb].have && mx > -INFINITY);
+                exp_block(qb);
+                redo = redo || !(lsum[qb] <= SUM_LIMIT) || !st[qb].have;
             }
-            if (__builtin_amdgcn_ballot_w64(raise) != 0) {       // wave-uniform: rare after the first block
+            if (__builtin_amdgcn_ballot_w64(redo) != 0) {        // wave-uniform; rare after the first block
 #pragma unroll
                 for (int qb = 0; qb < NQB; qb++) {
-                    const float tm = max_xor32(tmax[qb]);        // both halves of a query must agree
+                    float mx = s[qb][0];
+#pragma unroll
+                    for (int r = 1; r < 16; r++) mx = fmaxf(mx, s[qb][r]);
+                    const float tm = max_xor32(mx);              // both halves of a query must agree
                     float delta = 0.0f;
                     if (tm > -INFINITY) {
                         delta = st[qb].have ? fmaxf(tm, 0.0f) : tm;
@@ -327,56 +384,27 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                     st[qb].m += delta;
                     st[qb].l *= f;
 #pragma unroll
+                    for (int r = 0; r < 16; r++) negm[qb][r] = -st[qb].m;
+#pragma unroll
                     for (int db = 0; db < DB; db++)
 #pragma unroll
                         for (int r = 0; r < 16; r++) oacc[qb][db][r] *= f;
 #pragma unroll
                     for (int r = 0; r < 16; r++) s[qb][r] -= delta;
+                    exp_block(qb);
                 }
             }
-
-            // ---- P = 2^s in f16; the row sum is taken over the rounded values the MFMA will use -----------
-            half8 preg[NQB][2];
-            const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
-            for (int qb = 0; qb < NQB; qb++) {
-                float lsum = 0.0f;
-#pragma unroll
-                for (int r = 0; r < 16; r += 2) {
-                    half2v p2;
-                    p2[0] = (_Float16)__builtin_amdgcn_exp2f(s[qb][r]);
-                    p2[1] = (_Float16)__builtin_amdgcn_exp2f(s[qb][r + 1]);
-                    lsum = __builtin_amdgcn_fdot2(p2, ones, lsum, false);
-                    preg[qb][r >> 3][r & 7]       = p2[0];
-                    preg[qb][r >> 3][(r & 7) + 1] = p2[1];
-                }
-                st[qb].l += lsum;
-            }
+            for (int qb = 0; qb < NQB; qb++) st[qb].l += lsum[qb];
 
             // ---- O^T += V^T . P^T ------------------------------------------------------------------------------
 #pragma unroll
-            for (int k2 = 0; k2 < 2; k2++) {
-                const int kk = kb * 2 + k2;
+            for (int k2 = 0; k2 < 2; k2++)
 #pragma unroll
-                for (int db = 0; db < DB; db++) {
-                    // transpose read: lane i of a 16-lane block addresses 4 halves of key (i/4) at d0 + 4*(i%4)
-                    const int i16 = lane & 15;
-                    const int d0  = db * 32 + ((lane >> 4) & 1) * 16;
-                    const int kr  = kk * 16 + hh * 4 + (i16 >> 2);
-                    const _Float16 * p0 = &v_lds[buf][kr * PV + d0 + (i16 & 3) * 4];
-                    const _Float16 * p1 = p0 + 8 * PV;
-                    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p0);
-                    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p1);
-                    half8 va;
-                    const half4 lo4 = __builtin_bit_cast(half4, lo);
-                    const half4 hi4 = __builtin_bit_cast(half4, hi);
-                    va[0] = lo4[0]; va[1] = lo4[1]; va[2] = lo4[2]; va[3] = lo4[3];
-                    va[4] = hi4[0]; va[5] = hi4[1]; va[6] = hi4[2]; va[7] = hi4[3];
+                for (int db = 0; db < DB; db++)
 #pragma unroll
                     for (int qb = 0; qb < NQB; qb++)
-                        oacc[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, preg[qb][k2], oacc[qb][db], 0, 0, 0);
-                }
-            }
+                        oacc[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[k2][db], preg[qb][k2], oacc[qb][db], 0, 0, 0);
         }
     };
 
@@ -433,6 +461,13 @@ int launch(const FattnArgs & a, hipStream_t stream) {
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
         attr_set = true;
+    }
+    static const bool debug = getenv("MI355X_FATTN_DEBUG") != nullptr;
+    if (debug) {
+        int nb = -1;
+        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void *)fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP>, MMA_THREADS, lds);
+        fprintf(stderr, "[mi355x] fattn_mma<%d,%d,%d,%d,%d> grid %u lds %zu B, resident workgroups per CU: %d\n",
+                D, NQB, TYPE, (int)MASK, (int)SOFTCAP, grid.x, lds, nb);
     }
     hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
     return (int)hipGetLastError();

@@ -29,7 +29,8 @@ PREC_DEFAULT, PREC_F32 = 0, 10
 OK, ERR_UNSUPPORTED, ERR_INVALID, ERR_HIP, ERR_NO_DEVICE, ERR_WORKSPACE = range(6)
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmi355x_fattn.so")
+# MI355X_FATTN_LIB points at an alternative build of the same library (e.g. one compiled with other flags)
+LIB_PATH = os.environ.get("MI355X_FATTN_LIB") or os.path.join(_HERE, "libmi355x_fattn.so")
 
 
 class Mi355xError(RuntimeError):
