@@ -159,78 +159,113 @@ def cpu_baseline(args, ora, host0):
 
 
 def bench_decode(args, ca, ora, torch):
-    """HBM-bound decode shapes: per-call GB/s over all layers of a step with distinct per-layer
-    buffers (cache-cold: the rotating working set exceeds the 256 MB Infinity Cache)."""
+    """HBM-bound decode shapes.  Each figure is the mean time of one FLASH_ATTN_EXT call inside a HIP graph
+    that replays one call per layer over distinct per-layer buffers (no host launch overhead between
+    calls); `rotating_MB` says how much distinct K/V a replay touches, against the 256 MB Infinity Cache.
+    Bytes are the algorithmic ones: Q f32 + K,V in storage type once per KV head + mask f16 + out f32."""
     import numpy as np
     out = {}
 
-    def run(name, layers, scale, bytes_per_layer, reps):
+    def run(name, layers, scale, bytes_per_call, reps, note):
         def step():
             for dev in layers:
                 ca.flash_attn_ext(dev["q"], dev["k"], dev["v"], dev.get("mask"), scale, out=dev["out"])
-        for _ in range(3):
-            step()
+        for _ in range(2):
+            step()                                   # also sizes the library's split-KV scratch
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                step()
+        torch.cuda.synchronize()
+        graph.replay()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(reps):
-            step()
+            graph.replay()
         e1.record()
         torch.cuda.synchronize()
         us = e0.elapsed_time(e1) * 1e3 / (reps * len(layers))
-        gbs = bytes_per_layer / (us * 1e-6) / 1e9
+        gbs = bytes_per_call / (us * 1e-6) / 1e9
         kern, ns = ca.ggml.flash_attn_plan(layers[0]["q"], layers[0]["k"], layers[0]["v"], layers[0].get("mask"), scale)
         out[name] = {"us_per_call": us, "GB/s": gbs, "frac_of_hbm_peak": gbs / PEAK_HBM_GBS,
-                     "bytes_per_call": bytes_per_layer, "layers_rotated": len(layers), "kernel": kern, "n_splits": ns}
+                     "bytes_per_call": bytes_per_call, "calls_per_replay": len(layers),
+                     "rotating_MB": bytes_per_call * len(layers) / 1e6, "kernel": kern, "n_splits": ns, "note": note}
         log(f"[bench] decode {name}: {us:.2f} us/call, {gbs:.0f} GB/s ({100 * gbs / PEAK_HBM_GBS:.1f}% of HBM peak), "
             f"kernel {kern}, splits {ns}")
 
-    # Whisper large-v3 cross-attention, beam 5: 5 queries vs one shared 1500-entry f16 K/V, 20 heads x 64
-    D, H, Nkv, NL = 64, 20, 1500, 64
+    def f16_buf(n):
+        return torch.randn(n, device="cuda").half().view(torch.uint8)
+
+    def q8_buf(seed, n):
+        return torch.from_numpy(ora.quantize_q8_0(ora.randn(seed, (n,)))).cuda()
+
+    # Whisper large-v3 decoder step, beam 5, 20 heads x 64 (strides of the [token][head][dim] cache)
+    D, H = 64, 20
+    n_state = D * H
+    Nkv, NL = 1500, 64
     layers = []
     for l in range(NL):
-        k = torch.randn(Nkv * H * D, device="cuda").half().view(torch.uint8)
-        v = torch.randn(Nkv * H * D, device="cuda").half().view(torch.uint8)
-        q = torch.randn(5 * H * D, device="cuda").view(torch.uint8)
-        nbk = (2, 2 * H * D, 2 * D, 2 * H * D * Nkv)
-        layers.append({"q": ca.Tensor(q, ca.F32, (D, 5, H, 1), (4, 4 * H * D, 4 * D, 4 * H * D * 5)),
-                       "k": ca.Tensor(k, ca.F16, (D, Nkv, H, 1), nbk), "v": ca.Tensor(v, ca.F16, (D, Nkv, H, 1), nbk),
+        nbk = (2, 2 * n_state, 2 * D, 2 * n_state * Nkv)
+        layers.append({"q": ca.Tensor(torch.randn(5 * n_state, device="cuda").view(torch.uint8), ca.F32, (D, 5, H, 1),
+                                      (4, 4 * n_state, 4 * D, 4 * n_state * 5)),
+                       "k": ca.Tensor(f16_buf(Nkv * n_state), ca.F16, (D, Nkv, H, 1), nbk),
+                       "v": ca.Tensor(f16_buf(Nkv * n_state), ca.F16, (D, Nkv, H, 1), nbk),
                        "out": ca.Tensor.empty(ca.F32, (D, H, 5, 1))})
-    bytes_ = 2 * Nkv * H * D * 2 + 2 * 5 * H * D * 4
-    run("whisper_cross_beam5_f16", layers, 64 ** -0.25, bytes_, 20)
-
-    # Voxtral-style LLM decode: 32 q heads / 8 kv heads, D 128, Q8_0 cache of 663 entries
-    D, Hq, Hkv, Lk, NL = 128, 32, 8, 663, 60
+    run("whisper_cross_beam5_f16", layers, 64 ** -0.25, 2 * Nkv * n_state * 2 + 2 * 5 * n_state * 4, 10,
+        "5 queries vs one shared 1500-entry f16 K/V per layer")
+    Lk, NL = 224, 64
     layers = []
-    rs = 136
+    mask = np.zeros((5, 1, 1, Lk), np.float32)
+    for b in range(5):
+        mask[b, 0, 0, ora.randint(31, b, 1, Lk):] = -np.inf
+    mask_d = ca.Tensor.from_host(ora.fp32_to_fp16(mask), ca.F16, (Lk, 1, 1, 5))
     for l in range(NL):
-        kf = ora.randn(900 + l, (Hkv * Lk * D,))
-        raw = ora.quantize_q8_0(kf)
-        k = torch.from_numpy(raw).cuda()
-        v = torch.from_numpy(ora.quantize_q8_0(kf[::-1].copy())).cuda()
-        q = torch.randn(Hq * D, device="cuda").view(torch.uint8)
-        nbk = (34, rs, rs * Lk, rs * Lk * Hkv)
-        layers.append({"q": ca.Tensor(q, ca.F32, (D, 1, Hq, 1)),
-                       "k": ca.Tensor(k, ca.Q8_0, (D, Lk, Hkv, 1), nbk), "v": ca.Tensor(v, ca.Q8_0, (D, Lk, Hkv, 1), nbk),
-                       "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 1))})
-    bytes_ = 2 * Lk * Hkv * rs + 2 * Hq * D * 4
-    run("voxtral_decode_q8_0_gqa4", layers, 128 ** -0.5, bytes_, 20)
+        nbk = (2, 2 * n_state, 2 * D, 2 * n_state * Lk)
+        layers.append({"q": ca.Tensor(torch.randn(5 * n_state, device="cuda").view(torch.uint8), ca.F32, (D, 1, H, 5),
+                                      (4, 4 * n_state, 4 * D, 4 * n_state)),
+                       "k": ca.Tensor(f16_buf(5 * Lk * n_state), ca.F16, (D, Lk, H, 5), nbk),
+                       "v": ca.Tensor(f16_buf(5 * Lk * n_state), ca.F16, (D, Lk, H, 5), nbk),
+                       "mask": mask_d, "out": ca.Tensor.empty(ca.F32, (D, H, 1, 5))})
+    run("whisper_self_beam5_f16", layers, 1.0, 5 * (2 * Lk * n_state * 2 + 2 * n_state * 4 + Lk * 2), 10,
+        "1 query per beam vs its own 224-entry f16 cache, -inf mask beyond each beam's position")
 
-    # saturating variant: the same Q8_0 decode with 64 independent sequences (ne3) per call
-    Bs = 64
-    kf = ora.randn(990, (Bs * Hkv * Lk * D,))
-    k = torch.from_numpy(ora.quantize_q8_0(kf)).cuda()
-    v = torch.from_numpy(ora.quantize_q8_0(kf[::-1].copy())).cuda()
+    # Voxtral-style LLM decode: 32 q heads / 8 kv heads, D 128, Q8_0 cache of 663 entries (last of 256 steps)
+    D, Hq, Hkv, Lk, NL = 128, 32, 8, 663, 240
+    rs = 136
+    nbk = (34, rs, rs * Lk, rs * Lk * Hkv)
     layers = []
-    for l in range(8):
-        q = torch.randn(Bs * Hq * D, device="cuda").view(torch.uint8)
-        nbk = (34, rs, rs * Lk, rs * Lk * Hkv)
-        layers.append({"q": ca.Tensor(q, ca.F32, (D, 1, Hq, Bs)),
-                       "k": ca.Tensor(k.clone(), ca.Q8_0, (D, Lk, Hkv, Bs), nbk),
-                       "v": ca.Tensor(v.clone(), ca.Q8_0, (D, Lk, Hkv, Bs), nbk),
+    for l in range(NL):
+        layers.append({"q": ca.Tensor(torch.randn(Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, 1)),
+                       "k": ca.Tensor(q8_buf(900 + 2 * l, Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, 1), nbk),
+                       "v": ca.Tensor(q8_buf(901 + 2 * l, Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, 1), nbk),
+                       "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 1))})
+    per_call = 2 * Lk * Hkv * rs + 2 * Hq * D * 4
+    run("voxtral_decode_q8_0_gqa4", layers, 128 ** -0.5, per_call, 10,
+        "1 token, 32 q / 8 kv heads, Q8_0 K/V of 663 entries; 1.44 MB per call")
+
+    # saturating variants: the same kernels with many independent sequences per call (ne3), to show
+    # the bandwidth ceiling that single calls of 1-8 MB cannot reach
+    Bs = 64
+    layers = []
+    for l in range(6):
+        layers.append({"q": ca.Tensor(torch.randn(Bs * Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, Bs)),
+                       "k": ca.Tensor(q8_buf(990 + 2 * l, Bs * Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, Bs), nbk),
+                       "v": ca.Tensor(q8_buf(991 + 2 * l, Bs * Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, Bs), nbk),
                        "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, Bs))})
-    bytes_ = Bs * (2 * Lk * Hkv * rs + 2 * Hq * D * 4)
-    run("voxtral_decode_q8_0_gqa4_x64seq", layers, 128 ** -0.5, bytes_, 20)
+    run("voxtral_decode_q8_0_gqa4_x64seq", layers, 128 ** -0.5, Bs * per_call, 10, "64 sequences per call")
+    Lk = 4096
+    nbk = (2, 2 * D, 2 * D * Lk, 2 * D * Lk * Hkv)
+    layers = []
+    for l in range(6):
+        layers.append({"q": ca.Tensor(torch.randn(16 * Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, 16)),
+                       "k": ca.Tensor(f16_buf(16 * Hkv * Lk * D), ca.F16, (D, Lk, Hkv, 16), nbk),
+                       "v": ca.Tensor(f16_buf(16 * Hkv * Lk * D), ca.F16, (D, Lk, Hkv, 16), nbk),
+                       "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 16))})
+    run("llm_decode_f16_gqa4_4096x16seq", layers, 128 ** -0.5, 16 * (2 * Lk * Hkv * D * 2 + 2 * Hq * D * 4), 10,
+        "16 sequences x 4096-entry f16 cache per call")
     return out
 
 

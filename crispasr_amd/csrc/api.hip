@@ -177,6 +177,10 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
         kv16 = kv16 && !(k->nb[i] % 16) && !(v->nb[i] % 16);
     }
     a.q_aligned16 = q16 ? 1 : 0;
+    a.kv_aligned16 = kv16 ? 1 : 0;
+    bool kv4 = !((uintptr_t)k->data % 4) && !((uintptr_t)v->data % 4);
+    for (int i = 1; i < 4; i++) kv4 = kv4 && !(k->nb[i] % 4) && !(v->nb[i] % 4);
+    a.kv_aligned4 = kv4 ? 1 : 0;
     const bool al16 = q16 && kv16;
     if (a.mask) {
         a.Hm = (int)mask->ne[2]; a.Bm = (int)mask->ne[3];
@@ -201,26 +205,31 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
 void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Plan & plan) {
     int kernel = p->kernel;
     if (kernel == MI355X_FATTN_AUTO) {
-        kernel = (a.Nq >= 16 && fattn_mma_supported(a, ktype)) ? MI355X_FATTN_MMA : MI355X_FATTN_VEC;
+        if (fattn_decode_supported(a, ktype))                 kernel = MI355X_FATTN_DECODE_MMA;   // <= 16 rows per KV head
+        else if (a.Nq >= 16 && fattn_mma_supported(a, ktype)) kernel = MI355X_FATTN_MMA;
+        else                                                  kernel = MI355X_FATTN_VEC;
     }
     plan.kernel = kernel;
     plan.n_splits = 1;
     plan.keys_per_split = a.Nkv;
     plan.workspace = 0;
-    if (kernel == MI355X_FATTN_VEC) {
+    if (kernel == MI355X_FATTN_VEC || kernel == MI355X_FATTN_DECODE_MMA) {
         const int64_t rows = (int64_t)a.Nq * a.Hq * a.B;
+        // workgroups that exist before splitting, and the fewest keys worth a split
+        const int64_t groups   = kernel == MI355X_FATTN_VEC ? rows : (int64_t)a.Hkv * a.B;
+        const int     min_keys = kernel == MI355X_FATTN_VEC ? 128 : 256;
         int ns = p->n_splits;
         if (ns <= 0) {
-            // enough workgroups to fill the chip, but at least 128 keys per split
-            const int64_t target = (int64_t)device_cus() * 4;
-            ns = (int)((target + rows - 1) / (rows > 0 ? rows : 1));
-            const int max_by_keys = (a.Nkv + 127) / 128;
+            const int64_t target = (int64_t)device_cus() * (kernel == MI355X_FATTN_VEC ? 4 : 2);
+            ns = (int)((target + groups - 1) / (groups > 0 ? groups : 1));
+            const int max_by_keys = (a.Nkv + min_keys - 1) / min_keys;
             if (ns > max_by_keys) ns = max_by_keys;
         }
         if (ns > a.Nkv) ns = a.Nkv;
         if (ns < 1) ns = 1;
         if (ns > 256) ns = 256;
         int kps = (a.Nkv + ns - 1) / ns;
+        if (kernel == MI355X_FATTN_DECODE_MMA) kps = (kps + 31) / 32 * 32;     // whole wave steps
         if (kps < 1) kps = 1;
         ns = a.Nkv > 0 ? (a.Nkv + kps - 1) / kps : 1;
         plan.n_splits = ns;
@@ -353,7 +362,11 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
         if (e) return hip_fail((hipError_t)e, "fattn_mma launch");
         return MI355X_OK;
     }
-    if (plan.kernel != MI355X_FATTN_VEC) return fail(MI355X_ERR_UNSUPPORTED, "kernel %d not available", plan.kernel);
+    if (plan.kernel == MI355X_FATTN_DECODE_MMA) {
+        if (!fattn_decode_supported(a, k->type)) return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the decode kernel");
+    } else if (plan.kernel != MI355X_FATTN_VEC) {
+        return fail(MI355X_ERR_UNSUPPORTED, "kernel %d not available", plan.kernel);
+    }
 
     a.n_splits = plan.n_splits;
     a.keys_per_split = plan.keys_per_split;
@@ -370,8 +383,8 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
         a.part_acc = (float *)ws;
         a.part_ml  = a.part_acc + rows * plan.n_splits * a.D;
     }
-    int e = fattn_vec_launch(a, k->type, st);
-    if (e) return hip_fail((hipError_t)e, "fattn_vec launch");
+    int e = plan.kernel == MI355X_FATTN_VEC ? fattn_vec_launch(a, k->type, st) : fattn_decode_launch(a, k->type, st);
+    if (e) return hip_fail((hipError_t)e, "split-KV kernel launch");
     if (plan.n_splits > 1) {
         e = fattn_merge_launch(a, st);
         if (e) return hip_fail((hipError_t)e, "fattn_merge launch");

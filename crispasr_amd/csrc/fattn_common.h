@@ -34,6 +34,8 @@ struct FattnArgs {
 
     int32_t aligned16;   // q, k and v bases and strides are all multiples of 16 bytes
     int32_t q_aligned16; // q alone
+    int32_t kv_aligned16; // k and v alone
+    int32_t kv_aligned4;
     int32_t mask_al8;    // mask base and strides are multiples of 8 bytes
 
     // split-KV
@@ -104,5 +106,7 @@ int fattn_vec_launch(const FattnArgs & a, int ktype, hipStream_t stream);
 int fattn_merge_launch(const FattnArgs & a, hipStream_t stream);
 int fattn_mma_launch(const FattnArgs & a, int ktype, hipStream_t stream);
 bool fattn_mma_supported(const FattnArgs & a, int ktype);
+int fattn_decode_launch(const FattnArgs & a, int ktype, hipStream_t stream);
+bool fattn_decode_supported(const FattnArgs & a, int ktype);
 int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream);
 int set_rows_launch(const CpyArgs & a, int dtype, hipStream_t stream);

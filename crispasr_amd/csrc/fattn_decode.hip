@@ -1,0 +1,366 @@
+// Split-KV MFMA decode kernel for gfx950: few query rows per KV head (beams and/or a GQA group),
+// long KV cache, HBM-bound.
+//
+// A workgroup of 4 waves owns one (KV head, batch, KV split); the up-to-16 query rows that read
+// this KV head - all queries of all q heads in its GQA group - are the 16 columns of
+// v_mfma_f32_16x16x32_f16 tiles, so K and V are fetched from HBM once per KV head, not once per
+// query row.  Each wave walks its share of the split in steps of 32 keys:
+//
+//   S^T[key, row] = K[key, :] . Q[row, :]^T      A = K from global memory in operand layout
+//                                                 (128-bit loads: 16 rows x 64 contiguous bytes)
+//   O^T[d,   row] = V[:, d]^T . P^T[:, row]      A = V^T via a wave-private LDS stage written with
+//                                                 coalesced 128-bit rows and read back with
+//                                                 ds_read_b64_tr_b16; B = P straight from the
+//                                                 accumulator registers of the first product
+//
+// Q8_0 caches are dequantised in registers: the 8 int8 of a lane's chunk are fetched with three
+// aligned dword loads and a byte funnel shift (blocks are 34 bytes, so chunks sit at 2 mod 4),
+// widened to exact f16 integers with v_perm_b32 + one packed add, and scaled by the block's f16 d
+// with one packed multiply (one rounding, = f16(q*d)).  Loads of the next step are in flight while
+// the current one is consumed.  Waves are merged through LDS, splits by fattn_merge_kernel.
+#include "fattn_common.h"
+
+#include <type_traits>
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float    float4v __attribute__((ext_vector_type(4)));
+typedef short    short4v __attribute__((ext_vector_type(4)));
+
+constexpr int   DEC_WAVES   = 4;
+constexpr int   DEC_THREADS = DEC_WAVES * 64;
+constexpr int   STEP        = 32;                  // keys per wave step
+constexpr float LOG2E       = 1.4426950408889634f;
+constexpr float SUM_LIMIT   = 4096.0f;             // 8 probabilities per lane and step
+
+// ---- Q8_0 in registers ------------------------------------------------------------------
+
+// the 8 quants of chunk c (0..3) of block blk of a row whose address is a multiple of 4
+__device__ __forceinline__ uint2 q8_load_chunk(const char * row, int blk, int c) {
+    const int o  = blk * FATTN_Q8_0_BYTES + 2 + c * 8;
+    const int sh = o & 3;                                   // 0 or 2
+    const uint32_t * p = (const uint32_t *)(row + (o - sh));
+    const uint32_t u0 = p[0];
+    const uint32_t u1 = p[1];
+    const uint32_t u2 = sh ? p[2] : 0u;                     // never read past the row when aligned
+    uint2 r;
+    r.x = __builtin_amdgcn_alignbyte(u1, u0, sh);
+    r.y = __builtin_amdgcn_alignbyte(u2, u1, sh);
+    return r;
+}
+
+// 4 int8 packed in a dword -> 4 exact f16 integers: bytes become the low mantissa bits of
+// 1024 + (q + 128), then 1152 is subtracted
+__device__ __forceinline__ void q8_widen(uint32_t w, half2v & lo, half2v & hi) {
+    const uint32_t x = w ^ 0x80808080u;
+    const uint32_t a = __builtin_amdgcn_perm(x, 0x64646464u, 0x00050004u);   // {0x64, b1, 0x64, b0}
+    const uint32_t b = __builtin_amdgcn_perm(x, 0x64646464u, 0x00070006u);   // {0x64, b3, 0x64, b2}
+    const half2v off = {(_Float16)1152.0f, (_Float16)1152.0f};
+    lo = __builtin_bit_cast(half2v, a) - off;
+    hi = __builtin_bit_cast(half2v, b) - off;
+}
+
+__device__ __forceinline__ half8 q8_dequant(uint2 q, uint16_t dbits) {
+    const _Float16 d  = __builtin_bit_cast(_Float16, dbits);
+    const half2v   d2 = {d, d};
+    half2v h0, h1, h2, h3;
+    q8_widen(q.x, h0, h1);
+    q8_widen(q.y, h2, h3);
+    h0 *= d2; h1 *= d2; h2 *= d2; h3 *= d2;
+    half8 r;
+    r[0] = h0[0]; r[1] = h0[1]; r[2] = h1[0]; r[3] = h1[1];
+    r[4] = h2[0]; r[5] = h2[1]; r[6] = h3[0]; r[7] = h3[1];
+    return r;
+}
+
+// raw global data of one 8-element chunk
+struct Chunk {
+    uint4 v;         // f16: the 8 halves; q8_0: x,y = quants, z = scale bits
+};
+
+template <int TYPE>
+__device__ __forceinline__ Chunk load_chunk(const char * row, int c) {
+    Chunk r;
+    if (TYPE == MI355X_TYPE_F16) {
+        r.v = *(const uint4 *)(row + c * 16);
+    } else {
+        const uint2 q = q8_load_chunk(row, c >> 2, c & 3);
+        r.v.x = q.x;
+        r.v.y = q.y;
+        r.v.z = *(const uint16_t *)(row + (c >> 2) * FATTN_Q8_0_BYTES);
+        r.v.w = 0;
+    }
+    return r;
+}
+
+template <int TYPE>
+__device__ __forceinline__ half8 chunk_to_half8(const Chunk & r) {
+    if (TYPE == MI355X_TYPE_F16) return __builtin_bit_cast(half8, r.v);
+    return q8_dequant(make_uint2(r.v.x, r.v.y), (uint16_t)r.v.z);
+}
+
+template <int D, int TYPE, bool MASK>
+__global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const FattnArgs a) {
+    constexpr int KS  = D / 32;                    // reduction steps of Q.K^T (one Q8_0 block each)
+    constexpr int DBK = D / 16;                    // 16-wide blocks of the output's d
+    constexpr int CH  = D / 8;                     // chunks per row
+    constexpr int NV  = STEP * CH / 64;            // V chunks per lane and step
+    constexpr int PV  = D + 32;                    // LDS pitch in halves: 64 mod 128 bytes
+
+    // the per-wave V stages; after the key loop the same memory carries the cross-wave reduction
+    constexpr int STAGE_BYTES = DEC_WAVES * STEP * PV * 2;
+    constexpr int RED_BYTES   = DEC_WAVES * 16 * (D + 1 + 2) * 4;
+    __shared__ __attribute__((aligned(16))) char smem[STAGE_BYTES > RED_BYTES ? STAGE_BYTES : RED_BYTES];
+    _Float16 (*v_lds)[STEP * PV]   = (_Float16 (*)[STEP * PV])smem;
+    float (*red_o)[16][D + 1]      = (float (*)[16][D + 1])smem;
+    float (*red_ml)[16][2]         = (float (*)[16][2])(smem + DEC_WAVES * 16 * (D + 1) * 4);
+
+    const int tid  = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int j    = lane & 15;                    // query column
+    const int g4   = lane >> 4;
+
+    const int split = blockIdx.x % a.n_splits;
+    const int hk    = (blockIdx.x / a.n_splits) % a.Hkv;
+    const int b     = blockIdx.x / (a.n_splits * a.Hkv);
+    const int bk    = b / a.bq;
+
+    // column j = iq1 * gqa + gg  <->  query iq1 of q head hk*gqa + gg
+    const int  R      = a.Nq * a.gqa;
+    const bool col_ok = j < R;
+    const int  jc     = col_ok ? j : 0;
+    const int  iq1    = jc / a.gqa;
+    const int  h      = hk * a.gqa + jc % a.gqa;
+
+    const int k_begin = split * a.keys_per_split;
+    const int k_end   = min(a.Nkv, k_begin + a.keys_per_split);
+
+    // ---- Q -> f16 B operands in log2 units -----------------------------------------------------
+    half8 qreg[KS];
+    {
+        const float * qrow = (const float *)(a.q + (int64_t)iq1 * a.nbq1 + (int64_t)h * a.nbq2 + (int64_t)b * a.nbq3);
+        const float   qs   = a.scale * LOG2E;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            half8 v;
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] = (_Float16)(qrow[ks * 32 + g4 * 8 + e] * qs);
+            qreg[ks] = v;
+        }
+    }
+    const char * kbase = a.k + (int64_t)hk * a.nbk2 + (int64_t)bk * a.nbk3;
+    const char * vbase = a.v + (int64_t)hk * a.nbv2 + (int64_t)bk * a.nbv3;
+    const uint16_t * mrow = MASK
+        ? (const uint16_t *)(a.mask + (int64_t)iq1 * a.nbm1 + (int64_t)(h % a.Hm) * a.nbm2 + (int64_t)(b % a.Bm) * a.nbm3)
+        : nullptr;
+    const float mslope = MASK ? fattn_slope(a, h) * LOG2E : 0.0f;
+
+    float4v oacc[DBK];
+#pragma unroll
+    for (int db = 0; db < DBK; db++) oacc[db] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+    float m = 0.0f, l = 0.0f;
+    bool  have = false;
+
+    // loads of one step: K in operand layout (key = kb*16 + j, chunk = ks*4 + g4), V in row order
+    Chunk kraw[2][2][KS];
+    Chunk vraw[2][NV];
+    auto issue = [&](int j0, auto stage) {
+        constexpr int s = decltype(stage)::value;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            const int key = min(j0 + kb * 16 + j, k_end - 1);
+            const char * row = kbase + (int64_t)key * a.nbk1;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) kraw[s][kb][ks] = load_chunk<TYPE>(row, ks * 4 + g4);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int flat = i * 64 + lane;
+            const int key  = min(j0 + flat / CH, k_end - 1);
+            vraw[s][i] = load_chunk<TYPE>(vbase + (int64_t)key * a.nbv1, flat % CH);
+        }
+    };
+
+    const int n_steps = k_end > k_begin ? (k_end - k_begin + STEP - 1) / STEP : 0;
+    typedef std::integral_constant<int, 0> S0;
+    typedef std::integral_constant<int, 1> S1;
+
+    // one step of 32 keys out of register stage s; the following step is requested into the other stage
+    auto step = [&](const int it, auto stage) {
+        constexpr int s = decltype(stage)::value;
+        const int j0 = k_begin + it * STEP;
+        if (it + DEC_WAVES < n_steps) issue(j0 + DEC_WAVES * STEP, std::integral_constant<int, 1 - s>{});
+
+        // ---- S^T = K . Q^T ------------------------------------------------------------------
+        float4v sc[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            sc[kb] = float4v{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++)
+                sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_to_half8<TYPE>(kraw[s][kb][ks]), qreg[ks], sc[kb], 0, 0, 0);
+        }
+        // V rows into this wave's LDS stage (f16, dequantised when the cache is Q8_0)
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int flat = i * 64 + lane;
+            *(half8 *)&v_lds[wave][(flat / CH) * PV + (flat % CH) * 8] = chunk_to_half8<TYPE>(vraw[s][i]);
+        }
+        __builtin_amdgcn_wave_barrier();      // LDS runs a wave's instructions in order; keep the compiler from reordering
+
+        // lane holds keys j0 + kb*16 + g4*4 + r of column j
+        float sv[8];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int key = j0 + kb * 16 + g4 * 4 + r;
+                float x = sc[kb][r];
+                if (MASK) x = fmaf(mslope, h2f_bits(mrow[min(key, k_end - 1)]), x);
+                if (key >= k_end) x = -INFINITY;
+                sv[kb * 4 + r] = x - m;
+            }
+
+        // ---- P = 2^(s - m): no maximum unless the step's sum says the reference fell behind -----
+        half8 preg;
+        float lsum;
+        const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+        auto exp_step = [&]() {
+            float acc = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                half2v p2;
+                p2[0] = (_Float16)__builtin_amdgcn_exp2f(sv[e]);
+                p2[1] = (_Float16)__builtin_amdgcn_exp2f(sv[e + 1]);
+                acc = __builtin_amdgcn_fdot2(p2, ones, acc, false);
+                preg[e] = p2[0];
+                preg[e + 1] = p2[1];
+            }
+            lsum = acc;
+        };
+        exp_step();
+        const bool redo = !(lsum <= SUM_LIMIT) || !have;
+        if (__builtin_amdgcn_ballot_w64(redo) != 0) {
+            float mx = sv[0];
+#pragma unroll
+            for (int e = 1; e < 8; e++) mx = fmaxf(mx, sv[e]);
+            mx = fmaxf(mx, xor_shuffle(mx, 16));          // the four lanes of a column must agree
+            mx = fmaxf(mx, xor_shuffle(mx, 32));
+            float delta = 0.0f;
+            if (mx > -INFINITY) {
+                delta = have ? fmaxf(mx, 0.0f) : mx;
+                have = true;
+            }
+            const float f = __builtin_amdgcn_exp2f(-delta);
+            m += delta;
+            l *= f;
+#pragma unroll
+            for (int db = 0; db < DBK; db++) oacc[db] *= f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) sv[e] -= delta;
+            exp_step();
+        }
+        l += lsum;
+
+        // ---- O^T += V^T . P^T: transpose reads of the stage, 16 d at a time --------------------------
+        {
+            const int kr = g4 * 4 + (j >> 2);
+#pragma unroll
+            for (int db = 0; db < DBK; db++) {
+                const _Float16 * p0 = &v_lds[wave][kr * PV + db * 16 + (j & 3) * 4];
+                const _Float16 * p1 = p0 + 16 * PV;
+                const half4 lo = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p0));
+                const half4 hi = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p1));
+                const half8 va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                oacc[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, preg, oacc[db], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    if (wave < n_steps) issue(k_begin + wave * STEP, S0{});
+    for (int it = wave; it < n_steps; it += 2 * DEC_WAVES) {
+        step(it, S0{});
+        if (it + DEC_WAVES < n_steps) step(it + DEC_WAVES, S1{});
+    }
+
+    // ---- column totals, then the four waves through LDS ----------------------------------------------
+    l += xor_shuffle(l, 16);
+    l += xor_shuffle(l, 32);
+    if (!have) m = -INFINITY;
+    __syncthreads();                           // every wave is done with its stage
+#pragma unroll
+    for (int db = 0; db < DBK; db++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) red_o[wave][j][db * 16 + g4 * 4 + r] = oacc[db][r];
+    if (g4 == 0) {
+        red_ml[wave][j][0] = m;
+        red_ml[wave][j][1] = l;
+    }
+    __syncthreads();
+
+    // thread t: column t / 16, a strided set of d
+    const int col = tid >> 4;
+    if (col < R) {
+        float M = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; w++) M = fmaxf(M, red_ml[w][col][0]);
+        float f[DEC_WAVES];
+        float L = 0.0f;
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; w++) {
+            const float mw = red_ml[w][col][0];
+            f[w] = mw == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw - M);
+            L += red_ml[w][col][1] * f[w];
+        }
+        const int     ciq1 = col / a.gqa;
+        const int     ch   = hk * a.gqa + col % a.gqa;
+        const int64_t row  = ((int64_t)b * a.Nq + ciq1) * a.Hq + ch;
+        for (int d = tid & 15; d < D; d += 16) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int w = 0; w < DEC_WAVES; w++) acc += red_o[w][col][d] * f[w];
+            if (a.n_splits == 1) {
+                a.dst[row * D + d] = L > 0.0f ? acc / L : 0.0f;
+            } else {
+                a.part_acc[(row * a.n_splits + split) * D + d] = acc;
+            }
+        }
+        if (a.n_splits > 1 && (tid & 15) == 0) {
+            // the merge kernel works in natural-log units
+            float * pm = a.part_ml + (row * a.n_splits + split) * 2;
+            pm[0] = M == -INFINITY ? -INFINITY : M * 0.6931471805599453f;
+            pm[1] = L;
+        }
+    }
+}
+
+template <int D, int TYPE>
+int launch(const FattnArgs & a, hipStream_t stream) {
+    const dim3 grid((unsigned)(a.n_splits * a.Hkv * a.B));
+    if (a.mask) hipLaunchKernelGGL((fattn_decode_kernel<D, TYPE, true>), grid, dim3(DEC_THREADS), 0, stream, a);
+    else        hipLaunchKernelGGL((fattn_decode_kernel<D, TYPE, false>), grid, dim3(DEC_THREADS), 0, stream, a);
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+bool fattn_decode_supported(const FattnArgs & a, int ktype) {
+    if (a.D != 64 && a.D != 128) return false;
+    if (a.Nq < 1 || a.Nkv < 1) return false;
+    if ((int64_t)a.Nq * a.gqa > 16) return false;
+    if (a.softcap != 0.0f) return false;
+    if (ktype == MI355X_TYPE_F16) return a.kv_aligned16 != 0;
+    if (ktype == MI355X_TYPE_Q8_0) return a.kv_aligned4 != 0;
+    return false;
+}
+
+int fattn_decode_launch(const FattnArgs & a, int ktype, hipStream_t stream) {
+    if (ktype == MI355X_TYPE_F16) return a.D == 64 ? launch<64, MI355X_TYPE_F16>(a, stream) : launch<128, MI355X_TYPE_F16>(a, stream);
+    if (ktype == MI355X_TYPE_Q8_0) return a.D == 64 ? launch<64, MI355X_TYPE_Q8_0>(a, stream) : launch<128, MI355X_TYPE_Q8_0>(a, stream);
+    return (int)hipErrorInvalidValue;
+}

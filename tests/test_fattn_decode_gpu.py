@@ -1,0 +1,78 @@
+"""GPU parity of the split-KV MFMA decode kernel (few query rows per KV head) against the oracle."""
+import numpy as np
+import pytest
+
+import oracle as ora
+from cases import make_case, to_f32
+from crispasr_amd import ggml
+from gpu_util import assert_parity, run_gpu, run_oracle, upload
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    dict(seed=201, D=64, Nq=1, Nkv=224, Hq=20, B=5, mask="random_inf_batched"),                 # Whisper self-attn, one beam per batch
+    dict(seed=202, D=64, Nq=5, Nkv=1500, Hq=20, q_layout="thd", kv_layout="thd", kv_pad_rows=36,
+         scale=64 ** -0.25),                                                                   # Whisper cross-attn, 5 beams share K/V
+    dict(seed=203, D=64, Nq=5, Nkv=333, Hq=4, q_layout="thd", kv_layout="thd", mask="random_inf"),  # unified cache + beam mask
+    dict(seed=204, D=128, Nq=1, Nkv=663, Hq=32, Hkv=8, ktype=ora.Q8_0),                         # Voxtral-style decode, GQA 4
+    dict(seed=205, D=128, Nq=1, Nkv=408, Hq=32, Hkv=8, ktype=ora.F16),
+    dict(seed=206, D=128, Nq=3, Nkv=100, Hq=8, Hkv=2, B=2, ktype=ora.Q8_0, mask="causal"),      # 12 rows per KV head
+    dict(seed=207, D=128, Nq=4, Nkv=77, Hq=8, Hkv=2, ktype=ora.F16, mask="bias_perhead"),       # 16 rows per KV head
+    dict(seed=208, D=64, Nq=2, Nkv=31, Hq=6, Hkv=3, ktype=ora.Q8_0),
+    dict(seed=209, D=64, Nq=1, Nkv=1, Hq=2),
+    dict(seed=210, D=64, Nq=16, Nkv=257, Hq=2, mask="all_masked_rows"),
+    dict(seed=211, D=128, Nq=1, Nkv=300, Hq=8, B=4, Bk=2, ktype=ora.Q8_0, kv_layout="gap"),     # Canary-style strided quantised view
+    dict(seed=212, D=64, Nq=2, Nkv=500, Hq=8, Hkv=8, mask="bias", max_bias=8.0),
+    dict(seed=213, D=128, Nq=1, Nkv=4096, Hq=16, Hkv=2, ktype=ora.F16),
+]
+
+
+@pytest.mark.parametrize("n_splits", [1, 0, 3])
+@pytest.mark.parametrize("spec", SHAPES, ids=lambda s: "seed%d" % s["seed"])
+def test_decode_kernel_matches_oracle(spec, n_splits):
+    case = make_case(**spec)
+    print("case", spec, "n_splits", n_splits, flush=True)
+    ref = run_oracle(case)
+    got = run_gpu(case, kernel=ggml.KERNEL_DECODE_MMA, n_splits=n_splits)
+    assert_parity(got, ref, str(spec))
+
+
+def test_decode_is_what_auto_picks_and_more_than_16_rows_is_rejected():
+    dec = make_case(seed=221, D=128, Nq=1, Nkv=300, Hq=32, Hkv=8, ktype=ora.Q8_0)
+    kern, _ = ggml.flash_attn_plan(upload(dec["q"]), upload(dec["k"]), upload(dec["v"]), None, dec["scale"])
+    assert kern == ggml.KERNEL_DECODE_MMA
+    assert_parity(run_gpu(dec), run_oracle(dec), "auto decode")
+    wide = make_case(seed=222, D=128, Nq=5, Nkv=64, Hq=32, Hkv=8)      # 20 rows per KV head
+    with pytest.raises(ggml.UnsupportedError):
+        run_gpu(wide, kernel=ggml.KERNEL_DECODE_MMA)
+    assert_parity(run_gpu(wide), run_oracle(wide), "auto fallback")
+
+
+def test_decode_q8_0_dequantisation_in_registers_is_exact():
+    """One visible key per row: the output must equal f16(q*d) of that V row exactly - the byte funnel
+    shift, the int8 -> f16 widening and the packed scale multiply are all checked bit for bit."""
+    Nkv = 97
+    case = make_case(seed=223, D=128, Nq=1, Nkv=Nkv, Hq=8, Hkv=2, B=3, ktype=ora.Q8_0, std=3.0)
+    m = np.full((3, 1, 1, Nkv), -np.inf, np.float32)
+    pick = [0, 96, 41]
+    for b, jkey in enumerate(pick):
+        m[b, 0, 0, jkey] = 0.0
+    case["mask"] = ora.from_f32(m, ora.F16)
+    v = to_f32(case["v"])                                       # exact q*d in f32
+    expect = v.astype(np.float16).astype(np.float32)            # one rounding to f16
+    for ns in (1, 2):
+        got = run_gpu(case, kernel=ggml.KERNEL_DECODE_MMA, n_splits=ns)
+        for b in range(3):
+            for h in range(8):
+                assert np.array_equal(got[b, 0, h], expect[b, h // 4, pick[b]]), (ns, b, h)
+    # f16 caches come back bit-exactly
+    case = make_case(seed=224, D=64, Nq=2, Nkv=Nkv, Hq=4, B=3)
+    m = np.full((3, 1, 2, Nkv), -np.inf, np.float32)
+    for b, jkey in enumerate(pick):
+        m[b, 0, :, jkey] = 0.0
+    case["mask"] = ora.from_f32(m, ora.F16)
+    v = to_f32(case["v"])
+    got = run_gpu(case, kernel=ggml.KERNEL_DECODE_MMA)
+    for b in range(3):
+        for h in range(4):
+            assert np.array_equal(got[b, 0, h], v[b, h, pick[b]]) and np.array_equal(got[b, 1, h], v[b, h, pick[b]])
