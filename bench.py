@@ -119,10 +119,18 @@ def bench_encoder(args, ca, ora, torch):
     from cases import MAX_ABS_TOL, REL_L2_TOL
     parity_ok = max_abs <= MAX_ABS_TOL and rel <= REL_L2_TOL
 
+    # HBM bytes per launch of the same kernel from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE runs
+    traffic = None
+    try:
+        for ln in open(os.path.join(ROOT, "profiles", "fattn_mma_whisper_large_v3_encoder.txt")):
+            if ln.startswith("traffic_bytes_per_launch"):
+                traffic = float(ln.split()[1])
+    except OSError:
+        pass
     res = {
         "value": value, "ms_per_step": ms_per_step,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_F16_TFLOPS, "traffic": None,
+                     "frac": achieved / PEAK_F16_TFLOPS, "traffic": traffic,
                      "kernel": "fattn_mma_kernel<64,2,F16>", "us_per_launch": kernel_ms * 1e3,
                      "flops_per_launch": flops_layer},
         "parity": {"max_abs": max_abs, "rel_l2": rel, "ok": bool(parity_ok), "rows_checked": 50,
@@ -269,6 +277,27 @@ def bench_decode(args, ca, ora, torch):
     return out
 
 
+def copy_calibration(ca, torch):
+    """A plain copy of known size through the library's own CPY kernel: 256 MiB read + 256 MiB written.
+    It gives the counter-to-bytes factor for the rocprofv3 FETCH_SIZE / WRITE_SIZE traffic figures."""
+    n = 64 * 1024 * 1024
+    src = ca.Tensor(torch.ones(n, device="cuda").view(torch.uint8), ca.F32, (n,))
+    dst = ca.Tensor.empty(ca.F32, (n,))
+    for _ in range(2):
+        ca.cpy(src, dst)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        ca.cpy(src, dst)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / 5
+    gbs = 2 * 4 * n / (us * 1e-6) / 1e9
+    log(f"[bench] copy calibration (cpy_scalar_kernel<float,float>): {4 * n} B read + {4 * n} B written in {us:.1f} us = {gbs:.0f} GB/s")
+    return {"bytes_read": 4 * n, "bytes_written": 4 * n, "us": us, "GB/s": gbs}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -306,6 +335,7 @@ def main():
         "roofline": enc["roofline"], "parity": enc["parity"],
         "device": {"name": info["name"], "arch": info["arch"], "cus": info["compute_units"], "clock_khz": info["clock_khz"]},
     }
+    line["copy_calibration"] = copy_calibration(ca, torch)
     if not args.no_decode:
         line["decode"] = bench_decode(args, ca, ora, torch)
     if not args.no_cpu_baseline:

@@ -486,6 +486,18 @@ int mi355x_buffer_free(void * ptr) {
     return MI355X_OK;
 }
 
+int mi355x_host_buffer_alloc(size_t size, void ** ptr) {
+    if (!ptr) return fail(MI355X_ERR_INVALID, "null argument");
+    *ptr = nullptr;
+    HIP_TRY(hipHostMalloc(ptr, size ? size : 1, hipHostMallocMapped | hipHostMallocCoherent));
+    return MI355X_OK;
+}
+
+int mi355x_host_buffer_free(void * ptr) {
+    if (ptr) HIP_TRY(hipHostFree(ptr));
+    return MI355X_OK;
+}
+
 int mi355x_buffer_memset(void * ptr, int value, size_t size, void * stream) {
     if (size == 0) return MI355X_OK;
     HIP_TRY(hipMemsetAsync(ptr, value, size, (hipStream_t)stream));

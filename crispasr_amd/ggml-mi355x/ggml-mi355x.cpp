@@ -1,0 +1,254 @@
+// ggml-mi355x: a minimal ggml backend that claims GGML_OP_FLASH_ATTN_EXT (and the copies it needs) and runs
+// it through libmi355x_fattn.so; every other op stays on ggml-cpu, routed by ggml_backend_sched.
+//
+// NOT COMPILED IN THIS REPOSITORY: ggml's headers (ggml.h, ggml-backend.h, ggml-backend-impl.h) are an empty
+// submodule in the reference tree.  The vtable layouts below are written from the v0.17 API as recalled (the
+// buffer vtable's member order is the one the reference's own initialiser uses, src/core/gguf_loader.cpp:332-344)
+// and must be checked against the real headers before this file is trusted.  Build, once ggml is available:
+//   g++ -std=c++17 -fPIC -shared -DGGML_BACKEND_DL -I$GGML/include -I$GGML/src -I../../include \
+//       ggml-mi355x.cpp -L.. -lmi355x_fattn -o libggml-mi355x.so
+// and let ggml_backend_load_all() pick it up (examples/cli/cli.cpp:2416).
+#include "ggml-backend-impl.h"
+#include "ggml-backend.h"
+#include "ggml.h"
+
+#include "mi355x_fattn.h"
+
+#include <cstring>
+#include <string>
+
+// ---- helpers ---------------------------------------------------------------------------------------------
+
+static mi355x_tensor to_mi(const ggml_tensor * t) {
+    mi355x_tensor m;
+    m.data = t->data;
+    m.type = (int32_t)t->type;                  // GGML_TYPE_F32 = 0, F16 = 1, Q8_0 = 8: the ids the library uses
+    for (int i = 0; i < 4; i++) { m.ne[i] = t->ne[i]; m.nb[i] = t->nb[i]; }
+    return m;
+}
+
+static mi355x_fattn_params fa_params(const ggml_tensor * node) {
+    mi355x_fattn_params p;
+    std::memset(&p, 0, sizeof(p));
+    std::memcpy(&p.scale,         (const float *)node->op_params + 0, sizeof(float));
+    std::memcpy(&p.max_bias,      (const float *)node->op_params + 1, sizeof(float));
+    std::memcpy(&p.logit_softcap, (const float *)node->op_params + 2, sizeof(float));
+    p.prec = ((const int32_t *)node->op_params)[3];
+    return p;
+}
+
+// ---- buffer type: pinned, GPU-mapped host memory ------------------------------------------------------------
+// The runtimes place weights and KV caches in the first GPU device's default buffer type
+// (src/crispasr.cpp:1940-1944, 3942-3971; src/core/gguf_loader.cpp:722-741).  For ggml-cpu to keep running
+// every other op on those tensors the buffer must be host memory (is_host = true); the GPU addresses the same
+// pages.  Tensors that only attention reads (the scheduler's copies at split boundaries) live in HBM buffers
+// of the second buffer type below.
+
+struct mi355x_buffer_ctx { void * base; bool device; };
+
+static void   buf_free(ggml_backend_buffer_t b) {
+    auto * c = (mi355x_buffer_ctx *)b->context;
+    if (c->device) mi355x_buffer_free(c->base); else mi355x_host_buffer_free(c->base);
+    delete c;
+}
+static void * buf_base(ggml_backend_buffer_t b) { return ((mi355x_buffer_ctx *)b->context)->base; }
+static enum ggml_status buf_init_tensor(ggml_backend_buffer_t, ggml_tensor *) { return GGML_STATUS_SUCCESS; }
+static void buf_memset(ggml_backend_buffer_t, ggml_tensor * t, uint8_t v, size_t off, size_t n) {
+    mi355x_buffer_memset((char *)t->data + off, v, n, nullptr);
+    mi355x_stream_synchronize(nullptr);
+}
+static void buf_set(ggml_backend_buffer_t, ggml_tensor * t, const void * d, size_t off, size_t n) {
+    mi355x_buffer_set((char *)t->data + off, d, n, nullptr);
+}
+static void buf_get(ggml_backend_buffer_t, const ggml_tensor * t, void * d, size_t off, size_t n) {
+    mi355x_buffer_get(d, (const char *)t->data + off, n, nullptr);
+}
+static bool buf_cpy(ggml_backend_buffer_t, const ggml_tensor * src, ggml_tensor * dst) {
+    if (!ggml_backend_buffer_is_host(src->buffer) && src->buffer->iface.get_base != buf_base) return false;
+    mi355x_buffer_copy(dst->data, src->data, ggml_nbytes(src), nullptr);
+    mi355x_stream_synchronize(nullptr);
+    return true;
+}
+static void buf_clear(ggml_backend_buffer_t b, uint8_t v) {
+    mi355x_buffer_memset(buf_base(b), v, b->size, nullptr);
+    mi355x_stream_synchronize(nullptr);
+}
+
+static const ggml_backend_buffer_i mi355x_buffer_iface = {
+    /* .free_buffer   = */ buf_free,
+    /* .get_base      = */ buf_base,
+    /* .init_tensor   = */ buf_init_tensor,
+    /* .memset_tensor = */ buf_memset,
+    /* .set_tensor    = */ buf_set,
+    /* .get_tensor    = */ buf_get,
+    /* .set_tensor_2d = */ nullptr,
+    /* .get_tensor_2d = */ nullptr,
+    /* .cpy_tensor    = */ buf_cpy,
+    /* .clear         = */ buf_clear,
+    /* .reset         = */ nullptr,
+};
+
+template <bool DEVICE>
+static ggml_backend_buffer_t buft_alloc(ggml_backend_buffer_type_t buft, size_t size) {
+    void * p = nullptr;
+    const int rc = DEVICE ? mi355x_buffer_alloc(size, &p) : mi355x_host_buffer_alloc(size, &p);
+    if (rc != MI355X_OK) return nullptr;                      // allocation failures are NULL returns (src/voxtral.cpp:1138-1142)
+    return ggml_backend_buffer_init(buft, mi355x_buffer_iface, new mi355x_buffer_ctx{p, DEVICE}, size);
+}
+static const char * buft_host_name(ggml_backend_buffer_type_t) { return "MI355X_Host"; }
+static const char * buft_dev_name(ggml_backend_buffer_type_t)  { return "MI355X"; }
+static size_t buft_align(ggml_backend_buffer_type_t) { return 256; }
+static size_t buft_max(ggml_backend_buffer_type_t)   { return SIZE_MAX; }
+static size_t buft_alloc_size(ggml_backend_buffer_type_t, const ggml_tensor * t) { return ggml_nbytes(t); }
+static bool   buft_is_host(ggml_backend_buffer_type_t)  { return true; }
+static bool   buft_not_host(ggml_backend_buffer_type_t) { return false; }
+
+static ggml_backend_dev_t g_dev();
+static ggml_backend_buffer_type_t mi355x_host_buft() {
+    static ggml_backend_buffer_type t = {
+        { buft_host_name, buft_alloc<false>, buft_align, buft_max, buft_alloc_size, buft_is_host }, g_dev(), nullptr };
+    return &t;
+}
+static ggml_backend_buffer_type_t mi355x_dev_buft() {
+    static ggml_backend_buffer_type t = {
+        { buft_dev_name, buft_alloc<true>, buft_align, buft_max, buft_alloc_size, buft_not_host }, g_dev(), nullptr };
+    return &t;
+}
+
+// ---- supports_op: FLASH_ATTN_EXT and the copies it needs, nothing else ----------------------------------------
+
+static bool dev_supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
+    switch (op->op) {
+        case GGML_OP_FLASH_ATTN_EXT: {
+            if (op->src[4]) return false;                      // sinks
+            mi355x_tensor q = to_mi(op->src[0]), k = to_mi(op->src[1]), v = to_mi(op->src[2]), d = to_mi(op);
+            mi355x_tensor m;
+            if (op->src[3]) m = to_mi(op->src[3]);
+            const mi355x_fattn_params p = fa_params(op);
+            q.data = k.data = v.data = d.data = nullptr;        // planning happens before allocation
+            return mi355x_fattn_supports(&q, &k, &v, op->src[3] ? &m : nullptr, &d, &p) == MI355X_OK;
+        }
+        case GGML_OP_CPY: case GGML_OP_CONT: case GGML_OP_DUP: {
+            mi355x_tensor s = to_mi(op->src[0]), d = to_mi(op);
+            return mi355x_cpy_supports(&s, &d) == MI355X_OK;
+        }
+        case GGML_OP_NONE: case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE:
+            return true;                                        // no-ops on any backend
+        default:
+            return false;
+    }
+}
+static bool dev_supports_buft(ggml_backend_dev_t, ggml_backend_buffer_type_t buft) {
+    return buft == mi355x_host_buft() || buft == mi355x_dev_buft();
+}
+// keep CPY/CONT on the CPU unless their destination already lives in one of our buffers
+static bool dev_offload_op(ggml_backend_dev_t, const ggml_tensor * op) { return op->op == GGML_OP_FLASH_ATTN_EXT; }
+
+// ---- backend: graph_compute walks the split's nodes ---------------------------------------------------------------
+
+static const char * be_name(ggml_backend_t) { return "MI355X"; }
+static void be_free(ggml_backend_t b) { delete b; }
+static void be_sync(ggml_backend_t) { mi355x_stream_synchronize(nullptr); }
+
+static enum ggml_status be_graph_compute(ggml_backend_t, ggml_cgraph * g) {
+    for (int i = 0; i < ggml_graph_n_nodes(g); i++) {
+        ggml_tensor * n = ggml_graph_node(g, i);
+        int rc = MI355X_OK;
+        switch (n->op) {
+            case GGML_OP_FLASH_ATTN_EXT: {
+                const mi355x_tensor q = to_mi(n->src[0]), k = to_mi(n->src[1]), v = to_mi(n->src[2]), d = to_mi(n);
+                mi355x_tensor m;
+                if (n->src[3]) m = to_mi(n->src[3]);
+                const mi355x_fattn_params p = fa_params(n);
+                rc = mi355x_flash_attn_ext(&q, &k, &v, n->src[3] ? &m : nullptr, &d, &p, nullptr);
+                break;
+            }
+            case GGML_OP_CPY: case GGML_OP_CONT: case GGML_OP_DUP: {
+                const mi355x_tensor s = to_mi(n->src[0]), d = to_mi(n);
+                rc = mi355x_cpy(&s, &d, nullptr);
+                break;
+            }
+            default:
+                break;                                          // views and reshapes
+        }
+        if (rc != MI355X_OK) {
+            GGML_LOG_ERROR("ggml-mi355x: %s failed: %s\n", ggml_op_name(n->op), mi355x_last_error());
+            return GGML_STATUS_FAILED;                          // callers only test == GGML_STATUS_SUCCESS (src/crispasr.cpp:273)
+        }
+    }
+    // inputs may be overwritten by the caller as soon as compute returns (src/canary_ctc.cpp:959-963)
+    return mi355x_stream_synchronize(nullptr) == MI355X_OK ? GGML_STATUS_SUCCESS : GGML_STATUS_FAILED;
+}
+
+static const ggml_backend_i mi355x_backend_iface = {
+    /* .get_name           = */ be_name,
+    /* .free               = */ be_free,
+    /* .set_tensor_async   = */ nullptr,
+    /* .get_tensor_async   = */ nullptr,
+    /* .cpy_tensor_async   = */ nullptr,
+    /* .synchronize        = */ be_sync,
+    /* .graph_plan_create  = */ nullptr,
+    /* .graph_plan_free    = */ nullptr,
+    /* .graph_plan_update  = */ nullptr,
+    /* .graph_plan_compute = */ nullptr,
+    /* .graph_compute      = */ be_graph_compute,
+    /* .event_record       = */ nullptr,
+    /* .event_wait         = */ nullptr,
+    /* .graph_optimize     = */ nullptr,
+};
+
+static ggml_guid_t mi355x_guid() {
+    static ggml_guid guid = {0x6d, 0x69, 0x33, 0x35, 0x35, 0x78, 0x2d, 0x66, 0x61, 0x74, 0x74, 0x6e, 0x00, 0x00, 0x00, 0x01};
+    return &guid;
+}
+
+// ---- device + registry ---------------------------------------------------------------------------------------------
+
+static const char * dev_name(ggml_backend_dev_t) { return "MI355X0"; }
+static const char * dev_desc(ggml_backend_dev_t) {
+    static mi355x_device_info info;
+    static bool once = (mi355x_device_get_info(0, &info), true);
+    (void)once;
+    return info.name;
+}
+static void dev_memory(ggml_backend_dev_t, size_t * free, size_t * total) {
+    mi355x_device_info info;
+    mi355x_device_get_info(0, &info);
+    *free = info.free_memory; *total = info.total_memory;
+}
+static enum ggml_backend_dev_type dev_type(ggml_backend_dev_t) { return GGML_BACKEND_DEVICE_TYPE_GPU; }   // the runtimes only look at GPU|IGPU (src/core/gpu_backend_pref.h:116-163)
+static void dev_props(ggml_backend_dev_t d, ggml_backend_dev_props * p) {
+    p->name = dev_name(d); p->description = dev_desc(d); p->type = dev_type(d);
+    dev_memory(d, &p->memory_free, &p->memory_total);
+    p->caps = { /* async */ false, /* host_buffer */ true, /* buffer_from_host_ptr */ false, /* events */ false };
+}
+static ggml_backend_t dev_init(ggml_backend_dev_t d, const char *) {
+    if (mi355x_set_device(0) != MI355X_OK) return nullptr;     // callers fall back to the CPU backend (src/voxtral.cpp:842-845)
+    return new ggml_backend{ mi355x_guid(), mi355x_backend_iface, d, nullptr };
+}
+static ggml_backend_buffer_type_t dev_buft(ggml_backend_dev_t)      { return mi355x_host_buft(); }
+static ggml_backend_buffer_type_t dev_host_buft(ggml_backend_dev_t) { return mi355x_host_buft(); }
+
+static const ggml_backend_device_i mi355x_device_iface = {
+    dev_name, dev_desc, dev_memory, dev_type, dev_props, dev_init, dev_buft, dev_host_buft,
+    /* buffer_from_host_ptr */ nullptr, dev_supports_op, dev_supports_buft, dev_offload_op,
+    /* event_new */ nullptr, /* event_free */ nullptr, /* event_synchronize */ nullptr,
+};
+
+static const char * reg_name(ggml_backend_reg_t) { return "MI355X"; }
+static size_t reg_count(ggml_backend_reg_t) { int n = 0; mi355x_device_count(&n); return n > 0 ? 1 : 0; }
+static ggml_backend_dev_t reg_dev(ggml_backend_reg_t, size_t) { return g_dev(); }
+static void * reg_proc(ggml_backend_reg_t, const char *) { return nullptr; }
+
+extern "C" ggml_backend_reg_t ggml_backend_mi355x_reg(void) {
+    static ggml_backend_reg reg = { GGML_BACKEND_API_VERSION, { reg_name, reg_count, reg_dev, reg_proc }, nullptr };
+    return &reg;
+}
+static ggml_backend_dev_t g_dev() {
+    static ggml_backend_device dev = { mi355x_device_iface, ggml_backend_mi355x_reg(), nullptr };
+    return &dev;
+}
+
+#ifdef GGML_BACKEND_DL
+GGML_BACKEND_DL_IMPL(ggml_backend_mi355x_reg)
+#endif

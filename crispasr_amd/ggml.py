@@ -72,7 +72,7 @@ EXPORTS = [
     "mi355x_device_count", "mi355x_device_get_info", "mi355x_set_device", "mi355x_stream_synchronize",
     "mi355x_fattn_supports", "mi355x_flash_attn_ext", "mi355x_fattn_workspace_size", "mi355x_fattn_plan",
     "mi355x_cpy_supports", "mi355x_cpy", "mi355x_set_rows",
-    "mi355x_buffer_alloc", "mi355x_buffer_free", "mi355x_buffer_memset", "mi355x_buffer_set",
+    "mi355x_buffer_alloc", "mi355x_buffer_free", "mi355x_host_buffer_alloc", "mi355x_host_buffer_free", "mi355x_buffer_memset", "mi355x_buffer_set",
     "mi355x_buffer_get", "mi355x_buffer_copy",
 ]
 
@@ -107,6 +107,8 @@ def lib() -> ctypes.CDLL:
                                       ctypes.POINTER(ctypes.c_size_t), PT, ctypes.c_void_p]
         L.mi355x_buffer_alloc.argtypes = [ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]
         L.mi355x_buffer_free.argtypes = [ctypes.c_void_p]
+        L.mi355x_host_buffer_alloc.argtypes = [ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]
+        L.mi355x_host_buffer_free.argtypes = [ctypes.c_void_p]
         L.mi355x_buffer_memset.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p]
         L.mi355x_buffer_set.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         L.mi355x_buffer_get.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]

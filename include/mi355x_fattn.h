@@ -167,6 +167,10 @@ int mi355x_set_rows(const mi355x_tensor * src, const void * idx, int32_t idx_typ
 
 int mi355x_buffer_alloc(size_t size, void ** ptr);                 /* alloc_buffer (256-byte aligned) */
 int mi355x_buffer_free(void * ptr);                                /* free_buffer */
+/* pinned host memory the GPU can address at the same pointer (hipHostMalloc, mapped + coherent): the
+ * is_host buffer type a one-op backend needs so that ggml-cpu keeps running every other op on it */
+int mi355x_host_buffer_alloc(size_t size, void ** ptr);
+int mi355x_host_buffer_free(void * ptr);
 int mi355x_buffer_memset(void * ptr, int value, size_t size, void * stream);         /* memset_tensor / clear */
 int mi355x_buffer_set(void * dst, const void * host_src, size_t size, void * stream);   /* set_tensor  (sync) */
 int mi355x_buffer_get(void * host_dst, const void * src, size_t size, void * stream);   /* get_tensor  (sync) */
