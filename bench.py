@@ -90,8 +90,7 @@ def bench_encoder(args, ca, ora, torch):
 
     def step():
         for dev in layers:
-            ca.flash_attn_ext(dev["q"], dev["k"], dev["v"], None, scale, out=dev["out"],
-                              kernel=ca.ggml.KERNEL_MMA)
+            ca.flash_attn_ext(dev["q"], dev["k"], dev["v"], None, scale, out=dev["out"])
 
     for _ in range(args.warmup):
         step()

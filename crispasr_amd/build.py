@@ -9,7 +9,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmi355x_fattn.so")
-SOURCES = ["api.hip", "fattn_vec.hip", "fattn_mma.hip", "fattn_decode.hip", "cpy.hip"]
+SOURCES = ["api.hip", "fattn_vec.hip", "fattn_mma.hip", "fattn_mma_pipe.hip", "fattn_decode.hip", "cpy.hip"]
 
 # packed-fp32 VALU ops are switched off for all device code of this library
 HIPCC_FLAGS = [
@@ -26,9 +26,14 @@ def _hipcc() -> str:
     return "hipcc"
 
 
+# per-file flags: the pipelined kernel wants its MFMA results in ordinary VGPRs (they feed v_exp_f32 directly;
+# accumulation registers would cost two moves per score)
+PER_FILE_FLAGS = {"fattn_mma_pipe.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def _compile(src: str, extra) -> str:
     obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *PER_FILE_FLAGS.get(src, []), *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
     err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)

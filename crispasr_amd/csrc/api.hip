@@ -356,6 +356,12 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     make_plan(a, k->type, params, plan);
     hipStream_t st = (hipStream_t)stream;
 
+    if (plan.kernel == MI355X_FATTN_MMA_PIPE) {
+        if (!fattn_mma_pipe_supported(a, k->type)) return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the pipelined MFMA kernel");
+        const int e = fattn_mma_pipe_launch(a, k->type, st);
+        if (e) return hip_fail((hipError_t)e, "fattn_mma_pipe launch");
+        return MI355X_OK;
+    }
     if (plan.kernel == MI355X_FATTN_MMA) {
         if (!fattn_mma_supported(a, k->type)) return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the MFMA kernel");
         const int e = fattn_mma_launch(a, k->type, st);

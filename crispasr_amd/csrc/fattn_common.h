@@ -106,6 +106,8 @@ int fattn_vec_launch(const FattnArgs & a, int ktype, hipStream_t stream);
 int fattn_merge_launch(const FattnArgs & a, hipStream_t stream);
 int fattn_mma_launch(const FattnArgs & a, int ktype, hipStream_t stream);
 bool fattn_mma_supported(const FattnArgs & a, int ktype);
+int fattn_mma_pipe_launch(const FattnArgs & a, int ktype, hipStream_t stream);
+bool fattn_mma_pipe_supported(const FattnArgs & a, int ktype);
 int fattn_decode_launch(const FattnArgs & a, int ktype, hipStream_t stream);
 bool fattn_decode_supported(const FattnArgs & a, int ktype);
 int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream);

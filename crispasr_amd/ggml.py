@@ -23,7 +23,7 @@ QK8_0 = 32
 TYPE_SIZE = {F32: 4, F16: 2, Q8_0: 34}
 BLOCK_SIZE = {F32: 1, F16: 1, Q8_0: QK8_0}
 
-KERNEL_AUTO, KERNEL_VEC, KERNEL_MMA, KERNEL_DECODE_MMA = 0, 1, 2, 3
+KERNEL_AUTO, KERNEL_VEC, KERNEL_MMA, KERNEL_DECODE_MMA, KERNEL_MMA_PIPE = 0, 1, 2, 3, 4
 PREC_DEFAULT, PREC_F32 = 0, 10
 
 OK, ERR_UNSUPPORTED, ERR_INVALID, ERR_HIP, ERR_NO_DEVICE, ERR_WORKSPACE = range(6)

@@ -71,7 +71,47 @@ def test_auto_picks_the_tile_kernel_for_prefill_and_the_vector_kernel_for_decode
     pre = make_case(seed=122, D=64, Nq=200, Nkv=200, Hq=4)
     dec = make_case(seed=123, D=64, Nq=1, Nkv=200, Hq=4)
     odd = make_case(seed=124, D=80, Nq=200, Nkv=200, Hq=4)
-    for case, want in ((pre, ggml.KERNEL_MMA), (dec, ggml.KERNEL_VEC), (odd, ggml.KERNEL_VEC)):
+    for case, want in ((pre, ggml.KERNEL_MMA), (dec, ggml.KERNEL_DECODE_MMA), (odd, ggml.KERNEL_VEC)):
         kern, _ = ggml.flash_attn_plan(upload(case["q"]), upload(case["k"]), upload(case["v"]), None, case["scale"])
         assert kern == want
         assert_parity(run_gpu(case), run_oracle(case), "auto")
+
+
+PIPE_SHAPES = [
+    dict(seed=131, D=64, Nq=64, Nkv=64, Hq=2),
+    dict(seed=132, D=64, Nq=300, Nkv=333, Hq=3, B=2, q_layout="thd", kv_layout="thd"),
+    dict(seed=133, D=64, Nq=256, Nkv=1, Hq=2),
+    dict(seed=134, D=64, Nq=257, Nkv=65, Hq=2, ktype=ora.F32, kv_layout="gap"),
+    dict(seed=135, D=64, Nq=100, Nkv=128, Hq=4, Hkv=2, ktype=ora.Q8_0),
+    dict(seed=136, D=64, Nq=130, Nkv=200, Hq=2, kv_pad_rows=56, kv_layout="thd"),             # Whisper zero-pad rows
+    dict(seed=137, D=64, Nq=1500, Nkv=1500, Hq=2, scale=0.125),                                 # Whisper base geometry
+    dict(seed=138, D=64, Nq=512, Nkv=640, Hq=8, B=4, Bk=2, scale=0.125),
+    dict(seed=139, D=64, Nq=90, Nkv=192, Hq=2, std=1.5),                                         # sharp softmax: reference raises mid-way
+    dict(seed=140, D=64, Nq=90, Nkv=500, Hq=2, std=0.05),
+]
+
+
+@pytest.mark.parametrize("spec", PIPE_SHAPES, ids=lambda s: "seed%d" % s["seed"])
+def test_pipelined_mma_kernel_matches_oracle(spec):
+    case = make_case(**spec)
+    print("case", spec, flush=True)
+    ref = run_oracle(case)
+    got = run_gpu(case, kernel=ggml.KERNEL_MMA_PIPE)
+    err = assert_parity(got, ref, str(spec))
+    print("max_abs %.3e rel_l2 %.3e" % err, flush=True)
+
+
+def test_pipelined_kernel_with_growing_scores():
+    """Keys sorted so that every block raises the running maximum: exercises the redo path on every block,
+    including the adjustment of the scores of the block already in flight."""
+    case = make_case(seed=141, D=64, Nq=128, Nkv=448, Hq=2, std=2.0)
+    k = to_f32(case["k"])
+    ramp = np.linspace(0.2, 3.0, 448, dtype=np.float32)[None, None, :, None]
+    case["k"] = ora.from_f32(k * ramp, ora.F16)
+    q = to_f32(case["q"])
+    case["q"] = ora.from_f32(np.abs(q), ora.F32)
+    case["k"] = ora.from_f32(np.abs(to_f32(case["k"])), ora.F16)
+    ref = run_oracle(case)
+    amax = float(np.abs(ref).max())                 # outputs are a few units large here: scale the absolute bound
+    for kern in (ggml.KERNEL_MMA_PIPE, ggml.KERNEL_MMA):
+        assert_parity(run_gpu(case, kernel=kern), ref, "growing scores, kernel %d" % kern, max_abs_tol=2e-3 * max(1.0, amax))
