@@ -192,13 +192,14 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     const int sr = tid / CH;
 
     Raw kraw[NP], vraw[NP];
+    // Rows past Nkv re-read the last row: their scores are forced to -inf in the tail tile, so any finite
+    // stand-in will do, and branch-free loads let the waits on them be exact counts.
     auto load_tile = [&](int j0) {
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-            const int  key = j0 + sr + p * RPP;
-            const bool ok  = key < a.Nkv;
-            kraw[p] = load_chunk<TYPE>(kbase + (int64_t)key * a.nbk1, sc, ok);
-            vraw[p] = load_chunk<TYPE>(vbase + (int64_t)key * a.nbv1, sc, ok);
+            const int key = min(j0 + sr + p * RPP, a.Nkv - 1);
+            kraw[p] = load_chunk<TYPE>(kbase + (int64_t)key * a.nbk1, sc, true);
+            vraw[p] = load_chunk<TYPE>(vbase + (int64_t)key * a.nbv1, sc, true);
         }
     };
     auto store_tile = [&](int buf) {
