@@ -265,19 +265,30 @@ def bench_decode(args, ca, ora, torch):
     run("voxtral_decode_q8_0_gqa4_x64seq", layers, 128 ** -0.5, Bs * per_call, 10, "64 sequences per call")
     Lk = 4096
     nbk = (2, 2 * D, 2 * D * Lk, 2 * D * Lk * Hkv)
+    for Bs, nl in ((16, 6), (64, 2)):
+        layers = []
+        for l in range(nl):
+            layers.append({"q": ca.Tensor(torch.randn(Bs * Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, Bs)),
+                           "k": ca.Tensor(f16_buf(Bs * Hkv * Lk * D), ca.F16, (D, Lk, Hkv, Bs), nbk),
+                           "v": ca.Tensor(f16_buf(Bs * Hkv * Lk * D), ca.F16, (D, Lk, Hkv, Bs), nbk),
+                           "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, Bs))})
+        run(f"llm_decode_f16_gqa4_4096x{Bs}seq", layers, 128 ** -0.5, Bs * (2 * Lk * Hkv * D * 2 + 2 * Hq * D * 4), 10,
+            f"{Bs} sequences x 4096-entry f16 cache per call")
+        del layers
+    rs, nbk = 136, (34, 136, 136 * Lk, 136 * Lk * Hkv)
     layers = []
-    for l in range(6):
-        layers.append({"q": ca.Tensor(torch.randn(16 * Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, 16)),
-                       "k": ca.Tensor(f16_buf(16 * Hkv * Lk * D), ca.F16, (D, Lk, Hkv, 16), nbk),
-                       "v": ca.Tensor(f16_buf(16 * Hkv * Lk * D), ca.F16, (D, Lk, Hkv, 16), nbk),
-                       "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 16))})
-    run("llm_decode_f16_gqa4_4096x16seq", layers, 128 ** -0.5, 16 * (2 * Lk * Hkv * D * 2 + 2 * Hq * D * 4), 10,
-        "16 sequences x 4096-entry f16 cache per call")
+    for l in range(2):
+        layers.append({"q": ca.Tensor(torch.randn(64 * Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, 64)),
+                       "k": ca.Tensor(q8_buf(1100 + 2 * l, 64 * Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, 64), nbk),
+                       "v": ca.Tensor(q8_buf(1101 + 2 * l, 64 * Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, 64), nbk),
+                       "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 64))})
+    run("llm_decode_q8_0_gqa4_4096x64seq", layers, 128 ** -0.5, 64 * (2 * Lk * Hkv * rs + 2 * Hq * D * 4), 10,
+        "64 sequences x 4096-entry Q8_0 cache per call")
     return out
 
 
 def copy_calibration(ca, torch):
-    """A plain copy of known size through the library's own CPY kernel: 256 MiB read + 256 MiB written.
+    """A plain copy of known size through the library's own CPY kernel (128-bit path): 256 MiB read + 256 MiB written.
     It gives the counter-to-bytes factor for the rocprofv3 FETCH_SIZE / WRITE_SIZE traffic figures."""
     n = 64 * 1024 * 1024
     src = ca.Tensor(torch.ones(n, device="cuda").view(torch.uint8), ca.F32, (n,))
@@ -293,7 +304,7 @@ def copy_calibration(ca, torch):
     torch.cuda.synchronize()
     us = e0.elapsed_time(e1) * 1e3 / 5
     gbs = 2 * 4 * n / (us * 1e-6) / 1e9
-    log(f"[bench] copy calibration (cpy_scalar_kernel<float,float>): {4 * n} B read + {4 * n} B written in {us:.1f} us = {gbs:.0f} GB/s")
+    log(f"[bench] copy calibration (cpy_vec8_kernel<float,float>): {4 * n} B read + {4 * n} B written in {us:.1f} us = {gbs:.0f} GB/s")
     return {"bytes_read": 4 * n, "bytes_written": 4 * n, "us": us, "GB/s": gbs}
 
 

@@ -28,6 +28,23 @@ __global__ void __launch_bounds__(256) cpy_scalar_kernel(const CpyArgs a) {
     *(TD *)(a.dst + offset_of(i, a.dne, a.dnb, 1)) = (TD)x;     // f32 -> f16 is round-to-nearest-even
 }
 
+// 8 consecutive elements of dimension 0 per lane: 128-bit loads and stores for f16 <-> f32 and same-type copies.
+// Launched only when both sides have ne0 % 8 == 0, unit element stride and 16-byte aligned rows.
+template <typename TS, typename TD>
+__global__ void __launch_bounds__(256) cpy_vec8_kernel(const CpyArgs a) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= a.n) return;
+    const TS * sp = (const TS *)(a.src + offset_of(i, a.sne, a.snb, 8));
+    TD *       dp = (TD *)(a.dst + offset_of(i, a.dne, a.dnb, 8));
+    typedef TS vs8 __attribute__((ext_vector_type(8)));
+    typedef TD vd8 __attribute__((ext_vector_type(8)));
+    const vs8 x = *(const vs8 *)sp;
+    vd8 y;
+#pragma unroll
+    for (int e = 0; e < 8; e++) y[e] = (TD)x[e];
+    *(vd8 *)dp = y;
+}
+
 // quantise one block of 32 held one element per lane (32 consecutive lanes):
 // d = amax/127 (f32), q = rne(x * (1/d)), d stored as fp16
 // (called by every lane of the wave: the reduction runs before any divergence)
@@ -112,8 +129,29 @@ __global__ void __launch_bounds__(256) set_rows_kernel(const CpyArgs a) {
 
 }  // namespace
 
+static bool vec8_ok(const CpyArgs & a, int stype, int dtype) {
+    if (stype == MI355X_TYPE_Q8_0 || dtype == MI355X_TYPE_Q8_0) return false;
+    const int64_t ss = stype == MI355X_TYPE_F32 ? 4 : 2, ds = dtype == MI355X_TYPE_F32 ? 4 : 2;
+    if (a.sne[0] % 8 || a.dne[0] % 8 || a.snb[0] != ss || a.dnb[0] != ds) return false;
+    if (((uintptr_t)a.src % (8 * ss)) || ((uintptr_t)a.dst % (8 * ds))) return false;
+    for (int i = 1; i < 4; i++) {
+        if ((a.sne[i] > 1 && a.snb[i] % (8 * ss)) || (a.dne[i] > 1 && a.dnb[i] % (8 * ds))) return false;
+    }
+    return true;
+}
+
 int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream) {
     if (a.n == 0) return 0;
+    if (vec8_ok(a, stype, dtype)) {
+        CpyArgs v = a;
+        v.n = a.n / 8;
+        const unsigned g = (unsigned)((v.n + 255) / 256);
+        if (stype == MI355X_TYPE_F32 && dtype == MI355X_TYPE_F32)      hipLaunchKernelGGL((cpy_vec8_kernel<float, float>), dim3(g), dim3(256), 0, stream, v);
+        else if (stype == MI355X_TYPE_F32 && dtype == MI355X_TYPE_F16) hipLaunchKernelGGL((cpy_vec8_kernel<float, _Float16>), dim3(g), dim3(256), 0, stream, v);
+        else if (stype == MI355X_TYPE_F16 && dtype == MI355X_TYPE_F16) hipLaunchKernelGGL((cpy_vec8_kernel<_Float16, _Float16>), dim3(g), dim3(256), 0, stream, v);
+        else                                                          hipLaunchKernelGGL((cpy_vec8_kernel<_Float16, float>), dim3(g), dim3(256), 0, stream, v);
+        return (int)hipGetLastError();
+    }
     const unsigned g256 = (unsigned)((a.n + 255) / 256);
     const unsigned g8   = (unsigned)((a.n + 7) / 8);
     if (stype == MI355X_TYPE_F32 && dtype == MI355X_TYPE_F32)

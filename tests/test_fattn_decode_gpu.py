@@ -24,6 +24,9 @@ SHAPES = [
     dict(seed=211, D=128, Nq=1, Nkv=300, Hq=8, B=4, Bk=2, ktype=ora.Q8_0, kv_layout="gap"),     # Canary-style strided quantised view
     dict(seed=212, D=64, Nq=2, Nkv=500, Hq=8, Hkv=8, mask="bias", max_bias=8.0),
     dict(seed=213, D=128, Nq=1, Nkv=4096, Hq=16, Hkv=2, ktype=ora.F16),
+    dict(seed=214, D=64, Nq=1, Nkv=1237, Hq=12, Hkv=4, B=2, ktype=ora.Q8_0, mask="random_inf"),  # contiguous rows: streamed through LDS
+    dict(seed=215, D=128, Nq=2, Nkv=1031, Hq=8, Hkv=2, ktype=ora.Q8_0, kv_layout="thd"),         # head-interleaved rows: per-lane loads
+    dict(seed=216, D=128, Nq=1, Nkv=2049, Hq=8, Hkv=2, B=2, ktype=ora.Q8_0),
 ]
 
 
