@@ -135,6 +135,7 @@ def bench_encoder(args, ca, ora, torch):
         "parity": {"max_abs": max_abs, "rel_l2": rel, "ok": bool(parity_ok), "rows_checked": 50,
                    "oracle": "oracle/fattn_oracle.c exact mode"},
     }
+    res["scale_check"] = scale_check(ca, torch, layers[0])
     return res, host0
 
 
@@ -287,6 +288,154 @@ def bench_decode(args, ca, ora, torch):
     return out
 
 
+def _time_calls(torch, fn, reps):
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(5):                                # median of 5 batches of `reps` launches
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ts.append(e0.elapsed_time(e1) * 1e3 / reps)
+    return sorted(ts)[len(ts) // 2]
+
+
+def bench_configs(args, ca, ora, torch):
+    """The other configurations of the baseline file at their real shapes, one call each (back-to-back launches,
+    median of 5 batches), every one checked against the oracle (exact mode, all rows) before its time is reported.
+    FLOPs = 4*Nq*Nkv*D*Hq*B over the full rectangle; causal shapes also give the half-rectangle figure.
+    Bytes = Q f32 + K,V in storage type once per KV head + mask f16 + out f32."""
+    from cases import make_case, errors, MAX_ABS_TOL, REL_L2_TOL
+    res = {}
+
+    def run(name, spec, causal=False, note=""):
+        case = make_case(**spec)
+        q, k, v = (ca.Tensor.from_host(t.buf, t.type, t.ne, t.nb, t.offset) for t in (case["q"], case["k"], case["v"]))
+        mt = case["mask"]
+        m = ca.Tensor.from_host(mt.buf, mt.type, mt.ne, mt.nb, mt.offset) if mt is not None else None
+        D, Nq, Hq, B = q.ne
+        Nkv, Hkv, Bk = k.ne[1], k.ne[2], k.ne[3]
+        out = ca.Tensor.empty(ca.F32, (v.ne[0], Hq, Nq, B))
+        kern, ns = ca.ggml.flash_attn_plan(q, k, v, m, case["scale"])
+        fn = lambda: ca.flash_attn_ext(q, k, v, m, case["scale"], case["max_bias"], case["softcap"], out=out)
+        us = _time_calls(torch, fn, 20)
+        ref = ora.flash_attn_ext(case["q"], case["k"], case["v"], case["mask"], case["scale"], case["max_bias"],
+                                 case["softcap"], ora.MODE_EXACT)
+        max_abs, rel = errors(out.numpy_f32(), ref)
+        ok = bool(max_abs <= MAX_ABS_TOL and rel <= REL_L2_TOL)
+        row = ora.TYPE_SIZE[k.type] * D // (32 if k.type == ora.Q8_0 else 1)
+        nbytes = 2 * D * Nq * Hq * B * 4 + 2 * Nkv * Hkv * Bk * row + (mt.buf.size if mt is not None else 0)
+        flops = attn_flops(D, Nq, Nkv, Hq, B)
+        r = {"us_per_call": us if ok else None, "TFLOP/s": flops / us / 1e6 if ok else None,
+             "frac_of_f16_peak": flops / us / 1e6 / PEAK_F16_TFLOPS if ok else None,
+             "GB/s": nbytes / us / 1e3 if ok else None, "frac_of_hbm_peak": nbytes / us / 1e3 / PEAK_HBM_GBS if ok else None,
+             "flops": flops, "bytes": nbytes, "kernel": kern, "n_splits": ns,
+             "parity": {"max_abs": max_abs, "rel_l2": rel, "ok": ok}, "note": note}
+        if causal:
+            r["TFLOP/s_causal_half"] = r["TFLOP/s"] / 2 if ok else None
+        res[name] = r
+        log(f"[bench] {name}: {us:.1f} us/call, {flops / us / 1e6:.1f} TFLOP/s, {nbytes / us / 1e3:.0f} GB/s, kernel {kern} "
+            f"splits {ns}, parity max_abs={max_abs:.2e} rel_l2={rel:.2e} {'ok' if ok else 'FAIL: timing withheld'}")
+
+    run("C1_whisper_base_encoder", dict(seed=1, D=64, Nq=1500, Nkv=1500, Hq=8, scale=0.125, q_layout="thd", kv_layout="thd"),
+        note="8 heads x 64, 1500x1500, f16 K/V, Whisper strides, one window")
+    run("C1_kv_zero_padded_1536", dict(seed=1, D=64, Nq=1500, Nkv=1500, Hq=8, scale=0.125, q_layout="thd", kv_layout="thd",
+                                       kv_pad_rows=36), note="as the runtime calls it: 36 zero rows take part in the softmax")
+    run("C3_unified_cache_beam5", dict(seed=3, D=64, Nq=5, Nkv=1120, Hq=20, q_layout="thd", kv_layout="thd", mask="random_inf"),
+        note="5 beams vs one interleaved 1120-cell f16 cache, -inf mask picks each beam's cells (1 layer)")
+    for kt, nm in ((ora.Q8_0, "q8_0"), (ora.F16, "f16")):
+        run(f"C4_voxtral_prefill_{nm}", dict(seed=4, D=128, Nq=407, Nkv=407, Hq=32, Hkv=8, ktype=kt, mask="causal"), causal=True,
+            note="32 q / 8 kv heads x 128, T=407, causal f16 mask read from memory (1 layer)")
+    lengths = [ora.randint(5, b, 400, 750) for b in range(8)]
+    for kt, nm in ((ora.F16, "f16"), (ora.F32, "f32")):
+        run(f"C5_fastconformer_kv_{nm}", dict(seed=5, D=128, Nq=750, Nkv=750, Hq=8, B=8, ktype=kt, mask="bias_perhead_pad",
+                                              lengths=lengths),
+            note="8 heads x 128, T=750, batch 8, per-head f16 bias N(0, std 0.5) with -inf beyond each length (1 layer)")
+    return res
+
+
+def scale_check(ca, torch, layer):
+    """Halving the keys must about halve the time: a kernel that skipped work would not show it."""
+    D, N, H, B = layer["q"].ne
+    half = {n: layer[n].view((D, N // 2, H, B), layer[n].nb, 0) for n in ("k", "v")}
+    t_full = _time_calls(torch, lambda: ca.flash_attn_ext(layer["q"], layer["k"], layer["v"], None, 0.125, out=layer["out"]), 10)
+    t_half = _time_calls(torch, lambda: ca.flash_attn_ext(layer["q"], half["k"], half["v"], None, 0.125, out=layer["out"]), 10)
+    log(f"[bench] scale check: {N} keys: {t_full:.1f} us, {N // 2} keys: {t_half:.1f} us, ratio {t_full / t_half:.2f}")
+    return {"us_n_kv_full": t_full, "us_n_kv_half": t_half, "ratio": t_full / t_half}
+
+
+def bench_whisper_protocol(args, ca, ora, torch):
+    """Attention calls of the reference's Whisper bench protocol (examples/bench/bench.cpp:103-163) on a large-v3
+    decoder (32 layers, 20 heads x 64): heat, then 256 single-token decodes at n_past = i, 64 decodes of 5 tokens,
+    16 prompts of 256 tokens.  Each decode is 32 x (self-attention over the f16 cache with the causal f16 mask
+    + cross-attention over the 1536-row zero-padded encoder memory), launched call by call from the host as the
+    runtime does (it rebuilds its graph every call), so the figures include host launch cost."""
+    import numpy as np
+    D, H, L, CTX, NENC = 64, 20, 32, 448, 1536
+    n_state = D * H
+
+    def f16_buf(n):
+        return torch.randn(n, device="cuda").half().view(torch.uint8)
+
+    layers = []
+    for l in range(L):
+        kc, vc = f16_buf(NENC * n_state), f16_buf(NENC * n_state)
+        kc.view(torch.float16)[1500 * n_state:] = 0
+        vc.view(torch.float16)[1500 * n_state:] = 0
+        layers.append({"ks": f16_buf(CTX * n_state), "vs": f16_buf(CTX * n_state), "kc": kc, "vc": vc})
+    qbuf = torch.randn(256 * n_state, device="cuda").view(torch.uint8)
+    obuf = torch.empty(256 * n_state, device="cuda")
+    masks = {}
+
+    def mask_for(n_tok, n_past):
+        key = (n_tok, n_past)
+        if key not in masks:
+            n_kv = n_past + n_tok
+            m = np.zeros((n_tok, n_kv), np.float32)
+            for t in range(n_tok):
+                m[t, n_past + t + 1:] = -np.inf
+            masks[key] = ca.Tensor.from_host(ora.fp32_to_fp16(m), ca.F16, (n_kv, n_tok, 1, 1))
+        return masks[key]
+
+    def decode(n_tok, n_past):
+        n_kv = n_past + n_tok
+        q = ca.Tensor(qbuf, ca.F32, (D, n_tok, H, 1), (4, 4 * n_state, 4 * D, 4 * n_state * n_tok))
+        out = ca.Tensor(obuf.view(torch.uint8), ca.F32, (D, H, n_tok, 1))
+        m = mask_for(n_tok, n_past)
+        for lay in layers:
+            nbs = (2, 2 * n_state, 2 * D, 2 * n_state * n_kv)
+            nbc = (2, 2 * n_state, 2 * D, 2 * n_state * NENC)
+            ca.flash_attn_ext(q, ca.Tensor(lay["ks"], ca.F16, (D, n_kv, H, 1), nbs), ca.Tensor(lay["vs"], ca.F16, (D, n_kv, H, 1), nbs),
+                              m, 1.0, out=out)
+            ca.flash_attn_ext(q, ca.Tensor(lay["kc"], ca.F16, (D, NENC, H, 1), nbc), ca.Tensor(lay["vc"], ca.F16, (D, NENC, H, 1), nbc),
+                              None, 64 ** -0.25, out=out)
+
+    for _ in range(2):                                  # heat, as the protocol does
+        decode(256, 0)
+        for i in range(0, 256, 16):
+            decode(1, i)
+        decode(5, 0)
+    for i in range(256):
+        mask_for(1, i)
+    torch.cuda.synchronize()
+    res = {}
+    for name, n, fn in (("single_token_x256", 256, lambda i: decode(1, i)), ("batch5_x64", 64, lambda i: decode(5, 0)),
+                        ("prompt256_x16", 16, lambda i: decode(256, 0))):
+        t0 = time.perf_counter()
+        for i in range(n):
+            fn(i)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3
+        res[name] = {"ms_total": ms, "ms_per_decode": ms / n, "us_per_attention_call": ms * 1e3 / (n * 2 * L)}
+        log(f"[bench] whisper protocol {name}: {ms:.1f} ms total, {ms / n:.3f} ms per decode (64 attention calls), "
+            f"{ms * 1e3 / (n * 2 * L):.1f} us per call incl. host launch")
+    return res
+
+
 def copy_calibration(ca, torch):
     """A plain copy of known size through the library's own CPY kernel (128-bit path): 256 MiB read + 256 MiB written.
     It gives the counter-to-bytes factor for the rocprofv3 FETCH_SIZE / WRITE_SIZE traffic figures."""
@@ -315,6 +464,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="skip the other baseline configurations and the Whisper protocol")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU form in this build (heads and windows "
@@ -342,12 +492,15 @@ def main():
                                "1500x1500 non-causal), batch of 4 windows, Q f32 / K,V f16, scale 1/8; "
                                "N(0,1) per-layer seeded; FLOPs = 4*Nq*Nkv*D*H*B per layer",
                    "layers": 32, "heads": 20, "head_dim": 64, "n_q": 1500, "n_kv": 1500, "batch": 4},
-        "roofline": enc["roofline"], "parity": enc["parity"],
+        "roofline": enc["roofline"], "parity": enc["parity"], "scale_check": enc["scale_check"],
         "device": {"name": info["name"], "arch": info["arch"], "cus": info["compute_units"], "clock_khz": info["clock_khz"]},
     }
     line["copy_calibration"] = copy_calibration(ca, torch)
     if not args.no_decode:
         line["decode"] = bench_decode(args, ca, ora, torch)
+    if not args.no_configs:
+        line["configs"] = bench_configs(args, ca, ora, torch)
+        line["whisper_bench_protocol"] = bench_whisper_protocol(args, ca, ora, torch)
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args, ora, host0)
     if not enc["parity"]["ok"]:

@@ -55,14 +55,21 @@ __device__ __forceinline__ uint2 q8_load_chunk(const char * row, int blk, int c)
 }
 
 // the same from a raw copy of the rows in LDS (row_off = byte offset of the row inside the stage)
+// (row_off is a multiple of 4, so odd blocks start on a dword; UNIFORM_BLK says blk is the same in every lane)
+template <bool UNIFORM_BLK>
 __device__ __forceinline__ uint4 q8_lds_chunk(const char * stage, int row_off, int blk, int c) {
     const int o  = row_off + blk * FATTN_Q8_0_BYTES + 2 + c * 8;
-    const int sh = o & 3;
+    const int sh = (blk & 1) ? 0 : 2;
     const uint32_t * p = (const uint32_t *)(stage + (o - sh));
     const uint32_t u0 = p[0], u1 = p[1], u2 = p[2];         // the stage is padded: p[2] is always inside it
     uint4 r;
-    r.x = __builtin_amdgcn_alignbyte(u1, u0, sh);
-    r.y = __builtin_amdgcn_alignbyte(u2, u1, sh);
+    if (UNIFORM_BLK && (blk & 1)) {
+        r.x = u0;
+        r.y = u1;
+    } else {
+        r.x = __builtin_amdgcn_alignbyte(u1, u0, sh);
+        r.y = __builtin_amdgcn_alignbyte(u2, u1, sh);
+    }
     r.z = *(const uint16_t *)(stage + row_off + blk * FATTN_Q8_0_BYTES);
     r.w = 0;
     return r;
@@ -147,14 +154,14 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     // the per-wave stages; after the key loop the same memory carries the cross-wave reduction
     extern __shared__ __attribute__((aligned(16))) char smem[];
     constexpr int WAVE_BYTES = STEP * PV * 2 + (RAW ? 2 * RAWSZ : 0);
-    _Float16 * v_stage = (_Float16 *)(smem + (threadIdx.x >> 6) * WAVE_BYTES);
-    char * k_rawst     = smem + (threadIdx.x >> 6) * WAVE_BYTES + STEP * PV * 2;
+    _Float16 * v_stage = (_Float16 *)(smem + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * WAVE_BYTES);
+    char * k_rawst     = smem + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * WAVE_BYTES + STEP * PV * 2;
     char * v_rawst     = k_rawst + RAWSZ;
     float (*red_o)[16][D + 1]      = (float (*)[16][D + 1])smem;
     float (*red_ml)[16][2]         = (float (*)[16][2])(smem + DEC_WAVES * 16 * (D + 1) * 4);
 
     const int tid  = threadIdx.x;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // uniform: loop control and row bases stay scalar
     const int lane = tid & 63;
     const int j    = lane & 15;                    // query column
     const int g4   = lane >> 4;
@@ -174,19 +181,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     const int k_begin = split * a.keys_per_split;
     const int k_end   = min(a.Nkv, k_begin + a.keys_per_split);
 
-    // ---- Q -> f16 B operands in log2 units -----------------------------------------------------
     half8 qreg[KS];
-    {
-        const float * qrow = (const float *)(a.q + (int64_t)iq1 * a.nbq1 + (int64_t)h * a.nbq2 + (int64_t)b * a.nbq3);
-        const float   qs   = a.scale * LOG2E;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            half8 v;
-#pragma unroll
-            for (int e = 0; e < 8; e++) v[e] = (_Float16)(qrow[ks * 32 + g4 * 8 + e] * qs);
-            qreg[ks] = v;
-        }
-    }
     const char * kbase = a.k + (int64_t)hk * a.nbk2 + (int64_t)bk * a.nbk3;
     const char * vbase = a.v + (int64_t)hk * a.nbv2 + (int64_t)bk * a.nbv3;
     const uint16_t * mrow = MASK
@@ -205,19 +200,21 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     Chunk vraw[2][RAW ? 1 : NV];
     typedef typename std::conditional<UNIT == 8, uint2, uint32_t>::type unit_t;
     unit_t kun[2][RAW ? NU : 1], vun[2][RAW ? NU : 1];
-    auto issue = [&](int j0, auto stage) {
+    // a partial last step: its loads are clamped to the last valid row or unit (branch-free, in bounds) and the
+    // keys they stand for are excluded in the step
+    auto issue = [&](int it, auto stage) __attribute__((always_inline)) {
         constexpr int s = decltype(stage)::value;
+        const int j0 = k_begin + it * STEP;
         if (RAW) {
-            // one coalesced stream per tensor; units past the last valid row of a partial step re-read the last
-            // valid unit (branch-free, in bounds), the keys they belong to are excluded below
-            const int n_units = min(STEP, k_end - j0) * (RS / UNIT);
+            // one coalesced stream per tensor
+            const int last = min(STEP, k_end - j0) * (RS / UNIT) - 1;
             const char * kp = kbase + (int64_t)j0 * RS;
             const char * vp = vbase + (int64_t)j0 * RS;
 #pragma unroll
             for (int i = 0; i < NU; i++) {
-                const int u = min(i * 64 + lane, n_units - 1);
-                kun[s][i] = *(const unit_t *)(kp + u * UNIT);
-                vun[s][i] = *(const unit_t *)(vp + u * UNIT);
+                const uint32_t off = (uint32_t)min(i * 64 + lane, last) * UNIT;
+                kun[s][i] = *(const unit_t *)(kp + off);
+                vun[s][i] = *(const unit_t *)(vp + off);
             }
             return;
         }
@@ -241,16 +238,25 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     typedef std::integral_constant<int, 1> S1;
 
     // one step of 32 keys out of register stage s; the following step is requested into the other stage
-    auto step = [&](const int it, auto stage) {
+    auto step = [&](const int it, auto stage) __attribute__((always_inline)) {
         constexpr int s = decltype(stage)::value;
-        const int j0 = k_begin + it * STEP;
-        if (it + DEC_WAVES < n_steps) issue(j0 + DEC_WAVES * STEP, std::integral_constant<int, 1 - s>{});
+        const int  j0   = k_begin + it * STEP;
+        const bool tail = j0 + STEP > k_end;                  // wave-uniform
+        if (it + DEC_WAVES < n_steps) issue(it + DEC_WAVES, std::integral_constant<int, 1 - s>{});
 
         if (RAW) {
 #pragma unroll
             for (int i = 0; i < NU; i++) {
                 *(unit_t *)(k_rawst + (i * 64 + lane) * UNIT) = kun[s][i];
                 *(unit_t *)(v_rawst + (i * 64 + lane) * UNIT) = vun[s][i];
+            }
+            if (tail) {
+                // rows past k_end hold bytes of no row: a zero scale keeps what is made of them finite
+#pragma unroll
+                for (int t = 0; t < STEP * KS / 64; t++) {
+                    const int idx = t * 64 + lane;
+                    if (j0 + idx / KS >= k_end) *(uint16_t *)(v_rawst + (idx / KS) * RS + (idx % KS) * FATTN_Q8_0_BYTES) = 0;
+                }
             }
             __builtin_amdgcn_wave_barrier();
         }
@@ -262,7 +268,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
                 Chunk c;
-                if (RAW) c.v = q8_lds_chunk(k_rawst, (kb * 16 + j) * RS, ks, g4);
+                if (RAW) c.v = q8_lds_chunk<true>(k_rawst, (kb * 16 + j) * RS, ks, g4);
                 else     c = kraw[s][kb][ks];
                 sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_to_half8<TYPE>(c), qreg[ks], sc[kb], 0, 0, 0);
             }
@@ -273,8 +279,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
             const int flat = i * 64 + lane;
             Chunk c;
             if (RAW) {
-                c.v = q8_lds_chunk(v_rawst, (flat / CH) * RS, (flat % CH) >> 2, (flat % CH) & 3);
-                if (j0 + flat / CH >= k_end) c.v = make_uint4(0, 0, 0, 0);       // bytes of no row: keep them finite
+                c.v = q8_lds_chunk<false>(v_rawst, (flat / CH) * RS, (flat % CH) >> 2, (flat % CH) & 3);
             } else {
                 c = vraw[s][i];
             }
@@ -291,7 +296,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
                 const int key = j0 + kb * 16 + g4 * 4 + r;
                 float x = sc[kb][r];
                 if (MASK) x = fmaf(mslope, h2f_bits(mrow[min(key, k_end - 1)]), x);
-                if (key >= k_end) x = -INFINITY;
+                if (tail && key >= k_end) x = -INFINITY;
                 sv[kb * 4 + r] = x - m;
             }
 
@@ -351,8 +356,20 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
         }
         __builtin_amdgcn_wave_barrier();
     };
+    if (wave < n_steps) issue(wave, S0{});
 
-    if (wave < n_steps) issue(k_begin + wave * STEP, S0{});
+    // ---- Q -> f16 B operands in log2 units (after the first K/V request: the two cold misses overlap) ----
+    {
+        const float * qrow = (const float *)(a.q + (int64_t)iq1 * a.nbq1 + (int64_t)h * a.nbq2 + (int64_t)b * a.nbq3);
+        const float   qs   = a.scale * LOG2E;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            half8 v;
+#pragma unroll
+            for (int e = 0; e < 8; e++) v[e] = (_Float16)(qrow[ks * 32 + g4 * 8 + e] * qs);
+            qreg[ks] = v;
+        }
+    }
     for (int it = wave; it < n_steps; it += 2 * DEC_WAVES) {
         step(it, S0{});
         if (it + DEC_WAVES < n_steps) step(it + DEC_WAVES, S1{});
@@ -401,7 +418,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
             }
         }
         if (a.n_splits > 1 && (tid & 15) == 0) {
-            // the merge kernel works in natural-log units
+            // natural-log units, as the merge kernel expects them
             float * pm = a.part_ml + (row * a.n_splits + split) * 2;
             pm[0] = M == -INFINITY ? -INFINITY : M * 0.6931471805599453f;
             pm[1] = L;

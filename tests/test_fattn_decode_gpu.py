@@ -79,3 +79,20 @@ def test_decode_q8_0_dequantisation_in_registers_is_exact():
     for b in range(3):
         for h in range(4):
             assert np.array_equal(got[b, 0, h], v[b, h, pick[b]]) and np.array_equal(got[b, 1, h], v[b, h, pick[b]])
+
+
+def test_split_counts_and_caller_workspace():
+    """Any split count gives the same result, with the library's scratch or with a caller's workspace."""
+    import torch
+    case = make_case(seed=231, D=128, Nq=1, Nkv=1500, Hq=16, Hkv=4, B=3, ktype=ora.Q8_0)
+    ref = run_oracle(case)
+    for ns in (5, 2, 7):
+        assert_parity(run_gpu(case, kernel=ggml.KERNEL_DECODE_MMA, n_splits=ns), ref, "library scratch %d" % ns)
+    q, k, v = upload(case["q"]), upload(case["k"]), upload(case["v"])
+    ws = torch.empty(16 * 3 * 7 * (128 + 2), dtype=torch.float32, device="cuda")
+    for ns in (7, 4):
+        out = ggml.flash_attn_ext(q, k, v, None, case["scale"], kernel=ggml.KERNEL_DECODE_MMA, n_splits=ns, workspace=ws)
+        assert_parity(out.numpy_f32(), ref, "caller workspace %d" % ns)
+    small = torch.empty(16, dtype=torch.float32, device="cuda")
+    with pytest.raises(ggml.Mi355xError):
+        ggml.flash_attn_ext(q, k, v, None, case["scale"], kernel=ggml.KERNEL_DECODE_MMA, n_splits=4, workspace=small)
