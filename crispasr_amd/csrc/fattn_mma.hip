@@ -20,6 +20,12 @@
 // 32-byte row segments of four keys and each lane receives the four keys' values of its own
 // d - V's pitch is 64 mod 128 bytes so that those four segments tile the banks.
 //
+// F16 caches skip the registers on the way in (DIRECT): global_load_lds_dwordx4 writes each wave's 64 x 16
+// bytes straight into LDS.  Such a load fills 1 KiB of consecutive LDS, so rows cannot be padded; instead
+// the 16-byte chunks of a row are stored XOR-swizzled (each lane fetches the global chunk that belongs at
+// its LDS slot), with one swizzle for K (128-bit operand reads: 16 consecutive rows, one chunk column) and
+// one for V (transpose reads: 8 rows x 4 chunk columns), both conflict-free.
+//
 // Softmax runs in base 2: scale*log2(e) is folded into Q when it is converted to f16.
 #include "fattn_common.h"
 
@@ -117,8 +123,17 @@ struct RowState {
 // a block of 16 probabilities summing to more than this means the reference is > 9 behind
 constexpr float SUM_LIMIT = 8192.0f;
 
-template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP>
+// chunk swizzles of the unpadded DIRECT layout (r = key row inside the tile)
+template <int D> __device__ __forceinline__ int swz_k(int r) { return D == 64 ? (r >> 1) & 7 : r & 15; }
+template <int D> __device__ __forceinline__ int swz_v(int r) { return D == 64 ? r & 7 : (r & 3) << 2; }
+
+template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT>
 __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnArgs a, const int n_qtiles) {
+    static_assert(!DIRECT || TYPE == MI355X_TYPE_F16, "only f16 rows can go to LDS unconverted");
+    constexpr int ROWB  = D * 2;                   // DIRECT: bytes per (unpadded) row
+    constexpr int TILEB = BC * ROWB;               //         bytes per K or V tile; LDS = K0 K1 V0 V1
+    constexpr int NLD   = TILEB / 1024 / MMA_WAVES;   //      global->LDS loads per wave, tile and tensor
+
     constexpr int KS   = D / 16;                   // reduction steps of Q.K^T
     constexpr int DB   = D / 32;                   // 32-wide blocks of the output's d
     constexpr int CH   = D / 8;                    // 8-element chunks per row
@@ -134,7 +149,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     _Float16 (*v_lds)[BC * PV] = (_Float16 (*)[BC * PV])(lds_raw + 2 * BC * PK);
 
     const int tid  = threadIdx.x;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int l32  = lane & 31;
     const int hh   = lane >> 5;                    // which half of the wave
@@ -211,6 +226,49 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         }
     };
 
+    // DIRECT: lane's share of a tile is NLD 16-byte chunks per tensor; LDS slot L = (wave*NLD + j)*64 + lane
+    // holds chunk (L % CH) ^ swizzle of row L / CH.  Offsets are relative to the tile's first row.
+    uint32_t koff[DIRECT ? NLD : 1], voff[DIRECT ? NLD : 1];
+    uint32_t kaddr[DIRECT ? KS : 1], vaddr[DIRECT ? DB : 1];      // operand read offsets (bytes) inside a K / V buffer
+    if (DIRECT) {
+#pragma unroll
+        for (int j = 0; j < NLD; j++) {
+            const int L = (wave * NLD + j) * 64 + lane;
+            const int r = L / CH, c = L % CH;
+            koff[j] = (uint32_t)r * (uint32_t)a.nbk1 + (uint32_t)((c ^ swz_k<D>(r)) * 16);
+            voff[j] = (uint32_t)r * (uint32_t)a.nbv1 + (uint32_t)((c ^ swz_v<D>(r)) * 16);
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) kaddr[ks] = (uint32_t)((l32 * CH + ((ks * 2 + hh) ^ swz_k<D>(l32))) * 16);
+        const int i16 = lane & 15;
+        const int kr0 = hh * 4 + (i16 >> 2);
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+            const int c = db * 4 + ((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1);
+            vaddr[db] = (uint32_t)((kr0 * CH + (c ^ swz_v<D>(kr0))) * 16 + 8 * (i16 & 1));
+        }
+    }
+    typedef __attribute__((address_space(3))) void * lds_vptr;
+    typedef const __attribute__((address_space(1))) void * glb_vptr;
+    auto load_direct = [&](int j0, char * wk, char * wv, bool tail) __attribute__((always_inline)) {
+        const char * kp = kbase + (int64_t)j0 * a.nbk1;
+        const char * vp = vbase + (int64_t)j0 * a.nbv1;
+        char * lk = wk + wave * (NLD * 1024);
+        char * lv = wv + wave * (NLD * 1024);
+#pragma unroll
+        for (int j = 0; j < NLD; j++) {
+            uint32_t ko = koff[j], vo = voff[j];
+            if (tail) {       // rows past Nkv re-read the last row (their scores are excluded)
+                const int L = (wave * NLD + j) * 64 + lane;
+                const int r = L / CH, c = L % CH, rr = min(r, a.Nkv - 1 - j0);
+                ko = (uint32_t)rr * (uint32_t)a.nbk1 + (uint32_t)((c ^ swz_k<D>(r)) * 16);
+                vo = (uint32_t)rr * (uint32_t)a.nbv1 + (uint32_t)((c ^ swz_v<D>(r)) * 16);
+            }
+            __builtin_amdgcn_global_load_lds((glb_vptr)(kp + ko), (lds_vptr)(lk + j * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((glb_vptr)(vp + vo), (lds_vptr)(lv + j * 1024), 16, 0, 0);
+        }
+    };
+
     float16v oacc[NQB][DB];
     float16v negm[NQB];            // -m in all 16 slots: the C operand of the first Q.K^T MFMA
     RowState st[NQB];
@@ -228,8 +286,13 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     }
 
     // One tile of 64 keys.  TAIL: the tile runs past Nkv (keys beyond it are excluded).
-    auto tile = [&](const int j0, const int buf, auto tail_tag) {
+    // DIRECT: operands are read from rk / rv while the tile at key jn (if any) is requested into wk / wv.  The four
+    // are distinct buffers, and saying so (restrict) is what lets the compiler keep the operand reads from
+    // waiting on the loads that have just been issued.
+    auto tile = [&](const int j0, const int buf, auto tail_tag, const char * __restrict__ rk, const char * __restrict__ rv,
+                    char * __restrict__ wk, char * __restrict__ wv, const int jn, const bool tn) __attribute__((always_inline)) {
         constexpr bool TAIL = decltype(tail_tag)::value;
+        if (DIRECT && jn >= 0) load_direct(jn, wk, wv, tn);
 
         // additive mask values of this lane's 32 (key, query) pairs per query block, fetched early
         uint2 mraw[NQB][2][4];
@@ -257,7 +320,8 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         auto load_k = [&](int kb, half8 (&ka)[KS]) {
 #pragma unroll
             for (int ks = 0; ks < KS; ks++)
-                ka[ks] = *(const half8 *)&k_lds[buf][(kb * 32 + l32) * PK + ks * 16 + hh * 8];
+                ka[ks] = DIRECT ? *(const half8 *)(rk + kaddr[ks] + kb * 32 * ROWB)
+                                : *(const half8 *)&k_lds[buf][(kb * 32 + l32) * PK + ks * 16 + hh * 8];
         };
         // V^T operands of a 32-key block by transpose reads: lane i of a 16-lane block addresses
         // 4 halves of key (i/4) at d0 + 4*(i%4) and receives 4 keys' values of d0 + i
@@ -269,8 +333,9 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                 for (int db = 0; db < DB; db++) {
                     const int d0 = db * 32 + ((lane >> 4) & 1) * 16;
                     const int kr = (kb * 2 + k2) * 16 + hh * 4 + (i16 >> 2);
-                    const _Float16 * p0 = &v_lds[buf][kr * PV + d0 + (i16 & 3) * 4];
-                    const _Float16 * p1 = p0 + 8 * PV;
+                    const _Float16 * p0 = DIRECT ? (const _Float16 *)(rv + vaddr[db] + (kb * 2 + k2) * 16 * ROWB)
+                                                 : &v_lds[buf][kr * PV + d0 + (i16 & 3) * 4];
+                    const _Float16 * p1 = p0 + 8 * (DIRECT ? D : PV);
                     const half4 lo = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p0));
                     const half4 hi = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p1));
                     va[k2][db] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -411,6 +476,23 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
 
     const int n_tiles = (a.Nkv + BC - 1) / BC;
     const int n_full  = a.Nkv / BC;
+    if (DIRECT) {
+        char * const lb = (char *)lds_raw;               // K0 K1 V0 V1
+        load_direct(0, lb, lb + 2 * TILEB, n_full == 0);
+        __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): this wave's share of the tile is in LDS
+        __syncthreads();
+        for (int t = 0; t < n_full; t++) {
+            const int cur = (t & 1) * TILEB, nxt = TILEB - cur;
+            const int jn  = t + 1 < n_tiles ? (t + 1) * BC : -1;
+            tile(t * BC, 0, std::false_type{}, lb + cur, lb + 2 * TILEB + cur, lb + nxt, lb + 2 * TILEB + nxt, jn, t + 1 >= n_full);
+            __builtin_amdgcn_s_waitcnt(0x0F70);
+            __syncthreads();
+        }
+        if (n_full < n_tiles) {
+            const int cur = (n_full & 1) * TILEB;
+            tile(n_full * BC, 0, std::true_type{}, lb + cur, lb + 2 * TILEB + cur, nullptr, nullptr, -1, false);
+        }
+    } else {
     load_tile(0);
     store_tile(0);
     __syncthreads();
@@ -420,12 +502,13 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         const int  buf  = t & 1;
         const bool more = t + 1 < n_tiles;
         if (more) load_tile((t + 1) * BC);
-        tile(t * BC, buf, std::false_type{});
+        tile(t * BC, buf, std::false_type{}, nullptr, nullptr, nullptr, nullptr, -1, false);
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
     // at most one partial tile, already staged by the last iteration above (or the prologue)
-    if (n_full < n_tiles) tile(n_full * BC, n_full & 1, std::true_type{});
+    if (n_full < n_tiles) tile(n_full * BC, n_full & 1, std::true_type{}, nullptr, nullptr, nullptr, nullptr, -1, false);
+    }
 
     // ---- normalise and write dst[D, Hq, Nq, B] -------------------------------------------------------
 #pragma unroll
@@ -450,15 +533,16 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     }
 }
 
-template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP>
+template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT>
 int launch(const FattnArgs & a, hipStream_t stream) {
     const int bmg = 32 * NQB * MMA_WAVES;
     const int n_qtiles = (a.Nq + bmg - 1) / bmg;
     const dim3 grid((unsigned)(n_qtiles * a.Hq * a.B));
-    const size_t lds = (size_t)2 * BC * (Pitch<D>::K + Pitch<D>::V) * sizeof(_Float16);
+    const size_t lds = DIRECT ? (size_t)4 * BC * D * sizeof(_Float16)
+                              : (size_t)2 * BC * (Pitch<D>::K + Pitch<D>::V) * sizeof(_Float16);
     static bool attr_set = false;     // per instantiation; the attribute only matters above 64 KiB
     if (!attr_set && lds > 64 * 1024) {
-        const hipError_t e = hipFuncSetAttribute((const void *)fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP>,
+        const hipError_t e = hipFuncSetAttribute((const void *)fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP, DIRECT>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
         attr_set = true;
@@ -466,19 +550,28 @@ int launch(const FattnArgs & a, hipStream_t stream) {
     static const bool debug = getenv("MI355X_FATTN_DEBUG") != nullptr;
     if (debug) {
         int nb = -1;
-        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void *)fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP>, MMA_THREADS, lds);
-        fprintf(stderr, "[mi355x] fattn_mma<%d,%d,%d,%d,%d> grid %u lds %zu B, resident workgroups per CU: %d\n",
-                D, NQB, TYPE, (int)MASK, (int)SOFTCAP, grid.x, lds, nb);
+        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void *)fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP, DIRECT>, MMA_THREADS, lds);
+        fprintf(stderr, "[mi355x] fattn_mma<%d,%d,%d,%d,%d,%d> grid %u lds %zu B, resident workgroups per CU: %d\n",
+                D, NQB, TYPE, (int)MASK, (int)SOFTCAP, (int)DIRECT, grid.x, lds, nb);
     }
-    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
+    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP, DIRECT>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
     return (int)hipGetLastError();
+}
+
+template <int D, int NQB, int TYPE, bool DIRECT>
+int launch_mask(const FattnArgs & a, hipStream_t stream) {
+    const bool mask = a.mask != nullptr;
+    if (a.softcap != 0.0f) return mask ? launch<D, NQB, TYPE, true, true, DIRECT>(a, stream) : launch<D, NQB, TYPE, false, true, DIRECT>(a, stream);
+    return mask ? launch<D, NQB, TYPE, true, false, DIRECT>(a, stream) : launch<D, NQB, TYPE, false, false, DIRECT>(a, stream);
 }
 
 template <int D, int NQB, int TYPE>
 int launch_flags(const FattnArgs & a, hipStream_t stream) {
-    const bool mask = a.mask != nullptr;
-    if (a.softcap != 0.0f) return mask ? launch<D, NQB, TYPE, true, true>(a, stream) : launch<D, NQB, TYPE, false, true>(a, stream);
-    return mask ? launch<D, NQB, TYPE, true, false>(a, stream) : launch<D, NQB, TYPE, false, false>(a, stream);
+    // f16 rows go straight to LDS when a tile's row offsets fit 32 bits
+    static const bool no_direct = getenv("MI355X_FATTN_NO_DIRECT") != nullptr;       // experiments only
+    if (TYPE == MI355X_TYPE_F16 && !no_direct && a.nbk1 < (1u << 24) && a.nbv1 < (1u << 24))
+        return launch_mask<D, NQB, MI355X_TYPE_F16, true>(a, stream);
+    return launch_mask<D, NQB, TYPE, false>(a, stream);
 }
 
 template <int TYPE>
@@ -486,7 +579,8 @@ int launch_type(const FattnArgs & a, hipStream_t stream) {
     // two query blocks per wave halve the LDS operand traffic per MFMA; one block keeps more
     // workgroups in flight when there are few queries
     const int64_t wg2 = (int64_t)((a.Nq + 255) / 256) * a.Hq * a.B;
-    const bool two = wg2 >= 128;
+    static const char * force = getenv("MI355X_FATTN_NQB");          // experiments only
+    const bool two = force ? atoi(force) == 2 : wg2 >= 128;
     if (a.D == 64)  return two ? launch_flags<64, 2, TYPE>(a, stream) : launch_flags<64, 1, TYPE>(a, stream);
     if (a.D == 128) return launch_flags<128, 1, TYPE>(a, stream);
     return (int)hipErrorInvalidValue;

@@ -152,6 +152,7 @@ class Tensor:
         self.ne = tuple(int(x) for x in ne) + (1,) * (4 - len(ne))
         self.nb = tuple(int(x) for x in (nb if nb is not None else contiguous_nb(self.type, self.ne)))
         self.offset = int(offset)
+        self._c = None                      # the C descriptor, built once: a view never changes
         if buf is not None:
             assert buf.dtype == torch.uint8 and buf.dim() == 1 and buf.is_contiguous()
 
@@ -192,12 +193,19 @@ class Tensor:
         return self.buf.data_ptr() + self.offset
 
     def c(self) -> CTensor:
-        t = CTensor()
-        t.data = self.data_ptr()
-        t.type = self.type
-        t.ne = (ctypes.c_int64 * 4)(*self.ne)
-        t.nb = (ctypes.c_size_t * 4)(*self.nb)
-        return t
+        if self._c is None:
+            t = CTensor()
+            t.data = self.data_ptr()
+            t.type = self.type
+            t.ne = (ctypes.c_int64 * 4)(*self.ne)
+            t.nb = (ctypes.c_size_t * 4)(*self.nb)
+            self._c = (t, ctypes.byref(t))
+        return self._c[0]
+
+    def ref(self):
+        """pointer to the C descriptor, as the entry points take it"""
+        self.c()
+        return self._c[1]
 
     def to_host(self) -> np.ndarray:
         """ggml_backend_tensor_get of the whole underlying buffer (uint8)"""
@@ -209,6 +217,25 @@ class Tensor:
         n = self.ne[0] * self.ne[1] * self.ne[2] * self.ne[3]
         raw = self.buf[self.offset:self.offset + 4 * n].cpu().numpy()
         return raw.view(np.float32).reshape(self.ne[3], self.ne[2], self.ne[1], self.ne[0]).copy()
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(device):
+    """make `device` current for the call; no context switch when it already is"""
+    idx = device.index
+    if idx is None or idx == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 def _stream_handle(stream) -> int:
@@ -267,12 +294,9 @@ def flash_attn_ext(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor], scal
     if out is None:
         out = Tensor.empty(F32, (v.ne[0], q.ne[2], q.ne[1], q.ne[3]), device=q.buf.device)
     p = _params(scale, max_bias, logit_softcap, prec, kernel, n_splits, workspace)
-    cq, ck, cv, co = q.c(), k.c(), v.c(), out.c()
-    cm = mask.c() if mask is not None else None
-    with torch.cuda.device(q.buf.device):
-        _check(lib().mi355x_flash_attn_ext(ctypes.byref(cq), ctypes.byref(ck), ctypes.byref(cv),
-                                           ctypes.byref(cm) if cm is not None else None, ctypes.byref(co),
-                                           ctypes.byref(p), _stream_handle(stream)))
+    with _on_device(q.buf.device):
+        _check(lib().mi355x_flash_attn_ext(q.ref(), k.ref(), v.ref(), mask.ref() if mask is not None else None,
+                                           out.ref(), ctypes.byref(p), _stream_handle(stream)))
     return out
 
 
