@@ -188,6 +188,9 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
         bool m8 = !((uintptr_t)mask->data % 8);
         for (int i = 1; i < 4; i++) m8 = m8 && !(mask->nb[i] % 8);
         a.mask_al8 = m8 ? 1 : 0;
+        bool m4 = !((uintptr_t)mask->data % 4);
+        for (int i = 1; i < 4; i++) m4 = m4 && !(mask->nb[i] % 4);
+        a.mask_al4 = m4 ? 1 : 0;
     }
     a.aligned16 = al16 ? 1 : 0;
     a.softcap = p->logit_softcap;

@@ -26,6 +26,10 @@
 // its LDS slot), with one swizzle for K (128-bit operand reads: 16 consecutive rows, one chunk column) and
 // one for V (transpose reads: 8 rows x 4 chunk columns), both conflict-free.
 //
+// The mask of such a kernel takes the same road (MDMA): each wave fetches the 32 keys x its own queries that a
+// half tile needs into a private, swizzled LDS block half a tile before they are read, instead of having
+// every lane pull 8-byte pieces of 32 different rows through the vector cache.
+//
 // Softmax runs in base 2: scale*log2(e) is folded into Q when it is converted to f16.
 #include "fattn_common.h"
 
@@ -127,9 +131,14 @@ constexpr float SUM_LIMIT = 8192.0f;
 template <int D> __device__ __forceinline__ int swz_k(int r) { return D == 64 ? (r >> 1) & 7 : r & 15; }
 template <int D> __device__ __forceinline__ int swz_v(int r) { return D == 64 ? r & 7 : (r & 3) << 2; }
 
-template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT>
+template <int D> __device__ __forceinline__ int swz_m(int r) { return (r >> 2) & 3; }     // mask half tile: 4 chunks per row
+
+template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA>
 __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnArgs a, const int n_qtiles) {
     static_assert(!DIRECT || TYPE == MI355X_TYPE_F16, "only f16 rows can go to LDS unconverted");
+    static_assert(!MDMA || (DIRECT && MASK), "the mask goes through LDS only beside directly loaded K/V");
+    constexpr int NMH   = NQB * 2;                 // MDMA: loads per wave and half tile (16 rows x 64 bytes each)
+    constexpr int MHALF = NQB * 32 * 64;           //       bytes of a wave's half-tile block; a wave owns 2 of them
     constexpr int ROWB  = D * 2;                   // DIRECT: bytes per (unpadded) row
     constexpr int TILEB = BC * ROWB;               //         bytes per K or V tile; LDS = K0 K1 V0 V1
     constexpr int NLD   = TILEB / 1024 / MMA_WAVES;   //      global->LDS loads per wave, tile and tensor
@@ -250,6 +259,70 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     }
     typedef __attribute__((address_space(3))) void * lds_vptr;
     typedef const __attribute__((address_space(1))) void * glb_vptr;
+    // MDMA: slot (row, s) of a half-tile block holds the 8 keys of chunk s ^ swizzle(row) of query q0 + row
+    uint32_t moff[MDMA ? NMH : 1], maddr[MDMA ? 4 : 1];
+    const char * mhead = nullptr;
+    if (MDMA) {
+        mhead = a.mask + (int64_t)(h % a.Hm) * a.nbm2 + (int64_t)(b % a.Bm) * a.nbm3;
+#pragma unroll
+        for (int j = 0; j < NMH; j++) {
+            const int row = j * 16 + (lane >> 2);
+            moff[j] = (uint32_t)min(q0 + row, a.Nq - 1) * (uint32_t)a.nbm1 + (uint32_t)((((lane & 3) ^ swz_m<D>(row))) * 16);
+        }
+#pragma unroll
+        for (int g = 0; g < 4; g++) maddr[g] = (uint32_t)(l32 * 64 + ((g ^ swz_m<D>(l32)) * 16) + 8 * hh);
+    }
+    // half tile hf of the tile at key j0 -> this wave's block hf of mb.  `after` is a value the requests must not
+    // overtake: the empty asm ties the addresses to it, so the loads issue only once it has been computed.
+    auto load_mask_half = [&](int j0, int hf, char * mb, float after) __attribute__((always_inline)) {
+        const char * mp = mhead + (int64_t)(j0 + hf * 32) * 2;
+        char * lm = mb + wave * (2 * MHALF) + hf * MHALF;
+#pragma unroll
+        for (int j = 0; j < NMH; j++) {
+            uint32_t mo = moff[j];
+            asm volatile("" : "+v"(mo) : "v"(after));
+            __builtin_amdgcn_global_load_lds((glb_vptr)(mp + mo), (lds_vptr)(lm + j * 1024), 16, 0, 0);
+        }
+    };
+
+    // The tail tile's mask takes the same LDS layout through registers.  A chunk that would run past Nkv is fetched
+    // from the row's last 8 valid keys instead (Nkv is even and >= 64 here, so that address is dword-aligned and
+    // in bounds) and shifted down by the difference: branch-free, all loads in flight together, nothing read past
+    // Nkv; the positions shifted in from beyond belong to keys that the tail tile excludes.
+    typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+    auto stage_mask_tail = [&](int j0, char * mb) __attribute__((always_inline)) {
+        u32x4_a4 raw[2][NMH];
+        int      sh[2][NMH];
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+            for (int j = 0; j < NMH; j++) {
+                const int row = j * 16 + (lane >> 2);
+                const int cg  = (lane & 3) ^ swz_m<D>(row);
+                const int s0  = j0 + hf * 32 + 8 * cg;                     // first key of this lane's chunk
+                const int sc  = min(s0, a.Nkv - 8);
+                sh[hf][j] = min(s0 - sc, 8);                               // halfwords to shift out
+                // moff[j] = row offset + 16*cg, relative to key j0 + 32*hf of the head's mask
+                raw[hf][j] = *(const u32x4_a4 *)(mhead + (int64_t)(j0 + hf * 32) * 2 + moff[j] - (int64_t)(s0 - sc) * 2);
+            }
+#pragma unroll
+        for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+            for (int j = 0; j < NMH; j++) {
+                const int k = sh[hf][j];
+                uint32_t e[6] = {raw[hf][j][0], raw[hf][j][1], raw[hf][j][2], raw[hf][j][3], 0u, 0u};
+                if (k & 8) { e[0] = e[1] = e[2] = e[3] = 0u; }
+                if (k & 4) { e[0] = e[2]; e[1] = e[3]; e[2] = 0u; e[3] = 0u; }
+                if (k & 2) { e[0] = e[1]; e[1] = e[2]; e[2] = e[3]; e[3] = 0u; }
+                const uint32_t bs = (k & 1) * 2;                               // bytes
+                uint4 val;
+                val.x = __builtin_amdgcn_alignbyte(e[1], e[0], bs);
+                val.y = __builtin_amdgcn_alignbyte(e[2], e[1], bs);
+                val.z = __builtin_amdgcn_alignbyte(e[3], e[2], bs);
+                val.w = __builtin_amdgcn_alignbyte(e[4], e[3], bs);
+                *(uint4 *)(mb + wave * (2 * MHALF) + hf * MHALF + j * 1024 + lane * 16) = val;
+            }
+    };
     auto load_direct = [&](int j0, char * wk, char * wv, bool tail) __attribute__((always_inline)) {
         const char * kp = kbase + (int64_t)j0 * a.nbk1;
         const char * vp = vbase + (int64_t)j0 * a.nbv1;
@@ -290,13 +363,18 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     // are distinct buffers, and saying so (restrict) is what lets the compiler keep the operand reads from
     // waiting on the loads that have just been issued.
     auto tile = [&](const int j0, const int buf, auto tail_tag, const char * __restrict__ rk, const char * __restrict__ rv,
-                    char * __restrict__ wk, char * __restrict__ wv, const int jn, const bool tn) __attribute__((always_inline)) {
+                    char * __restrict__ wk, char * __restrict__ wv, const int jn, const bool tn, char * __restrict__ mb,
+                    const bool mn) __attribute__((always_inline)) {
         constexpr bool TAIL = decltype(tail_tag)::value;
+        constexpr bool MLDS = MDMA;                   // this tile's mask is in LDS (mn: so will the next tile's be)
+        // mask of keys 32..63 of this tile: its block was last read before the barrier that ended the previous tile
+        // (the tail tile's mask is staged whole before the tile starts)
+        if (MLDS && !TAIL) load_mask_half(j0, 1, mb, 0.0f);
         if (DIRECT && jn >= 0) load_direct(jn, wk, wv, tn);
 
         // additive mask values of this lane's 32 (key, query) pairs per query block, fetched early
-        uint2 mraw[NQB][2][4];
-        if (MASK) {
+        uint2 mraw[MLDS ? 1 : NQB][2][4];
+        if (MASK && !MLDS) {
 #pragma unroll
             for (int qb = 0; qb < NQB; qb++)
 #pragma unroll
@@ -304,12 +382,18 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
                         const int key = j0 + kb * 32 + g * 8 + hh * 4;
+                        // Past Nkv the loads are clamped to the row's last valid pair (or element): branch-free and in
+                        // bounds; what they return belongs to keys that the tail tile excludes anyway.
                         if (!TAIL && a.mask_al8) {
                             mraw[qb][kb][g] = *(const uint2 *)(mrow[qb] + key);
+                        } else if (a.mask_al4 && !(a.Nkv & 1)) {
+                            const int k0 = TAIL ? min(key, a.Nkv - 2) : key, k1 = TAIL ? min(key + 2, a.Nkv - 2) : key + 2;
+                            mraw[qb][kb][g].x = *(const uint32_t *)(mrow[qb] + k0);
+                            mraw[qb][kb][g].y = *(const uint32_t *)(mrow[qb] + k1);
                         } else {
                             uint16_t mv[4];
 #pragma unroll
-                            for (int e = 0; e < 4; e++) mv[e] = (!TAIL || key + e < a.Nkv) ? mrow[qb][key + e] : (uint16_t)0;
+                            for (int e = 0; e < 4; e++) mv[e] = mrow[qb][TAIL ? min(key + e, a.Nkv - 1) : key + e];
                             mraw[qb][kb][g].x = (uint32_t)mv[0] | ((uint32_t)mv[1] << 16);
                             mraw[qb][kb][g].y = (uint32_t)mv[2] | ((uint32_t)mv[3] << 16);
                         }
@@ -354,7 +438,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             float16v s[NQB];
 #pragma unroll
             for (int qb = 0; qb < NQB; qb++) {
-                if (MASK || SOFTCAP) {
+                if (SOFTCAP) {          // the cap applies to the raw score: m is subtracted afterwards
 #pragma unroll
                     for (int r = 0; r < 16; r++) s[qb][r] = 0.0f;
                 } else {
@@ -371,7 +455,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             load_v(kb, va);
             if (kb == 0) load_k(1, ka[K_AHEAD ? 1 : 0]);
 
-            // ---- soft cap, mask (these paths subtract m explicitly), key tail -----------------------
+            // ---- soft cap (this path subtracts m explicitly), mask, key tail -----------------------------
             if (SOFTCAP) {
                 const float c2 = a.softcap * LOG2E;
 #pragma unroll
@@ -379,20 +463,27 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
 #pragma unroll
                     for (int r = 0; r < 16; r++) s[qb][r] = c2 * fast_tanh(s[qb][r]);
             }
+            if (MLDS && kb == 1 && !TAIL) {
+                // the second half was requested when the tile began; the only requests that can be younger than
+                // it are the next tile's first mask half (they follow block 0's exponentials)
+                if (mn) __builtin_amdgcn_s_waitcnt(0x0F70 | NMH);
+                else    __builtin_amdgcn_s_waitcnt(0x0F70);
+            }
             if (MASK) {
 #pragma unroll
                 for (int qb = 0; qb < NQB; qb++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        const uint32_t w[2] = {mraw[qb][kb][g].x, mraw[qb][kb][g].y};
+                        // f16 halves enter the FMA directly (mixed-precision FMA, no separate conversion)
+                        const uint2 mv = MLDS ? *(const uint2 *)(mb + wave * (2 * MHALF) + kb * MHALF + qb * 2048 + maddr[g])
+                                              : mraw[MLDS ? 0 : qb][kb][g];
+                        const half2v w[2] = {__builtin_bit_cast(half2v, mv.x), __builtin_bit_cast(half2v, mv.y)};
 #pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            const float mv = h2f_bits((uint16_t)(w[e >> 1] >> (16 * (e & 1))));
-                            s[qb][g * 4 + e] = fmaf(mslope, mv, s[qb][g * 4 + e]);
-                        }
+                        for (int e = 0; e < 4; e++)
+                            s[qb][g * 4 + e] = fmaf(mslope, (float)w[e >> 1][e & 1], s[qb][g * 4 + e]);
                     }
             }
-            if (MASK || SOFTCAP) {
+            if (SOFTCAP) {
 #pragma unroll
                 for (int qb = 0; qb < NQB; qb++)
 #pragma unroll
@@ -462,6 +553,11 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             }
 #pragma unroll
             for (int qb = 0; qb < NQB; qb++) st[qb].l += lsum[qb];
+            if (MLDS && kb == 0 && !TAIL && mn) {
+                // block 0's mask has been consumed - the sums below depend on every value of it - so its LDS
+                // block can take the next tile's
+                load_mask_half(j0 + BC, 0, mb, lsum[0] + lsum[NQB - 1]);
+            }
 
             // ---- O^T += V^T . P^T ------------------------------------------------------------------------------
 #pragma unroll
@@ -477,20 +573,25 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     const int n_tiles = (a.Nkv + BC - 1) / BC;
     const int n_full  = a.Nkv / BC;
     if (DIRECT) {
-        char * const lb = (char *)lds_raw;               // K0 K1 V0 V1
+        char * const lb = (char *)lds_raw;               // K0 K1 V0 V1 [mask: per wave 2 half-tile blocks]
+        char * const mb = lb + 4 * TILEB;
         load_direct(0, lb, lb + 2 * TILEB, n_full == 0);
+        if (MDMA && n_full > 0) load_mask_half(0, 0, mb, 0.0f);
         __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): this wave's share of the tile is in LDS
         __syncthreads();
         for (int t = 0; t < n_full; t++) {
-            const int cur = (t & 1) * TILEB, nxt = TILEB - cur;
-            const int jn  = t + 1 < n_tiles ? (t + 1) * BC : -1;
-            tile(t * BC, 0, std::false_type{}, lb + cur, lb + 2 * TILEB + cur, lb + nxt, lb + 2 * TILEB + nxt, jn, t + 1 >= n_full);
+            const int  cur = (t & 1) * TILEB, nxt = TILEB - cur;
+            const int  jn  = t + 1 < n_tiles ? (t + 1) * BC : -1;
+            const bool mn  = MDMA && t + 1 < n_full;
+            tile(t * BC, 0, std::false_type{}, lb + cur, lb + 2 * TILEB + cur, lb + nxt, lb + 2 * TILEB + nxt, jn, t + 1 >= n_full, mb, mn);
+            // everything requested during the tile has had at least half a tile to land
             __builtin_amdgcn_s_waitcnt(0x0F70);
             __syncthreads();
         }
         if (n_full < n_tiles) {
             const int cur = (n_full & 1) * TILEB;
-            tile(n_full * BC, 0, std::true_type{}, lb + cur, lb + 2 * TILEB + cur, nullptr, nullptr, -1, false);
+            if (MDMA) stage_mask_tail(n_full * BC, mb);
+            tile(n_full * BC, 0, std::true_type{}, lb + cur, lb + 2 * TILEB + cur, nullptr, nullptr, -1, false, mb, false);
         }
     } else {
     load_tile(0);
@@ -502,12 +603,12 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         const int  buf  = t & 1;
         const bool more = t + 1 < n_tiles;
         if (more) load_tile((t + 1) * BC);
-        tile(t * BC, buf, std::false_type{}, nullptr, nullptr, nullptr, nullptr, -1, false);
+        tile(t * BC, buf, std::false_type{}, nullptr, nullptr, nullptr, nullptr, -1, false, nullptr, false);
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
     // at most one partial tile, already staged by the last iteration above (or the prologue)
-    if (n_full < n_tiles) tile(n_full * BC, n_full & 1, std::true_type{}, nullptr, nullptr, nullptr, nullptr, -1, false);
+    if (n_full < n_tiles) tile(n_full * BC, n_full & 1, std::true_type{}, nullptr, nullptr, nullptr, nullptr, -1, false, nullptr, false);
     }
 
     // ---- normalise and write dst[D, Hq, Nq, B] -------------------------------------------------------
@@ -533,16 +634,16 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     }
 }
 
-template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT>
+template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA>
 int launch(const FattnArgs & a, hipStream_t stream) {
     const int bmg = 32 * NQB * MMA_WAVES;
     const int n_qtiles = (a.Nq + bmg - 1) / bmg;
     const dim3 grid((unsigned)(n_qtiles * a.Hq * a.B));
-    const size_t lds = DIRECT ? (size_t)4 * BC * D * sizeof(_Float16)
+    const size_t lds = DIRECT ? (size_t)4 * BC * D * sizeof(_Float16) + (MDMA ? (size_t)MMA_WAVES * NQB * 4096 : 0)
                               : (size_t)2 * BC * (Pitch<D>::K + Pitch<D>::V) * sizeof(_Float16);
     static bool attr_set = false;     // per instantiation; the attribute only matters above 64 KiB
     if (!attr_set && lds > 64 * 1024) {
-        const hipError_t e = hipFuncSetAttribute((const void *)fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP, DIRECT>,
+        const hipError_t e = hipFuncSetAttribute((const void *)fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP, DIRECT, MDMA>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
         attr_set = true;
@@ -550,19 +651,25 @@ int launch(const FattnArgs & a, hipStream_t stream) {
     static const bool debug = getenv("MI355X_FATTN_DEBUG") != nullptr;
     if (debug) {
         int nb = -1;
-        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void *)fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP, DIRECT>, MMA_THREADS, lds);
-        fprintf(stderr, "[mi355x] fattn_mma<%d,%d,%d,%d,%d,%d> grid %u lds %zu B, resident workgroups per CU: %d\n",
-                D, NQB, TYPE, (int)MASK, (int)SOFTCAP, (int)DIRECT, grid.x, lds, nb);
+        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void *)fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP, DIRECT, MDMA>, MMA_THREADS, lds);
+        fprintf(stderr, "[mi355x] fattn_mma<%d,%d,%d,%d,%d,%d,%d> grid %u lds %zu B, resident workgroups per CU: %d\n",
+                D, NQB, TYPE, (int)MASK, (int)SOFTCAP, (int)DIRECT, (int)MDMA, grid.x, lds, nb);
     }
-    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP, DIRECT>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
+    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP, DIRECT, MDMA>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
     return (int)hipGetLastError();
 }
 
 template <int D, int NQB, int TYPE, bool DIRECT>
 int launch_mask(const FattnArgs & a, hipStream_t stream) {
     const bool mask = a.mask != nullptr;
-    if (a.softcap != 0.0f) return mask ? launch<D, NQB, TYPE, true, true, DIRECT>(a, stream) : launch<D, NQB, TYPE, false, true, DIRECT>(a, stream);
-    return mask ? launch<D, NQB, TYPE, true, false, DIRECT>(a, stream) : launch<D, NQB, TYPE, false, false, DIRECT>(a, stream);
+    if (a.softcap != 0.0f) return mask ? launch<D, NQB, TYPE, true, true, DIRECT, false>(a, stream) : launch<D, NQB, TYPE, false, true, DIRECT, false>(a, stream);
+    if (!mask) return launch<D, NQB, TYPE, false, false, DIRECT, false>(a, stream);
+    // the mask follows K/V through LDS when its rows start on dwords, Nkv is even (the tail tile's dword-aligned
+    // stand-in chunk) and a wave's row offsets fit 32 bits
+    static const bool no_mdma = getenv("MI355X_FATTN_NO_MDMA") != nullptr;          // experiments only
+    if (DIRECT && !no_mdma && a.mask_al4 && a.Nkv >= 64 && !(a.Nkv & 1) && (uint64_t)a.Nq * a.nbm1 < (1ull << 31))
+        return launch<D, NQB, TYPE, true, false, DIRECT, DIRECT>(a, stream);
+    return launch<D, NQB, TYPE, true, false, DIRECT, false>(a, stream);
 }
 
 template <int D, int NQB, int TYPE>
