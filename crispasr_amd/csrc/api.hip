@@ -109,6 +109,7 @@ struct Plan {
     int     n_splits;
     int     keys_per_split;
     size_t  workspace;
+    bool    kv_to_f16;       // F32 K/V are converted to f16 in the workspace first (tile kernel only)
 };
 
 int check(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
@@ -216,6 +217,14 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
     plan.n_splits = 1;
     plan.keys_per_split = a.Nkv;
     plan.workspace = 0;
+    plan.kv_to_f16 = false;
+    // The tile kernel rounds F32 K/V to f16 on their way into LDS anyway.  With enough queries to share the work it
+    // is cheaper to do that once, in a copy of its own, and let the f16 path (which moves tiles global->LDS without
+    // touching registers) read the result: same values, same rounding.
+    if (kernel == MI355X_FATTN_MMA && ktype == MI355X_TYPE_F32 && a.Nq >= 128 && a.kv_aligned16) {
+        plan.kv_to_f16 = true;
+        plan.workspace = (size_t)2 * a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t);
+    }
     if (kernel == MI355X_FATTN_VEC || kernel == MI355X_FATTN_DECODE_MMA) {
         const int64_t rows = (int64_t)a.Nq * a.Hq * a.B;
         // workgroups that exist before splitting, and the fewest keys worth a split
@@ -367,7 +376,44 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     }
     if (plan.kernel == MI355X_FATTN_MMA) {
         if (!fattn_mma_supported(a, k->type)) return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the MFMA kernel");
-        const int e = fattn_mma_launch(a, k->type, st);
+        int ktype = k->type;
+        if (plan.kv_to_f16) {
+            void * ws = params->workspace;
+            if (ws) {
+                if (params->workspace_size < plan.workspace)
+                    return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, plan.workspace);
+            } else {
+                rc = get_scratch(plan.workspace, &ws);
+                if (rc) return rc;
+            }
+            const mi355x_tensor * src[2] = {k, v};
+            const size_t half = plan.workspace / 2;
+            for (int t = 0; t < 2; t++) {
+                CpyArgs c;
+                memset(&c, 0, sizeof(c));
+                c.src = (const char *)src[t]->data;
+                c.dst = (char *)ws + t * half;
+                int64_t nb = sizeof(uint16_t);
+                c.n = 1;
+                for (int i = 0; i < 4; i++) {
+                    c.sne[i] = c.dne[i] = src[t]->ne[i];
+                    c.snb[i] = (int64_t)src[t]->nb[i];
+                    c.dnb[i] = nb;
+                    nb *= src[t]->ne[i];
+                    c.n *= src[t]->ne[i];
+                }
+                const int e = cpy_launch(c, MI355X_TYPE_F32, MI355X_TYPE_F16, st);
+                if (e) return hip_fail((hipError_t)e, "K/V conversion launch");
+            }
+            // the same call on the f16 copies: contiguous [D, Nkv, Hkv, Bk]
+            a.k = (const char *)ws;
+            a.v = (const char *)ws + half;
+            a.nbk1 = a.nbv1 = (size_t)a.D * 2;
+            a.nbk2 = a.nbv2 = a.nbk1 * a.Nkv;
+            a.nbk3 = a.nbv3 = a.nbk2 * a.Hkv;
+            ktype = MI355X_TYPE_F16;
+        }
+        const int e = fattn_mma_launch(a, ktype, st);
         if (e) return hip_fail((hipError_t)e, "fattn_mma launch");
         return MI355X_OK;
     }

@@ -5,7 +5,7 @@ import pytest
 import oracle as ora
 from cases import make_case, to_f32
 from crispasr_amd import ggml
-from gpu_util import assert_parity, run_gpu, run_oracle
+from gpu_util import assert_parity, run_gpu, run_oracle, upload
 
 pytestmark = pytest.mark.gpu
 
@@ -115,3 +115,22 @@ def test_pipelined_kernel_with_growing_scores():
     amax = float(np.abs(ref).max())                 # outputs are a few units large here: scale the absolute bound
     for kern in (ggml.KERNEL_MMA_PIPE, ggml.KERNEL_MMA):
         assert_parity(run_gpu(case, kernel=kern), ref, "growing scores, kernel %d" % kern, max_abs_tol=2e-3 * max(1.0, amax))
+
+
+def test_f32_cache_is_converted_once_and_matches_with_any_workspace():
+    """F32 K/V with many queries: the library rounds them to f16 in a workspace and runs the f16 path.  Strided
+    views, a shared K/V batch and a per-head mask; the library's scratch and a caller's workspace give the same
+    result, a workspace that is too small is refused."""
+    import torch
+    spec = dict(seed=151, D=128, Nq=300, Nkv=333, Hq=4, Hkv=2, B=2, Bk=1, ktype=ora.F32, kv_layout="thd", mask="bias_perhead")
+    case = make_case(**spec)
+    ref = run_oracle(case)
+    got = run_gpu(case, kernel=ggml.KERNEL_MMA)
+    assert_parity(got, ref, "library scratch")
+    q, k, v, m = upload(case["q"]), upload(case["k"]), upload(case["v"]), upload(case["mask"])
+    need = 2 * 128 * 333 * 2 * 1 * 2
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    out = ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_MMA, workspace=ws)
+    assert np.array_equal(out.numpy_f32(), got)
+    with pytest.raises(ggml.Mi355xError):
+        ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_MMA, workspace=ws[: need - 16])
