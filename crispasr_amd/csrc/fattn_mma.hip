@@ -181,7 +181,9 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
 
     // ---- Q -> f16 B operands, scaled so that the MFMA result is already in log2 units ----
     const float qscale = SOFTCAP ? a.scale : a.scale * LOG2E;   // a.scale is scale/softcap when capped
+    // (called after the first K/V tile has been requested, so the two cold misses overlap)
     half8 qreg[NQB][KS];
+    auto load_q = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int qb = 0; qb < NQB; qb++) {
         const int qi = min(q0 + qb * 32 + l32, a.Nq - 1);
@@ -198,6 +200,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             qreg[qb][ks] = v;
         }
     }
+    };
 
     const char * kbase = a.k + (int64_t)hk * a.nbk2 + (int64_t)bk * a.nbk3;
     const char * vbase = a.v + (int64_t)hk * a.nbv2 + (int64_t)bk * a.nbv3;
@@ -577,6 +580,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         char * const mb = lb + 4 * TILEB;
         load_direct(0, lb, lb + 2 * TILEB, n_full == 0);
         if (MDMA && n_full > 0) load_mask_half(0, 0, mb, 0.0f);
+        load_q();
         __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): this wave's share of the tile is in LDS
         __syncthreads();
         for (int t = 0; t < n_full; t++) {
@@ -595,6 +599,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         }
     } else {
     load_tile(0);
+    load_q();
     store_tile(0);
     __syncthreads();
 
