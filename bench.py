@@ -436,6 +436,23 @@ def bench_whisper_protocol(args, ca, ora, torch):
     return res
 
 
+def bench_whisper_protocol_native():
+    """The same protocol driven by the native host driver (C++ above the C ABI, no Python between the calls): what a
+    ggml backend's graph_compute would pay per node.  Runs as a child process."""
+    import subprocess
+    exe = os.path.join(ROOT, "crispasr_amd", "host", "mi355x_attn_protocol")
+    if not os.path.exists(exe):
+        return {"error": "host driver not built"}
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    if res.returncode != 0:
+        return {"error": "exit code %d: %s" % (res.returncode, res.stderr[-300:])}
+    out = json.loads(res.stdout.strip().splitlines()[-1])
+    for k in ("single_token_x256", "batch5_x64", "prompt256_x16"):
+        log(f"[bench] whisper protocol, native host driver, {k}: {out[k]['ms_per_decode']:.3f} ms per decode, "
+            f"{out[k]['us_per_attention_call']:.1f} us per call incl. host launch")
+    return out
+
+
 def copy_calibration(ca, torch):
     """A plain copy of known size through the library's own CPY kernel (128-bit path): 256 MiB read + 256 MiB written.
     It gives the counter-to-bytes factor for the rocprofv3 FETCH_SIZE / WRITE_SIZE traffic figures."""
@@ -502,6 +519,7 @@ def main():
     if not args.no_configs:
         line["configs"] = bench_configs(args, ca, ora, torch)
         line["whisper_bench_protocol"] = bench_whisper_protocol(args, ca, ora, torch)
+        line["whisper_bench_protocol_native"] = bench_whisper_protocol_native()
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args, ora, host0)
     if not enc["parity"]["ok"]:

@@ -54,5 +54,20 @@ def build_library(extra_flags=(), jobs: int = 4) -> str:
     return LIB
 
 
+HOST_SRC = os.path.join(HERE, "host", "attn_protocol.cpp")
+HOST_BIN = os.path.join(HERE, "host", "mi355x_attn_protocol")
+
+
+def build_host_driver() -> str:
+    """The native host driver above the C ABI (plain g++; it links only libmi355x_fattn.so)."""
+    cmd = ["g++", "-O2", "-std=c++17", "-Wall", "-I", os.path.join(os.path.dirname(HERE), "include"), HOST_SRC, "-o", HOST_BIN,
+           "-L", HERE, "-lmi355x_fattn", "-Wl,-rpath,$ORIGIN/.."]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("host driver build failed:\n" + res.stderr)
+    return HOST_BIN
+
+
 if __name__ == "__main__":
     print(build_library(sys.argv[1:]))
+    print(build_host_driver())

@@ -99,3 +99,18 @@ def test_cpy_supports_matrix():
     assert ok(ca.F32, ca.F16, (64, 4, 2, 1), (512, 1, 1, 1)) == ggml.OK          # reshape with equal counts
     assert ok(ca.F32, ca.F16, (64, 4, 2, 1), (64, 5, 2, 1)) == ggml.ERR_INVALID
     assert ok(ca.F32, ca.Q8_0, (48, 4, 2, 1)) == ggml.ERR_INVALID
+
+
+@pytest.mark.gpu
+def test_native_host_driver_runs_the_bench_protocol():
+    """The C++ driver links only the C-ABI library, checks one masked call against its own double-precision loop
+    and runs the reference's decode protocol at attention level; exit code 0 = self-check within 2e-3."""
+    import json
+    import subprocess
+    exe = os.path.join(ROOT, "crispasr_amd", "host", "mi355x_attn_protocol")
+    assert os.path.exists(exe), "host driver not built (python -c 'import __graft_entry__ as g; g.build()')"
+    res = subprocess.run([exe, "4"], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr
+    out = json.loads(res.stdout.strip().splitlines()[-1])
+    assert out["layers"] == 4 and out["self_check_max_abs"] <= 2e-3
+    assert out["single_token_x256"]["us_per_attention_call"] > 0
