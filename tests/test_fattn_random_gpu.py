@@ -1,0 +1,62 @@
+"""Randomised GPU parity: seeded shapes, layouts, cache types and masks, through AUTO and through each kernel that
+accepts the shape.  The draws are made to hit the tile kernel's paths in every combination: K/V moved global->LDS
+directly or through registers, masks with dword-aligned and unaligned rows, even and odd Nkv, full and partial
+last tiles, few and many queries (the F32 -> f16 pre-conversion starts at 128)."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle as ora
+from cases import make_case
+from crispasr_amd import ggml
+from gpu_util import assert_parity, run_gpu, run_oracle
+
+pytestmark = pytest.mark.gpu
+
+MASKS = [None, None, "causal", "random_inf", "random_inf_batched", "bias", "bias_perhead", "bias_perhead_pad", "all_masked_rows"]
+
+
+def draw(seed: int) -> dict:
+    r = np.random.default_rng(1000 + seed)
+    D = int(r.choice([64, 128]))
+    gqa = int(r.choice([1, 1, 2, 4]))
+    Hkv = int(r.integers(1, 4))
+    B = int(r.integers(1, 4))
+    Bk = B if r.random() < 0.7 else 1
+    big = r.random() < 0.5
+    Nq = int(r.integers(1, 420)) if big else int(r.integers(1, 40))
+    Nkv = int(r.choice([int(r.integers(1, 450)), 64 * int(r.integers(1, 6)), 2 * int(r.integers(1, 200)), 64 * int(r.integers(1, 5)) + 8]))
+    mask = MASKS[int(r.integers(0, len(MASKS)))]
+    spec = dict(seed=5000 + seed, D=D, Nq=Nq, Nkv=Nkv, Hq=Hkv * gqa, Hkv=Hkv, B=B, Bk=Bk,
+                ktype=int(r.choice([ora.F16, ora.F16, ora.F32, ora.Q8_0])), mask=mask,
+                q_layout=str(r.choice(["contig", "thd"])), kv_layout=str(r.choice(["contig", "thd", "gap"])))
+    if mask is None and r.random() < 0.3:
+        spec["kv_pad_rows"] = int(r.integers(1, 40))
+    if mask == "bias_perhead_pad":
+        spec["lengths"] = [int(r.integers(1, Nkv + 1)) for _ in range(B)]
+    if r.random() < 0.2:
+        spec["scale"] = float(r.choice([0.5, 1.5])) * D ** -0.5      # score std 0.5 or 1.5 (at 2 the f16 operands bring max-abs to the tolerance)
+    if mask is not None and r.random() < 0.15:
+        spec["max_bias"] = 8.0
+    if r.random() < 0.1:
+        spec["softcap"] = 20.0
+    return spec
+
+
+N_CASES = int(os.environ.get("FATTN_RANDOM_CASES", "150"))        # more for a longer hunt
+
+
+@pytest.mark.parametrize("seed", range(N_CASES))
+def test_random_shape_matches_oracle_on_every_kernel(seed):
+    spec = draw(seed)
+    print("case", spec, flush=True)
+    case = make_case(**spec)
+    ref = run_oracle(case)
+    assert_parity(run_gpu(case), ref, "auto %s" % spec)
+    for kern in (ggml.KERNEL_VEC, ggml.KERNEL_MMA, ggml.KERNEL_DECODE_MMA):
+        try:
+            got = run_gpu(case, kernel=kern)
+        except ggml.UnsupportedError:
+            continue
+        assert_parity(got, ref, "kernel %d %s" % (kern, spec))
