@@ -194,6 +194,7 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
         a.mask_al4 = m4 ? 1 : 0;
     }
     a.aligned16 = al16 ? 1 : 0;
+    a.n_cus = device_cus();
     a.softcap = p->logit_softcap;
     a.scale   = p->logit_softcap != 0.0f ? p->scale / p->logit_softcap : p->scale;
     a.max_bias = p->max_bias;

@@ -38,6 +38,7 @@ struct FattnArgs {
     int32_t kv_aligned4;
     int32_t mask_al8;    // mask base and strides are multiples of 8 bytes
     int32_t mask_al4;    // ... of 4 bytes
+    int32_t n_cus;       // compute units of the device
 
     // split-KV
     int32_t n_splits;

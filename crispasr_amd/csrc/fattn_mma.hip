@@ -583,7 +583,17 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         load_q();
         __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): this wave's share of the tile is in LDS
         __syncthreads();
+        // Two workgroups share a CU, and the SIMD's arbiter prefers the older wave: left alone, the first
+        // workgroup runs at full speed and the second finishes its last third alone, at one wave per SIMD.  Waves
+        // therefore take the higher priority in alternating time slices (workgroups i and i + n_cus are the ones
+        // that meet on a CU), so that both finish together.
+        const int  prio_phase = a.n_cus > 0 ? (blockIdx.x / a.n_cus) & 1 : 0;
+        const bool shared_cu  = a.n_cus > 0 && (int)gridDim.x > a.n_cus;
         for (int t = 0; t < n_full; t++) {
+            if (shared_cu) {
+                if (((int)(clock64() >> 12) ^ prio_phase) & 1) __builtin_amdgcn_s_setprio(2);
+                else                                            __builtin_amdgcn_s_setprio(0);
+            }
             const int  cur = (t & 1) * TILEB, nxt = TILEB - cur;
             const int  jn  = t + 1 < n_tiles ? (t + 1) * BC : -1;
             const bool mn  = MDMA && t + 1 < n_full;
@@ -592,6 +602,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             __builtin_amdgcn_s_waitcnt(0x0F70);
             __syncthreads();
         }
+        __builtin_amdgcn_s_setprio(0);
         if (n_full < n_tiles) {
             const int cur = (n_full & 1) * TILEB;
             if (MDMA) stage_mask_tail(n_full * BC, mb);
