@@ -108,7 +108,8 @@ struct Plan {
     int     kernel;
     int     n_splits;
     int     keys_per_split;
-    size_t  workspace;
+    size_t  workspace;       // bytes in all: [f16 copies of K and V][split partials]
+    size_t  ws_partials;     // offset of the split partials inside the workspace
     bool    kv_to_f16;       // F32 K/V are converted to f16 in the workspace first (tile kernel only)
 };
 
@@ -222,9 +223,38 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
     // The tile kernel rounds F32 K/V to f16 on their way into LDS anyway.  With enough queries to share the work it
     // is cheaper to do that once, in a copy of its own, and let the f16 path (which moves tiles global->LDS without
     // touching registers) read the result: same values, same rounding.
+    plan.ws_partials = 0;
     if (kernel == MI355X_FATTN_MMA && ktype == MI355X_TYPE_F32 && a.Nq >= 128 && a.kv_aligned16) {
         plan.kv_to_f16 = true;
-        plan.workspace = (size_t)2 * a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t);
+        plan.workspace = ((size_t)2 * a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t) + 255) / 256 * 256;
+        plan.ws_partials = plan.workspace;
+    }
+    if (kernel == MI355X_FATTN_MMA) {
+        // Very few query tiles and many keys (a short prompt against a long cache): split the keys into ranges of whole
+        // 64-key tiles, one workgroup per CU.  Every split repeats the Q load and writes a partial per row, and the merge
+        // is a launch of its own - measured on the Whisper-base encoder (96 tiles x 24 key tiles) any split is a loss -
+        // so only grids below a quarter of the CUs are split, into ranges of at least four tiles.
+        const int64_t rows    = (int64_t)a.Nq * a.Hq * a.B;
+        const int64_t wgs     = (int64_t)((a.Nq + 127) / 128) * a.Hq * a.B;
+        const int     n_tiles = (a.Nkv + 63) / 64;
+        int ns = p->n_splits;
+        if (ns <= 0) {
+            ns = 1;
+            const int cus = device_cus();
+            if (wgs * 4 <= cus) {
+                int want = (int)(cus / wgs);
+                if (want > n_tiles / 4) want = n_tiles / 4;
+                if (want >= 2) ns = want;
+            }
+        }
+        if (ns > n_tiles) ns = n_tiles;
+        if (ns < 1) ns = 1;
+        if (ns > 64) ns = 64;
+        const int tps = (n_tiles + ns - 1) / ns;
+        ns = (n_tiles + tps - 1) / tps;
+        plan.n_splits = ns;
+        plan.keys_per_split = ns > 1 ? tps * 64 : a.Nkv;
+        if (ns > 1) plan.workspace += (size_t)rows * ns * (a.D + 2) * sizeof(float);
     }
     if (kernel == MI355X_FATTN_VEC || kernel == MI355X_FATTN_DECODE_MMA) {
         const int64_t rows = (int64_t)a.Nq * a.Hq * a.B;
@@ -378,8 +408,9 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     if (plan.kernel == MI355X_FATTN_MMA) {
         if (!fattn_mma_supported(a, k->type)) return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the MFMA kernel");
         int ktype = k->type;
-        if (plan.kv_to_f16) {
-            void * ws = params->workspace;
+        void * ws = nullptr;
+        if (plan.workspace) {
+            ws = params->workspace;
             if (ws) {
                 if (params->workspace_size < plan.workspace)
                     return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, plan.workspace);
@@ -387,8 +418,10 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
                 rc = get_scratch(plan.workspace, &ws);
                 if (rc) return rc;
             }
+        }
+        if (plan.kv_to_f16) {
             const mi355x_tensor * src[2] = {k, v};
-            const size_t half = plan.workspace / 2;
+            const size_t half = (size_t)a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t);
             for (int t = 0; t < 2; t++) {
                 CpyArgs c;
                 memset(&c, 0, sizeof(c));
@@ -414,8 +447,19 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
             a.nbk3 = a.nbv3 = a.nbk2 * a.Hkv;
             ktype = MI355X_TYPE_F16;
         }
-        const int e = fattn_mma_launch(a, ktype, st);
+        a.n_splits = plan.n_splits;
+        a.keys_per_split = plan.keys_per_split;
+        if (plan.n_splits > 1) {
+            const size_t rows = (size_t)a.Nq * a.Hq * a.B;
+            a.part_acc = (float *)((char *)ws + plan.ws_partials);
+            a.part_ml  = a.part_acc + rows * plan.n_splits * a.D;
+        }
+        int e = fattn_mma_launch(a, ktype, st);
         if (e) return hip_fail((hipError_t)e, "fattn_mma launch");
+        if (plan.n_splits > 1) {
+            e = fattn_merge_launch(a, st);
+            if (e) return hip_fail((hipError_t)e, "fattn_merge launch");
+        }
         return MI355X_OK;
     }
     if (plan.kernel == MI355X_FATTN_DECODE_MMA) {

@@ -171,6 +171,12 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         const int per = nb / 8;
         if (bid < per * 8) bid = (bid % 8) * per + bid / 8;
     }
+    // key range of this workgroup: everything, or one of n_splits ranges of whole tiles (few query tiles on many
+    // CUs; the partial results then go through fattn_merge_kernel)
+    const int split = bid % a.n_splits;
+    bid /= a.n_splits;
+    const int k_begin = split * a.keys_per_split;
+    const int k_end   = min(a.Nkv, k_begin + a.keys_per_split);
     const int qt = bid % n_qtiles;
     const int h  = (bid / n_qtiles) % a.Hq;
     const int b  = bid / (n_qtiles * a.Hq);
@@ -224,7 +230,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     auto load_tile = [&](int j0) {
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-            const int key = min(j0 + sr + p * RPP, a.Nkv - 1);
+            const int key = min(j0 + sr + p * RPP, k_end - 1);
             kraw[p] = load_chunk<TYPE>(kbase + (int64_t)key * a.nbk1, sc, true);
             vraw[p] = load_chunk<TYPE>(vbase + (int64_t)key * a.nbv1, sc, true);
         }
@@ -303,7 +309,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                 const int row = j * 16 + (lane >> 2);
                 const int cg  = (lane & 3) ^ swz_m<D>(row);
                 const int s0  = j0 + hf * 32 + 8 * cg;                     // first key of this lane's chunk
-                const int sc  = min(s0, a.Nkv - 8);
+                const int sc  = min(s0, k_end - 8);
                 sh[hf][j] = min(s0 - sc, 8);                               // halfwords to shift out
                 // moff[j] = row offset + 16*cg, relative to key j0 + 32*hf of the head's mask
                 raw[hf][j] = *(const u32x4_a4 *)(mhead + (int64_t)(j0 + hf * 32) * 2 + moff[j] - (int64_t)(s0 - sc) * 2);
@@ -336,7 +342,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             uint32_t ko = koff[j], vo = voff[j];
             if (tail) {       // rows past Nkv re-read the last row (their scores are excluded)
                 const int L = (wave * NLD + j) * 64 + lane;
-                const int r = L / CH, c = L % CH, rr = min(r, a.Nkv - 1 - j0);
+                const int r = L / CH, c = L % CH, rr = min(r, k_end - 1 - j0);
                 ko = (uint32_t)rr * (uint32_t)a.nbk1 + (uint32_t)((c ^ swz_k<D>(r)) * 16);
                 vo = (uint32_t)rr * (uint32_t)a.nbv1 + (uint32_t)((c ^ swz_v<D>(r)) * 16);
             }
@@ -389,14 +395,14 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                         // bounds; what they return belongs to keys that the tail tile excludes anyway.
                         if (!TAIL && a.mask_al8) {
                             mraw[qb][kb][g] = *(const uint2 *)(mrow[qb] + key);
-                        } else if (a.mask_al4 && !(a.Nkv & 1)) {
-                            const int k0 = TAIL ? min(key, a.Nkv - 2) : key, k1 = TAIL ? min(key + 2, a.Nkv - 2) : key + 2;
+                        } else if (a.mask_al4 && !(k_end & 1)) {
+                            const int k0 = TAIL ? min(key, k_end - 2) : key, k1 = TAIL ? min(key + 2, k_end - 2) : key + 2;
                             mraw[qb][kb][g].x = *(const uint32_t *)(mrow[qb] + k0);
                             mraw[qb][kb][g].y = *(const uint32_t *)(mrow[qb] + k1);
                         } else {
                             uint16_t mv[4];
 #pragma unroll
-                            for (int e = 0; e < 4; e++) mv[e] = mrow[qb][TAIL ? min(key + e, a.Nkv - 1) : key + e];
+                            for (int e = 0; e < 4; e++) mv[e] = mrow[qb][TAIL ? min(key + e, k_end - 1) : key + e];
                             mraw[qb][kb][g].x = (uint32_t)mv[0] | ((uint32_t)mv[1] << 16);
                             mraw[qb][kb][g].y = (uint32_t)mv[2] | ((uint32_t)mv[3] << 16);
                         }
@@ -496,7 +502,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int key = j0 + kb * 32 + (r >> 2) * 8 + hh * 4 + (r & 3);
-                    if (key >= a.Nkv) {
+                    if (key >= k_end) {
 #pragma unroll
                         for (int qb = 0; qb < NQB; qb++) s[qb][r] = -INFINITY;
                     }
@@ -573,13 +579,13 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         }
     };
 
-    const int n_tiles = (a.Nkv + BC - 1) / BC;
-    const int n_full  = a.Nkv / BC;
+    const int n_tiles = (k_end - k_begin + BC - 1) / BC;
+    const int n_full  = (k_end - k_begin) / BC;
     if (DIRECT) {
         char * const lb = (char *)lds_raw;               // K0 K1 V0 V1 [mask: per wave 2 half-tile blocks]
         char * const mb = lb + 4 * TILEB;
-        load_direct(0, lb, lb + 2 * TILEB, n_full == 0);
-        if (MDMA && n_full > 0) load_mask_half(0, 0, mb, 0.0f);
+        load_direct(k_begin, lb, lb + 2 * TILEB, n_full == 0);
+        if (MDMA && n_full > 0) load_mask_half(k_begin, 0, mb, 0.0f);
         load_q();
         __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): this wave's share of the tile is in LDS
         __syncthreads();
@@ -595,9 +601,9 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                 else                                            __builtin_amdgcn_s_setprio(0);
             }
             const int  cur = (t & 1) * TILEB, nxt = TILEB - cur;
-            const int  jn  = t + 1 < n_tiles ? (t + 1) * BC : -1;
+            const int  jn  = t + 1 < n_tiles ? k_begin + (t + 1) * BC : -1;
             const bool mn  = MDMA && t + 1 < n_full;
-            tile(t * BC, 0, std::false_type{}, lb + cur, lb + 2 * TILEB + cur, lb + nxt, lb + 2 * TILEB + nxt, jn, t + 1 >= n_full, mb, mn);
+            tile(k_begin + t * BC, 0, std::false_type{}, lb + cur, lb + 2 * TILEB + cur, lb + nxt, lb + 2 * TILEB + nxt, jn, t + 1 >= n_full, mb, mn);
             // everything requested during the tile has had at least half a tile to land
             __builtin_amdgcn_s_waitcnt(0x0F70);
             __syncthreads();
@@ -605,11 +611,11 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         __builtin_amdgcn_s_setprio(0);
         if (n_full < n_tiles) {
             const int cur = (n_full & 1) * TILEB;
-            if (MDMA) stage_mask_tail(n_full * BC, mb);
-            tile(n_full * BC, 0, std::true_type{}, lb + cur, lb + 2 * TILEB + cur, nullptr, nullptr, -1, false, mb, false);
+            if (MDMA) stage_mask_tail(k_begin + n_full * BC, mb);
+            tile(k_begin + n_full * BC, 0, std::true_type{}, lb + cur, lb + 2 * TILEB + cur, nullptr, nullptr, -1, false, mb, false);
         }
     } else {
-    load_tile(0);
+    load_tile(k_begin);
     load_q();
     store_tile(0);
     __syncthreads();
@@ -618,23 +624,24 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     for (int t = 0; t < n_full; t++) {
         const int  buf  = t & 1;
         const bool more = t + 1 < n_tiles;
-        if (more) load_tile((t + 1) * BC);
-        tile(t * BC, buf, std::false_type{}, nullptr, nullptr, nullptr, nullptr, -1, false, nullptr, false);
+        if (more) load_tile(k_begin + (t + 1) * BC);
+        tile(k_begin + t * BC, buf, std::false_type{}, nullptr, nullptr, nullptr, nullptr, -1, false, nullptr, false);
         if (more) store_tile(buf ^ 1);
         __syncthreads();
     }
     // at most one partial tile, already staged by the last iteration above (or the prologue)
-    if (n_full < n_tiles) tile(n_full * BC, n_full & 1, std::true_type{}, nullptr, nullptr, nullptr, nullptr, -1, false, nullptr, false);
+    if (n_full < n_tiles) tile(k_begin + n_full * BC, n_full & 1, std::true_type{}, nullptr, nullptr, nullptr, nullptr, -1, false, nullptr, false);
     }
 
-    // ---- normalise and write dst[D, Hq, Nq, B] -------------------------------------------------------
+    // ---- normalise and write dst[D, Hq, Nq, B], or hand the unnormalised partial to the merge kernel --------------
 #pragma unroll
     for (int qb = 0; qb < NQB; qb++) {
         const float ltot = sum_xor32(st[qb].l);
-        const float inv  = ltot > 0.0f ? 1.0f / ltot : 0.0f;
+        const float inv  = a.n_splits > 1 ? 1.0f : (ltot > 0.0f ? 1.0f / ltot : 0.0f);
         const int   qi   = q0 + qb * 32 + l32;
         if (qi < a.Nq) {
-            float * out = a.dst + (((int64_t)b * a.Nq + qi) * a.Hq + h) * D;
+            const int64_t row = ((int64_t)b * a.Nq + qi) * a.Hq + h;
+            float * out = a.n_splits > 1 ? a.part_acc + (row * a.n_splits + split) * D : a.dst + row * D;
 #pragma unroll
             for (int db = 0; db < DB; db++)
 #pragma unroll
@@ -646,6 +653,12 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                     o.w = oacc[qb][db][g * 4 + 3] * inv;
                     *(float4 *)(out + db * 32 + g * 8 + hh * 4) = o;
                 }
+            if (a.n_splits > 1 && hh == 0) {
+                // (reference, sum) in natural-log units; a range with no visible key contributes nothing
+                float * pm = a.part_ml + (row * a.n_splits + split) * 2;
+                pm[0] = st[qb].have ? st[qb].m * 0.6931471805599453f : -INFINITY;
+                pm[1] = ltot;
+            }
         }
     }
 }
@@ -654,7 +667,7 @@ template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool M
 int launch(const FattnArgs & a, hipStream_t stream) {
     const int bmg = 32 * NQB * MMA_WAVES;
     const int n_qtiles = (a.Nq + bmg - 1) / bmg;
-    const dim3 grid((unsigned)(n_qtiles * a.Hq * a.B));
+    const dim3 grid((unsigned)(n_qtiles * a.Hq * a.B * a.n_splits));
     const size_t lds = DIRECT ? (size_t)4 * BC * D * sizeof(_Float16) + (MDMA ? (size_t)MMA_WAVES * NQB * 4096 : 0)
                               : (size_t)2 * BC * (Pitch<D>::K + Pitch<D>::V) * sizeof(_Float16);
     static bool attr_set = false;     // per instantiation; the attribute only matters above 64 KiB

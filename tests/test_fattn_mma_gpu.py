@@ -134,3 +134,29 @@ def test_f32_cache_is_converted_once_and_matches_with_any_workspace():
     assert np.array_equal(out.numpy_f32(), got)
     with pytest.raises(ggml.Mi355xError):
         ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_MMA, workspace=ws[: need - 16])
+
+
+@pytest.mark.parametrize("n_splits", [2, 5])
+@pytest.mark.parametrize("spec", [
+    dict(seed=161, D=64, Nq=300, Nkv=1500, Hq=2, q_layout="thd", kv_layout="thd"),                       # Whisper-base-like, few heads
+    dict(seed=162, D=128, Nq=200, Nkv=407, Hq=8, Hkv=2, ktype=ora.Q8_0, mask="causal"),
+    dict(seed=163, D=128, Nq=130, Nkv=700, Hq=2, B=2, ktype=ora.F32, mask="bias_perhead_pad", lengths=[700, 333]),
+    dict(seed=164, D=64, Nq=17, Nkv=129, Hq=3, mask="all_masked_rows"),
+], ids=lambda s: "seed%d" % s["seed"])
+def test_tile_kernel_with_split_keys(spec, n_splits):
+    """Key ranges of whole tiles per workgroup + the merge pass give the unsplit result (also together with the
+    F32 -> f16 pre-conversion, which shares the workspace)."""
+    case = make_case(**spec)
+    ref = run_oracle(case)
+    assert_parity(run_gpu(case, kernel=ggml.KERNEL_MMA, n_splits=n_splits), ref, "splits %d %s" % (n_splits, spec))
+
+
+def test_auto_splits_keys_only_when_query_tiles_are_very_few():
+    few = make_case(seed=165, D=64, Nq=100, Nkv=2100, Hq=4, q_layout="thd", kv_layout="thd")      # 4 workgroups x 33 key tiles
+    q, k, v = upload(few["q"]), upload(few["k"]), upload(few["v"])
+    kern, ns = ggml.flash_attn_plan(q, k, v, None, few["scale"])
+    assert kern == ggml.KERNEL_MMA and ns > 1
+    assert_parity(run_gpu(few), run_oracle(few), "auto split")
+    base = make_case(seed=166, D=64, Nq=1500, Nkv=1500, Hq=8, q_layout="thd", kv_layout="thd")     # Whisper base encoder: 96 workgroups
+    kern, ns = ggml.flash_attn_plan(upload(base["q"]), upload(base["k"]), upload(base["v"]), None, base["scale"])
+    assert kern == ggml.KERNEL_MMA and ns == 1

@@ -60,3 +60,5 @@ def test_random_shape_matches_oracle_on_every_kernel(seed):
         except ggml.UnsupportedError:
             continue
         assert_parity(got, ref, "kernel %d %s" % (kern, spec))
+        if kern == ggml.KERNEL_MMA and spec["Nkv"] > 64:       # key ranges of whole tiles + merge pass
+            assert_parity(run_gpu(case, kernel=kern, n_splits=2 + seed % 3), ref, "tile kernel, split keys %s" % spec)
