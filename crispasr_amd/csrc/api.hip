@@ -183,6 +183,9 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
     bool kv4 = !((uintptr_t)k->data % 4) && !((uintptr_t)v->data % 4);
     for (int i = 1; i < 4; i++) kv4 = kv4 && !(k->nb[i] % 4) && !(v->nb[i] % 4);
     a.kv_aligned4 = kv4 ? 1 : 0;
+    bool kv2 = !((uintptr_t)k->data % 2) && !((uintptr_t)v->data % 2);
+    for (int i = 1; i < 4; i++) kv2 = kv2 && !(k->nb[i] % 2) && !(v->nb[i] % 2);
+    a.kv_aligned2 = kv2 ? 1 : 0;
     const bool al16 = q16 && kv16;
     if (a.mask) {
         a.Hm = (int)mask->ne[2]; a.Bm = (int)mask->ne[3];
@@ -220,11 +223,12 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
     plan.keys_per_split = a.Nkv;
     plan.workspace = 0;
     plan.kv_to_f16 = false;
-    // The tile kernel rounds F32 K/V to f16 on their way into LDS anyway.  With enough queries to share the work it
+    // The tile kernel rounds F32 and Q8_0 K/V to f16 on their way into LDS anyway.  With enough queries to share the work it
     // is cheaper to do that once, in a copy of its own, and let the f16 path (which moves tiles global->LDS without
     // touching registers) read the result: same values, same rounding.
     plan.ws_partials = 0;
-    if (kernel == MI355X_FATTN_MMA && ktype == MI355X_TYPE_F32 && a.Nq >= 128 && a.kv_aligned16) {
+    const bool convertible = (ktype == MI355X_TYPE_F32 && a.kv_aligned16) || (ktype == MI355X_TYPE_Q8_0 && a.kv_aligned2);
+    if (kernel == MI355X_FATTN_MMA && convertible && a.Nq >= 128) {
         plan.kv_to_f16 = true;
         plan.workspace = ((size_t)2 * a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t) + 255) / 256 * 256;
         plan.ws_partials = plan.workspace;
@@ -420,31 +424,17 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
             }
         }
         if (plan.kv_to_f16) {
-            const mi355x_tensor * src[2] = {k, v};
             const size_t half = (size_t)a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t);
-            for (int t = 0; t < 2; t++) {
-                CpyArgs c;
-                memset(&c, 0, sizeof(c));
-                c.src = (const char *)src[t]->data;
-                c.dst = (char *)ws + t * half;
-                int64_t nb = sizeof(uint16_t);
-                c.n = 1;
-                for (int i = 0; i < 4; i++) {
-                    c.sne[i] = c.dne[i] = src[t]->ne[i];
-                    c.snb[i] = (int64_t)src[t]->nb[i];
-                    c.dnb[i] = nb;
-                    nb *= src[t]->ne[i];
-                    c.n *= src[t]->ne[i];
-                }
-                const int e = cpy_launch(c, MI355X_TYPE_F32, MI355X_TYPE_F16, st);
-                if (e) return hip_fail((hipError_t)e, "K/V conversion launch");
-            }
+            const int e = kv_to_f16_launch(a, k->type, ws, st);
+            if (e) return hip_fail((hipError_t)e, "K/V conversion launch");
             // the same call on the f16 copies: contiguous [D, Nkv, Hkv, Bk]
             a.k = (const char *)ws;
             a.v = (const char *)ws + half;
             a.nbk1 = a.nbv1 = (size_t)a.D * 2;
             a.nbk2 = a.nbv2 = a.nbk1 * a.Nkv;
             a.nbk3 = a.nbv3 = a.nbk2 * a.Hkv;
+            a.kv_aligned16 = a.kv_aligned4 = a.kv_aligned2 = 1;
+            a.aligned16 = a.q_aligned16;
             ktype = MI355X_TYPE_F16;
         }
         a.n_splits = plan.n_splits;

@@ -127,7 +127,57 @@ __global__ void __launch_bounds__(256) set_rows_kernel(const CpyArgs a) {
     }
 }
 
+// K and V of one attention call -> two contiguous f16 tensors [D, Nkv, Hkv, Bk] (K first, V right behind it), one
+// launch for both.  One lane per 8 elements of a row: two 128-bit loads (F32) or 8 quants and the block's scale
+// (Q8_0), one 128-bit store.  Rounding is the tile kernel's own: f32 -> f16 round-to-nearest-even, q*d exact in f32
+// and then rounded once.
+template <int TYPE>
+__global__ void __launch_bounds__(256) kv_to_f16_kernel(const FattnArgs a, char * dst) {
+    const int     cpr  = a.D / 8;                                  // chunks per row
+    const int64_t half = (int64_t)cpr * a.Nkv * a.Hkv * a.Bk;      // chunks per tensor
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= 2 * half) return;
+    const bool is_v = i >= half;
+    if (is_v) i -= half;
+    const int     c = (int)(i % cpr);
+    int64_t       r = i / cpr;
+    const int64_t j = r % a.Nkv;  r /= a.Nkv;
+    const int64_t h = r % a.Hkv;
+    const int64_t b = r / a.Hkv;
+    const char * row = is_v ? a.v + j * a.nbv1 + h * a.nbv2 + b * a.nbv3
+                            : a.k + j * a.nbk1 + h * a.nbk2 + b * a.nbk3;
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    h8 y;
+    if (TYPE == MI355X_TYPE_F32) {
+        const float4 x0 = *(const float4 *)(row + c * 32);
+        const float4 x1 = *(const float4 *)(row + c * 32 + 16);
+        y[0] = (_Float16)x0.x; y[1] = (_Float16)x0.y; y[2] = (_Float16)x0.z; y[3] = (_Float16)x0.w;
+        y[4] = (_Float16)x1.x; y[5] = (_Float16)x1.y; y[6] = (_Float16)x1.z; y[7] = (_Float16)x1.w;
+    } else {
+        const char *     blk = row + (c >> 2) * FATTN_Q8_0_BYTES;
+        const uint16_t * qs  = (const uint16_t *)(blk + 2 + (c & 3) * 8);      // blocks are only 2-byte aligned
+        const float      d   = h2f_bits(*(const uint16_t *)blk);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const uint32_t w = qs[e];
+            y[2 * e]     = (_Float16)((float)(int8_t)(w & 0xff) * d);
+            y[2 * e + 1] = (_Float16)((float)(int8_t)(w >> 8) * d);
+        }
+    }
+    *(h8 *)(dst + ((is_v ? half : 0) + i) * 16) = y;
+}
+
 }  // namespace
+
+int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t stream) {
+    const int64_t n = 2 * (int64_t)(a.D / 8) * a.Nkv * a.Hkv * a.Bk;
+    if (n == 0) return 0;
+    const unsigned g = (unsigned)((n + 255) / 256);
+    if (ktype == MI355X_TYPE_F32)       hipLaunchKernelGGL((kv_to_f16_kernel<MI355X_TYPE_F32>), dim3(g), dim3(256), 0, stream, a, (char *)dst);
+    else if (ktype == MI355X_TYPE_Q8_0) hipLaunchKernelGGL((kv_to_f16_kernel<MI355X_TYPE_Q8_0>), dim3(g), dim3(256), 0, stream, a, (char *)dst);
+    else return (int)hipErrorInvalidValue;
+    return (int)hipGetLastError();
+}
 
 static bool vec8_ok(const CpyArgs & a, int stype, int dtype) {
     if (stype == MI355X_TYPE_Q8_0 || dtype == MI355X_TYPE_Q8_0) return false;

@@ -36,6 +36,7 @@ struct FattnArgs {
     int32_t q_aligned16; // q alone
     int32_t kv_aligned16; // k and v alone
     int32_t kv_aligned4;
+    int32_t kv_aligned2;  // k and v: base and strides even (what the Q8_0 halfword reads need)
     int32_t mask_al8;    // mask base and strides are multiples of 8 bytes
     int32_t mask_al4;    // ... of 4 bytes
     int32_t n_cus;       // compute units of the device
@@ -114,3 +115,5 @@ int fattn_decode_launch(const FattnArgs & a, int ktype, hipStream_t stream);
 bool fattn_decode_supported(const FattnArgs & a, int ktype);
 int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream);
 int set_rows_launch(const CpyArgs & a, int dtype, hipStream_t stream);
+// K and V (F32 or Q8_0, any strides) -> contiguous f16 [D, Nkv, Hkv, Bk] at dst and right behind it
+int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t stream);

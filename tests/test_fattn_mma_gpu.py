@@ -117,12 +117,13 @@ def test_pipelined_kernel_with_growing_scores():
         assert_parity(run_gpu(case, kernel=kern), ref, "growing scores, kernel %d" % kern, max_abs_tol=2e-3 * max(1.0, amax))
 
 
-def test_f32_cache_is_converted_once_and_matches_with_any_workspace():
-    """F32 K/V with many queries: the library rounds them to f16 in a workspace and runs the f16 path.  Strided
-    views, a shared K/V batch and a per-head mask; the library's scratch and a caller's workspace give the same
-    result, a workspace that is too small is refused."""
+@pytest.mark.parametrize("ktype", [ora.F32, ora.Q8_0], ids=["f32", "q8_0"])
+def test_f32_and_q8_0_caches_are_converted_once_and_match_with_any_workspace(ktype):
+    """F32 or Q8_0 K/V with many queries: the library rounds them to f16 in a workspace and runs the f16 path.
+    Strided views, a shared K/V batch and a per-head mask; the library's scratch and a caller's workspace give the
+    same result, a workspace that is too small is refused."""
     import torch
-    spec = dict(seed=151, D=128, Nq=300, Nkv=333, Hq=4, Hkv=2, B=2, Bk=1, ktype=ora.F32, kv_layout="thd", mask="bias_perhead")
+    spec = dict(seed=151, D=128, Nq=300, Nkv=333, Hq=4, Hkv=2, B=2, Bk=1, ktype=ktype, kv_layout="thd", mask="bias_perhead")
     case = make_case(**spec)
     ref = run_oracle(case)
     got = run_gpu(case, kernel=ggml.KERNEL_MMA)
