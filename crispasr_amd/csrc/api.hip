@@ -503,6 +503,158 @@ static int cpy_check(const mi355x_tensor * src, const mi355x_tensor * dst) {
     return MI355X_OK;
 }
 
+// ---- FastConformer relative-position mask --------------------------------------------------------------------
+
+static bool aligned16_view(const mi355x_tensor * t) {
+    if ((uintptr_t)t->data % 16) return false;
+    for (int i = 1; i < 4; i++)
+        if (t->ne[i] > 1 && t->nb[i] % 16) return false;
+    return true;
+}
+
+static int relpos_check(const mi355x_tensor * qv, const mi355x_tensor * r, const mi355x_tensor * add,
+                        const mi355x_tensor * dst) {
+    if (!qv || !r || !dst) return fail(MI355X_ERR_INVALID, "null argument");
+    if (qv->type != MI355X_TYPE_F32 || qv->nb[0] != 4) return fail(MI355X_ERR_UNSUPPORTED, "q_v must be F32 with unit element stride");
+    if (r->type != MI355X_TYPE_F32 && r->type != MI355X_TYPE_F16) return fail(MI355X_ERR_UNSUPPORTED, "r type %d not covered", r->type);
+    if (r->nb[0] != type_size(r->type)) return fail(MI355X_ERR_UNSUPPORTED, "r rows must be contiguous");
+    if (dst->type != MI355X_TYPE_F16 || dst->nb[0] != 2) return fail(MI355X_ERR_INVALID, "dst must be F16 with contiguous rows");
+    const int64_t D = qv->ne[0], Nq = qv->ne[1], H = qv->ne[2], B = qv->ne[3];
+    const int64_t Nkv = dst->ne[0];
+    if (D != 64 && D != 128) return fail(MI355X_ERR_UNSUPPORTED, "head size %lld not covered (64, 128)", (long long)D);
+    if (dst->ne[1] != Nq || dst->ne[2] != H || dst->ne[3] != B) return fail(MI355X_ERR_INVALID, "dst shape does not match q_v");
+    if (Nq < 0 || Nkv < 0 || H <= 0 || B <= 0) return fail(MI355X_ERR_INVALID, "bad extents");
+    if (Nq > 0 && Nkv > 0 && (r->ne[0] != D || r->ne[1] != Nq + Nkv - 1))
+        return fail(MI355X_ERR_INVALID, "r must be [D, Nq+Nkv-1, ..]: got [%lld, %lld], want [%lld, %lld]",
+                    (long long)r->ne[0], (long long)r->ne[1], (long long)D, (long long)(Nq + Nkv - 1));
+    if (r->ne[2] <= 0 || r->ne[3] <= 0 || H % r->ne[2] || B % r->ne[3]) return fail(MI355X_ERR_INVALID, "r heads / batch do not divide q_v's");
+    if (Nq + Nkv > (1 << 24) || H * B > (1 << 24)) return fail(MI355X_ERR_UNSUPPORTED, "extent too large");
+    if (qv->data && !aligned16_view(qv)) return fail(MI355X_ERR_UNSUPPORTED, "q_v must be 16-byte aligned");
+    if (r->data && !aligned16_view(r)) return fail(MI355X_ERR_UNSUPPORTED, "r must be 16-byte aligned");
+    if (dst->nb[1] < (size_t)Nkv * 2 || (dst->nb[1] & 1) || (dst->nb[2] & 1) || (dst->nb[3] & 1)) return fail(MI355X_ERR_INVALID, "bad dst strides");
+    if (add && add->ne[0] > 0) {
+        if (add->type != MI355X_TYPE_F32 && add->type != MI355X_TYPE_F16) return fail(MI355X_ERR_UNSUPPORTED, "add type %d not covered", add->type);
+        if (add->nb[0] != type_size(add->type)) return fail(MI355X_ERR_UNSUPPORTED, "add rows must be contiguous");
+        if (add->ne[0] < Nkv || add->ne[1] < Nq) return fail(MI355X_ERR_INVALID, "add is smaller than [Nkv, Nq]");
+        if (add->ne[2] <= 0 || add->ne[3] <= 0 || H % add->ne[2] || B % add->ne[3]) return fail(MI355X_ERR_INVALID, "add heads / batch do not divide q_v's");
+        const size_t es = type_size(add->type);
+        if ((add->data && (uintptr_t)add->data % es) || add->nb[1] % es || add->nb[2] % es || add->nb[3] % es) return fail(MI355X_ERR_UNSUPPORTED, "add is not element-aligned");
+    }
+    return MI355X_OK;
+}
+
+static int relpos_run(const mi355x_tensor * qv, const mi355x_tensor * r, const mi355x_tensor * add,
+                      const mi355x_tensor * dst, float scale, hipStream_t st) {
+    RelposArgs a;
+    memset(&a, 0, sizeof(a));
+    a.D = (int)qv->ne[0]; a.Nq = (int)qv->ne[1]; a.H = (int)qv->ne[2]; a.B = (int)qv->ne[3];
+    a.Nkv = (int)dst->ne[0];
+    if ((int64_t)a.Nq * a.Nkv * a.H * a.B == 0) return MI355X_OK;
+    const bool has_add = add && add->ne[0] > 0;
+    if (!qv->data || !r->data || !dst->data || (has_add && !add->data)) return fail(MI355X_ERR_INVALID, "null data pointer");
+    a.qv = (const char *)qv->data; a.nbq1 = qv->nb[1]; a.nbq2 = qv->nb[2]; a.nbq3 = qv->nb[3];
+    a.r  = (const char *)r->data;  a.nbr1 = r->nb[1];  a.nbr2 = r->nb[2];  a.nbr3 = r->nb[3];
+    a.Hr = (int)r->ne[2]; a.Br = (int)r->ne[3];
+    a.Ha = a.Ba = 1;
+    if (has_add) {
+        a.add = (const char *)add->data; a.nba1 = add->nb[1]; a.nba2 = add->nb[2]; a.nba3 = add->nb[3];
+        a.Ha = (int)add->ne[2]; a.Ba = (int)add->ne[3];
+        a.add_f16 = add->type == MI355X_TYPE_F16;
+    }
+    a.out = (char *)dst->data; a.nbo1 = dst->nb[1]; a.nbo2 = dst->nb[2]; a.nbo3 = dst->nb[3];
+    a.out_al4 = !((uintptr_t)dst->data % 4) && !(dst->nb[1] % 4) && !(dst->nb[2] % 4) && !(dst->nb[3] % 4);
+    a.scale = scale;
+    const int e = relpos_bias_launch(a, r->type, st);
+    if (e) return hip_fail((hipError_t)e, "relpos_bias launch");
+    return MI355X_OK;
+}
+
+int mi355x_relpos_bias_supports(const mi355x_tensor * q_v, const mi355x_tensor * r, const mi355x_tensor * add,
+                                const mi355x_tensor * dst) {
+    return relpos_check(q_v, r, add, dst);
+}
+
+int mi355x_relpos_bias(const mi355x_tensor * q_v, const mi355x_tensor * r, const mi355x_tensor * add,
+                       const mi355x_tensor * dst, float scale, void * stream) {
+    const int rc = relpos_check(q_v, r, add, dst);
+    if (rc) return rc;
+    return relpos_run(q_v, r, add, dst, scale, (hipStream_t)stream);
+}
+
+// the mask the fused call keeps in its workspace: [Nkv, Nq, H, B] with rows padded to 16 bytes
+static void relpos_mask_view(const mi355x_tensor * q_u, const mi355x_tensor * k, void * data, mi355x_tensor * m) {
+    memset(m, 0, sizeof(*m));
+    m->data = data;
+    m->type = MI355X_TYPE_F16;
+    m->ne[0] = k->ne[1]; m->ne[1] = q_u->ne[1]; m->ne[2] = q_u->ne[2]; m->ne[3] = q_u->ne[3];
+    m->nb[0] = 2;
+    m->nb[1] = ((size_t)k->ne[1] * 2 + 15) / 16 * 16;
+    m->nb[2] = m->nb[1] * (size_t)q_u->ne[1];
+    m->nb[3] = m->nb[2] * (size_t)q_u->ne[2];
+}
+
+static int relpos_fused_check(const mi355x_tensor * q_u, const mi355x_tensor * q_v, const mi355x_tensor * k,
+                              const mi355x_tensor * v, const mi355x_tensor * r, const mi355x_tensor * add,
+                              const mi355x_tensor * dst, const mi355x_fattn_params * params, mi355x_tensor * m,
+                              size_t * mask_bytes, size_t * inner_bytes) {
+    if (!q_u || !q_v || !k || !v || !r || !params) return fail(MI355X_ERR_INVALID, "null argument");
+    if (params->max_bias != 0.0f || params->logit_softcap != 0.0f)
+        return fail(MI355X_ERR_UNSUPPORTED, "relative-position attention takes neither max_bias nor logit_softcap");
+    for (int i = 0; i < 4; i++)
+        if (q_u->ne[i] != q_v->ne[i]) return fail(MI355X_ERR_INVALID, "q_u and q_v shapes differ");
+    relpos_mask_view(q_u, k, nullptr, m);
+    int rc = relpos_check(q_v, r, add, m);
+    if (rc) return rc;
+    rc = check(q_u, k, v, m, dst, params);
+    if (rc) return rc;
+    *mask_bytes = (m->nb[3] * (size_t)q_u->ne[3] + 255) / 256 * 256;
+    FattnArgs a;
+    fill_args(a, q_u, k, v, m, nullptr, params);
+    Plan plan;
+    make_plan(a, k->type, params, plan);
+    *inner_bytes = plan.workspace;
+    return MI355X_OK;
+}
+
+int mi355x_fattn_relpos_workspace_size(const mi355x_tensor * q_u, const mi355x_tensor * q_v, const mi355x_tensor * k,
+                                       const mi355x_tensor * v, const mi355x_tensor * r, const mi355x_tensor * add,
+                                       const mi355x_fattn_params * params, size_t * bytes) {
+    if (!bytes) return fail(MI355X_ERR_INVALID, "null argument");
+    mi355x_tensor m;
+    size_t mb = 0, ib = 0;
+    const int rc = relpos_fused_check(q_u, q_v, k, v, r, add, nullptr, params, &m, &mb, &ib);
+    if (rc) return rc;
+    *bytes = mb + ib;
+    return MI355X_OK;
+}
+
+int mi355x_flash_attn_relpos(const mi355x_tensor * q_u, const mi355x_tensor * q_v, const mi355x_tensor * k,
+                             const mi355x_tensor * v, const mi355x_tensor * r, const mi355x_tensor * add,
+                             const mi355x_tensor * dst, const mi355x_fattn_params * params, void * stream) {
+    if (!dst) return fail(MI355X_ERR_INVALID, "null dst");
+    mi355x_tensor m;
+    size_t mb = 0, ib = 0;
+    int rc = relpos_fused_check(q_u, q_v, k, v, r, add, dst, params, &m, &mb, &ib);
+    if (rc) return rc;
+    if ((int64_t)q_u->ne[1] * q_u->ne[2] * q_u->ne[3] == 0) return MI355X_OK;
+    void * ws = params->workspace;
+    if (ws) {
+        if (params->workspace_size < mb + ib)
+            return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, mb + ib);
+        if ((uintptr_t)ws % 16) return fail(MI355X_ERR_WORKSPACE, "workspace must be 16-byte aligned");
+    } else {
+        rc = get_scratch(mb + ib, &ws);
+        if (rc) return rc;
+    }
+    m.data = ws;
+    rc = relpos_run(q_v, r, add, &m, params->scale, (hipStream_t)stream);
+    if (rc) return rc;
+    mi355x_fattn_params inner = *params;
+    inner.workspace      = ib ? (char *)ws + mb : nullptr;      // never the library scratch again: the mask lives there
+    inner.workspace_size = ib;
+    return mi355x_flash_attn_ext(q_u, k, v, &m, dst, &inner, stream);
+}
+
 int mi355x_cpy_supports(const mi355x_tensor * src, const mi355x_tensor * dst) { return cpy_check(src, dst); }
 
 int mi355x_cpy(const mi355x_tensor * src, const mi355x_tensor * dst, void * stream) {

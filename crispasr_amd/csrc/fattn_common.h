@@ -104,6 +104,19 @@ struct CpyArgs {
     int64_t ine[3], inb[3];
 };
 
+// The relative-position mask of a FastConformer attention block (relpos.hip).
+struct RelposArgs {
+    const char * qv;  size_t nbq1, nbq2, nbq3;                  // F32 [D, Nq, H, B]
+    const char * r;   size_t nbr1, nbr2, nbr3; int32_t Hr, Br;   // F32 | F16 [D, Nq+Nkv-1, Hr, Br]
+    const char * add; size_t nba1, nba2, nba3; int32_t Ha, Ba;   // optional F32 | F16 [>=Nkv, >=Nq, Ha, Ba]
+    int32_t add_f16;
+    char *       out; size_t nbo1, nbo2, nbo3;                  // F16 [Nkv, Nq, H, B], rows contiguous
+    int32_t out_al4;                                            // out base and strides are multiples of 4 bytes
+    int32_t D, Nq, Nkv, H, B;
+    float   scale;
+    int32_t n_qblocks, n_chunks;                                // filled in by the launcher
+};
+
 // Launchers implemented next to their kernels; all return hipError_t as int.
 int fattn_vec_launch(const FattnArgs & a, int ktype, hipStream_t stream);
 int fattn_merge_launch(const FattnArgs & a, hipStream_t stream);
@@ -116,4 +129,5 @@ bool fattn_decode_supported(const FattnArgs & a, int ktype);
 int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream);
 int set_rows_launch(const CpyArgs & a, int dtype, hipStream_t stream);
 // K and V (F32 or Q8_0, any strides) -> contiguous f16 [D, Nkv, Hkv, Bk] at dst and right behind it
+int relpos_bias_launch(RelposArgs a, int rtype, hipStream_t stream);
 int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t stream);

@@ -71,6 +71,7 @@ EXPORTS = [
     "mi355x_api_version", "mi355x_status_string", "mi355x_last_error",
     "mi355x_device_count", "mi355x_device_get_info", "mi355x_set_device", "mi355x_stream_synchronize",
     "mi355x_fattn_supports", "mi355x_flash_attn_ext", "mi355x_fattn_workspace_size", "mi355x_fattn_plan",
+    "mi355x_relpos_bias_supports", "mi355x_relpos_bias", "mi355x_flash_attn_relpos", "mi355x_fattn_relpos_workspace_size",
     "mi355x_cpy_supports", "mi355x_cpy", "mi355x_set_rows",
     "mi355x_buffer_alloc", "mi355x_buffer_free", "mi355x_host_buffer_alloc", "mi355x_host_buffer_free", "mi355x_buffer_memset", "mi355x_buffer_set",
     "mi355x_buffer_get", "mi355x_buffer_copy",
@@ -101,6 +102,10 @@ def lib() -> ctypes.CDLL:
         L.mi355x_flash_attn_ext.argtypes = [PT, PT, PT, PT, PT, PP, ctypes.c_void_p]
         L.mi355x_fattn_workspace_size.argtypes = [PT, PT, PT, PT, PP, ctypes.POINTER(ctypes.c_size_t)]
         L.mi355x_fattn_plan.argtypes = [PT, PT, PT, PT, PP, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]
+        L.mi355x_relpos_bias_supports.argtypes = [PT, PT, PT, PT]
+        L.mi355x_relpos_bias.argtypes = [PT, PT, PT, PT, ctypes.c_float, ctypes.c_void_p]
+        L.mi355x_flash_attn_relpos.argtypes = [PT, PT, PT, PT, PT, PT, PT, PP, ctypes.c_void_p]
+        L.mi355x_fattn_relpos_workspace_size.argtypes = [PT, PT, PT, PT, PT, PT, PP, ctypes.POINTER(ctypes.c_size_t)]
         L.mi355x_cpy_supports.argtypes = [PT, PT]
         L.mi355x_cpy.argtypes = [PT, PT, ctypes.c_void_p]
         L.mi355x_set_rows.argtypes = [PT, ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_int64),
@@ -298,6 +303,44 @@ def flash_attn_ext(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor], scal
         _check(lib().mi355x_flash_attn_ext(q.ref(), k.ref(), v.ref(), mask.ref() if mask is not None else None,
                                            out.ref(), ctypes.byref(p), _stream_handle(stream)))
     return out
+
+
+def relpos_bias(q_v: Tensor, r: Tensor, add: Optional[Tensor], scale: float, n_kv: Optional[int] = None, *,
+                out: Optional[Tensor] = None, stream=None) -> Tensor:
+    """The F16 mask core_conformer::build_block builds for its flash-attention call (src/core/fastconformer.h:880-918):
+    cast_f16(scale * rel_shift(mul_mat(cont(R), Q_v)) [+ add]).  Returns it with ne = [n_kv, Nq, H, B]."""
+    if out is None:
+        if n_kv is None:
+            n_kv = r.ne[1] - q_v.ne[1] + 1
+        out = Tensor.empty(F16, (n_kv, q_v.ne[1], q_v.ne[2], q_v.ne[3]), device=q_v.buf.device)
+    with _on_device(q_v.buf.device):
+        _check(lib().mi355x_relpos_bias(q_v.ref(), r.ref(), add.ref() if add is not None else None, out.ref(),
+                                        float(scale), _stream_handle(stream)))
+    return out
+
+
+def flash_attn_relpos(q_u: Tensor, q_v: Tensor, k: Tensor, v: Tensor, r: Tensor, add: Optional[Tensor], scale: float, *,
+                      kernel: int = KERNEL_AUTO, n_splits: int = 0, out: Optional[Tensor] = None,
+                      workspace: Optional[torch.Tensor] = None, stream=None) -> Tensor:
+    """The flash branch of a FastConformer attention block (src/core/fastconformer.h:876-934) in one call:
+    softmax(scale * (q_u.k^T + rel_shift(q_v.r^T)) + add) . v, result ne = [DV, H, Nq, B]."""
+    if out is None:
+        out = Tensor.empty(F32, (v.ne[0], q_u.ne[2], q_u.ne[1], q_u.ne[3]), device=q_u.buf.device)
+    p = _params(scale, 0.0, 0.0, PREC_DEFAULT, kernel, n_splits, workspace)
+    with _on_device(q_u.buf.device):
+        _check(lib().mi355x_flash_attn_relpos(q_u.ref(), q_v.ref(), k.ref(), v.ref(), r.ref(),
+                                              add.ref() if add is not None else None, out.ref(), ctypes.byref(p),
+                                              _stream_handle(stream)))
+    return out
+
+
+def flash_attn_relpos_workspace_size(q_u: Tensor, q_v: Tensor, k: Tensor, v: Tensor, r: Tensor, add: Optional[Tensor],
+                                     scale: float, kernel: int = KERNEL_AUTO, n_splits: int = 0) -> int:
+    p = _params(scale, 0.0, 0.0, PREC_DEFAULT, kernel, n_splits, None)
+    n = ctypes.c_size_t(0)
+    _check(lib().mi355x_fattn_relpos_workspace_size(q_u.ref(), q_v.ref(), k.ref(), v.ref(), r.ref(),
+                                                    add.ref() if add is not None else None, ctypes.byref(p), ctypes.byref(n)))
+    return n.value
 
 
 def cpy(src: Tensor, dst: Tensor, stream=None) -> Tensor:

@@ -143,6 +143,44 @@ int mi355x_fattn_plan(const mi355x_tensor * q, const mi355x_tensor * k, const mi
                       const mi355x_tensor * mask, const mi355x_fattn_params * params,
                       int32_t * kernel, int32_t * n_splits);
 
+/* ---- FastConformer relative-position attention (src/core/fastconformer.h:876-935) ---------- */
+
+/*
+ * The mask that core_conformer::build_block computes for its flash_attn_ext call, as one launch:
+ *
+ *   dst[j, i, h, b] = f16( scale * <q_v[:, i, h, b], r[:, Nq-1+j-i, h % Hr, b % Br]>  +  add[j, i, h % Ha, b % Ba] )
+ *
+ * It replaces the graph nodes  mul_mat(cont(R), Q_v) -> rel_shift view (fastconformer.h:98-102) -> cont -> scale
+ * -> add(local_attn_mask) -> cast F16  (fastconformer.h:880-895, 918); dst is the BD_mask tensor of that graph.
+ *
+ *   q_v  F32 [D, Nq, H, B]            nb[0] == 4, base and strides multiples of 16 bytes; D = 64 or 128
+ *   r    F32 | F16 [D, Nq+Nkv-1, Hr, Br]   rows contiguous and 16-byte aligned; H % Hr == 0, B % Br == 0
+ *   add  NULL, or F32 | F16 [>=Nkv, >=Nq, Ha, Ba]  (0 / -inf / -1e9 pad and window masks), rows contiguous
+ *   dst  F16 [Nkv, Nq, H, B]          rows contiguous (nb[0] == 2); nb[1] may exceed 2*Nkv
+ *
+ * The dot products take f16-rounded inputs and accumulate in f32; scale, add and the rounding to f16 follow the
+ * graph (f32 multiply, f32 add, round to nearest even, overflow to -inf).
+ */
+int mi355x_relpos_bias_supports(const mi355x_tensor * q_v, const mi355x_tensor * r, const mi355x_tensor * add,
+                                const mi355x_tensor * dst);
+int mi355x_relpos_bias(const mi355x_tensor * q_v, const mi355x_tensor * r, const mi355x_tensor * add,
+                       const mi355x_tensor * dst, float scale, void * stream);
+
+/*
+ * The whole flash branch of that block (fastconformer.h:915-934) in one call:
+ *   dst = softmax(scale * (q_u.k^T + BD) + add) . v,   BD[j, i] = <q_v[i], r[Nq-1+j-i]>
+ * computed as mi355x_relpos_bias into the workspace (rows padded to 16 bytes) followed by mi355x_flash_attn_ext
+ * with that mask: same values as the two calls made separately.  q_u, k, v, dst, params as for
+ * mi355x_flash_attn_ext (max_bias and logit_softcap must be 0); Nkv = k->ne[1].
+ */
+int mi355x_flash_attn_relpos(const mi355x_tensor * q_u, const mi355x_tensor * q_v, const mi355x_tensor * k,
+                             const mi355x_tensor * v, const mi355x_tensor * r, const mi355x_tensor * add,
+                             const mi355x_tensor * dst, const mi355x_fattn_params * params, void * stream);
+/* bytes of workspace the call above uses (the mask plus what the attention call itself needs) */
+int mi355x_fattn_relpos_workspace_size(const mi355x_tensor * q_u, const mi355x_tensor * q_v, const mi355x_tensor * k,
+                                       const mi355x_tensor * v, const mi355x_tensor * r, const mi355x_tensor * add,
+                                       const mi355x_fattn_params * params, size_t * bytes);
+
 /* ---- GGML_OP_CPY / CONT / DUP with the destination in a device buffer --------------------- */
 
 /*

@@ -77,6 +77,9 @@ def lib() -> ctypes.CDLL:
         L.ora_cpy_f32.restype = ctypes.c_int
         L.ora_cpy_f32.argtypes = [ctypes.POINTER(_CTensor), ctypes.c_void_p, ctypes.c_int32,
                                   ctypes.POINTER(ctypes.c_int64), ctypes.c_int]
+        L.ora_relpos_bias.restype = ctypes.c_int
+        L.ora_relpos_bias.argtypes = [ctypes.POINTER(_CTensor), ctypes.POINTER(_CTensor), ctypes.POINTER(_CTensor),
+                                      ctypes.c_float, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int]
         L.ora_max_threads.restype = ctypes.c_int
         _lib = L
     return _lib
@@ -226,3 +229,18 @@ def cpy_f32(src: Tensor, dst: Tensor, rounding: int = ROUND_NEAREST_EVEN) -> Non
     rc = lib().ora_cpy_f32(ctypes.byref(cs), dst.buf.ctypes.data + dst.offset, dst.type, nb, rounding)
     if rc != 0:
         raise ValueError(f"ora_cpy_f32 rejected the arguments (code {rc})")
+
+
+def relpos_bias(qv: Tensor, r: Tensor, add: Optional[Tensor], scale: float, n_kv: int, n_threads: int = 0) -> Tensor:
+    """FastConformer's rel-pos mask f16(scale * rel_shift(R^T Q_v) + add) as an F16 tensor ne [n_kv, Nq, H, B]."""
+    Nq, H, B = qv.ne[1], qv.ne[2], qv.ne[3]
+    out = np.zeros(B * H * Nq * n_kv, dtype=np.uint16)
+    if n_threads <= 0:
+        n_threads = max_threads()
+    cq, cr = qv.c(), r.c()
+    ca = add.c() if add is not None else None
+    rc = lib().ora_relpos_bias(ctypes.byref(cq), ctypes.byref(cr), ctypes.byref(ca) if ca is not None else None,
+                               scale, n_kv, out.ctypes.data, n_threads)
+    if rc != 0:
+        raise ValueError(f"ora_relpos_bias rejected the arguments (code {rc})")
+    return Tensor(out.view(np.uint8).reshape(-1), F16, (n_kv, Nq, H, B))

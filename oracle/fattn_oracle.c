@@ -452,3 +452,70 @@ int ora_cpy_f32(const ora_tensor * src, void * dst_data, int32_t dst_type, const
     free(tmp);
     return 0;
 }
+
+/* ------------------------------------------------ FastConformer rel-pos mask -- */
+
+/* The F16 mask that core_conformer::build_block hands to ggml_flash_attn_ext, restated node by
+ * node (src/core/fastconformer.h:876-918):
+ *   BD_raw    = ggml_mul_mat(ggml_cont(R), Q_v)      ne = [NR, Nq, H], NR = 2T-1 (here Nq+Nkv-1)
+ *   BD        = rel_shift(BD_raw)                    a VIEW (fastconformer.h:98-102): ne = [T, T, H],
+ *                                                    nb1 = nb1_raw - nb0, nb2 = nb2_raw, offset (T-1)*nb0
+ *   BD_scaled = ggml_scale(ggml_cont(BD), scale)     f32
+ *   BD_scaled = ggml_add(BD_scaled, local_attn_mask) optional f32 [T, T] (0 / -inf / -1e9), all heads
+ *   BD_mask   = ggml_cast(BD_scaled, F16)            round to nearest even, overflow to -inf
+ * The view is applied literally, as byte offsets into the BD_raw buffer, so that its index map
+ * (element (j, i) of BD = element (T-1+j-i, i) of BD_raw) is a consequence, not an assumption.
+ * The dot products are accumulated in double and rounded once to f32 (ggml's own summation order
+ * inside mul_mat is not fixed by anything in the reference's tree).
+ * Generalised to Nq != Nkv: the view offset is (Nq-1)*nb0 and NR = Nq+Nkv-1.
+ * dst: f16 [Nkv, Nq, H, B] contiguous.  add may be NULL; F32 or F16, ne = [Nkv, Nq, 1|H, 1|B]. */
+int ora_relpos_bias(const ora_tensor * qv, const ora_tensor * r, const ora_tensor * add,
+                    float scale, int64_t n_kv, uint16_t * dst, int n_threads) {
+    if (!qv || !r || !dst) return -1;
+    if (add && !add->data) add = NULL;
+    if (qv->type != ORA_TYPE_F32 || (r->type != ORA_TYPE_F32 && r->type != ORA_TYPE_F16)) return -2;
+    if (add && add->type != ORA_TYPE_F32 && add->type != ORA_TYPE_F16) return -2;
+    const int64_t D = qv->ne[0], Nq = qv->ne[1], H = qv->ne[2], B = qv->ne[3];
+    const int64_t NR = Nq + n_kv - 1;
+    if (r->ne[0] != D || r->ne[1] != NR || r->ne[2] <= 0 || r->ne[3] <= 0 || H % r->ne[2] || B % r->ne[3]) return -3;
+    if (add && (add->ne[0] < n_kv || add->ne[1] < Nq || H % add->ne[2] || B % add->ne[3])) return -4;
+    int nt = n_threads > 0 ? n_threads : 1;
+#ifndef _OPENMP
+    nt = 1;
+#endif
+#pragma omp parallel num_threads(nt)
+    {
+        float * raw  = (float *)malloc((size_t)(NR * Nq > 0 ? NR * Nq : 1) * sizeof(float));
+        float * qrow = (float *)malloc((size_t)(D > 0 ? D : 1) * sizeof(float));
+        float * rrow = (float *)malloc((size_t)(D > 0 ? D : 1) * sizeof(float));
+#pragma omp for schedule(dynamic, 1)
+        for (int64_t hb = 0; hb < H * B; hb++) {
+            const int64_t h = hb % H, b = hb / H;
+            /* BD_raw[p, i] = <R[:, p], Q_v[:, i]>, contiguous: nb0 = 4, nb1 = NR*4 */
+            for (int64_t i = 0; i < Nq; i++) {
+                row_to_f32(row_ptr(qv, i, h, b), ORA_TYPE_F32, D, qrow);
+                for (int64_t p = 0; p < NR; p++) {
+                    row_to_f32(row_ptr(r, p, h % r->ne[2], b % r->ne[3]), r->type, D, rrow);
+                    double acc = 0.0;
+                    for (int64_t d = 0; d < D; d++) acc += (double)rrow[d] * (double)qrow[d];
+                    raw[i * NR + p] = (float)acc;
+                }
+            }
+            /* the rel_shift view of that buffer, then scale, add, cast */
+            const int64_t nb0 = 4, nb1 = NR * 4 - nb0, off = (Nq - 1) * nb0;
+            for (int64_t i = 0; i < Nq; i++)
+                for (int64_t j = 0; j < n_kv; j++) {
+                    const float bd = *(const float *)((const char *)raw + off + j * nb0 + i * nb1);
+                    float x = bd * scale;
+                    if (add) {
+                        const char * ap = (const char *)add->data + j * add->nb[0] + i * add->nb[1] +
+                                          (h % add->ne[2]) * add->nb[2] + (b % add->ne[3]) * add->nb[3];
+                        x += add->type == ORA_TYPE_F32 ? *(const float *)ap : h2f(*(const uint16_t *)ap);
+                    }
+                    dst[((b * H + h) * Nq + i) * n_kv + j] = f2h(x);
+                }
+        }
+        free(raw); free(qrow); free(rrow);
+    }
+    return 0;
+}

@@ -26,6 +26,10 @@
  *       max_bias (ALiBi) slope formula : PARITY UNPINNED - recalled
  *       behaviour of ggml-cpu that no file, test or fixture of the reference
  *       holds.  logit_softcap is pinned by its closed form only.
+ *   ora_relpos_bias : pinned by the reference's own graph (src/core/fastconformer.h:98-102,
+ *       876-918, every node of which is restated literally, the rel_shift view as byte strides)
+ *       and by the mathematics: numpy matmul + numpy.lib.stride_tricks.as_strided with the
+ *       view's strides, and the closed form BD[j, i] = <Q_v[i], R[T-1+j-i]>, on small shapes.
  */
 #ifndef FATTN_ORACLE_H
 #define FATTN_ORACLE_H
@@ -85,6 +89,12 @@ int ora_flash_attn_ext(const ora_tensor * q, const ora_tensor * k, const ora_ten
  * are contiguous): src and dst have equal ne, src is F32. */
 int ora_cpy_f32(const ora_tensor * src, void * dst_data, int32_t dst_type, const int64_t dst_nb[4],
                 int rounding);
+
+/* FastConformer's relative-position mask: f16( scale * rel_shift(R^T Q_v) + add ), see the .c file.
+ * qv F32 [D, Nq, H, B]; r F32/F16 [D, Nq+n_kv-1, 1|H.., 1|B..]; add NULL or F32/F16 [n_kv, Nq, 1|H, 1|B];
+ * dst f16 [n_kv, Nq, H, B] contiguous. */
+int ora_relpos_bias(const ora_tensor * qv, const ora_tensor * r, const ora_tensor * add,
+                    float scale, int64_t n_kv, uint16_t * dst, int n_threads);
 
 int ora_max_threads(void);
 

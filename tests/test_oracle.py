@@ -364,3 +364,90 @@ def test_cpy_f32_into_strided_cache_view(dtype):
     # rows outside [n_past, n_past+T) untouched
     c = cache.reshape(H, ctx, rs)
     assert np.all(c[:, :n_past] == 0xAB) and np.all(c[:, n_past + T:] == 0xAB)
+
+
+# ----------------------------------------------------------------------------- FastConformer rel-pos mask
+
+
+def _relpos_inputs(seed, D, Nq, Nkv, H, B, Br=1, with_add=None):
+    qv = ora.randn(seed, (B, H, Nq, D))
+    r = ora.randn(seed + 1000, (Br, H, Nq + Nkv - 1, D))
+    add = None
+    if with_add == "pad":          # pad keys are -inf for every query (src/canary_ctc.cpp:988-996)
+        add = np.zeros((1, 1, Nq, Nkv), np.float32)
+        add[..., Nkv - 3:] = -np.inf
+    elif with_add == "local":      # finite "minus infinity" of the local-attention mask (src/core/fastconformer.h:139-163)
+        add = np.full((1, 1, Nq, Nkv), -1e9, np.float32)
+        for i in range(Nq):
+            add[0, 0, i, max(0, i - 2):min(Nkv, i + 3)] = 0.0
+    return qv, r, add
+
+
+@pytest.mark.parametrize("spec", [
+    dict(seed=31, D=64, Nq=9, Nkv=9, H=2, B=1),
+    dict(seed=32, D=128, Nq=17, Nkv=17, H=3, B=2, with_add="pad"),
+    dict(seed=33, D=32, Nq=12, Nkv=12, H=1, B=2, Br=2, with_add="local"),
+], ids=lambda s: "seed%d" % s["seed"])
+def test_relpos_bias_equals_numpy_matmul_seen_through_the_rel_shift_view(spec):
+    """mul_mat -> rel_shift view -> scale -> add -> cast, with numpy doing the matmul and
+    as_strided doing the view with the strides of src/core/fastconformer.h:98-102."""
+    D, Nq, Nkv, H, B = spec["D"], spec["Nq"], spec["Nkv"], spec["H"], spec["B"]
+    qv, r, add = _relpos_inputs(**spec)
+    scale = np.float32(1.0 / math.sqrt(D))
+    got = ora.relpos_bias(ora.from_f32(qv), ora.from_f32(r), ora.from_f32(add) if add is not None else None,
+                          float(scale), Nkv)
+    got = got.buf.view(np.uint16).reshape(B, H, Nq, Nkv)
+    T, NR = Nq, Nq + Nkv - 1
+    for b in range(B):
+        for h in range(H):
+            raw = (qv[b, h].astype(np.float64) @ r[b % r.shape[0], h].astype(np.float64).T).astype(np.float32)   # [T, NR]: ne = [NR, T]
+            raw = np.ascontiguousarray(raw)
+            view = np.lib.stride_tricks.as_strided(raw.reshape(-1)[T - 1:], shape=(T, T), strides=(NR * 4 - 4, 4))
+            x = view * scale
+            if add is not None:
+                x = x + add[0, 0]
+            with np.errstate(over="ignore"):
+                want = x.astype(np.float16).view(np.uint16)
+            assert np.array_equal(got[b, h], want), (b, h)
+
+
+def test_relpos_bias_closed_form_and_direction_of_the_shift():
+    """BD[j, i] = <Q_v[i], R[Nq-1+j-i]>: with every query equal the mask is Toeplitz, its diagonal is row Nq-1
+    of R, keys to the right of the diagonal (j > i) take later rows.  Also the rectangular generalisation."""
+    D, Nq, Nkv = 32, 7, 11
+    qv = np.ones((1, 1, Nq, D), np.float32)
+    r = np.zeros((1, 1, Nq + Nkv - 1, D), np.float32)
+    r[0, 0, :, 0] = np.arange(Nq + Nkv - 1, dtype=np.float32) - (Nq - 1)      # <q, R[p]> = p - (Nq-1) = j - i
+    got = ora.relpos_bias(ora.from_f32(qv), ora.from_f32(r), None, 1.0, Nkv)
+    m = ora.fp16_to_fp32(got.buf.view(np.uint16)).reshape(Nq, Nkv)
+    for i in range(Nq):
+        for j in range(Nkv):
+            assert m[i, j] == j - i
+    # random rectangular case against the per-element closed form
+    qv, r, _ = _relpos_inputs(34, 64, 5, 13, 2, 1)
+    got = ora.relpos_bias(ora.from_f32(qv), ora.from_f32(r, ora.F16), None, 0.125, 13)
+    m = got.buf.view(np.uint16).reshape(2, 5, 13)
+    r16 = ora.fp16_to_fp32(ora.fp32_to_fp16(r))
+    for h in range(2):
+        for i in range(5):
+            for j in range(13):
+                bd = np.float32(np.dot(qv[0, h, i].astype(np.float64), r16[0, h, 5 - 1 + j - i].astype(np.float64)))
+                assert m[h, i, j] == np.float16(bd * np.float32(0.125)).view(np.uint16)
+
+
+def test_relpos_mask_in_attention_equals_manual_softmax_of_ac_plus_bd():
+    """softmax((Q_u K^T + BD) * scale) V (src/core/fastconformer.h:883-885, the manual branch :897-914) against
+    flash_attn_ext with mask = BD*scale: equal up to the f16 rounding of the mask."""
+    D, T, H = 64, 10, 2
+    qu = ora.randn(41, (1, H, T, D)); k = ora.randn(42, (1, H, T, D)); v = ora.randn(43, (1, H, T, D))
+    qv, r, _ = _relpos_inputs(44, D, T, T, H, 1)
+    scale = 1.0 / math.sqrt(D)
+    mask = ora.relpos_bias(ora.from_f32(qv), ora.from_f32(r), None, scale, T)
+    got = ora.flash_attn_ext(ora.from_f32(qu), ora.from_f32(k), ora.from_f32(v), mask, scale)[0]      # [T, H, D]
+    for h in range(H):
+        ac = qu[0, h].astype(np.float64) @ k[0, h].astype(np.float64).T
+        bd = np.array([[np.dot(qv[0, h, i].astype(np.float64), r[0, h, T - 1 + j - i]) for j in range(T)] for i in range(T)])
+        s = (ac + bd) * scale
+        p = np.exp(s - s.max(axis=1, keepdims=True)); p /= p.sum(axis=1, keepdims=True)
+        want = p @ v[0, h].astype(np.float64)
+        assert np.abs(got[:, h] - want).max() < 3e-3

@@ -1,0 +1,143 @@
+"""GPU parity of FastConformer's relative-position mask kernel and of the fused rel-pos attention call against the
+CPU oracle's node-by-node restatement of the graph (src/core/fastconformer.h:98-102, 876-934)."""
+import math
+
+import numpy as np
+import pytest
+
+import oracle as ora
+from crispasr_amd import ggml
+from gpu_util import assert_parity, upload
+
+pytestmark = pytest.mark.gpu
+
+NEG_INF_BITS = 0xFC00
+
+
+def strided(x: np.ndarray, layout: str) -> ora.Tensor:
+    """f32 numpy [B, H, N, D] -> ggml tensor ne [D, N, H, B]; "thd" stores it as [B, N, H, D] (the permuted view of a
+    [d_model, T] activation that the reference passes, src/core/fastconformer.h:849-852)."""
+    B, H, N, D = x.shape
+    if layout == "thd":
+        raw = np.ascontiguousarray(x.transpose(0, 2, 1, 3)).view(np.uint8).reshape(-1)
+        return ora.Tensor(raw, ora.F32, (D, N, H, B), (4, H * D * 4, D * 4, N * H * D * 4))
+    return ora.from_f32(x)
+
+
+def make(seed, D, Nq, Nkv, H, B, Br=1, rtype=ora.F32, add=None, layout="cont", add_type=ora.F32, qgain=1.0):
+    qv = np.float32(qgain) * ora.randn(seed, (B, H, Nq, D))
+    r = ora.randn(seed + 1, (Br, H, Nq + Nkv - 1, D))
+    a = None
+    if add == "pad":                                   # per-sequence key padding, -inf (src/canary_ctc.cpp:988-996)
+        a = np.zeros((B, 1, Nq, Nkv), np.float32)
+        for b in range(B):
+            a[b, :, :, Nkv - 1 - (7 * b + 3) % max(1, Nkv // 2):] = -np.inf
+    elif add == "local":                               # window mask with the finite -1e9 (src/core/fastconformer.h:139-163)
+        a = np.full((1, 1, Nq, Nkv), -1e9, np.float32)
+        for i in range(Nq):
+            a[0, 0, i, max(0, i - 40):min(Nkv, i + 41)] = 0.0
+    elif add == "perhead":
+        a = 0.25 * ora.randn(seed + 2, (1, H, Nq, Nkv))
+    return dict(qv=strided(qv, layout), r=ora.from_f32(r, rtype), add=None if a is None else ora.from_f32(a, add_type),
+                D=D, Nq=Nq, Nkv=Nkv, H=H, B=B, scale=1.0 / math.sqrt(D))
+
+
+def check_mask(got_bits: np.ndarray, ref_bits: np.ndarray, what: str):
+    assert got_bits.shape == ref_bits.shape
+    inf_ref = ref_bits == NEG_INF_BITS
+    assert np.array_equal(got_bits == NEG_INF_BITS, inf_ref), f"{what}: -inf positions differ"
+    g, r = ora.fp16_to_fp32(got_bits), ora.fp16_to_fp32(ref_bits)
+    fin = ~inf_ref
+    assert np.isfinite(g[fin]).all(), f"{what}: non-finite value at a finite position"
+    err = np.abs(g[fin] - r[fin])
+    # inputs of the products are rounded to f16 (relative 2^-11 each) before an f32 accumulation, and the result
+    # is rounded to f16 again: a few f16 ulps at most, under one on average
+    tol = 4e-3 * np.maximum(1.0, np.abs(r[fin]))
+    assert (err <= tol).all(), f"{what}: max err {err.max():.3e}"
+    assert err.mean() < 6e-4, f"{what}: mean err {err.mean():.3e}"
+
+
+SPECS = [
+    dict(seed=301, D=128, Nq=75, Nkv=75, H=2, B=2, add="pad"),                       # odd Nkv: halfword stores
+    dict(seed=302, D=64, Nq=300, Nkv=300, H=2, B=1),                                 # 5 key tiles: two chunks per query block
+    dict(seed=303, D=64, Nq=70, Nkv=334, H=3, B=1, rtype=ora.F16, add="local"),      # rectangular, f16 table, -1e9 window
+    dict(seed=304, D=128, Nq=130, Nkv=130, H=4, B=2, Br=2, layout="thd", add="perhead", add_type=ora.F16),
+    dict(seed=305, D=128, Nq=33, Nkv=64, H=1, B=1, layout="thd"),
+    dict(seed=306, D=64, Nq=1, Nkv=1, H=2, B=1),
+    dict(seed=307, D=128, Nq=750, Nkv=750, H=2, B=1, add="pad", layout="thd"),        # FastConformer's real T
+]
+
+
+@pytest.mark.parametrize("spec", SPECS, ids=lambda s: "seed%d" % s["seed"])
+def test_relpos_mask_matches_the_graph_restatement(spec):
+    c = make(**spec)
+    ref = ora.relpos_bias(c["qv"], c["r"], c["add"], c["scale"], c["Nkv"])
+    got = ggml.relpos_bias(upload(c["qv"]), upload(c["r"]), upload(c["add"]) if c["add"] is not None else None,
+                           c["scale"], c["Nkv"])
+    n = c["Nkv"] * c["Nq"] * c["H"] * c["B"]
+    got_bits = got.to_host()[: 2 * n].view(np.uint16)
+    check_mask(got_bits, ref.buf.view(np.uint16), str(spec))
+
+
+def test_relpos_mask_into_a_padded_destination_leaves_the_padding_alone():
+    import torch
+    c = make(seed=311, D=64, Nq=40, Nkv=75, H=2, B=1)
+    pitch = 160                                                                      # 75 keys = 150 bytes, padded to 16
+    buf = torch.full((pitch * 40 * 2,), 0x5A, dtype=torch.uint8, device="cuda")
+    dst = ggml.Tensor(buf, ggml.F16, (75, 40, 2, 1), (2, pitch, pitch * 40, pitch * 80))
+    ggml.relpos_bias(upload(c["qv"]), upload(c["r"]), None, c["scale"], out=dst)
+    raw = buf.cpu().numpy().reshape(80, pitch)
+    assert (raw[:, 150:] == 0x5A).all()
+    ref = ora.relpos_bias(c["qv"], c["r"], None, c["scale"], 75).buf.view(np.uint16).reshape(80, 75)
+    check_mask(np.ascontiguousarray(raw[:, :150]).view(np.uint16), ref, "padded rows")
+
+
+ATTN = [
+    dict(seed=321, D=128, Nq=150, Nkv=150, H=4, B=2, add="pad", layout="thd", ktype=ora.F32),      # as the reference calls it
+    dict(seed=322, D=64, Nq=257, Nkv=257, H=2, B=1, ktype=ora.F16),
+    dict(seed=323, D=128, Nq=20, Nkv=90, H=2, B=1, add="local", ktype=ora.F16),                    # few queries: not the tile kernel's mask path
+]
+
+
+@pytest.mark.parametrize("spec", ATTN, ids=lambda s: "seed%d" % s["seed"])
+def test_fused_relpos_attention_matches_oracle_and_the_two_separate_calls(spec):
+    import torch
+    spec = dict(spec)
+    ktype = spec.pop("ktype")
+    # content and position terms of std 0.7 each: scores of unit variance, the level the op's tolerance is quoted at
+    c = make(qgain=0.7, **spec)
+    D, Nq, Nkv, H, B = c["D"], c["Nq"], c["Nkv"], c["H"], c["B"]
+    qu = strided(np.float32(0.7) * ora.randn(spec["seed"] + 10, (B, H, Nq, D)), spec.get("layout", "cont"))
+    k = ora.from_f32(ora.randn(spec["seed"] + 11, (B, H, Nkv, D)), ktype)
+    v = ora.from_f32(ora.randn(spec["seed"] + 12, (B, H, Nkv, D)), ktype)
+    mask = ora.relpos_bias(c["qv"], c["r"], c["add"], c["scale"], Nkv)
+    ref = ora.flash_attn_ext(qu, k, v, mask, c["scale"])
+    dq, dqv, dk, dv, dr = upload(qu), upload(c["qv"]), upload(k), upload(v), upload(c["r"])
+    da = upload(c["add"]) if c["add"] is not None else None
+    got = ggml.flash_attn_relpos(dq, dqv, dk, dv, dr, da, c["scale"]).numpy_f32()
+    assert_parity(got, ref, "fused " + str(spec))
+    # the same through a caller's workspace, and as two calls: identical bits
+    need = ggml.flash_attn_relpos_workspace_size(dq, dqv, dk, dv, dr, da, c["scale"])
+    pitch = (Nkv * 2 + 15) // 16 * 16
+    assert need >= pitch * Nq * H * B
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    got_ws = ggml.flash_attn_relpos(dq, dqv, dk, dv, dr, da, c["scale"], workspace=ws).numpy_f32()
+    assert np.array_equal(got_ws, got)
+    with pytest.raises(ggml.Mi355xError):
+        ggml.flash_attn_relpos(dq, dqv, dk, dv, dr, da, c["scale"], workspace=ws[: need - 256])
+    mbuf = torch.empty(pitch * Nq * H * B, dtype=torch.uint8, device="cuda")
+    m = ggml.Tensor(mbuf, ggml.F16, (Nkv, Nq, H, B), (2, pitch, pitch * Nq, pitch * Nq * H))
+    ggml.relpos_bias(dqv, dr, da, c["scale"], out=m)
+    two = ggml.flash_attn_ext(dq, dk, dv, m, c["scale"]).numpy_f32()
+    assert np.array_equal(two, got)
+
+
+def test_relpos_contract_violations_are_reported():
+    c = make(seed=331, D=64, Nq=10, Nkv=10, H=1, B=1)
+    qv, r = upload(c["qv"]), upload(c["r"])
+    short = ggml.Tensor(r.buf, ggml.F32, (64, 18, 1, 1))                               # needs Nq+Nkv-1 = 19 rows
+    with pytest.raises(ggml.InvalidError):
+        ggml.relpos_bias(qv, short, None, 0.125, 10)
+    c80 = dict(qv=ora.from_f32(ora.randn(1, (1, 1, 4, 80))), r=ora.from_f32(ora.randn(2, (1, 1, 7, 80))))
+    with pytest.raises(ggml.UnsupportedError):
+        ggml.relpos_bias(upload(c80["qv"]), upload(c80["r"]), None, 0.1, 4)
