@@ -350,7 +350,61 @@ def bench_configs(args, ca, ora, torch):
         run(f"C5_fastconformer_kv_{nm}", dict(seed=5, D=128, Nq=750, Nkv=750, Hq=8, B=8, ktype=kt, mask="bias_perhead_pad",
                                               lengths=lengths),
             note="8 heads x 128, T=750, batch 8, per-head f16 bias N(0, std 0.5) with -inf beyond each length (1 layer)")
+    res["C5_fastconformer_relpos_f32"] = bench_relpos(ca, ora, torch, lengths)
     return res
+
+
+def bench_relpos(ca, ora, torch, lengths):
+    """The flash branch of a FastConformer block as the reference builds it (src/core/fastconformer.h:876-934) at the
+    Parakeet / Canary-CTC shape: Q_u, Q_v, K, V F32 views [128, 750, 8] of [1024, 750] activations, R F32 [128, 1499, 8],
+    F32 pad mask [750, 750] per sequence with -inf beyond its length, batch 8.  Times the mask kernel alone and the
+    fused call (mask kernel + attention).  Content and position terms are drawn with std 0.7 each (unit-variance
+    scores).  Parity: the oracle's node-by-node mask and exact attention, on the first and the last sequence."""
+    import numpy as np
+    from cases import errors, MAX_ABS_TOL, REL_L2_TOL
+    D, T, H, B = 128, 750, 8, 8
+    dm = D * H
+    scale = 1.0 / D ** 0.5
+
+    def act(seed, n, gain=1.0):          # [B, n, d_model] activations seen as ne [D, n, H, B]
+        x = (np.float32(gain) * ora.randn(seed, (B, n, dm))).astype(np.float32)
+        return ora.Tensor(x.view(np.uint8).reshape(-1), ora.F32, (D, n, H, B), (4, dm * 4, D * 4, n * dm * 4))
+
+    qu, qv, k, v = act(51, T, 0.7), act(52, T, 0.7), act(53, T), act(54, T)
+    r1 = ora.randn(55, (1, 2 * T - 1, dm)).astype(np.float32)
+    r = ora.Tensor(r1.view(np.uint8).reshape(-1), ora.F32, (D, 2 * T - 1, H, 1), (4, dm * 4, D * 4, (2 * T - 1) * dm * 4))
+    pad = np.zeros((B, 1, T, T), np.float32)
+    for b in range(B):
+        pad[b, :, :, lengths[b]:] = -np.inf
+    add = ora.from_f32(pad)
+    up = lambda t: ca.Tensor.from_host(t.buf, t.type, t.ne, t.nb, t.offset)
+    dqu, dqv, dk, dv, dr, da = (up(t) for t in (qu, qv, k, v, r, add))
+    out = ca.Tensor.empty(ca.F32, (D, H, T, B))
+    pitch = (T * 2 + 15) // 16 * 16
+    mbuf = torch.empty(pitch * T * H * B, dtype=torch.uint8, device="cuda")
+    dm_t = ca.Tensor(mbuf, ca.F16, (T, T, H, B), (2, pitch, pitch * T, pitch * T * H))
+    us_mask = _time_calls(torch, lambda: ca.ggml.relpos_bias(dqv, dr, da, scale, out=dm_t), 20)
+    us_all = _time_calls(torch, lambda: ca.ggml.flash_attn_relpos(dqu, dqv, dk, dv, dr, da, scale, out=out), 20)
+    got = out.numpy_f32()
+    worst = [0.0, 0.0]
+    for b in (0, B - 1):
+        sub = lambda t: ora.Tensor(t.buf, t.type, t.ne[:3] + (1,), t.nb, t.offset + b * t.nb[3])
+        mask = ora.relpos_bias(sub(qv), r, sub(add), scale, T)
+        ref = ora.flash_attn_ext(sub(qu), sub(k), sub(v), mask, scale)
+        ma, rel = errors(got[b:b + 1], ref)
+        worst = [max(worst[0], ma), max(worst[1], rel)]
+    ok = bool(worst[0] <= MAX_ABS_TOL and worst[1] <= REL_L2_TOL)
+    flops = attn_flops(D, T, T, H, B) * 1.5                     # + one 2*D-flop dot per (query, key) for the position term
+    nbytes = (4 * T + 2 * T - 1) * dm * 4 + 4 * T * dm * 4 * (B - 1) + T * T * 4 * B + T * dm * 4 * B
+    log(f"[bench] C5_fastconformer_relpos_f32: mask kernel {us_mask:.1f} us, fused call {us_all:.1f} us, "
+        f"{flops / us_all / 1e6:.1f} TFLOP/s, parity (2 of 8 sequences) max_abs={worst[0]:.2e} rel_l2={worst[1]:.2e} "
+        f"{'ok' if ok else 'FAIL: timing withheld'}")
+    return {"us_per_call": us_all if ok else None, "us_mask_kernel": us_mask if ok else None,
+            "TFLOP/s": flops / us_all / 1e6 if ok else None, "GB/s": nbytes / us_all / 1e3 if ok else None,
+            "flops": flops, "bytes": nbytes, "mask_workspace_bytes": pitch * T * H * B,
+            "parity": {"max_abs": worst[0], "rel_l2": worst[1], "ok": ok, "sequences_checked": 2},
+            "note": "8 heads x 128, T=750, batch 8: Q_u/Q_v/K/V F32 strided views, R F32 [128,1499,8], F32 pad mask; "
+                    "mask kernel + attention in one call, nothing computed on the host"}
 
 
 def scale_check(ca, torch, layer):

@@ -529,6 +529,10 @@ static int relpos_check(const mi355x_tensor * qv, const mi355x_tensor * r, const
                     (long long)r->ne[0], (long long)r->ne[1], (long long)D, (long long)(Nq + Nkv - 1));
     if (r->ne[2] <= 0 || r->ne[3] <= 0 || H % r->ne[2] || B % r->ne[3]) return fail(MI355X_ERR_INVALID, "r heads / batch do not divide q_v's");
     if (Nq + Nkv > (1 << 24) || H * B > (1 << 24)) return fail(MI355X_ERR_UNSUPPORTED, "extent too large");
+    const uint64_t lim = (uint64_t)1 << 31;      // the kernel keeps 32-bit offsets inside a (head, batch) plane
+    if ((uint64_t)Nq * qv->nb[1] >= lim || (uint64_t)(Nq + Nkv) * D * 2 >= lim || (uint64_t)Nq * dst->nb[1] >= lim ||
+        (add && add->ne[0] > 0 && (uint64_t)Nq * add->nb[1] >= lim))
+        return fail(MI355X_ERR_UNSUPPORTED, "a (head, batch) plane exceeds 2 GiB");
     if (qv->data && !aligned16_view(qv)) return fail(MI355X_ERR_UNSUPPORTED, "q_v must be 16-byte aligned");
     if (r->data && !aligned16_view(r)) return fail(MI355X_ERR_UNSUPPORTED, "r must be 16-byte aligned");
     if (dst->nb[1] < (size_t)Nkv * 2 || (dst->nb[1] & 1) || (dst->nb[2] & 1) || (dst->nb[3] & 1)) return fail(MI355X_ERR_INVALID, "bad dst strides");
@@ -543,8 +547,15 @@ static int relpos_check(const mi355x_tensor * qv, const mi355x_tensor * r, const
     return MI355X_OK;
 }
 
+// bytes of the contiguous f16 copy the kernel reads (0 for an F16 table with contiguous rows, which is read in place)
+static size_t relpos_table_bytes(const mi355x_tensor * r) {
+    if (r->type == MI355X_TYPE_F16 && r->nb[1] == (size_t)r->ne[0] * 2) return 0;
+    return ((size_t)r->ne[0] * r->ne[1] * r->ne[2] * r->ne[3] * 2 + 255) / 256 * 256;
+}
+
+// r16: room for relpos_table_bytes(r), or NULL to take it from the library's scratch
 static int relpos_run(const mi355x_tensor * qv, const mi355x_tensor * r, const mi355x_tensor * add,
-                      const mi355x_tensor * dst, float scale, hipStream_t st) {
+                      const mi355x_tensor * dst, float scale, void * r16, hipStream_t st) {
     RelposArgs a;
     memset(&a, 0, sizeof(a));
     a.D = (int)qv->ne[0]; a.Nq = (int)qv->ne[1]; a.H = (int)qv->ne[2]; a.B = (int)qv->ne[3];
@@ -555,16 +566,42 @@ static int relpos_run(const mi355x_tensor * qv, const mi355x_tensor * r, const m
     a.qv = (const char *)qv->data; a.nbq1 = qv->nb[1]; a.nbq2 = qv->nb[2]; a.nbq3 = qv->nb[3];
     a.r  = (const char *)r->data;  a.nbr1 = r->nb[1];  a.nbr2 = r->nb[2];  a.nbr3 = r->nb[3];
     a.Hr = (int)r->ne[2]; a.Br = (int)r->ne[3];
+    if (relpos_table_bytes(r)) {
+        // the kernel multiplies f16 values anyway: round the table once, into a contiguous [D, NR, Hr, Br] copy
+        if (!r16) {
+            const int rc = get_scratch(relpos_table_bytes(r), &r16);
+            if (rc) return rc;
+        }
+        CpyArgs c;
+        memset(&c, 0, sizeof(c));
+        c.src = (const char *)r->data;
+        c.dst = (char *)r16;
+        int64_t nb = 2;
+        c.n = 1;
+        for (int i = 0; i < 4; i++) {
+            c.sne[i] = c.dne[i] = r->ne[i];
+            c.snb[i] = (int64_t)r->nb[i];
+            c.dnb[i] = nb;
+            nb *= r->ne[i];
+            c.n *= r->ne[i];
+        }
+        const int e = cpy_launch(c, r->type, MI355X_TYPE_F16, st);
+        if (e) return hip_fail((hipError_t)e, "table conversion launch");
+        a.r = (const char *)r16;
+        a.nbr1 = (size_t)a.D * 2; a.nbr2 = a.nbr1 * (size_t)r->ne[1]; a.nbr3 = a.nbr2 * (size_t)r->ne[2];
+    }
     a.Ha = a.Ba = 1;
     if (has_add) {
         a.add = (const char *)add->data; a.nba1 = add->nb[1]; a.nba2 = add->nb[2]; a.nba3 = add->nb[3];
         a.Ha = (int)add->ne[2]; a.Ba = (int)add->ne[3];
         a.add_f16 = add->type == MI355X_TYPE_F16;
+        const size_t pair = 2 * type_size(add->type);
+        a.add_vec = !((uintptr_t)add->data % pair) && !(add->nb[1] % pair) && !(add->nb[2] % pair) && !(add->nb[3] % pair);
     }
     a.out = (char *)dst->data; a.nbo1 = dst->nb[1]; a.nbo2 = dst->nb[2]; a.nbo3 = dst->nb[3];
     a.out_al4 = !((uintptr_t)dst->data % 4) && !(dst->nb[1] % 4) && !(dst->nb[2] % 4) && !(dst->nb[3] % 4);
     a.scale = scale;
-    const int e = relpos_bias_launch(a, r->type, st);
+    const int e = relpos_bias_launch(a, MI355X_TYPE_F16, st);
     if (e) return hip_fail((hipError_t)e, "relpos_bias launch");
     return MI355X_OK;
 }
@@ -578,7 +615,7 @@ int mi355x_relpos_bias(const mi355x_tensor * q_v, const mi355x_tensor * r, const
                        const mi355x_tensor * dst, float scale, void * stream) {
     const int rc = relpos_check(q_v, r, add, dst);
     if (rc) return rc;
-    return relpos_run(q_v, r, add, dst, scale, (hipStream_t)stream);
+    return relpos_run(q_v, r, add, dst, scale, nullptr, (hipStream_t)stream);
 }
 
 // the mask the fused call keeps in its workspace: [Nkv, Nq, H, B] with rows padded to 16 bytes
@@ -607,7 +644,7 @@ static int relpos_fused_check(const mi355x_tensor * q_u, const mi355x_tensor * q
     if (rc) return rc;
     rc = check(q_u, k, v, m, dst, params);
     if (rc) return rc;
-    *mask_bytes = (m->nb[3] * (size_t)q_u->ne[3] + 255) / 256 * 256;
+    *mask_bytes = (m->nb[3] * (size_t)q_u->ne[3] + 255) / 256 * 256 + relpos_table_bytes(r);      // the mask, then the f16 table
     FattnArgs a;
     fill_args(a, q_u, k, v, m, nullptr, params);
     Plan plan;
@@ -647,7 +684,7 @@ int mi355x_flash_attn_relpos(const mi355x_tensor * q_u, const mi355x_tensor * q_
         if (rc) return rc;
     }
     m.data = ws;
-    rc = relpos_run(q_v, r, add, &m, params->scale, (hipStream_t)stream);
+    rc = relpos_run(q_v, r, add, &m, params->scale, (char *)ws + mb - relpos_table_bytes(r), (hipStream_t)stream);
     if (rc) return rc;
     mi355x_fattn_params inner = *params;
     inner.workspace      = ib ? (char *)ws + mb : nullptr;      // never the library scratch again: the mask lives there
