@@ -380,7 +380,7 @@ def bench_relpos(ca, ora, torch, lengths):
     up = lambda t: ca.Tensor.from_host(t.buf, t.type, t.ne, t.nb, t.offset)
     dqu, dqv, dk, dv, dr, da = (up(t) for t in (qu, qv, k, v, r, add))
     out = ca.Tensor.empty(ca.F32, (D, H, T, B))
-    pitch = (T * 2 + 15) // 16 * 16
+    pitch = (T * 2 + 127) // 128 * 128
     mbuf = torch.empty(pitch * T * H * B, dtype=torch.uint8, device="cuda")
     dm_t = ca.Tensor(mbuf, ca.F16, (T, T, H, B), (2, pitch, pitch * T, pitch * T * H))
     us_mask = _time_calls(torch, lambda: ca.ggml.relpos_bias(dqv, dr, da, scale, out=dm_t), 20)
@@ -532,6 +532,8 @@ def main():
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-scale-check", action="store_true", help="skip the half-size launches (keeps profiler means per kernel clean)")
     ap.add_argument("--no-configs", action="store_true", help="skip the other baseline configurations and the Whisper protocol")
+    ap.add_argument("--relpos-only", action="store_true",
+                    help="run only the FastConformer rel-pos configuration and print its figures as the JSON line (profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU form in this build (heads and windows "
@@ -548,6 +550,11 @@ def main():
     info = ca.ggml.device_info(0)
     log(f"[bench] device {info['name']} {info['arch']} CUs={info['compute_units']} clock={info['clock_khz']} kHz; "
         f"roofline constants: f16 dense MFMA {PEAK_F16_TFLOPS} TFLOP/s, HBM {PEAK_HBM_GBS} GB/s")
+
+    if args.relpos_only:
+        lengths = [ora.randint(5, b, 400, 750) for b in range(8)]
+        print(json.dumps({"config": "C5_fastconformer_relpos_f32", **bench_relpos(ca, ora, torch, lengths)}), flush=True)
+        return
 
     enc, host0 = bench_encoder(args, ca, ora, torch)
     line = {

@@ -618,14 +618,14 @@ int mi355x_relpos_bias(const mi355x_tensor * q_v, const mi355x_tensor * r, const
     return relpos_run(q_v, r, add, dst, scale, nullptr, (hipStream_t)stream);
 }
 
-// the mask the fused call keeps in its workspace: [Nkv, Nq, H, B] with rows padded to 16 bytes
+// the mask the fused call keeps in its workspace: [Nkv, Nq, H, B] with rows padded to whole 128-byte lines
 static void relpos_mask_view(const mi355x_tensor * q_u, const mi355x_tensor * k, void * data, mi355x_tensor * m) {
     memset(m, 0, sizeof(*m));
     m->data = data;
     m->type = MI355X_TYPE_F16;
     m->ne[0] = k->ne[1]; m->ne[1] = q_u->ne[1]; m->ne[2] = q_u->ne[2]; m->ne[3] = q_u->ne[3];
     m->nb[0] = 2;
-    m->nb[1] = ((size_t)k->ne[1] * 2 + 15) / 16 * 16;
+    m->nb[1] = ((size_t)k->ne[1] * 2 + 127) / 128 * 128;
     m->nb[2] = m->nb[1] * (size_t)q_u->ne[1];
     m->nb[3] = m->nb[2] * (size_t)q_u->ne[2];
 }

@@ -169,7 +169,7 @@ int mi355x_relpos_bias(const mi355x_tensor * q_v, const mi355x_tensor * r, const
 /*
  * The whole flash branch of that block (fastconformer.h:915-934) in one call:
  *   dst = softmax(scale * (q_u.k^T + BD) + add) . v,   BD[j, i] = <q_v[i], r[Nq-1+j-i]>
- * computed as mi355x_relpos_bias into the workspace (rows padded to 16 bytes) followed by mi355x_flash_attn_ext
+ * computed as mi355x_relpos_bias into the workspace (rows padded to whole 128-byte lines) followed by mi355x_flash_attn_ext
  * with that mask: same values as the two calls made separately.  q_u, k, v, dst, params as for
  * mi355x_flash_attn_ext (max_bias and logit_softcap must be 0); Nkv = k->ne[1].
  */

@@ -118,7 +118,7 @@ def test_fused_relpos_attention_matches_oracle_and_the_two_separate_calls(spec):
     assert_parity(got, ref, "fused " + str(spec))
     # the same through a caller's workspace, and as two calls: identical bits
     need = ggml.flash_attn_relpos_workspace_size(dq, dqv, dk, dv, dr, da, c["scale"])
-    pitch = (Nkv * 2 + 15) // 16 * 16
+    pitch = (Nkv * 2 + 127) // 128 * 128
     assert need >= pitch * Nq * H * B
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")
     got_ws = ggml.flash_attn_relpos(dq, dqv, dk, dv, dr, da, c["scale"], workspace=ws).numpy_f32()
