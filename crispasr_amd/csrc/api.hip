@@ -236,8 +236,10 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
     if (kernel == MI355X_FATTN_MMA) {
         // Very few query tiles and many keys (a short prompt against a long cache): split the keys into ranges of whole
         // 64-key tiles, one workgroup per CU.  Every split repeats the Q load and writes a partial per row, and the merge
-        // is a launch of its own - measured on the Whisper-base encoder (96 tiles x 24 key tiles) any split is a loss -
-        // so only grids below a quarter of the CUs are split, into ranges of at least four tiles.
+        // is a launch of its own, so grids below a quarter of the CUs are split into ranges of at least four tiles, and
+        // grids below half of the CUs in two when a workgroup would otherwise walk 16 tiles or more (measured: the
+        // Whisper-base encoder, 96 workgroups x 24 key tiles, 25.0 -> 22.0 us in two ranges and slower again in three;
+        // a 407-token prefill, 128 workgroups x 7 tiles, loses 2.5 us to any split).
         const int64_t rows    = (int64_t)a.Nq * a.Hq * a.B;
         const int64_t wgs     = (int64_t)((a.Nq + 127) / 128) * a.Hq * a.B;
         const int     n_tiles = (a.Nkv + 63) / 64;
@@ -249,6 +251,8 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
                 int want = (int)(cus / wgs);
                 if (want > n_tiles / 4) want = n_tiles / 4;
                 if (want >= 2) ns = want;
+            } else if (wgs * 2 <= cus && n_tiles >= 16) {
+                ns = 2;
             }
         }
         if (ns > n_tiles) ns = n_tiles;
@@ -264,12 +268,15 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
         const int64_t rows = (int64_t)a.Nq * a.Hq * a.B;
         // workgroups that exist before splitting, and the fewest keys worth a split
         const int64_t groups   = kernel == MI355X_FATTN_VEC ? rows : (int64_t)a.Hkv * a.B;
-        const int     min_keys = kernel == MI355X_FATTN_VEC ? 128 : 256;
+        // decode kernel: a split must be worth the merge launch (about 2.5 us): measured on Whisper cross-attention
+        // (64-wide heads, 1500 keys: best at 8 splits) and a Q8_0 LLM cache (128-wide, 663 keys: best at 6 to 8),
+        // while 224 keys are fastest unsplit
+        const int     min_keys = kernel == MI355X_FATTN_VEC ? 128 : (a.D <= 64 ? 192 : 96);
         int ns = p->n_splits;
         if (ns <= 0) {
             const int64_t target = (int64_t)device_cus() * (kernel == MI355X_FATTN_VEC ? 4 : 2);
             ns = (int)((target + groups - 1) / (groups > 0 ? groups : 1));
-            const int max_by_keys = (a.Nkv + min_keys - 1) / min_keys;
+            const int max_by_keys = kernel == MI355X_FATTN_VEC ? (a.Nkv + min_keys - 1) / min_keys : a.Nkv / min_keys;
             if (ns > max_by_keys) ns = max_by_keys;
         }
         if (ns > a.Nkv) ns = a.Nkv;
@@ -418,6 +425,7 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
             if (ws) {
                 if (params->workspace_size < plan.workspace)
                     return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, plan.workspace);
+                if ((uintptr_t)ws % 16) return fail(MI355X_ERR_WORKSPACE, "workspace must be 16-byte aligned");
             } else {
                 rc = get_scratch(plan.workspace, &ws);
                 if (rc) return rc;
@@ -465,6 +473,7 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
         if (ws) {
             if (params->workspace_size < plan.workspace)
                 return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, plan.workspace);
+            if ((uintptr_t)ws % 16) return fail(MI355X_ERR_WORKSPACE, "workspace must be 16-byte aligned");
         } else {
             rc = get_scratch(plan.workspace, &ws);
             if (rc) return rc;

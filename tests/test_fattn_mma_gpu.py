@@ -152,12 +152,19 @@ def test_tile_kernel_with_split_keys(spec, n_splits):
     assert_parity(run_gpu(case, kernel=ggml.KERNEL_MMA, n_splits=n_splits), ref, "splits %d %s" % (n_splits, spec))
 
 
-def test_auto_splits_keys_only_when_query_tiles_are_very_few():
+def test_auto_splits_keys_only_when_the_grid_leaves_half_the_cus_idle():
     few = make_case(seed=165, D=64, Nq=100, Nkv=2100, Hq=4, q_layout="thd", kv_layout="thd")      # 4 workgroups x 33 key tiles
     q, k, v = upload(few["q"]), upload(few["k"]), upload(few["v"])
     kern, ns = ggml.flash_attn_plan(q, k, v, None, few["scale"])
     assert kern == ggml.KERNEL_MMA and ns > 1
     assert_parity(run_gpu(few), run_oracle(few), "auto split")
-    base = make_case(seed=166, D=64, Nq=1500, Nkv=1500, Hq=8, q_layout="thd", kv_layout="thd")     # Whisper base encoder: 96 workgroups
+    base = make_case(seed=166, D=64, Nq=1500, Nkv=1500, Hq=8, q_layout="thd", kv_layout="thd")     # Whisper base encoder: 96 workgroups x 24 tiles
     kern, ns = ggml.flash_attn_plan(upload(base["q"]), upload(base["k"]), upload(base["v"]), None, base["scale"])
+    assert kern == ggml.KERNEL_MMA and ns == 2
+    assert_parity(run_gpu(base), run_oracle(base), "two ranges")
+    full = make_case(seed=167, D=64, Nq=1500, Nkv=1500, Hq=20, q_layout="thd", kv_layout="thd")    # Whisper large encoder window: no split
+    kern, ns = ggml.flash_attn_plan(upload(full["q"]), upload(full["k"]), upload(full["v"]), None, full["scale"])
+    assert kern == ggml.KERNEL_MMA and ns == 1
+    short = make_case(seed=168, D=128, Nq=407, Nkv=407, Hq=32, Hkv=8, mask="causal")                # 128 workgroups x 7 tiles: no split
+    kern, ns = ggml.flash_attn_plan(upload(short["q"]), upload(short["k"]), upload(short["v"]), upload(short["mask"]), short["scale"])
     assert kern == ggml.KERNEL_MMA and ns == 1
