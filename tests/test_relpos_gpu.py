@@ -141,3 +141,25 @@ def test_relpos_contract_violations_are_reported():
     c80 = dict(qv=ora.from_f32(ora.randn(1, (1, 1, 4, 80))), r=ora.from_f32(ora.randn(2, (1, 1, 7, 80))))
     with pytest.raises(ggml.UnsupportedError):
         ggml.relpos_bias(upload(c80["qv"]), upload(c80["r"]), None, 0.1, 4)
+
+
+def _draw(seed: int) -> dict:
+    """a seeded random rel-pos case: sizes off the tile grid, broadcast tables, both table and add types, layouts"""
+    r = lambda i, lo, hi: ora.randint(9000 + seed, i, lo, hi)
+    H = r(0, 1, 4)
+    B = r(1, 1, 3)
+    return dict(seed=400 + seed, D=(64, 128)[r(2, 0, 1)], Nq=r(3, 1, 150), Nkv=r(4, 1, 330), H=H, B=B,
+                Br=(1, B)[r(5, 0, 1)], rtype=(ora.F32, ora.F16)[r(6, 0, 1)],
+                add=(None, "pad", "local", "perhead")[r(7, 0, 3)], layout=("cont", "thd")[r(8, 0, 1)],
+                add_type=(ora.F32, ora.F16)[r(9, 0, 1)])
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_relpos_mask_random_shapes(seed):
+    spec = _draw(seed)
+    c = make(**spec)
+    ref = ora.relpos_bias(c["qv"], c["r"], c["add"], c["scale"], c["Nkv"])
+    got = ggml.relpos_bias(upload(c["qv"]), upload(c["r"]), upload(c["add"]) if c["add"] is not None else None,
+                           c["scale"], c["Nkv"])
+    n = c["Nkv"] * c["Nq"] * c["H"] * c["B"]
+    check_mask(got.to_host()[: 2 * n].view(np.uint16), ref.buf.view(np.uint16), str(spec))
