@@ -604,12 +604,11 @@ static int relpos_run(const mi355x_tensor * qv, const mi355x_tensor * r, const m
         a.add = (const char *)add->data; a.nba1 = add->nb[1]; a.nba2 = add->nb[2]; a.nba3 = add->nb[3];
         a.Ha = (int)add->ne[2]; a.Ba = (int)add->ne[3];
         a.add_f16 = add->type == MI355X_TYPE_F16;
-        const size_t pair = 2 * type_size(add->type);
-        a.add_vec = !((uintptr_t)add->data % pair) && !(add->nb[1] % pair) && !(add->nb[2] % pair) && !(add->nb[3] % pair);
     }
     a.out = (char *)dst->data; a.nbo1 = dst->nb[1]; a.nbo2 = dst->nb[2]; a.nbo3 = dst->nb[3];
     a.out_al4 = !((uintptr_t)dst->data % 4) && !(dst->nb[1] % 4) && !(dst->nb[2] % 4) && !(dst->nb[3] % 4);
     a.scale = scale;
+    a.n_cus = device_cus();
     const int e = relpos_bias_launch(a, MI355X_TYPE_F16, st);
     if (e) return hip_fail((hipError_t)e, "relpos_bias launch");
     return MI355X_OK;

@@ -110,12 +110,12 @@ struct RelposArgs {
     const char * r;   size_t nbr1, nbr2, nbr3; int32_t Hr, Br;   // F32 | F16 [D, Nq+Nkv-1, Hr, Br]
     const char * add; size_t nba1, nba2, nba3; int32_t Ha, Ba;   // optional F32 | F16 [>=Nkv, >=Nq, Ha, Ba]
     int32_t add_f16;
-    int32_t add_vec;                                            // a pair of add values can be read with one load (alignment)
     char *       out; size_t nbo1, nbo2, nbo3;                  // F16 [Nkv, Nq, H, B], rows contiguous
     int32_t out_al4;                                            // out base and strides are multiples of 4 bytes
     int32_t D, Nq, Nkv, H, B;
     float   scale;
-    int32_t n_qblocks, n_chunks;                                // filled in by the launcher
+    int32_t n_cus;                                              // CUs of the device (0 = unknown)
+    int32_t n_qblocks, n_chunks, chunk_tiles;                   // filled in by the launcher
 };
 
 // Launchers implemented next to their kernels; all return hipError_t as int.

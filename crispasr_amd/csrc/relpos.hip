@@ -7,19 +7,25 @@
 // ggml_flash_attn_ext as its mask.  The products run on v_mfma_f32_32x32x16_f16 (Q_v and R rounded to f16, f32
 // accumulation); scale, add and the final rounding are done in f32 exactly as the graph does them.
 //
-// A wave owns 32 queries of one (head, batch) and a run of 64-key tiles.  It walks R in blocks of 32 rows:
-// block n x the 32 queries is one 32x32 accumulator whose element (row, query il) belongs to key
-// j = 32n + row + il - 31 (relative to the wave's first query) - a shift that differs per lane, so the block is
-// scattered into a wave-private LDS ring [query][key mod 128] and the finished 64-key tile is read back row-wise
-// and written out in full 128-byte rows.  Tile t needs blocks 2t, 2t+1, 2t+2; block 2t+2 is also tile t+1's
-// first, so each further tile costs two blocks.
+// A workgroup of 4 waves owns 128 consecutive queries of one (head, batch) - 32 per wave - and a run of 32-key
+// tiles.  R is walked in blocks of 32 rows: block n x a wave's 32 queries is one 32x32 accumulator whose element
+// (row, query il) belongs to key j = 32n + row + il - 31 (relative to the wave's first query) - a shift that differs
+// per lane.  Tile t (keys 32t .. 32t+31) is made of the lower-right triangle of block t (row + il >= 31) and the
+// upper-left triangle of block t+1 (row + il <= 30): for one accumulator slot the two candidate columns differ by
+// exactly 32, so exactly one of the two blocks owns that slot's place in the tile.  A wave therefore keeps the
+// previous block's accumulator in registers, computes one new block per tile, selects per slot, and writes the
+// 32x32 tile into a wave-private LDS square from which it is read back row-wise, scaled, added to the optional mask
+// and stored with 128-bit stores.  One block of MFMAs per 32 keys, no result computed twice.
 //
-// MFMA operands want lane = row with 8 consecutive d, which as a global access pattern is 64 scattered 16-byte
-// pieces per instruction.  Rows are therefore fetched coalesced (adjacent lanes = adjacent 16 bytes of a row), 64
-// values of d at a time, converted to f16 and passed through a wave-private 32 x 64 staging block in LDS
-// (16-byte chunks XOR-swizzled so that both the row-wise writes and the operand reads are conflict-free); the next
-// block's global loads are in flight while the current one is multiplied and scattered.  Waves never synchronise with each other.
+// The four waves need the same rows of R one step apart (wave w's block n is wave 0's block n - w), so the table
+// blocks are staged once per workgroup: every step all 256 threads fetch one new block coalesced (adjacent lanes =
+// adjacent 16 bytes of a row) into a ring of six f16 blocks in LDS (16-byte chunks XOR-swizzled so that the row-wise
+// writes and the MFMA operand reads - lane = row, 8 consecutive d - are both conflict-free), one barrier per step;
+// each wave reads its operands from the slot that holds its block.  A quarter of the table traffic and of the
+// staging work of a wave-private scheme.  Q_v goes through the same slots once, before the loop.
 #include "fattn_common.h"
+
+#include <stdlib.h>
 
 namespace {
 
@@ -29,11 +35,9 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float    float16v __attribute__((ext_vector_type(16)));
 
 constexpr int RP_WAVES       = 4;
-constexpr int RP_CHUNK_TILES = 4;      // 64-key tiles per wave
-constexpr int RP_RING        = 128;    // keys per ring row
-constexpr int RP_RING_BYTES  = 32 * RP_RING * 4;
-constexpr int RP_STAGE_BYTES = 32 * 64 * 2;
-constexpr int RP_LDS_BYTES   = RP_WAVES * (RP_RING_BYTES + RP_STAGE_BYTES);
+constexpr int RP_TILE_BYTES  = 32 * 32 * 4;
+constexpr int RP_SLAB_BYTES  = 32 * 64 * 2;            // 32 rows x 64 values of d, f16
+constexpr int RP_SLOTS       = 6;                      // table blocks resident per workgroup
 
 // swizzle of the staging block's eight 16-byte chunks per row
 __device__ __forceinline__ int rp_swz(int r) { return (r >> 1) & 7; }
@@ -90,11 +94,14 @@ __device__ __forceinline__ void slab_operands(const char * stage, int l32, int h
 
 template <int D, int RTYPE>
 __global__ void __launch_bounds__(RP_WAVES * 64, 2) relpos_bias_kernel(const RelposArgs a) {
-    constexpr int NSLAB = D / 64;                 // slabs per 32-row block
-    extern __shared__ __attribute__((aligned(16))) char rp_lds[];
+    constexpr int NSLAB      = D / 64;                 // slabs per 32-row block
+    constexpr int SLOT_BYTES = NSLAB * RP_SLAB_BYTES;
+    constexpr int NLD        = SLOT_BYTES / 16 / (RP_WAVES * 64);      // 16-byte pieces per thread and block
+    extern __shared__ __attribute__((aligned(16))) char rp_lds[];        // RP_SLOTS table blocks, then 2 squares per wave
 
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63;
+    const int tid  = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
     const int l32  = lane & 31;
     const int hh   = lane >> 5;
 
@@ -106,23 +113,26 @@ __global__ void __launch_bounds__(RP_WAVES * 64, 2) relpos_bias_kernel(const Rel
     const int n_qgroups = (a.n_qblocks + RP_WAVES - 1) / RP_WAVES;
     const int64_t s_idx = blockIdx.x >> 3;
     const int64_t group = (s_idx / per_group) * 8 + (blockIdx.x & 7);
-    if (group >= (int64_t)n_qgroups * a.B) return;                // waves are independent: no barriers below
+    if (group >= (int64_t)n_qgroups * a.B) return;                // the whole workgroup leaves
     const int w  = (int)(s_idx % per_group);
     const int h  = w % a.H;
     const int ch = w / a.H;
     const int b  = (int)(group / n_qgroups);
-    const int qb = (int)(group % n_qgroups) * RP_WAVES + wave;
-    if (qb >= a.n_qblocks) return;
-
-    const int i0      = qb * 32;
-    const int n_tiles = (a.Nkv + 63) / 64;
-    const int t_begin = ch * RP_CHUNK_TILES;
-    const int t_end   = min(n_tiles, t_begin + RP_CHUNK_TILES);
+    const int qg = (int)(group % n_qgroups);
+    // a wave whose query block lies past Nq keeps step with the others (barriers, table loads) and stores nothing
+    const int i0      = (qg * RP_WAVES + wave) * 32;
+    const int n_tiles = (a.Nkv + 31) / 32;
+    const int t_begin = ch * a.chunk_tiles;                       // even: chunk_tiles is
+    const int t_end   = min(n_tiles, t_begin + a.chunk_tiles);
     const int NR      = a.Nq + a.Nkv - 1;
-    const int p_base  = a.Nq - 1 - i0 - 31;            // R row of (block 0, row 0); may be negative
+    // table row of (block m, row 0) in wave 0's numbering; wave w's block n is block m = n - w.  May be negative.
+    const int p_base0 = a.Nq - 1 - qg * RP_WAVES * 32 - 31;
+    const int m_first = t_begin - (RP_WAVES - 1);                 // first block the workgroup stages
 
-    float * ring  = (float *)(rp_lds + wave * RP_RING_BYTES);
-    char *  stage = rp_lds + RP_WAVES * RP_RING_BYTES + wave * RP_STAGE_BYTES;
+    typedef __attribute__((address_space(3))) float lds_float;
+    char *  slots = rp_lds;
+    float * tile  = (float *)(rp_lds + RP_SLOTS * SLOT_BYTES + wave * 2 * RP_TILE_BYTES);      // squares of an even and an odd tile
+    auto slot_of = [&](int m) { return slots + ((m - m_first) % RP_SLOTS) * SLOT_BYTES; };
 
     const char * qbase = a.qv + (int64_t)h * a.nbq2 + (int64_t)b * a.nbq3;
     const char * rbase = a.r + (int64_t)(h % a.Hr) * a.nbr2 + (int64_t)(b % a.Br) * a.nbr3;
@@ -135,179 +145,195 @@ __global__ void __launch_bounds__(RP_WAVES * 64, 2) relpos_bias_kernel(const Rel
     // outside [0, Nq) x [0, Nkv), which are never stored.
     auto qrow = [&](int row) { return qbase + (uint32_t)min(i0 + row, a.Nq - 1) * (uint32_t)a.nbq1; };
 
-    // B operands: the wave's 32 queries, all of d, through the staging block (all loads in flight together)
+    // Piece j of a block for this thread: 16 bytes = chunk c of row `row` of slab sl (table rows are contiguous f16,
+    // the launcher sees to it)
+    u32x4 piece[NLD];
+    auto request = [&](int m) __attribute__((always_inline)) {
+        const int p0 = p_base0 + 32 * m;
+#pragma unroll
+        for (int j = 0; j < NLD; j++) {
+            const int idx = j * (RP_WAVES * 64) + tid;
+            const int sl = idx >> 8, row = (idx & 255) >> 3, c = idx & 7;
+            const int p = min(max(p0 + row, 0), NR - 1);
+            piece[j] = *(const u32x4 *)(rbase + (uint32_t)p * (2u * D) + (uint32_t)(sl * 128 + c * 16));
+        }
+    };
+    // blocks m_first .. t_begin + 1 (what the first step of all four waves needs) are requested right away, together
+    // with Q_v: one memory latency for the whole prologue
+    u32x4 first[RP_WAVES + 1][NLD];
+#pragma unroll
+    for (int i = 0; i <= RP_WAVES; i++) {
+        request(m_first + i);
+#pragma unroll
+        for (int j = 0; j < NLD; j++) first[i][j] = piece[j];
+    }
+
+    // B operands: the wave's 32 queries, all of d, through the wave's own slot (all loads in flight together)
     half8 qv[NSLAB][4];
     {
+        char * mine = slots + wave * SLOT_BYTES;
         RawSlab<MI355X_TYPE_F32> qraw[NSLAB];
 #pragma unroll
         for (int sl = 0; sl < NSLAB; sl++) slab_load<MI355X_TYPE_F32>(qraw[sl], lane, sl * 64, qrow);
 #pragma unroll
-        for (int sl = 0; sl < NSLAB; sl++) {
-            slab_store<MI355X_TYPE_F32>(qraw[sl], lane, stage);
-            __builtin_amdgcn_wave_barrier();
-            slab_operands(stage, l32, hh, qv[sl]);
-            __builtin_amdgcn_wave_barrier();
-        }
+        for (int sl = 0; sl < NSLAB; sl++) slab_store<MI355X_TYPE_F32>(qraw[sl], lane, mine + sl * RP_SLAB_BYTES);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int sl = 0; sl < NSLAB; sl++) slab_operands(mine + sl * RP_SLAB_BYTES, l32, hh, qv[sl]);
     }
 
-    // accumulator slot gg*4+e of lane (l32, hh) = row 8gg + 4hh + e of the block, query l32.  Byte address in the
-    // ring = row base | ((4*column) mod 512): the wave's ring is 512-byte aligned, so the OR is an addition.
-    typedef __attribute__((address_space(3))) float lds_float;
-    const uint32_t ring_row = (uint32_t)(uintptr_t)(lds_float *)ring + (uint32_t)l32 * (RP_RING * 4);
-    auto scatter = [&](int n, const float16v & g) __attribute__((always_inline)) {
-        const uint32_t x4 = (uint32_t)(32 * n + 4 * hh + l32 - 31) * 4u;
+    auto stage = [&](int m) __attribute__((always_inline)) {
+        char * dst = slot_of(m);
 #pragma unroll
-        for (int gg = 0; gg < 4; gg++)
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-                *(lds_float *)(uintptr_t)(ring_row | ((x4 + (uint32_t)(8 * gg + e) * 4u) & (RP_RING * 4 - 1))) = g[gg * 4 + e];
-    };
-
-    // A tile is written out in 16 steps of 2 query rows x 64 keys: lane (l32, hh) handles keys 2*l32, 2*l32+1 of
-    // row 2k + hh.  Whole tiles of whole query blocks (the common case) take a path without per-element tests.
-    const bool rows_full = i0 + 32 <= a.Nq;
-    float ad[16][2];               // add values of the next tile to be written, requested a tile ahead
-#pragma unroll
-    for (int k = 0; k < 16; k++) ad[k][0] = ad[k][1] = 0.0f;
-    auto request_add = [&](int t) __attribute__((always_inline)) {
-        if (!abase) return;
-        const int j = 64 * t + 2 * l32;
-        if (rows_full && 64 * t + 64 <= a.Nkv && a.add_vec) {
-            uint32_t off = (uint32_t)(i0 + hh) * (uint32_t)a.nba1 + (uint32_t)j * (a.add_f16 ? 2u : 4u);
-            const uint32_t step = 2u * (uint32_t)a.nba1;
-            if (a.add_f16) {
-#pragma unroll
-                for (int k = 0; k < 16; k++, off += step) {
-                    const half2v w = *(const half2v *)(abase + off);
-                    ad[k][0] = (float)w[0]; ad[k][1] = (float)w[1];
-                }
-            } else {
-#pragma unroll
-                for (int k = 0; k < 16; k++, off += step) {
-                    const float2 w = *(const float2 *)(abase + off);
-                    ad[k][0] = w.x; ad[k][1] = w.y;
-                }
-            }
-            return;
-        }
-        const bool two = j + 1 < a.Nkv;
-#pragma unroll
-        for (int k = 0; k < 16; k++) {
-            ad[k][0] = ad[k][1] = 0.0f;
-            const int i = i0 + 2 * k + hh;
-            if (i < a.Nq && j < a.Nkv) {
-                const char * ap = abase + (uint32_t)i * (uint32_t)a.nba1;
-                if (a.add_f16) {
-                    ad[k][0] = (float)*(const _Float16 *)(ap + j * 2);
-                    if (two) ad[k][1] = (float)*(const _Float16 *)(ap + j * 2 + 2);
-                } else {
-                    ad[k][0] = *(const float *)(ap + j * 4);
-                    if (two) ad[k][1] = *(const float *)(ap + j * 4 + 4);
-                }
-            }
+        for (int j = 0; j < NLD; j++) {
+            const int idx = j * (RP_WAVES * 64) + tid;
+            const int sl = idx >> 8, row = (idx & 255) >> 3, c = idx & 7;
+            *(u32x4 *)(dst + sl * RP_SLAB_BYTES + row * 128 + ((c ^ rp_swz(row)) * 16)) = piece[j];
         }
     };
-    // scale, add and the rounding to f16 as the graph's nodes do them: an f32 multiply, an f32 add (not fused), RNE
-    auto finish = [&](float g, float add) { return (_Float16)__fadd_rn(__fmul_rn(g, a.scale), add); };
-    auto flush = [&](int t) __attribute__((always_inline)) {
-        __builtin_amdgcn_wave_barrier();
-        const int j = 64 * t + 2 * l32;
-        const float * rp = ring + hh * RP_RING + (j & (RP_RING - 1));
-        if (rows_full && 64 * t + 64 <= a.Nkv && a.out_al4) {
-            uint32_t off = (uint32_t)(i0 + hh) * (uint32_t)a.nbo1 + (uint32_t)j * 2u;
-            const uint32_t step = 2u * (uint32_t)a.nbo1;
-#pragma unroll
-            for (int k = 0; k < 16; k++, off += step) {
-                const float2 g2 = *(const float2 *)(rp + k * 2 * RP_RING);
-                half2v hv;
-                hv[0] = finish(g2.x, ad[k][0]);
-                hv[1] = finish(g2.y, ad[k][1]);
-                *(half2v *)(obase + off) = hv;
-            }
-        } else {
-            const bool two = j + 1 < a.Nkv;
-#pragma unroll
-            for (int k = 0; k < 16; k++) {
-                const int i = i0 + 2 * k + hh;
-                const float2 g2 = *(const float2 *)(rp + k * 2 * RP_RING);
-                if (i < a.Nq && j < a.Nkv) {
-                    const _Float16 h0 = finish(g2.x, ad[k][0]), h1 = finish(g2.y, ad[k][1]);
-                    char * op = obase + (uint32_t)i * (uint32_t)a.nbo1 + (uint32_t)j * 2u;
-                    if (two && a.out_al4) {
-                        half2v hv = {h0, h1};
-                        *(half2v *)op = hv;
-                    } else {
-                        *(_Float16 *)op = h0;
-                        if (two) *(_Float16 *)(op + 2) = h1;
-                    }
-                }
-            }
-        }
-        __builtin_amdgcn_wave_barrier();
-        if (t + 1 < t_end) request_add(t + 1);
-    };
-
-    // blocks 2*t_begin .. 2*t_end in order (an even count plus one); the rows of two blocks ahead are in flight
-    // while one is multiplied and scattered
-    const int n0 = 2 * t_begin, n_last = 2 * t_end;
-    // The table's rows are contiguous f16 (the launcher sees to it), so a block that lies inside the table is a
-    // wave-uniform base plus a fixed lane offset; only the first and last blocks need their rows clamped.
-    const uint32_t lane_roff = (uint32_t)(lane >> 3) * (2u * D) + (uint32_t)(lane & 7) * 16u;
-    auto request = [&](int n, RawSlab<RTYPE> (&raw)[NSLAB]) __attribute__((always_inline)) {
-        const int p0 = p_base + 32 * n;
-        if (p0 >= 0 && p0 + 31 <= NR - 1) {
-            const char * bp = rbase + (uint32_t)p0 * (2u * D);
-#pragma unroll
-            for (int sl = 0; sl < NSLAB; sl++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) raw[sl].v[j] = *(const u32x4 *)(bp + lane_roff + (uint32_t)(j * 8 * 2 * D + sl * 128));
-        } else {
-            auto rrow = [&](int row) { return rbase + (uint32_t)min(max(p0 + row, 0), NR - 1) * (2u * D); };
-#pragma unroll
-            for (int sl = 0; sl < NSLAB; sl++) slab_load<RTYPE>(raw[sl], lane, sl * 64, rrow);
-        }
-    };
-    // stage the block held in raw, refill raw with block n_next (if any), multiply, scatter
-    auto block = [&](int n, int n_next, RawSlab<RTYPE> (&raw)[NSLAB]) __attribute__((always_inline)) {
-        float16v g;
+    // this wave's block n (= staged block n - wave) -> accumulator
+    auto multiply = [&](int n, float16v & g) __attribute__((always_inline)) {
+        const char * src = slot_of(n - wave);
 #pragma unroll
         for (int e = 0; e < 16; e++) g[e] = 0.0f;
 #pragma unroll
         for (int sl = 0; sl < NSLAB; sl++) {
             half8 ra[4];
-            slab_store<RTYPE>(raw[sl], lane, stage);
-            __builtin_amdgcn_wave_barrier();
-            slab_operands(stage, l32, hh, ra);
-            __builtin_amdgcn_wave_barrier();
-            if (sl == NSLAB - 1 && n_next <= n_last) request(n_next, raw);
+            slab_operands(src + sl * RP_SLAB_BYTES, l32, hh, ra);
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) g = __builtin_amdgcn_mfma_f32_32x32x16_f16(ra[ks], qv[sl][ks], g, 0, 0, 0);
         }
-        scatter(n, g);
     };
-    RawSlab<RTYPE> raw_even[NSLAB], raw_odd[NSLAB];
-    request(n0, raw_even);
-    request(n0 + 1, raw_odd);            // n_last >= n0 + 2: a chunk holds at least one tile
+
+    // Accumulator slot gg*4+e of lane (l32, hh) is row rho = 8gg + 4hh + e of its block, query l32.  Its place in
+    // tile t is column rho + l32 - 31 if that is >= 0 (the value of block t), else that column + 32 (block t+1).
+    const uint32_t tile_row = (uint32_t)(uintptr_t)(lds_float *)tile + (uint32_t)l32 * 128u;
+    const int      c_lane   = 4 * hh + l32 - 31;
+    auto compose = [&](const float16v & g_lo, const float16v & g_hi, int odd) __attribute__((always_inline)) {
+#pragma unroll
+        for (int gg = 0; gg < 4; gg++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int   c = c_lane + 8 * gg + e;
+                const float x = c >= 0 ? g_lo[gg * 4 + e] : g_hi[gg * 4 + e];
+                *(lds_float *)(uintptr_t)(tile_row + (uint32_t)odd * RP_TILE_BYTES + (((uint32_t)c & 31u) << 2)) = x;
+            }
+    };
+
+    // Tiles are written out in pairs (an even tile and the odd one after it: 64 keys, whole 128-byte lines when the
+    // output rows are padded to lines) in 4 steps of 8 query rows: lane handles keys 8*(lane%8) .. +7 of the pair in
+    // row 8k + lane/8 - a 128-bit store and 2 x 128-bit loads of the add mask when all 8 keys exist and the output
+    // rows are dword-aligned, element by element otherwise (the end of a row, odd layouts).  Rows past Nq are
+    // computed from the clamped last row and not stored.  The add values of a pair are requested a pair ahead.
+    typedef float    f32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+    typedef _Float16 f16x8_a4 __attribute__((ext_vector_type(8), aligned(4)));
+    typedef _Float16 f16x8_a2 __attribute__((ext_vector_type(8), aligned(2)));
+    const int frow = lane >> 3, fkey = 8 * (lane & 7);               // fkey: key offset inside the pair
+    auto keys_left = [&](int t) { return min(max(a.Nkv - (32 * t + fkey), 0), 8); };      // t even; of this lane's 8
+    float ad[4][8];
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) ad[k][e] = 0.0f;
+    auto request_add = [&](int t) __attribute__((always_inline)) {
+        if (!abase || keys_left(t) < 8) return;                      // partial lanes read theirs element by element
+        const uint32_t es = a.add_f16 ? 2u : 4u;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t off = (uint32_t)min(i0 + frow + 8 * k, a.Nq - 1) * (uint32_t)a.nba1 + (uint32_t)(32 * t + fkey) * es;
+            if (a.add_f16) {
+                const f16x8_a2 wv = *(const f16x8_a2 *)(abase + off);
+#pragma unroll
+                for (int e = 0; e < 8; e++) ad[k][e] = (float)wv[e];
+            } else {
+                const f32x4_a4 w0 = *(const f32x4_a4 *)(abase + off), w1 = *(const f32x4_a4 *)(abase + off + 16);
+#pragma unroll
+                for (int e = 0; e < 4; e++) { ad[k][e] = w0[e]; ad[k][4 + e] = w1[e]; }
+            }
+        }
+    };
+    // scale, add and the rounding to f16 as the graph's nodes do them: an f32 multiply, an f32 add (not fused), RNE
+    auto finish = [&](float g, float add) { return (_Float16)__fadd_rn(__fmul_rn(g, a.scale), add); };
+    auto flush = [&](int t) __attribute__((always_inline)) {         // t even: tiles t and t + 1
+        __builtin_amdgcn_wave_barrier();
+        const int nk = keys_left(t);
+        const float * rp = tile + (fkey >> 5) * (RP_TILE_BYTES / 4) + frow * 32 + (fkey & 31);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int i = i0 + frow + 8 * k;
+            const float4 x0 = *(const float4 *)(rp + k * 8 * 32), x1 = *(const float4 *)(rp + k * 8 * 32 + 4);
+            const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+            if (i < a.Nq && nk > 0) {
+                char * op = obase + (uint32_t)i * (uint32_t)a.nbo1 + (uint32_t)(32 * t + fkey) * 2u;
+                if (nk == 8 && a.out_al4) {
+                    f16x8_a4 hv;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) hv[e] = finish(x[e], ad[k][e]);
+                    *(f16x8_a4 *)op = hv;
+                } else {
+                    const char * ap = abase ? abase + (uint32_t)i * (uint32_t)a.nba1 + (uint32_t)(32 * t + fkey) * (a.add_f16 ? 2u : 4u) : nullptr;
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        if (e < nk) {
+                            float av = 0.0f;
+                            if (ap) av = nk == 8 ? ad[k][e] : (a.add_f16 ? (float)((const _Float16 *)ap)[e] : ((const float *)ap)[e]);
+                            ((_Float16 *)op)[e] = finish(x[e], av);
+                        }
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (t + 2 < t_end) request_add(t + 2);
+    };
+
+    // Prologue: the Q_v slots are free once every wave has its operands; then the blocks requested at the start
+    // are staged.
+    __syncthreads();
+    {
+#pragma unroll
+        for (int i = 0; i <= RP_WAVES; i++) {
+#pragma unroll
+            for (int j = 0; j < NLD; j++) piece[j] = first[i][j];
+            stage(m_first + i);
+        }
+    }
+    if (t_begin + 2 <= t_end) request(t_begin + 2);
     request_add(t_begin);
-    for (int n = n0; n <= n_last; n += 2) {
-        block(n, n + 2, raw_even);
-        if (n > n0) flush(n / 2 - 1);
-        if (n + 1 <= n_last) block(n + 1, n + 3, raw_odd);
+    __syncthreads();
+    float16v g0, g1;
+    multiply(t_begin, g0);
+    // Step t: block t + 2 (requested a step ago) goes into the slot whose last readers finished two steps ago - the
+    // barrier of the step between makes that safe - and block t + 3 is requested; the wave multiplies its block t + 1,
+    // which was staged a step ago and published by that step's barrier.  Unrolled by two so that both accumulators
+    // stay in registers.
+    auto step = [&](int t, const float16v & g_lo, float16v & g_hi, int odd) __attribute__((always_inline)) {
+        if (t + 2 <= t_end) stage(t + 2);
+        if (t + 3 <= t_end) request(t + 3);
+        __syncthreads();
+        multiply(t + 1, g_hi);
+        compose(g_lo, g_hi, odd);
+    };
+    for (int t = t_begin; t < t_end; t += 2) {          // t_begin is even: pairs start on 64-key boundaries
+        step(t, g0, g1, 0);
+        if (t + 1 < t_end) step(t + 1, g1, g0, 1);
+        flush(t);                                       // a missing odd tile lies past Nkv: its lanes store nothing
     }
 }
 
 template <int D, int RTYPE>
 int launch_dt(const RelposArgs & a, hipStream_t stream) {
-    static bool attr_set = false;     // per instantiation: the dynamic LDS exceeds the 64 KiB default
-    if (!attr_set) {
+    constexpr int LDS = RP_SLOTS * (D / 64) * RP_SLAB_BYTES + RP_WAVES * 2 * RP_TILE_BYTES;
+    static bool attr_set = false;     // per instantiation; the attribute only matters above 64 KiB
+    if (!attr_set && LDS > 64 * 1024) {
         const hipError_t e = hipFuncSetAttribute((const void *)relpos_bias_kernel<D, RTYPE>,
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, RP_LDS_BYTES);
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
         if (e != hipSuccess) return (int)e;
         attr_set = true;
     }
     const int64_t groups = (int64_t)((a.n_qblocks + RP_WAVES - 1) / RP_WAVES) * a.B;
     const dim3 grid((unsigned)((groups + 7) / 8 * 8 * a.n_chunks * a.H));
-    hipLaunchKernelGGL((relpos_bias_kernel<D, RTYPE>), grid, dim3(RP_WAVES * 64), RP_LDS_BYTES, stream, a);
+    hipLaunchKernelGGL((relpos_bias_kernel<D, RTYPE>), grid, dim3(RP_WAVES * 64), LDS, stream, a);
     return (int)hipGetLastError();
 }
 
@@ -324,7 +350,26 @@ int launch_d(const RelposArgs & a, int rtype, hipStream_t stream) {
 int relpos_bias_launch(RelposArgs a, int rtype, hipStream_t stream) {
     if (a.Nq <= 0 || a.Nkv <= 0 || a.H <= 0 || a.B <= 0) return 0;
     a.n_qblocks = (a.Nq + 31) / 32;
-    a.n_chunks  = ((a.Nkv + 63) / 64 + RP_CHUNK_TILES - 1) / RP_CHUNK_TILES;
+    // Keys are cut into chunks of an even number of 32-key tiles, one workgroup per (4 query blocks, head, chunk).
+    // A workgroup costs a prologue worth about 6 tiles (Q_v, the first table blocks) plus its tiles, and workgroups run
+    // in rounds of `slots` at a time: take the chunk size with the cheapest rounds x (6 + tiles), the longer on a tie
+    // (measured at 8 heads x 128, T = 750, batch 8: 24 tiles 50 us, 12: 52, 8: 53, 6: 57, 4: 59).
+    {
+        const int     n_tiles = (a.Nkv + 31) / 32;
+        const int64_t groups  = (int64_t)((a.n_qblocks + RP_WAVES - 1) / RP_WAVES) * a.B * a.H;
+        const int64_t slots   = (int64_t)(a.n_cus > 0 ? a.n_cus : 256) * (a.D == 64 ? 3 : 2);
+        int64_t best_cost = -1;
+        int     best = 2;
+        for (int c = 2; c <= ((n_tiles + 1) & ~1); c += 2) {
+            const int64_t wgs  = groups * ((n_tiles + c - 1) / c);
+            const int64_t cost = ((wgs + slots - 1) / slots) * (6 + c);
+            if (best_cost < 0 || cost < best_cost || (cost == best_cost && c > best)) { best_cost = cost; best = c; }
+        }
+        static const char * force = getenv("MI355X_RELPOS_CHUNK");          // experiments only
+        if (force && atoi(force) >= 2) best = atoi(force) & ~1;
+        a.chunk_tiles = best;
+        a.n_chunks    = (n_tiles + best - 1) / best;
+    }
     if ((int64_t)a.n_qblocks * a.n_chunks * a.H * a.B > ((int64_t)1 << 33)) return (int)hipErrorInvalidValue;
     // 32-bit offsets inside a (head, batch) plane
     const uint64_t lim = (uint64_t)1 << 31;
