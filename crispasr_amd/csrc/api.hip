@@ -153,6 +153,7 @@ int check(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor 
         if (dst->ne[0] != D || dst->ne[1] != Hq || dst->ne[2] != Nq || dst->ne[3] != B)
             return fail(MI355X_ERR_INVALID, "dst must be [DV, Hq, Nq, B]");
         if (!is_contiguous(dst)) return fail(MI355X_ERR_UNSUPPORTED, "dst must be contiguous");
+        if ((uintptr_t)dst->data % 16) return fail(MI355X_ERR_UNSUPPORTED, "dst must be 16-byte aligned (128-bit stores)");
     }
     if (Nq * Hq * B > (int64_t)1 << 26 || Nkv > (int64_t)1 << 30) return fail(MI355X_ERR_UNSUPPORTED, "problem too large");
     if (p->prec != 0 && p->prec != 10) return fail(MI355X_ERR_INVALID, "unknown prec %d", p->prec);

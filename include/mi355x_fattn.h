@@ -110,7 +110,7 @@ int mi355x_stream_synchronize(void * stream);
 /* ---- GGML_OP_FLASH_ATTN_EXT ------------------------------------------------------------ */
 
 /*
- * dst[DV, Hq, Nq, B] (f32, contiguous) = softmax(scale * q.k^T [soft-capped] + slope(h) * mask) . v
+ * dst[DV, Hq, Nq, B] (f32, contiguous, 16-byte aligned) = softmax(scale * q.k^T [soft-capped] + slope(h) * mask) . v
  *
  *   q    F32  [D,  Nq,  Hq,  B ]   any strides with nb[0] == 4
  *   k    F16 | F32 | Q8_0 [D,  Nkv, Hkv, Bk]   rows contiguous (nb[0] == type size)

@@ -114,3 +114,26 @@ def test_native_host_driver_runs_the_bench_protocol():
     out = json.loads(res.stdout.strip().splitlines()[-1])
     assert out["layers"] == 4 and out["self_check_max_abs"] <= 2e-3
     assert out["single_token_x256"]["us_per_attention_call"] > 0
+
+
+def test_relpos_bias_supports_predicate():
+    """the predicate a backend's supports_op would ask before claiming FastConformer's mask-building node chain"""
+    L = ggml.lib()
+
+    def sup(qv, r, add, dst):
+        return L.mi355x_relpos_bias_supports(qv.ref(), r.ref(), add.ref() if add is not None else None, dst.ref())
+
+    T, H = 750, 8
+    qv = _t(ca.F32, (128, T, H, 1), (4, 1024 * 4, 128 * 4, T * 1024 * 4))          # permuted view of a [1024, T] activation
+    r = _t(ca.F32, (128, 2 * T - 1, H, 1), (4, 1024 * 4, 128 * 4, (2 * T - 1) * 1024 * 4))
+    dst = _t(ca.F16, (T, T, H, 1))
+    assert sup(qv, r, None, dst) == ggml.OK
+    assert sup(qv, r, _t(ca.F32, (T, T, 1, 1)), dst) == ggml.OK                      # pad / window mask, all heads
+    assert sup(qv, _t(ca.F16, (128, 2 * T - 1, H, 1)), None, dst) == ggml.OK
+    assert sup(qv, _t(ca.F32, (128, 2 * T - 2, H, 1)), None, dst) == ggml.ERR_INVALID    # table one row short
+    assert sup(qv, r, _t(ca.F32, (T - 1, T, 1, 1)), dst) == ggml.ERR_INVALID             # add narrower than the keys
+    assert sup(qv, r, None, _t(ca.F32, (T, T, H, 1))) == ggml.ERR_INVALID                # the mask is F16
+    assert sup(qv, r, None, _t(ca.F16, (T, T, H, 2))) == ggml.ERR_INVALID                # batch mismatch
+    q80 = _t(ca.F32, (80, 16, 2, 1))
+    assert sup(q80, _t(ca.F32, (80, 31, 2, 1)), None, _t(ca.F16, (16, 16, 2, 1))) == ggml.ERR_UNSUPPORTED   # head size
+    assert sup(_t(ca.F16, (128, T, H, 1)), r, None, dst) == ggml.ERR_UNSUPPORTED         # Q_v must be F32
