@@ -34,7 +34,7 @@ SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("n_splits", [1, 0, 3])
+@pytest.mark.parametrize("n_splits", [1, 0, 3, 11])       # 11: more splits than the merge kernel fetches in one batch
 @pytest.mark.parametrize("spec", SHAPES, ids=lambda s: "seed%d" % s["seed"])
 def test_vec_kernel_matches_oracle(spec, n_splits):
     case = make_case(**spec)
@@ -54,7 +54,7 @@ def test_vec_one_hot_mask_is_exact_and_all_masked_rows_are_zero():
         m[b, 0, i, j] = 0.0
     case["mask"] = ora.from_f32(m, ora.F16)
     v = to_f32(case["v"])                       # exact dequantisation, [B, H, Nkv, D]
-    for ns in (1, 4):
+    for ns in (1, 4, 19):
         print("one-hot n_splits", ns, flush=True)
         got = run_gpu(case, kernel=ggml.KERNEL_VEC, n_splits=ns)
         for b in range(2):
