@@ -527,7 +527,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=20,
+                    help="untimed steps first; the launch time of this kernel settles after about 14 steps (30 ms) from an idle GPU")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-scale-check", action="store_true", help="skip the half-size launches (keeps profiler means per kernel clean)")
