@@ -160,6 +160,10 @@ int mi355x_fattn_plan(const mi355x_tensor * q, const mi355x_tensor * k, const mi
  *
  * The dot products take f16-rounded inputs and accumulate in f32; scale, add and the rounding to f16 follow the
  * graph (f32 multiply, f32 add, round to nearest even, overflow to -inf).
+ * An F16 table with contiguous rows is read in place.  An F32 (or strided) table is first copied to contiguous f16
+ * in the library's per-device scratch block (2 bytes per element; see mi355x_fattn_params.workspace for when that
+ * block may be shared); a table that does not change between calls - it depends on the layer and on T only - is
+ * best converted once by the caller (mi355x_cpy to F16) and passed as F16.
  */
 int mi355x_relpos_bias_supports(const mi355x_tensor * q_v, const mi355x_tensor * r, const mi355x_tensor * add,
                                 const mi355x_tensor * dst);
