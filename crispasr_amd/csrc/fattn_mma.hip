@@ -43,6 +43,7 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float    float16v __attribute__((ext_vector_type(16)));
+typedef float    float4v __attribute__((ext_vector_type(4)));
 typedef short    short4v __attribute__((ext_vector_type(4)));
 typedef unsigned uint2v __attribute__((ext_vector_type(2)));
 
@@ -515,18 +516,34 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             half8 preg[NQB][2];
             float lsum[NQB];
             const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+            // With 64-wide heads the sum goes through the matrix pipe as well: v_mfma_f32_4x4x4_16b_f16 with A = ones
+            // adds the four f16 values a lane supplies as B into that lane's own f32 accumulators (16 independent 4x4
+            // blocks, lane = (block, column); all four rows of the result are equal) - exact products, f32
+            // accumulation, and the VALU, the busier pipe of that loop, has 32 instructions less per tile.  128-wide
+            // heads have no registers to spare for the accumulators and keep the packed dot product.
+            constexpr bool MFMA_SUMS = D == 64;
             auto exp_block = [&](int qb) {
-                float acc = 0.0f;
+                float dsum = 0.0f;
 #pragma unroll
                 for (int r = 0; r < 16; r += 2) {
                     half2v p2;
                     p2[0] = (_Float16)__builtin_amdgcn_exp2f(s[qb][r]);
                     p2[1] = (_Float16)__builtin_amdgcn_exp2f(s[qb][r + 1]);
-                    acc = __builtin_amdgcn_fdot2(p2, ones, acc, false);
+                    if (!MFMA_SUMS) dsum = __builtin_amdgcn_fdot2(p2, ones, dsum, false);
                     preg[qb][r >> 3][r & 7]       = p2[0];
                     preg[qb][r >> 3][(r & 7) + 1] = p2[1];
                 }
-                lsum[qb] = acc;
+                if (MFMA_SUMS) {
+                    const half4 ones4 = {(_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f, (_Float16)1.0f};
+                    float4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ones4, __builtin_shufflevector(preg[qb][h], preg[qb][h], 0, 1, 2, 3), acc, 0, 0, 0);
+                        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ones4, __builtin_shufflevector(preg[qb][h], preg[qb][h], 4, 5, 6, 7), acc, 0, 0, 0);
+                    }
+                    dsum = acc[0];
+                }
+                lsum[qb] = dsum;
             };
             bool redo = false;
 #pragma unroll
