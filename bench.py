@@ -208,7 +208,7 @@ def bench_decode(args, ca, ora, torch):
     # Whisper large-v3 decoder step, beam 5, 20 heads x 64 (strides of the [token][head][dim] cache)
     D, H = 64, 20
     n_state = D * H
-    Nkv, NL = 1500, 136                 # 136 x 7.7 MB = 1.05 GB of distinct K/V per replay
+    Nkv, NL = 1500, 64
     layers = []
     for l in range(NL):
         nbk = (2, 2 * n_state, 2 * D, 2 * n_state * Nkv)
@@ -219,7 +219,7 @@ def bench_decode(args, ca, ora, torch):
                        "out": ca.Tensor.empty(ca.F32, (D, H, 5, 1))})
     run("whisper_cross_beam5_f16", layers, 64 ** -0.25, 2 * Nkv * n_state * 2 + 2 * 5 * n_state * 4, 10,
         "5 queries vs one shared 1500-entry f16 K/V per layer")
-    Lk, NL = 224, 180                   # 180 x 5.8 MB = 1.04 GB
+    Lk, NL = 224, 64
     layers = []
     mask = np.zeros((5, 1, 1, Lk), np.float32)
     for b in range(5):
@@ -236,15 +236,14 @@ def bench_decode(args, ca, ora, torch):
         "1 query per beam vs its own 224-entry f16 cache, -inf mask beyond each beam's position")
 
     # Voxtral-style LLM decode: 32 q heads / 8 kv heads, D 128, Q8_0 cache of 663 entries (last of 256 steps)
-    D, Hq, Hkv, Lk, NL = 128, 32, 8, 663, 700       # 700 x 1.48 MB = 1.03 GB (48 distinct contents, 1400 distinct buffers)
+    D, Hq, Hkv, Lk, NL = 128, 32, 8, 663, 240
     rs = 136
     nbk = (34, rs, rs * Lk, rs * Lk * Hkv)
     layers = []
-    pool = [q8_buf(900 + i, Hkv * Lk * D) for i in range(48)]
     for l in range(NL):
         layers.append({"q": ca.Tensor(torch.randn(Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, 1)),
-                       "k": ca.Tensor(pool[(2 * l) % len(pool)].clone(), ca.Q8_0, (D, Lk, Hkv, 1), nbk),
-                       "v": ca.Tensor(pool[(2 * l + 1) % len(pool)].clone(), ca.Q8_0, (D, Lk, Hkv, 1), nbk),
+                       "k": ca.Tensor(q8_buf(900 + 2 * l, Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, 1), nbk),
+                       "v": ca.Tensor(q8_buf(901 + 2 * l, Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, 1), nbk),
                        "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 1))})
     per_call = 2 * Lk * Hkv * rs + 2 * Hq * D * 4
     run("voxtral_decode_q8_0_gqa4", layers, 128 ** -0.5, per_call, 10,
