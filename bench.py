@@ -9,7 +9,8 @@ resident in HBM before the timed region starts.  Prints ONE JSON line.
 Extra keys beside the contract's: `roofline` (dominant kernel against the f16 dense MFMA peak),
 `cpu_baseline` (the CPU oracle's ggml-like mode on a bounded sample, host cores of this box),
 `parity` (the timed configuration checked against the oracle on a sample of rows) and
-`decode` (the HBM-bound decode shapes, GB/s against 8 TB/s).
+`decode` (the HBM-bound decode shapes, GB/s against 8 TB/s) and `host_resident` (the same calls on
+pinned host buffers: link-inclusive rates, never `value`).
 """
 from __future__ import annotations
 
@@ -280,6 +281,65 @@ def bench_decode(args, ca, ora, torch):
                        "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 64))})
     run("llm_decode_q8_0_gqa4_4096x64seq", layers, 128 ** -0.5, 64 * (2 * Lk * Hkv * rs + 2 * Hq * D * 4), 10,
         "64 sequences x 4096-entry Q8_0 cache per call")
+    return out
+
+
+def bench_host_resident(ca, ora, torch):
+    """The same kernels with every tensor in pinned, GPU-mapped host memory (the is_host buffer type a backend
+    that implements one op gives ggml, so that ggml-cpu keeps running the other ops on weights and caches):
+    each call then pulls its K/V over the host link.  These are the link-inclusive rates; they are never
+    `value`."""
+    import numpy as np
+    out = {}
+
+    def host(nbytes):
+        return ca.HostBuffer(nbytes)
+
+    def timed(name, fn, bytes_per_call, reps, note):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        us = _time_calls(torch, fn, reps)
+        gbs = bytes_per_call / (us * 1e-6) / 1e9
+        out[name] = {"us_per_call": us, "GB/s_link_inclusive": gbs, "bytes_per_call": bytes_per_call, "note": note}
+        log(f"[bench] host-resident {name}: {us:.1f} us/call, {gbs:.1f} GB/s over the host link")
+
+    # Whisper large-v3 cross-attention for 5 beams: 1500-entry f16 K/V of one layer
+    D, H, Nkv = 64, 20, 1500
+    n_state = D * H
+    nbk = (2, 2 * n_state, 2 * D, 2 * n_state * Nkv)
+    kv = [host(Nkv * n_state * 2) for _ in range(2)]
+    rng = np.random.default_rng(7)
+    for b in kv:
+        b.array[:] = rng.standard_normal(Nkv * n_state, dtype=np.float32).astype(np.float16).view(np.uint8)
+    qh = host(5 * n_state * 4)
+    qh.array[:] = rng.standard_normal(5 * n_state, dtype=np.float32).view(np.uint8)
+    q = ca.Tensor(qh, ca.F32, (D, 5, H, 1), (4, 4 * n_state, 4 * D, 4 * n_state * 5))
+    k, v = ca.Tensor(kv[0], ca.F16, (D, Nkv, H, 1), nbk), ca.Tensor(kv[1], ca.F16, (D, Nkv, H, 1), nbk)
+    o = ca.Tensor(host(5 * n_state * 4), ca.F32, (D, H, 5, 1))
+    timed("whisper_cross_beam5_f16", lambda: ca.flash_attn_ext(q, k, v, None, 64 ** -0.25, out=o),
+          2 * Nkv * n_state * 2 + 2 * 5 * n_state * 4, 20, "q, K/V and dst in host memory; 7.7 MB per call")
+    # the device-resident result of the same bytes must be identical
+    kd = ca.Tensor.from_host(kv[0].array, ca.F16, (D, Nkv, H, 1), nbk)
+    vd = ca.Tensor.from_host(kv[1].array, ca.F16, (D, Nkv, H, 1), nbk)
+    qd = ca.Tensor.from_host(qh.array, ca.F32, q.ne, q.nb)
+    ref = ca.flash_attn_ext(qd, kd, vd, None, 64 ** -0.25).numpy_f32()
+    torch.cuda.synchronize()
+    out["whisper_cross_beam5_f16"]["equals_device_resident"] = bool(np.array_equal(o.numpy_f32(), ref))
+
+    # one encoder layer of the headline workload, one window, everything in host memory
+    N = 1500
+    bufs = [host(N * n_state * (4 if i in (0, 3) else 2)) for i in range(4)]           # q, k, v, out
+    bufs[0].array[:] = rng.standard_normal(N * n_state, dtype=np.float32).view(np.uint8)
+    for b in bufs[1:3]:
+        b.array[:] = rng.standard_normal(N * n_state, dtype=np.float32).astype(np.float16).view(np.uint8)
+    q = ca.Tensor(bufs[0], ca.F32, (D, N, H, 1), (4, 4 * n_state, 4 * D, 4 * n_state * N))
+    k = ca.Tensor(bufs[1], ca.F16, (D, N, H, 1), (2, 2 * n_state, 2 * D, 2 * n_state * N))
+    v = ca.Tensor(bufs[2], ca.F16, (D, N, H, 1), (2, 2 * n_state, 2 * D, 2 * n_state * N))
+    o = ca.Tensor(bufs[3], ca.F32, (D, H, N, 1))
+    timed("encoder_layer_1_window", lambda: ca.flash_attn_ext(q, k, v, None, 0.125, out=o),
+          N * n_state * (4 + 2 + 2 + 4), 10, "large-v3 encoder layer, one window (20 heads, 1500x1500): 23 MB per call")
+    out["encoder_layer_1_window"]["TFLOP/s"] = attn_flops(D, N, N, H, 1) / (out["encoder_layer_1_window"]["us_per_call"] * 1e-6) / 1e12
     return out
 
 
@@ -574,6 +634,7 @@ def main():
     if not args.no_decode:
         line["decode"] = bench_decode(args, ca, ora, torch)
     if not args.no_configs:
+        line["host_resident"] = bench_host_resident(ca, ora, torch)
         line["configs"] = bench_configs(args, ca, ora, torch)
         line["whisper_bench_protocol"] = bench_whisper_protocol(args, ca, ora, torch)
         line["whisper_bench_protocol_native"] = bench_whisper_protocol_native()

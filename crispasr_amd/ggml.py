@@ -147,18 +147,45 @@ def contiguous_nb(type_: int, ne: Sequence[int]) -> tuple:
     return (TYPE_SIZE[type_], nb1, nb1 * ne[1], nb1 * ne[1] * ne[2])
 
 
-class Tensor:
-    """A ggml tensor (or view) living in a device buffer."""
+class HostBuffer:
+    """Pinned host memory that the GPU addresses at the same pointer (mi355x_host_buffer_alloc): the
+    is_host buffer type a one-op backend gives ggml, so that ggml-cpu keeps running every other op on the
+    tensors in it.  ``array`` is the CPU's view of the bytes; the kernels read and write them in place."""
 
-    def __init__(self, buf: Optional[torch.Tensor], type_: int, ne: Sequence[int],
+    def __init__(self, nbytes: int, device=None):
+        self.device = torch.device("cuda", torch.cuda.current_device() if device is None else torch.device(device).index or 0)
+        self.nbytes = max(int(nbytes), 1)
+        p = ctypes.c_void_p()
+        with torch.cuda.device(self.device):
+            _check(lib().mi355x_host_buffer_alloc(self.nbytes, ctypes.byref(p)))
+        self.ptr = p.value
+        self.array = np.ctypeslib.as_array((ctypes.c_uint8 * self.nbytes).from_address(self.ptr))
+
+    def numel(self) -> int:
+        return self.nbytes
+
+    def data_ptr(self) -> int:
+        return self.ptr
+
+    def __del__(self):
+        if getattr(self, "ptr", None):
+            self.array = None
+            lib().mi355x_host_buffer_free(self.ptr)
+            self.ptr = None
+
+
+class Tensor:
+    """A ggml tensor (or view) living in a device buffer (a torch uint8 tensor) or in a HostBuffer."""
+
+    def __init__(self, buf, type_: int, ne: Sequence[int],
                  nb: Optional[Sequence[int]] = None, offset: int = 0):
-        self.buf = buf                      # 1-D uint8 device tensor, or None (planning only)
+        self.buf = buf                      # 1-D uint8 device tensor, a HostBuffer, or None (planning only)
         self.type = int(type_)
         self.ne = tuple(int(x) for x in ne) + (1,) * (4 - len(ne))
         self.nb = tuple(int(x) for x in (nb if nb is not None else contiguous_nb(self.type, self.ne)))
         self.offset = int(offset)
         self._c = None                      # the C descriptor, built once: a view never changes
-        if buf is not None:
+        if buf is not None and not isinstance(buf, HostBuffer):
             assert buf.dtype == torch.uint8 and buf.dim() == 1 and buf.is_contiguous()
 
     # -- construction ---------------------------------------------------------------------
@@ -176,6 +203,14 @@ class Tensor:
         buf = torch.from_numpy(raw.copy()).to(device)
         if buf.numel() == 0:
             buf = torch.zeros(1, dtype=torch.uint8, device=device)
+        return Tensor(buf, type_, ne, nb, offset)
+
+    @staticmethod
+    def in_host_buffer(raw: np.ndarray, type_: int, ne, nb=None, offset: int = 0) -> "Tensor":
+        """the same view over a fresh HostBuffer: set_tensor on an is_host buffer is a memcpy by the CPU"""
+        raw = np.ascontiguousarray(raw).view(np.uint8).reshape(-1)
+        buf = HostBuffer(raw.size)
+        buf.array[:raw.size] = raw
         return Tensor(buf, type_, ne, nb, offset)
 
     def view(self, ne, nb, offset: int = 0, type_: Optional[int] = None) -> "Tensor":
@@ -214,13 +249,18 @@ class Tensor:
 
     def to_host(self) -> np.ndarray:
         """ggml_backend_tensor_get of the whole underlying buffer (uint8)"""
+        if isinstance(self.buf, HostBuffer):
+            return self.buf.array.copy()
         return self.buf.cpu().numpy()
 
     def numpy_f32(self) -> np.ndarray:
         """contiguous F32 tensor -> numpy [ne3, ne2, ne1, ne0]"""
         assert self.type == F32 and self.nb == contiguous_nb(F32, self.ne)
         n = self.ne[0] * self.ne[1] * self.ne[2] * self.ne[3]
-        raw = self.buf[self.offset:self.offset + 4 * n].cpu().numpy()
+        if isinstance(self.buf, HostBuffer):
+            raw = self.buf.array[self.offset:self.offset + 4 * n]
+        else:
+            raw = self.buf[self.offset:self.offset + 4 * n].cpu().numpy()
         return raw.view(np.float32).reshape(self.ne[3], self.ne[2], self.ne[1], self.ne[0]).copy()
 
 
