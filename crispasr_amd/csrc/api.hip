@@ -22,6 +22,7 @@ int fail(int status, const char * fmt, ...) {
 }
 
 int hip_fail(hipError_t e, const char * what) {
+    (void)hipGetLastError();      // reported here: the launchers read the last error after each launch and must not see this one again
     return fail(MI355X_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
@@ -788,12 +789,16 @@ int mi355x_host_buffer_free(void * ptr) {
 
 int mi355x_buffer_memset(void * ptr, int value, size_t size, void * stream) {
     if (size == 0) return MI355X_OK;
-    HIP_TRY(hipMemsetAsync(ptr, value, size, (hipStream_t)stream));
+    if (!ptr) return fail(MI355X_ERR_INVALID, "null argument");
+    // a fill kernel, not hipMemsetAsync: safe to record into a graph the caller captures
+    const int e = fill_launch(ptr, value, size, (hipStream_t)stream);
+    if (e) return hip_fail((hipError_t)e, "fill launch");
     return MI355X_OK;
 }
 
 int mi355x_buffer_set(void * dst, const void * host_src, size_t size, void * stream) {
     if (size == 0) return MI355X_OK;
+    if (!dst || !host_src) return fail(MI355X_ERR_INVALID, "null argument");
     HIP_TRY(hipMemcpyAsync(dst, host_src, size, hipMemcpyHostToDevice, (hipStream_t)stream));
     HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
     return MI355X_OK;
@@ -801,6 +806,7 @@ int mi355x_buffer_set(void * dst, const void * host_src, size_t size, void * str
 
 int mi355x_buffer_get(void * host_dst, const void * src, size_t size, void * stream) {
     if (size == 0) return MI355X_OK;
+    if (!host_dst || !src) return fail(MI355X_ERR_INVALID, "null argument");
     HIP_TRY(hipMemcpyAsync(host_dst, src, size, hipMemcpyDeviceToHost, (hipStream_t)stream));
     HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
     return MI355X_OK;
@@ -808,6 +814,7 @@ int mi355x_buffer_get(void * host_dst, const void * src, size_t size, void * str
 
 int mi355x_buffer_copy(void * dst, const void * src, size_t size, void * stream) {
     if (size == 0) return MI355X_OK;
+    if (!dst || !src) return fail(MI355X_ERR_INVALID, "null argument");
     HIP_TRY(hipMemcpyAsync(dst, src, size, hipMemcpyDeviceToDevice, (hipStream_t)stream));
     return MI355X_OK;
 }

@@ -167,7 +167,31 @@ __global__ void __launch_bounds__(256) kv_to_f16_kernel(const FattnArgs a, char 
     *(h8 *)(dst + ((is_v ? half : 0) + i) * 16) = y;
 }
 
+// memset as a kernel: a memset node recorded into a captured graph is what a fill kernel avoids.
+// 16-byte stores over the aligned middle, single bytes for the (< 16-byte) head and tail.
+__global__ void __launch_bounds__(256) fill_kernel(unsigned char * p, unsigned value, size_t head, size_t n16, size_t tail) {
+    typedef unsigned u4 __attribute__((ext_vector_type(4)));
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const unsigned w = value * 0x01010101u;
+    if (i < n16) *(u4 *)(p + head + i * 16) = u4{w, w, w, w};
+    if (i < head) p[i] = (unsigned char)value;
+    if (i < tail) p[head + n16 * 16 + i] = (unsigned char)value;
+}
+
 }  // namespace
+
+int fill_launch(void * ptr, int value, size_t size, hipStream_t stream) {
+    if (size == 0) return 0;
+    size_t head = (16 - (uintptr_t)ptr % 16) % 16;
+    if (head > size) head = size;
+    const size_t n16  = (size - head) / 16;
+    const size_t tail = size - head - n16 * 16;
+    const size_t threads = n16 > 16 ? n16 : 16;                    // head and tail are below 16 bytes each
+    if ((threads + 255) / 256 > 0x7fffffffu) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(fill_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream,
+                       (unsigned char *)ptr, (unsigned)(value & 0xff), head, n16, tail);
+    return (int)hipGetLastError();
+}
 
 int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t stream) {
     const int64_t n = 2 * (int64_t)(a.D / 8) * a.Nkv * a.Hkv * a.Bk;

@@ -129,6 +129,7 @@ int fattn_decode_launch(const FattnArgs & a, int ktype, hipStream_t stream);
 bool fattn_decode_supported(const FattnArgs & a, int ktype);
 int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream);
 int set_rows_launch(const CpyArgs & a, int dtype, hipStream_t stream);
+int fill_launch(void * ptr, int value, size_t size, hipStream_t stream);      // memset by a kernel
 // K and V (F32 or Q8_0, any strides) -> contiguous f16 [D, Nkv, Hkv, Bk] at dst and right behind it
 int relpos_bias_launch(RelposArgs a, int rtype, hipStream_t stream);
 int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t stream);

@@ -214,7 +214,8 @@ int mi355x_buffer_free(void * ptr);                                /* free_buffe
  * is_host buffer type a one-op backend needs so that ggml-cpu keeps running every other op on it */
 int mi355x_host_buffer_alloc(size_t size, void ** ptr);
 int mi355x_host_buffer_free(void * ptr);
-int mi355x_buffer_memset(void * ptr, int value, size_t size, void * stream);         /* memset_tensor / clear */
+/* memset_tensor / clear: asynchronous on the stream, done by a fill kernel (no memset node if the caller captures a graph) */
+int mi355x_buffer_memset(void * ptr, int value, size_t size, void * stream);
 int mi355x_buffer_set(void * dst, const void * host_src, size_t size, void * stream);   /* set_tensor  (sync) */
 int mi355x_buffer_get(void * host_dst, const void * src, size_t size, void * stream);   /* get_tensor  (sync) */
 int mi355x_buffer_copy(void * dst, const void * src, size_t size, void * stream);      /* cpy_tensor D2D */
