@@ -796,10 +796,11 @@ int mi355x_buffer_memset(void * ptr, int value, size_t size, void * stream) {
     return MI355X_OK;
 }
 
+// The copies below name no direction: a buffer is HBM or pinned host memory and the runtime tells them apart by address.
 int mi355x_buffer_set(void * dst, const void * host_src, size_t size, void * stream) {
     if (size == 0) return MI355X_OK;
     if (!dst || !host_src) return fail(MI355X_ERR_INVALID, "null argument");
-    HIP_TRY(hipMemcpyAsync(dst, host_src, size, hipMemcpyHostToDevice, (hipStream_t)stream));
+    HIP_TRY(hipMemcpyAsync(dst, host_src, size, hipMemcpyDefault, (hipStream_t)stream));
     HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
     return MI355X_OK;
 }
@@ -807,7 +808,7 @@ int mi355x_buffer_set(void * dst, const void * host_src, size_t size, void * str
 int mi355x_buffer_get(void * host_dst, const void * src, size_t size, void * stream) {
     if (size == 0) return MI355X_OK;
     if (!host_dst || !src) return fail(MI355X_ERR_INVALID, "null argument");
-    HIP_TRY(hipMemcpyAsync(host_dst, src, size, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    HIP_TRY(hipMemcpyAsync(host_dst, src, size, hipMemcpyDefault, (hipStream_t)stream));
     HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
     return MI355X_OK;
 }
@@ -815,7 +816,7 @@ int mi355x_buffer_get(void * host_dst, const void * src, size_t size, void * str
 int mi355x_buffer_copy(void * dst, const void * src, size_t size, void * stream) {
     if (size == 0) return MI355X_OK;
     if (!dst || !src) return fail(MI355X_ERR_INVALID, "null argument");
-    HIP_TRY(hipMemcpyAsync(dst, src, size, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+    HIP_TRY(hipMemcpyAsync(dst, src, size, hipMemcpyDefault, (hipStream_t)stream));
     return MI355X_OK;
 }
 

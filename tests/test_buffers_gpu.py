@@ -51,6 +51,28 @@ def test_set_get_round_trip_and_device_copy():
         K.lib().mi355x_buffer_free(p)
 
 
+def test_set_get_copy_on_a_pinned_host_buffer():
+    # the is_host buffer type goes through the same vtable entries
+    n = 100000
+    data = np.random.default_rng(4).integers(0, 256, n, dtype=np.uint8)
+    h = ca.HostBuffer(n)
+    d = _alloc(n)
+    assert K.lib().mi355x_buffer_set(h.ptr, data.ctypes.data, n, None) == K.OK
+    assert np.array_equal(h.array, data)                                   # the CPU sees it in place
+    assert np.array_equal(_get(h.ptr, n), data)
+    assert K.lib().mi355x_buffer_copy(d, h.ptr, n, None) == K.OK           # host buffer -> HBM (a split-boundary copy)
+    assert K.lib().mi355x_stream_synchronize(None) == K.OK
+    assert np.array_equal(_get(d, n), data)
+    assert K.lib().mi355x_buffer_memset(h.ptr + 5, 0x77, 1001, None) == K.OK
+    assert K.lib().mi355x_buffer_copy(h.ptr + 50000, d, 100, None) == K.OK  # and back
+    assert K.lib().mi355x_stream_synchronize(None) == K.OK
+    want = data.copy()
+    want[5:1006] = 0x77
+    want[50000:50100] = data[:100]
+    assert np.array_equal(h.array, want)
+    K.lib().mi355x_buffer_free(d)
+
+
 @pytest.mark.parametrize("off,size", [(0, 0), (0, 1), (3, 5), (1, 15), (15, 2), (16, 16), (7, 4096), (0, 1 << 20), (34, 999999)])
 def test_memset_any_alignment_and_size(off, size):
     n = (1 << 20) + 256
