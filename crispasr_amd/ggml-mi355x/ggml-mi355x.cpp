@@ -132,6 +132,12 @@ static bool dev_supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
             mi355x_tensor s = to_mi(op->src[0]), d = to_mi(op);
             return mi355x_cpy_supports(&s, &d) == MI355X_OK;
         }
+        case GGML_OP_SET_ROWS: {                                // the write into a quantised KV cache (src/core/attention.h:366-376)
+            const ggml_tensor * src = op->src[0], * idx = op->src[1];
+            if (src->type != GGML_TYPE_F32 || (idx->type != GGML_TYPE_I64 && idx->type != GGML_TYPE_I32)) return false;
+            if (op->type != GGML_TYPE_F32 && op->type != GGML_TYPE_F16 && op->type != GGML_TYPE_Q8_0) return false;
+            return src->nb[0] == sizeof(float) && op->nb[0] == ggml_type_size(op->type);
+        }
         case GGML_OP_NONE: case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE:
             return true;                                        // no-ops on any backend
         default:
@@ -166,6 +172,14 @@ static enum ggml_status be_graph_compute(ggml_backend_t, ggml_cgraph * g) {
             case GGML_OP_CPY: case GGML_OP_CONT: case GGML_OP_DUP: {
                 const mi355x_tensor s = to_mi(n->src[0]), d = to_mi(n);
                 rc = mi355x_cpy(&s, &d, nullptr);
+                break;
+            }
+            case GGML_OP_SET_ROWS: {                            // the node is a view of the destination; src[0] = rows, src[1] = indices
+                const ggml_tensor * idx = n->src[1];
+                const mi355x_tensor s = to_mi(n->src[0]), d = to_mi(n);
+                const int64_t ine[3] = {idx->ne[0], idx->ne[1], idx->ne[2]};
+                const size_t  inb[3] = {idx->nb[0], idx->nb[1], idx->nb[2]};
+                rc = mi355x_set_rows(&s, idx->data, idx->type == GGML_TYPE_I64 ? 64 : 32, ine, inb, &d, nullptr);
                 break;
             }
             default:
