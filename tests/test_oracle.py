@@ -451,3 +451,57 @@ def test_relpos_mask_in_attention_equals_manual_softmax_of_ac_plus_bd():
         p = np.exp(s - s.max(axis=1, keepdims=True)); p /= p.sum(axis=1, keepdims=True)
         want = p @ v[0, h].astype(np.float64)
         assert np.abs(got[:, h] - want).max() < 3e-3
+
+
+# ---- the reference's own cross-attention unit test, through the flash path -------------------------------------
+
+class _RefTestRng:
+    """the generator of tests/test-core-cross-attn.cpp:26-31 (xorshift64, values in [-1, 1] on a 1e-4 grid)"""
+
+    def __init__(self, seed):
+        self.s = seed
+
+    def sym(self):
+        m = (1 << 64) - 1
+        self.s ^= (self.s << 13) & m
+        self.s ^= self.s >> 7
+        self.s ^= (self.s << 17) & m
+        nx = (self.s >> 11) & 0xFFFFFFFF
+        return np.float32((nx % 20001) / 10000.0 - 1.0)
+
+
+@pytest.mark.parametrize("scaled", [False, True])
+def test_reference_cross_attn_unit_test_shapes_and_fill(scaled):
+    # tests/test-core-cross-attn.cpp:35-145 checks core_cross_attn's manual path against a plain C++ MHA at 1e-4;
+    # core_cross_attn::cross_attn_step (src/core/cross_attn.h:119-153) is the same block with flash_attn_ext in the
+    # middle (scale 1/sqrt(head_dim), no mask).  Same shapes, same fill order, same tolerance, attention by the oracle.
+    d_model, head_dim, n_heads, T_enc = 8, 4, 2, 3
+    qd = n_heads * head_dim
+    rng = _RefTestRng(0x5151)
+    dec, q_proj, o_proj, cK, cV = (np.array([rng.sym() for _ in range(n)], np.float32)
+                                   for n in (d_model, d_model * qd, qd * d_model, head_dim * T_enc * n_heads,
+                                             head_dim * T_enc * n_heads))
+    scale = 1.0 / np.sqrt(head_dim) if scaled else 1.0
+    # the test's plain C++ reference, line by line (f32 accumulators as there)
+    QP = q_proj.reshape(qd, d_model)                     # qp[d, o] = q_proj[o*d_model + d]
+    K = cK.reshape(n_heads, T_enc, head_dim)
+    V = cV.reshape(n_heads, T_enc, head_dim)
+    head_out = np.zeros(qd, np.float32)
+    Q = np.zeros((n_heads, head_dim), np.float32)
+    for h in range(n_heads):
+        for hd in range(head_dim):
+            Q[h, hd] = np.float32(sum(np.float32(QP[h * head_dim + hd, d] * dec[d]) for d in range(d_model)))
+        sc = np.array([sum(K[h, te, hd] * Q[h, hd] for hd in range(head_dim)) for te in range(T_enc)], np.float32) * np.float32(scale)
+        p = np.exp(sc - sc.max())
+        p /= p.sum()
+        head_out[h * head_dim:(h + 1) * head_dim] = p @ V[h]
+    ref = o_proj.reshape(d_model, qd) @ head_out         # op[i, dm] = o_proj[dm*qd + i]
+    # the flash path: Q (head_dim, T_dec, n_heads) is a permuted view of the projection, K/V F32 [head_dim, T_enc, n_kv]
+    q_t = ora.Tensor(Q.reshape(-1).view(np.uint8).copy(), ora.F32, (head_dim, 1, n_heads, 1),
+                     (4, 4 * head_dim * n_heads, 4 * head_dim, 4 * head_dim * n_heads))
+    k_t = ora.Tensor(cK.view(np.uint8).copy(), ora.F32, (head_dim, T_enc, n_heads, 1))
+    v_t = ora.Tensor(cV.view(np.uint8).copy(), ora.F32, (head_dim, T_enc, n_heads, 1))
+    for mode in (ora.MODE_EXACT, ora.MODE_GGML_LIKE):
+        attn = ora.flash_attn_ext(q_t, k_t, v_t, None, float(scale), 0.0, 0.0, mode)      # [1, T_dec, n_heads, head_dim]
+        got = o_proj.reshape(d_model, qd) @ attn.reshape(qd).astype(np.float32)          # reshape_2d(attn, n_heads*head_dim, T_dec)
+        assert np.abs(got - ref).max() < 1e-4, (mode, np.abs(got - ref).max())
