@@ -35,6 +35,57 @@ def build() -> str:
     return _LIB_PATH
 
 
+REFERENCE_HEADER = "/root/reference/src/core/cpu_attention.h"
+_REF_LIB_PATH = os.path.join(_HERE, "_ref", "libref_cpu_attention.so")
+
+
+def build_ref() -> Optional[str]:
+    """Compile the reference's own scalar attention helpers into oracle/_ref/ (only where the reference tree is
+    present); returns the library's path, or None when there is nothing to build from."""
+    if not os.path.exists(REFERENCE_HEADER):
+        return _REF_LIB_PATH if os.path.exists(_REF_LIB_PATH) else None
+    subprocess.check_call(["make", "-C", _HERE, "-B", "ref"], stdout=subprocess.DEVNULL)
+    return _REF_LIB_PATH
+
+
+_ref_lib = None
+
+
+def ref_lib() -> Optional[ctypes.CDLL]:
+    """The compiled reference helpers, or None when they have not been built."""
+    global _ref_lib
+    if _ref_lib is None and os.path.exists(_REF_LIB_PATH):
+        L = ctypes.CDLL(_REF_LIB_PATH)
+        fp = ctypes.POINTER(ctypes.c_float)
+        L.ref_mha_f32.restype = None
+        L.ref_mha_f32.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, fp, fp, fp, ctypes.c_float, fp]
+        L.ref_relpos_mha_f32.restype = None
+        L.ref_relpos_mha_f32.argtypes = [ctypes.c_int] * 4 + [fp] * 7
+        _ref_lib = L
+    return _ref_lib
+
+
+def _fp(a: np.ndarray):
+    assert a.dtype == np.float32 and a.flags.c_contiguous
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_float))
+
+
+def ref_mha(q: np.ndarray, k: np.ndarray, v: np.ndarray, n_heads: int, scale: float) -> np.ndarray:
+    """q, k, v f32 [T, n_heads*head_dim] -> [T, n_heads*head_dim] by the reference's compiled helpers"""
+    T, H = q.shape
+    out = np.zeros((T, H), np.float32)
+    ref_lib().ref_mha_f32(T, n_heads, H // n_heads, _fp(q), _fp(k), _fp(v), float(scale), _fp(out))
+    return out
+
+
+def ref_relpos_mha(q, k, v, p, bu, bv, n_heads: int) -> np.ndarray:
+    """FireRed's relative-position attention: q, k, v [T, d], p [T_pe, d], bu / bv [n_heads, head_dim]"""
+    T, d = q.shape
+    out = np.zeros((T, d), np.float32)
+    ref_lib().ref_relpos_mha_f32(T, p.shape[0], n_heads, d // n_heads, _fp(q), _fp(k), _fp(v), _fp(p), _fp(bu), _fp(bv), _fp(out))
+    return out
+
+
 class _CTensor(ctypes.Structure):
     _fields_ = [
         ("data", ctypes.c_void_p),

@@ -26,6 +26,8 @@
  *       max_bias (ALiBi) slope formula : PARITY UNPINNED - recalled
  *       behaviour of ggml-cpu that no file, test or fixture of the reference
  *       holds.  logit_softcap is pinned by its closed form only.
+ *       Exact and ggml-like mode with F32 K/V are also held against the reference's own compiled scalar attention
+ *       (src/core/cpu_attention.h via oracle/ref_cpu_attention.cpp -> oracle/_ref/), where its tree is present.
  *   ora_relpos_bias : pinned by the reference's own graph (src/core/fastconformer.h:98-102,
  *       876-918, every node of which is restated literally, the rel_shift view as byte strides)
  *       and by the mathematics: numpy matmul + numpy.lib.stride_tricks.as_strided with the
