@@ -157,9 +157,25 @@ def cpu_baseline(args, ora, host0):
     tflops = attn_flops(D, N, N, H, B) / med / 1e12
     log(f"[bench] cpu baseline: {med * 1e3:.1f} ms per layer ({B} windows) on {threads} threads = {tflops * 1e3:.1f} GFLOP/s "
         f"({len(times)} runs, {sum(times):.1f} s of CPU work)")
-    return {"value": tflops, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"1 of 32 layers, all {B} windows (20 heads, 1500x1500), median of {len(times)} runs ({sum(times):.1f} s), "
-                      f"oracle ggml-like mode (restatement of ggml-cpu; real ggml is absent)"}
+    res = {"value": tflops, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+           "sample": f"1 of 32 layers, all {B} windows (20 heads, 1500x1500), median of {len(times)} runs ({sum(times):.1f} s), "
+                     f"oracle ggml-like mode (restatement of ggml-cpu; real ggml is absent)"}
+    if ora.ref_lib() is not None:
+        # the reference's own scalar attention helpers (compiled into oracle/_ref/), one thread, 2 heads of one window
+        Hs, n = 2, 3
+        qkv = [ora.randn(77 + i, (N, Hs * D)) for i in range(3)]
+        ts = []
+        for _ in range(n):
+            t0 = time.perf_counter()
+            ora.ref_mha(qkv[0], qkv[1], qkv[2], Hs, 0.125)
+            ts.append(time.perf_counter() - t0)
+        t = float(np.median(ts))
+        res["reference_scalar_helpers"] = {"value": attn_flops(D, N, N, Hs, 1) / t / 1e12, "unit": "TFLOP/s", "cores": 1,
+                                           "kind": "reference",
+                                           "sample": f"{Hs} heads x 1500x1500 of one window, median of {n} runs ({sum(ts):.1f} s), "
+                                                     "src/core/cpu_attention.h as the reference's CPU-loop backends call it"}
+        log(f"[bench] reference scalar helpers, 1 thread: {res['reference_scalar_helpers']['value'] * 1e3:.2f} GFLOP/s")
+    return res
 
 
 def bench_decode(args, ca, ora, torch):
