@@ -49,3 +49,22 @@ def test_relpos_bias_matches_golden():
     err = np.abs(g - w)
     # the kernel rounds Q_v and R to f16 before an f32 accumulation: a few f16 ulps at most, under one on average
     assert (err <= 4e-3 * np.maximum(1.0, np.abs(w))).all() and err.mean() < 6e-4, (err.max(), err.mean())
+
+
+@pytest.mark.skipif(ora.ref_lib() is None, reason="oracle/_ref not built (needs the reference tree)")
+@pytest.mark.parametrize("T,n_heads,hd,kernel", [(300, 3, 64, K.KERNEL_MMA), (150, 2, 128, K.KERNEL_MMA),
+                                                  (40, 2, 80, K.KERNEL_VEC), (12, 4, 64, K.KERNEL_AUTO)])
+def test_kernels_match_the_reference_scalar_attention(T, n_heads, hd, kernel):
+    # compiled reference code as the checker: src/core/cpu_attention.h driven as src/wav2vec2-ggml.cpp:1908-1924 does,
+    # Q/K/V [T, n_heads*hd] row-major F32 (the kernels see them as strided ggml views of the same bytes)
+    H = n_heads * hd
+    q, k, v = (ora.randn(9400 + i, (T, H)) for i in range(3))
+    scale = 1.0 / np.sqrt(hd)
+    want = ora.ref_mha(q, k, v, n_heads, scale)
+
+    def heads(x):
+        return upload(ora.Tensor(x.view(np.uint8).reshape(-1).copy(), ora.F32, (hd, T, n_heads, 1), (4, 4 * H, 4 * hd, 4 * H * T)))
+
+    print("kernel", kernel, "vs reference scalar attention", T, n_heads, hd, flush=True)
+    out = ca.flash_attn_ext(heads(q), heads(k), heads(v), None, float(scale), kernel=kernel)
+    assert_parity(out.numpy_f32().reshape(T, H), want, "vs reference scalar attention")

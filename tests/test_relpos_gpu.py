@@ -164,3 +164,28 @@ def test_relpos_mask_random_shapes(seed):
                            c["scale"], c["Nkv"])
     n = c["Nkv"] * c["Nq"] * c["H"] * c["B"]
     check_mask(got.to_host()[: 2 * n].view(np.uint16), ref.buf.view(np.uint16), str(spec))
+
+
+@pytest.mark.skipif(ora.ref_lib() is None, reason="oracle/_ref not built (needs the reference tree)")
+@pytest.mark.parametrize("T,n_heads,hd", [(150, 2, 128), (97, 3, 64)])
+def test_fused_relpos_attention_matches_the_reference_relpos_attention(T, n_heads, hd):
+    # the device path end to end against compiled reference code: FireRed's conformer attention
+    # (src/firered_asr.cpp:1525-1577 over src/core/cpu_attention.h), score = ((q+bu).k + (q+bv).p[T-1-tq+tk]) / sqrt(hd)
+    d = n_heads * hd
+    q, k, v = (0.7 * ora.randn(9300 + i, (T, d)) for i in range(3))
+    p = 0.7 * ora.randn(9303, (2 * T - 1, d))
+    bu, bv = 0.3 * ora.randn(9304, (n_heads, hd)), 0.3 * ora.randn(9305, (n_heads, hd))
+    want = ora.ref_relpos_mha(q, k, v, p, bu, bv, n_heads)
+
+    def heads(x):          # [rows, d] row-major -> ggml view ne [hd, rows, n_heads, 1] over the same bytes
+        rows = x.shape[0]
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        return upload(ora.Tensor(x.view(np.uint8).reshape(-1).copy(), ora.F32, (hd, rows, n_heads, 1),
+                                 (4, 4 * d, 4 * hd, 4 * d * rows)))
+
+    qu = (q.reshape(T, n_heads, hd) + bu[None]).reshape(T, d)
+    qv = (q.reshape(T, n_heads, hd) + bv[None]).reshape(T, d)
+    print("fused rel-pos attention vs reference helpers", T, n_heads, hd, flush=True)
+    out = ggml.flash_attn_relpos(heads(qu), heads(qv), heads(k), heads(v), heads(p), None, 1.0 / math.sqrt(hd))
+    got = out.numpy_f32()                                  # [1, T, n_heads, hd]
+    assert_parity(got.reshape(T, d), want, "fused rel-pos attention vs reference helpers")
