@@ -170,6 +170,7 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
     a.D = (int)q->ne[0]; a.Nq = (int)q->ne[1]; a.Hq = (int)q->ne[2]; a.B = (int)q->ne[3];
     a.Nkv = (int)k->ne[1]; a.Hkv = (int)k->ne[2]; a.Bk = (int)k->ne[3];
     a.gqa = a.Hq / a.Hkv; a.bq = a.B / a.Bk;
+    a.q_chunks = (int32_t)(((int64_t)a.Nq * a.gqa + 15) / 16);
     a.nbq1 = q->nb[1]; a.nbq2 = q->nb[2]; a.nbq3 = q->nb[3];
     a.nbk1 = k->nb[1]; a.nbk2 = k->nb[2]; a.nbk3 = k->nb[3];
     a.nbv1 = v->nb[1]; a.nbv2 = v->nb[2]; a.nbv3 = v->nb[3];
@@ -216,7 +217,15 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
 void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Plan & plan) {
     int kernel = p->kernel;
     if (kernel == MI355X_FATTN_AUTO) {
-        if (fattn_decode_supported(a, ktype))                 kernel = MI355X_FATTN_DECODE_MMA;   // <= 16 rows per KV head
+        // The decode kernel takes the Nq * gqa rows that share a KV head 16 at a time, each chunk streaming the head's K/V
+        // again.  Up to 16 rows that is the whole job.  Beyond, it still beats the tile kernel on a short prompt against
+        // a short Q8_0 cache (Canary's decoder reads its quantised cache directly, src/canary.cpp:966-972): no conversion
+        // pass, one round of workgroups (measured at 128 x 128 and 256 x 256, 32 q / 8 kv heads: 14.0 -> 8.6 and
+        // 18.0 -> 14.3 us; 24 x 300, 8 heads: 14.2 -> 10.9 us; at 407 x 407, 816 chunks, the tile kernel wins 29 to 31).
+        // With f16 K/V the two are within a microsecond of each other and the tile kernel keeps the shape.
+        const int64_t chunk_wgs = (int64_t)a.q_chunks * a.Hkv * a.B;
+        const bool    chunked   = ktype == MI355X_TYPE_Q8_0 && chunk_wgs <= 2 * (int64_t)device_cus() && a.Nkv <= 1024;
+        if (fattn_decode_supported(a, ktype) && (a.q_chunks <= 1 || chunked)) kernel = MI355X_FATTN_DECODE_MMA;
         else if (a.Nq >= 16 && fattn_mma_supported(a, ktype)) kernel = MI355X_FATTN_MMA;
         else                                                  kernel = MI355X_FATTN_VEC;
     }
@@ -269,7 +278,7 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
     if (kernel == MI355X_FATTN_VEC || kernel == MI355X_FATTN_DECODE_MMA) {
         const int64_t rows = (int64_t)a.Nq * a.Hq * a.B;
         // workgroups that exist before splitting, and the fewest keys worth a split
-        const int64_t groups   = kernel == MI355X_FATTN_VEC ? rows : (int64_t)a.Hkv * a.B;
+        const int64_t groups   = kernel == MI355X_FATTN_VEC ? rows : (int64_t)a.Hkv * a.B * a.q_chunks;
         // decode kernel: a split must be worth the merge launch (about 2.5 us): measured on Whisper cross-attention
         // (64-wide heads, 1500 keys: best at 8 splits) and a Q8_0 LLM cache (128-wide, 663 keys: best at 6 to 8),
         // while 224 keys are fastest unsplit
@@ -277,7 +286,9 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
         int ns = p->n_splits;
         if (ns <= 0) {
             const int64_t target = (int64_t)device_cus() * (kernel == MI355X_FATTN_VEC ? 4 : 2);
-            ns = (int)((target + groups - 1) / (groups > 0 ? groups : 1));
+            // whole splits only while they still fit the target: past it a split doubles the grid and adds the merge
+            ns = kernel == MI355X_FATTN_VEC ? (int)((target + groups - 1) / (groups > 0 ? groups : 1))
+                                            : (int)(target / (groups > 0 ? groups : 1));
             const int max_by_keys = kernel == MI355X_FATTN_VEC ? (a.Nkv + min_keys - 1) / min_keys : a.Nkv / min_keys;
             if (ns > max_by_keys) ns = max_by_keys;
         }

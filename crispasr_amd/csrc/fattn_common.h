@@ -20,6 +20,7 @@ struct FattnArgs {
     int32_t D, Nq, Hq, B, Nkv, Hkv, Bk;
     int32_t gqa;         // Hq / Hkv
     int32_t bq;          // B / Bk
+    int32_t q_chunks;    // decode kernel: 16-row chunks of the Nq * gqa query rows that share a KV head
     int32_t Hm, Bm;      // mask broadcast extents
 
     int64_t nbq1, nbq2, nbq3;

@@ -1,10 +1,11 @@
 // Split-KV MFMA decode kernel for gfx950: few query rows per KV head (beams and/or a GQA group),
 // long KV cache, HBM-bound.
 //
-// A workgroup of 4 waves owns one (KV head, batch, KV split); the up-to-16 query rows that read
-// this KV head - all queries of all q heads in its GQA group - are the 16 columns of
-// v_mfma_f32_16x16x32_f16 tiles, so K and V are fetched from HBM once per KV head, not once per
-// query row.  Each wave walks its share of the split in steps of 32 keys:
+// A workgroup of 4 waves owns one (KV head, batch, KV split, chunk of 16 query rows); the query rows
+// that read this KV head - all queries of all q heads in its GQA group, 16 of them per chunk - are
+// the 16 columns of v_mfma_f32_16x16x32_f16 tiles, so K and V are fetched once per KV head and chunk,
+// not once per query row (decode steps have one chunk; a short prompt has a few, and each streams the
+// head's K/V again).  Each wave walks its share of the split in steps of 32 keys:
 //
 //   S^T[key, row] = K[key, :] . Q[row, :]^T      A = K from global memory in operand layout
 //                                                 (128-bit loads: 16 rows x 64 contiguous bytes)
@@ -166,15 +167,18 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     const int j    = lane & 15;                    // query column
     const int g4   = lane >> 4;
 
+    // workgroup = (split, 16-row chunk, KV head, batch), splits fastest
     const int split = blockIdx.x % a.n_splits;
-    const int hk    = (blockIdx.x / a.n_splits) % a.Hkv;
-    const int b     = blockIdx.x / (a.n_splits * a.Hkv);
+    const int chunk = (blockIdx.x / a.n_splits) % a.q_chunks;
+    const int hk    = (blockIdx.x / (a.n_splits * a.q_chunks)) % a.Hkv;
+    const int b     = blockIdx.x / (a.n_splits * a.q_chunks * a.Hkv);
     const int bk    = b / a.bq;
 
-    // column j = iq1 * gqa + gg  <->  query iq1 of q head hk*gqa + gg
+    // row r = iq1 * gqa + gg of this KV head  <->  query iq1 of q head hk*gqa + gg; column j is row chunk*16 + j
     const int  R      = a.Nq * a.gqa;
-    const bool col_ok = j < R;
-    const int  jc     = col_ok ? j : 0;
+    const int  row0   = chunk * 16;
+    const bool col_ok = row0 + j < R;
+    const int  jc     = col_ok ? row0 + j : row0;
     const int  iq1    = jc / a.gqa;
     const int  h      = hk * a.gqa + jc % a.gqa;
 
@@ -392,7 +396,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
 
     // thread t: column t / 16, a strided set of d
     const int col = tid >> 4;
-    if (col < R) {
+    if (row0 + col < R) {
         float M = -INFINITY;
 #pragma unroll
         for (int w = 0; w < DEC_WAVES; w++) M = fmaxf(M, red_ml[w][col][0]);
@@ -404,8 +408,8 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
             f[w] = mw == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw - M);
             L += red_ml[w][col][1] * f[w];
         }
-        const int     ciq1 = col / a.gqa;
-        const int     ch   = hk * a.gqa + col % a.gqa;
+        const int     ciq1 = (row0 + col) / a.gqa;
+        const int     ch   = hk * a.gqa + (row0 + col) % a.gqa;
         const int64_t row  = ((int64_t)b * a.Nq + ciq1) * a.Hq + ch;
         for (int d = tid & 15; d < D; d += 16) {
             float acc = 0.0f;
@@ -428,7 +432,9 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
 
 template <int D, int TYPE, bool MASK, bool RAW>
 int launch_one(const FattnArgs & a, hipStream_t stream) {
-    const dim3 grid((unsigned)(a.n_splits * a.Hkv * a.B));
+    const int64_t wgs = (int64_t)a.n_splits * a.q_chunks * a.Hkv * a.B;
+    if (wgs > 0x7fffffff || a.q_chunks != (a.Nq * a.gqa + 15) / 16) return (int)hipErrorInvalidValue;
+    const dim3 grid((unsigned)wgs);
     constexpr int lds = decode_lds_bytes<D, RAW>();
     static bool attr_set = false;
     if (!attr_set && lds > 64 * 1024) {
@@ -463,7 +469,7 @@ int launch(const FattnArgs & a, hipStream_t stream) {
 bool fattn_decode_supported(const FattnArgs & a, int ktype) {
     if (a.D != 64 && a.D != 128) return false;
     if (a.Nq < 1 || a.Nkv < 1) return false;
-    if ((int64_t)a.Nq * a.gqa > 16) return false;
+    if ((int64_t)a.Nq * a.gqa > ((int64_t)1 << 20)) return false;      // 16-row chunks of the rows that share a KV head
     if (a.softcap != 0.0f) return false;
     if (ktype == MI355X_TYPE_F16) return a.kv_aligned16 != 0;
     if (ktype == MI355X_TYPE_Q8_0) return a.kv_aligned4 != 0;

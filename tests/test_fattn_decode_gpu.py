@@ -40,15 +40,49 @@ def test_decode_kernel_matches_oracle(spec, n_splits):
     assert_parity(got, ref, str(spec))
 
 
-def test_decode_is_what_auto_picks_and_more_than_16_rows_is_rejected():
+def test_decode_is_what_auto_picks_for_up_to_16_rows():
     dec = make_case(seed=221, D=128, Nq=1, Nkv=300, Hq=32, Hkv=8, ktype=ora.Q8_0)
     kern, _ = ggml.flash_attn_plan(upload(dec["q"]), upload(dec["k"]), upload(dec["v"]), None, dec["scale"])
     assert kern == ggml.KERNEL_DECODE_MMA
     assert_parity(run_gpu(dec), run_oracle(dec), "auto decode")
-    wide = make_case(seed=222, D=128, Nq=5, Nkv=64, Hq=32, Hkv=8)      # 20 rows per KV head
-    with pytest.raises(ggml.UnsupportedError):
-        run_gpu(wide, kernel=ggml.KERNEL_DECODE_MMA)
-    assert_parity(run_gpu(wide), run_oracle(wide), "auto fallback")
+
+
+# more than 16 rows per KV head: 16-row chunks, each its own workgroup
+CHUNKED = [
+    dict(seed=231, D=128, Nq=5, Nkv=64, Hq=32, Hkv=8),                                              # 20 rows: a chunk of 4
+    dict(seed=232, D=128, Nq=24, Nkv=300, Hq=8, ktype=ora.Q8_0),                                    # Canary prompt: rows = queries
+    dict(seed=233, D=128, Nq=37, Nkv=129, Hq=8, Hkv=2, B=2, ktype=ora.Q8_0, mask="causal"),         # 148 rows, chunks straddle q heads
+    dict(seed=234, D=64, Nq=50, Nkv=333, Hq=6, Hkv=3, B=2, Bk=1, mask="random_inf_batched", q_layout="thd", kv_layout="thd"),
+    dict(seed=235, D=64, Nq=33, Nkv=70, Hq=4, mask="bias_perhead"),
+    dict(seed=236, D=128, Nq=128, Nkv=128, Hq=32, Hkv=8, ktype=ora.Q8_0, mask="causal"),            # 32 chunks x 8 heads
+    dict(seed=237, D=64, Nq=17, Nkv=1, Hq=2, mask="all_masked_rows"),
+    dict(seed=238, D=128, Nq=19, Nkv=700, Hq=4, Hkv=4, ktype=ora.Q8_0, kv_layout="gap"),
+]
+
+
+@pytest.mark.parametrize("n_splits", [1, 0, 3])
+@pytest.mark.parametrize("spec", CHUNKED, ids=lambda s: "seed%d" % s["seed"])
+def test_decode_kernel_in_16_row_chunks_matches_oracle(spec, n_splits):
+    case = make_case(**spec)
+    print("chunked case", spec, "n_splits", n_splits, flush=True)
+    assert_parity(run_gpu(case, kernel=ggml.KERNEL_DECODE_MMA, n_splits=n_splits), run_oracle(case), str(spec))
+
+
+def test_auto_takes_short_q8_0_prompts_to_the_decode_kernel_and_long_ones_to_the_tile_kernel():
+    def plan(**spec):
+        c = make_case(**spec)
+        m = upload(c["mask"]) if c["mask"] is not None else None
+        return c, ggml.flash_attn_plan(upload(c["q"]), upload(c["k"]), upload(c["v"]), m, c["scale"])
+    short, (kern, ns) = plan(seed=241, D=128, Nq=24, Nkv=300, Hq=8, ktype=ora.Q8_0)                  # a prompt into Canary's cache
+    assert kern == ggml.KERNEL_DECODE_MMA
+    assert_parity(run_gpu(short), run_oracle(short), "auto, short Q8_0 prompt")
+    mid, (kern, ns) = plan(seed=242, D=128, Nq=100, Nkv=100, Hq=32, Hkv=8, ktype=ora.Q8_0, mask="causal")   # 200 chunks, no split
+    assert (kern, ns) == (ggml.KERNEL_DECODE_MMA, 1)
+    assert_parity(run_gpu(mid), run_oracle(mid), "auto, 100-token Q8_0 prefill")
+    _, (kern, _) = plan(seed=243, D=128, Nq=407, Nkv=407, Hq=32, Hkv=8, ktype=ora.Q8_0, mask="causal")   # 816 chunks
+    assert kern == ggml.KERNEL_MMA
+    _, (kern, _) = plan(seed=244, D=128, Nq=24, Nkv=300, Hq=8)                                         # f16: the tile kernel keeps it
+    assert kern == ggml.KERNEL_MMA
 
 
 def test_decode_q8_0_dequantisation_in_registers_is_exact():
