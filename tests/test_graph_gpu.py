@@ -1,0 +1,90 @@
+"""The entry points recorded into a HIP graph: replays must give what eager calls give, replay after replay, with
+eager work and synchronisations in between and with new input contents each time.  Callers that capture pass their
+own workspaces (the library's scratch may have to grow, which a capture cannot do)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import crispasr_amd as ca
+import oracle as ora
+from cases import make_case
+from crispasr_amd import ggml
+from gpu_util import assert_parity, run_oracle, upload
+
+pytestmark = pytest.mark.gpu
+
+
+def _ws(q, k, v, m, scale, kernel, ns):
+    p = ggml._params(scale, 0.0, 0.0, ggml.PREC_DEFAULT, kernel, ns, None)
+    n = ctypes.c_size_t(0)
+    ggml._check(ggml.lib().mi355x_fattn_workspace_size(q.ref(), k.ref(), v.ref(), m.ref() if m is not None else None,
+                                                       ctypes.byref(p), ctypes.byref(n)))
+    return torch.empty(max(n.value, 16), dtype=torch.uint8, device="cuda")
+
+
+def test_graph_replays_match_eager_calls():
+    # a decode step as a runtime issues it: write the new K/V rows into the f16 cache, split-KV attention over the cache;
+    # next to it a prefill on a Q8_0 cache (conversion pass + tile kernel) and a buffer clear
+    D, H, ctx, n_past = 64, 8, 640, 600
+    dec = make_case(seed=951, D=D, Nq=1, Nkv=n_past + 1, Hq=H, q_layout="thd")
+    cache_k = ca.Tensor.empty(ca.F16, (D, ctx, H, 1))
+    cache_v = ca.Tensor.empty(ca.F16, (D, ctx, H, 1))
+    for c in (cache_k, cache_v):
+        c.buf.copy_(torch.from_numpy(ora.fp32_to_fp16(ora.randn(952, (c.buf.numel() // 2,))).view(np.uint8)).cuda())
+    new_k = upload(ora.from_f32(ora.randn(953, (1, H, 1, D)), ora.F32))
+    new_v = upload(ora.from_f32(ora.randn(954, (1, H, 1, D)), ora.F32))
+    rs = 2 * D
+    row = lambda c: c.view((D, 1, H, 1), (2, rs, rs * ctx, rs * ctx * H), n_past * rs)          # noqa: E731
+    hist = lambda c: c.view((D, n_past + 1, H, 1), (2, rs, rs * ctx, rs * ctx * H))            # noqa: E731
+    q = upload(dec["q"])
+    pre = make_case(seed=955, D=128, Nq=160, Nkv=200, Hq=8, Hkv=2, ktype=ora.Q8_0, mask="causal")
+    pq, pk, pv, pm = upload(pre["q"]), upload(pre["k"]), upload(pre["v"]), upload(pre["mask"])
+    ws_dec = _ws(q, hist(cache_k), hist(cache_v), None, dec["scale"], ggml.KERNEL_DECODE_MMA, 4)
+    ws_pre = _ws(pq, pk, pv, pm, pre["scale"], ggml.KERNEL_MMA, 0)
+    scratch = torch.full((4099,), 7, dtype=torch.uint8, device="cuda")
+
+    def step(out_dec, out_pre, stream=None):
+        ca.cpy(new_k, row(cache_k), stream=stream)
+        ca.cpy(new_v, row(cache_v), stream=stream)
+        ggml.flash_attn_ext(q, hist(cache_k), hist(cache_v), None, dec["scale"], kernel=ggml.KERNEL_DECODE_MMA, n_splits=4,
+                            out=out_dec, workspace=ws_dec, stream=stream)
+        ggml.flash_attn_ext(pq, pk, pv, pm, pre["scale"], kernel=ggml.KERNEL_MMA, out=out_pre, workspace=ws_pre, stream=stream)
+        ggml._check(ggml.lib().mi355x_buffer_memset(scratch.data_ptr() + 3, 0x5A, 4090, ggml._stream_handle(stream)))
+
+    g_dec, g_pre = ca.Tensor.empty(ca.F32, (D, H, 1, 1)), ca.Tensor.empty(ca.F32, (128, 8, 160, 1))
+    e_dec, e_pre = ca.Tensor.empty(ca.F32, (D, H, 1, 1)), ca.Tensor.empty(ca.F32, (128, 8, 160, 1))
+    step(e_dec, e_pre)                                             # eager warm-up: modules loaded before the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            step(g_dec, g_pre, stream=side)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(5)
+    for replay in range(4):
+        # new contents in the same buffers, written by eager torch work between the replays
+        for t, n in ((q, D * H), (new_k, D * H), (new_v, D * H), (pq, 128 * 160 * 8)):
+            t.buf.copy_(torch.from_numpy(rng.standard_normal(n, dtype=np.float32).view(np.uint8)).cuda())
+        scratch.fill_(7)
+        g_dec.buf.zero_()
+        g_pre.buf.zero_()
+        torch.cuda.synchronize()
+        print("replay", replay, flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        got_dec, got_pre, got_fill = g_dec.numpy_f32(), g_pre.numpy_f32(), scratch.cpu().numpy().copy()
+        scratch.fill_(7)
+        step(e_dec, e_pre)
+        torch.cuda.synchronize()
+        assert np.array_equal(got_dec, e_dec.numpy_f32()), f"decode differs on replay {replay}"
+        assert np.array_equal(got_pre, e_pre.numpy_f32()), f"prefill differs on replay {replay}"
+        assert np.array_equal(got_fill, scratch.cpu().numpy()) and got_fill[2] == 7 and got_fill[3] == 0x5A and got_fill[4093] == 7
+    # and the last state against the oracle: the cache row really holds the new K/V
+    host_case = dict(dec)
+    kc = ora.Tensor(cache_k.to_host(), ora.F16, (D, n_past + 1, H, 1), (2, rs, rs * ctx, rs * ctx * H))
+    vc = ora.Tensor(cache_v.to_host(), ora.F16, (D, n_past + 1, H, 1), (2, rs, rs * ctx, rs * ctx * H))
+    host_case.update(q=ora.Tensor(q.to_host(), ora.F32, dec["q"].ne, dec["q"].nb), k=kc, v=vc)
+    assert_parity(e_dec.numpy_f32(), run_oracle(host_case), "decode step after the replays")
