@@ -77,7 +77,9 @@ typedef struct mi355x_fattn_params {
     int32_t prec;            /* GGML_PREC_DEFAULT = 0, GGML_PREC_F32 = 10; accumulation is f32 either way */
     int32_t kernel;          /* mi355x_fattn_kernel */
     int32_t n_splits;        /* 0 = choose; forces the KV split count of the split-KV kernels */
-    void *  workspace;       /* NULL = library-owned scratch (grown with hipMalloc when needed); else 16-byte aligned */
+    void *  workspace;       /* NULL = library-owned scratch (grown with hipMalloc when needed); else 16-byte aligned.
+                              * With a caller's workspace of mi355x_fattn_workspace_size bytes the call allocates nothing
+                              * and launches kernels only (no memset or copy nodes): it may be recorded into a HIP graph. */
     size_t  workspace_size;
 } mi355x_fattn_params;
 
