@@ -88,3 +88,40 @@ def test_graph_replays_match_eager_calls():
     vc = ora.Tensor(cache_v.to_host(), ora.F16, (D, n_past + 1, H, 1), (2, rs, rs * ctx, rs * ctx * H))
     host_case.update(q=ora.Tensor(q.to_host(), ora.F32, dec["q"].ne, dec["q"].nb), k=kc, v=vc)
     assert_parity(e_dec.numpy_f32(), run_oracle(host_case), "decode step after the replays")
+
+
+def test_graph_replays_of_the_relpos_attention_call_match_eager_calls():
+    # a FastConformer block's attention (F32 K/V views, F32 table, pad mask) recorded with a caller's workspace:
+    # table copy, mask kernel, K/V conversion and the tile kernel are all kernel nodes
+    from test_relpos_gpu import make, strided
+    c = make(seed=961, D=128, Nq=150, Nkv=150, H=2, B=2, add="pad", layout="thd", qgain=0.7)
+    qu = strided(np.float32(0.7) * ora.randn(962, (2, 2, 150, 128)), "thd")
+    k, v = strided(ora.randn(963, (2, 2, 150, 128)), "thd"), strided(ora.randn(964, (2, 2, 150, 128)), "thd")
+    dq, dqv, dk, dv, dr, da = (upload(t) for t in (qu, c["qv"], k, v, c["r"], c["add"]))
+    need = ggml.flash_attn_relpos_workspace_size(dq, dqv, dk, dv, dr, da, c["scale"])
+    ws_g = torch.empty(need, dtype=torch.uint8, device="cuda")
+    ws_e = torch.empty(need, dtype=torch.uint8, device="cuda")
+    out_g, out_e = ca.Tensor.empty(ca.F32, (128, 2, 150, 2)), ca.Tensor.empty(ca.F32, (128, 2, 150, 2))
+    ggml.flash_attn_relpos(dq, dqv, dk, dv, dr, da, c["scale"], out=out_e, workspace=ws_e)        # eager warm-up
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            ggml.flash_attn_relpos(dq, dqv, dk, dv, dr, da, c["scale"], out=out_g, workspace=ws_g, stream=side)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(6)
+    for replay in range(3):
+        for t in (dq, dqv):
+            t.buf.copy_(torch.from_numpy((0.7 * rng.standard_normal(t.buf.numel() // 4)).astype(np.float32).view(np.uint8)).cuda())
+        out_g.buf.zero_()
+        torch.cuda.synchronize()
+        print("relpos replay", replay, flush=True)
+        graph.replay()
+        torch.cuda.synchronize()
+        ggml.flash_attn_relpos(dq, dqv, dk, dv, dr, da, c["scale"], out=out_e, workspace=ws_e)
+        torch.cuda.synchronize()
+        assert np.array_equal(out_g.numpy_f32(), out_e.numpy_f32()), f"replay {replay} differs from the eager call"
+    host = dict(qu=ora.Tensor(dq.to_host(), ora.F32, qu.ne, qu.nb), qv=ora.Tensor(dqv.to_host(), ora.F32, c["qv"].ne, c["qv"].nb))
+    mask = ora.relpos_bias(host["qv"], c["r"], c["add"], c["scale"], 150)
+    assert_parity(out_e.numpy_f32(), ora.flash_attn_ext(host["qu"], k, v, mask, c["scale"]), "rel-pos attention after the replays")
