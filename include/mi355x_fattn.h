@@ -64,7 +64,7 @@ enum mi355x_fattn_kernel {
     MI355X_FATTN_AUTO       = 0,
     MI355X_FATTN_VEC        = 1,  /* split-KV vector kernel: any supported shape */
     MI355X_FATTN_MMA        = 2,  /* f16 MFMA tile kernel: prefill / encoder shapes */
-    MI355X_FATTN_DECODE_MMA = 3,  /* split-KV MFMA kernel: few query rows per KV head */
+    MI355X_FATTN_DECODE_MMA = 3,  /* split-KV MFMA kernel: the query rows of a KV head 16 at a time (decode steps, short prompts) */
     MI355X_FATTN_MMA_PIPE   = 4   /* software-pipelined variant of the tile kernel (head size 64, no mask); never chosen by AUTO */
 };
 
