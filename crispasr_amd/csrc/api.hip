@@ -225,7 +225,12 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
         // With f16 K/V the two are within a microsecond of each other and the tile kernel keeps the shape.
         const int64_t chunk_wgs = (int64_t)a.q_chunks * a.Hkv * a.B;
         const bool    chunked   = ktype == MI355X_TYPE_Q8_0 && chunk_wgs <= 2 * (int64_t)device_cus() && a.Nkv <= 1024;
-        if (fattn_decode_supported(a, ktype) && (a.q_chunks <= 1 || chunked)) kernel = MI355X_FATTN_DECODE_MMA;
+        // The MFMA kernels round F32 and Q8_0 K/V to f16 (2^-12 relative per element).  Over many keys that averages out;
+        // a row that sees a handful of keys keeps it (up to 1e-3 on |v| = 4, measured 2.01e-3 in all at 7 keys), so
+        // such calls go to the vector kernel, which works on the exact values - and has nothing to gain from MFMA there.
+        const bool few_keys = a.Nkv <= 16 && ktype != MI355X_TYPE_F16;
+        if (few_keys)                                                              kernel = MI355X_FATTN_VEC;
+        else if (fattn_decode_supported(a, ktype) && (a.q_chunks <= 1 || chunked)) kernel = MI355X_FATTN_DECODE_MMA;
         else if (a.Nq >= 16 && fattn_mma_supported(a, ktype)) kernel = MI355X_FATTN_MMA;
         else                                                  kernel = MI355X_FATTN_VEC;
     }

@@ -53,12 +53,21 @@ def test_random_shape_matches_oracle_on_every_kernel(seed):
     print("case", spec, flush=True)
     case = make_case(**spec)
     ref = run_oracle(case)
-    assert_parity(run_gpu(case), ref, "auto %s" % spec)
+    # The tolerance is quoted at unit-variance scores.  The MFMA kernels round q * scale to f16, an error in a score
+    # that grows with the score: at score std 1.5 a row that sees few keys (nothing to average over) can reach
+    # 2.3e-3 - plain f16-operand arithmetic in numpy gives the same figure to four digits (seed 1801) - so those
+    # draws are held to 3e-3.
+    hot = spec.get("scale", 0.0) * spec["D"] ** 0.5 > 1.2
+    tol = dict(max_abs_tol=3e-3) if hot else {}
+    assert_parity(run_gpu(case), ref, "auto %s" % spec, **tol)
     for kern in (ggml.KERNEL_VEC, ggml.KERNEL_MMA, ggml.KERNEL_DECODE_MMA):
         try:
             got = run_gpu(case, kernel=kern)
         except ggml.UnsupportedError:
             continue
-        assert_parity(got, ref, "kernel %d %s" % (kern, spec))
+        # a handful of keys in F32 or Q8_0: the automatic choice is the vector kernel (exact values); an MFMA kernel forced
+        # onto such a call rounds K/V to f16 with nothing to average the rounding over (2.01e-3 at 7 keys, seed 1932)
+        few = spec["Nkv"] <= 16 and spec["ktype"] != ora.F16 and kern != ggml.KERNEL_VEC
+        assert_parity(got, ref, "kernel %d %s" % (kern, spec), **(dict(max_abs_tol=3e-3) if few else tol))
         if kern == ggml.KERNEL_MMA and spec["Nkv"] > 64:       # key ranges of whole tiles + merge pass
-            assert_parity(run_gpu(case, kernel=kern, n_splits=2 + seed % 3), ref, "tile kernel, split keys %s" % spec)
+            assert_parity(run_gpu(case, kernel=kern, n_splits=2 + seed % 3), ref, "tile kernel, split keys %s" % spec, **tol)
