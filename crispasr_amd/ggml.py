@@ -328,6 +328,17 @@ def flash_attn_plan(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor] = No
     return kern.value, ns.value
 
 
+def flash_attn_workspace_size(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor] = None, scale: float = 1.0,
+                              max_bias: float = 0.0, logit_softcap: float = 0.0, kernel: int = KERNEL_AUTO,
+                              n_splits: int = 0) -> int:
+    """Bytes of workspace the call would use (split-KV partials, f16 copies of F32 / Q8_0 K/V); 0 if none."""
+    p = _params(scale, max_bias, logit_softcap, PREC_DEFAULT, kernel, n_splits, None)
+    n = ctypes.c_size_t(0)
+    _check(lib().mi355x_fattn_workspace_size(q.ref(), k.ref(), v.ref(), mask.ref() if mask is not None else None,
+                                             ctypes.byref(p), ctypes.byref(n)))
+    return n.value
+
+
 def flash_attn_ext(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor], scale: float,
                    max_bias: float = 0.0, logit_softcap: float = 0.0, *, prec: int = PREC_DEFAULT,
                    kernel: int = KERNEL_AUTO, n_splits: int = 0, out: Optional[Tensor] = None,

@@ -2,7 +2,6 @@
 (docs/concurrency.md:52-61, src/core/ggml_cpu_backend.h:202-204), so calls arrive from several host threads.
 The library keeps no per-call state besides the per-device scratch; threads that use their own streams pass their
 own workspaces.  Results must be the ones a single thread gets, and mi355x_last_error() is per thread."""
-import ctypes
 import threading
 
 import numpy as np
@@ -18,11 +17,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _workspace_bytes(q, k, v, m, scale, kernel, n_splits):
-    p = ggml._params(scale, 0.0, 0.0, ggml.PREC_DEFAULT, kernel, n_splits, None)
-    n = ctypes.c_size_t(0)
-    ggml._check(ggml.lib().mi355x_fattn_workspace_size(q.ref(), k.ref(), v.ref(), m.ref() if m is not None else None,
-                                                       ctypes.byref(p), ctypes.byref(n)))
-    return n.value
+    return ggml.flash_attn_workspace_size(q, k, v, m, scale, kernel=kernel, n_splits=n_splits)
 
 
 def test_two_host_threads_on_their_own_streams_and_workspaces():

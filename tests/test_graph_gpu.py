@@ -1,8 +1,6 @@
 """The entry points recorded into a HIP graph: replays must give what eager calls give, replay after replay, with
 eager work and synchronisations in between and with new input contents each time.  Callers that capture pass their
 own workspaces (the library's scratch may have to grow, which a capture cannot do)."""
-import ctypes
-
 import numpy as np
 import pytest
 import torch
@@ -17,11 +15,8 @@ pytestmark = pytest.mark.gpu
 
 
 def _ws(q, k, v, m, scale, kernel, ns):
-    p = ggml._params(scale, 0.0, 0.0, ggml.PREC_DEFAULT, kernel, ns, None)
-    n = ctypes.c_size_t(0)
-    ggml._check(ggml.lib().mi355x_fattn_workspace_size(q.ref(), k.ref(), v.ref(), m.ref() if m is not None else None,
-                                                       ctypes.byref(p), ctypes.byref(n)))
-    return torch.empty(max(n.value, 16), dtype=torch.uint8, device="cuda")
+    n = ggml.flash_attn_workspace_size(q, k, v, m, scale, kernel=kernel, n_splits=ns)
+    return torch.empty(max(n, 16), dtype=torch.uint8, device="cuda")
 
 
 def test_graph_replays_match_eager_calls():
