@@ -427,6 +427,17 @@ def bench_configs(args, ca, ora, torch):
                                               lengths=lengths),
             note="8 heads x 128, T=750, batch 8, per-head f16 bias N(0, std 0.5) with -inf beyond each length (1 layer)")
     res["C5_fastconformer_relpos_f32"] = bench_relpos(ca, ora, torch, lengths)
+    # the reference's other call sites of the op, at their shapes
+    run("voxtral_audio_encoder_f32", dict(seed=6, D=64, Nq=1500, Nkv=1500, Hq=20, ktype=ora.F32, q_layout="thd", kv_layout="thd"),
+        note="core_attn::encoder_self_attn (src/core/attention.h:517-580, src/voxtral.cpp:676-687): 20 heads x 64, "
+             "Q/K/V F32 views of [1280, 1500] activations, no mask; K/V rounded to f16 once, then the tile kernel")
+    run("canary_decoder_self_q8_0_view", dict(seed=7, D=128, Nq=1, Nkv=300, Hq=8, ktype=ora.Q8_0, kv_layout="gap"),
+        note="src/canary.cpp:953-972: one token against a strided view of the Q8_0 cache, 8 heads x 128, 300 entries")
+    run("canary_decoder_prompt_q8_0_view", dict(seed=8, D=128, Nq=24, Nkv=24, Hq=8, ktype=ora.Q8_0, kv_layout="gap", mask="causal"),
+        note="the same cache on the prompt step: 24 tokens, causal mask (decode kernel in 16-row chunks)")
+    run("decoder_cross_attn_f16", dict(seed=9, D=128, Nq=1, Nkv=375, Hq=8, q_layout="thd"),
+        note="core_cross_attn::cross_attn_step (src/core/cross_attn.h:119-153): one decoder token against 375 encoder "
+             "frames of f16 K/V, 8 heads x 128, no mask")
     return res
 
 
