@@ -408,6 +408,16 @@ def bench_configs(args, ca, ora, torch):
              "parity": {"max_abs": max_abs, "rel_l2": rel, "ok": ok}, "note": note}
         if causal:
             r["TFLOP/s_causal_half"] = r["TFLOP/s"] / 2 if ok else None
+        if k.type == ora.Q8_0 and D % 32 == 0:
+            # against the oracle's ggml-like mode (query rows quantised to Q8_0, as ggml-cpu is recalled to do for Q8_0 K):
+            # the default call, and the comparison mode that quantises the query rows the same way
+            like = ora.flash_attn_ext(case["q"], case["k"], case["v"], case["mask"], case["scale"], case["max_bias"],
+                                      case["softcap"], ora.MODE_GGML_LIKE)
+            d0 = errors(out.numpy_f32(), like)
+            qq = ca.flash_attn_ext(q, k, v, m, case["scale"], case["max_bias"], case["softcap"], q_quant=ca.Q8_0).numpy_f32()
+            d1 = errors(qq, like)
+            r["vs_ggml_like_oracle"] = {"default": {"max_abs": d0[0], "rel_l2": d0[1]},
+                                        "q_quant_q8_0": {"max_abs": d1[0], "rel_l2": d1[1]}}
         res[name] = r
         log(f"[bench] {name}: {us:.1f} us/call, {flops / us / 1e6:.1f} TFLOP/s, {nbytes / us / 1e3:.0f} GB/s, kernel {kern} "
             f"splits {ns}, parity max_abs={max_abs:.2e} rel_l2={rel:.2e} {'ok' if ok else 'FAIL: timing withheld'}")

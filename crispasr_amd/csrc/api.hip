@@ -158,6 +158,8 @@ int check(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor 
     }
     if (Nq * Hq * B > (int64_t)1 << 26 || Nkv > (int64_t)1 << 30) return fail(MI355X_ERR_UNSUPPORTED, "problem too large");
     if (p->prec != 0 && p->prec != 10) return fail(MI355X_ERR_INVALID, "unknown prec %d", p->prec);
+    if (p->q_quant != 0 && p->q_quant != MI355X_TYPE_Q8_0) return fail(MI355X_ERR_INVALID, "unknown q_quant %d", p->q_quant);
+    if (p->q_quant == MI355X_TYPE_Q8_0 && q->ne[0] % FATTN_QK8_0) return fail(MI355X_ERR_INVALID, "q_quant needs D %% 32 == 0");
     return MI355X_OK;
 }
 
@@ -310,6 +312,42 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
     }
 }
 
+// q_quant: the query rows rounded to Q8_0 and back, as contiguous F32 [D, Nq, Hq, B] at ws + q8_bytes
+size_t qq_q8_bytes(const mi355x_tensor * q) {
+    return ((size_t)q->ne[0] / FATTN_QK8_0 * FATTN_Q8_0_BYTES * q->ne[1] * q->ne[2] * q->ne[3] + 255) / 256 * 256;
+}
+size_t qq_f32_bytes(const mi355x_tensor * q) {
+    return ((size_t)q->ne[0] * q->ne[1] * q->ne[2] * q->ne[3] * sizeof(float) + 255) / 256 * 256;
+}
+void qq_view(const mi355x_tensor * q, void * data, mi355x_tensor * out) {
+    *out = *q;
+    out->data = data;
+    out->nb[0] = sizeof(float);
+    out->nb[1] = (size_t)q->ne[0] * sizeof(float);
+    out->nb[2] = out->nb[1] * (size_t)q->ne[1];
+    out->nb[3] = out->nb[2] * (size_t)q->ne[2];
+}
+int qq_run(const mi355x_tensor * q, void * ws, hipStream_t st) {
+    CpyArgs c;
+    memset(&c, 0, sizeof(c));
+    int64_t blocks = 1;
+    for (int i = 0; i < 4; i++) { c.sne[i] = c.dne[i] = q->ne[i]; c.snb[i] = (int64_t)q->nb[i]; }
+    const int64_t rs = q->ne[0] / FATTN_QK8_0 * FATTN_Q8_0_BYTES;
+    c.dnb[0] = FATTN_Q8_0_BYTES; c.dnb[1] = rs; c.dnb[2] = rs * q->ne[1]; c.dnb[3] = c.dnb[2] * q->ne[2];
+    blocks = q->ne[0] / FATTN_QK8_0 * q->ne[1] * q->ne[2] * q->ne[3];
+    c.src = (const char *)q->data; c.dst = (char *)ws; c.n = blocks;
+    int e = cpy_launch(c, MI355X_TYPE_F32, MI355X_TYPE_Q8_0, st);
+    if (e) return hip_fail((hipError_t)e, "query quantisation launch");
+    CpyArgs d;
+    memset(&d, 0, sizeof(d));
+    for (int i = 0; i < 4; i++) { d.sne[i] = d.dne[i] = q->ne[i]; d.snb[i] = c.dnb[i]; }
+    d.dnb[0] = 4; d.dnb[1] = 4 * q->ne[0]; d.dnb[2] = d.dnb[1] * q->ne[1]; d.dnb[3] = d.dnb[2] * q->ne[2];
+    d.src = (const char *)ws; d.dst = (char *)ws + qq_q8_bytes(q); d.n = blocks;
+    e = cpy_launch(d, MI355X_TYPE_Q8_0, MI355X_TYPE_F32, st);
+    if (e) return hip_fail((hipError_t)e, "query dequantisation launch");
+    return MI355X_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -408,7 +446,7 @@ int mi355x_fattn_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k
     fill_args(a, q, k, v, mask, nullptr, params);
     Plan plan;
     make_plan(a, k->type, params, plan);
-    *bytes = plan.workspace;
+    *bytes = plan.workspace + (params->q_quant ? qq_q8_bytes(q) + qq_f32_bytes(q) : 0);
     return MI355X_OK;
 }
 
@@ -420,6 +458,31 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     if (rc) return rc;
     if (q->ne[1] != 0 && (!q->data || !k->data || !v->data || !dst->data || (has_mask(mask) && !mask->data)))
         return fail(MI355X_ERR_INVALID, "null data pointer");
+    if (params->q_quant && (int64_t)q->ne[1] * q->ne[2] * q->ne[3] > 0) {
+        // the rounded query rows go to the head of the workspace; the call proper runs on them with what is left of it
+        const size_t qb = qq_q8_bytes(q) + qq_f32_bytes(q);
+        mi355x_fattn_params inner = *params;
+        inner.q_quant = 0;
+        size_t need = 0;
+        rc = mi355x_fattn_workspace_size(q, k, v, mask, &inner, &need);
+        if (rc) return rc;
+        void * ws = params->workspace;
+        if (ws) {
+            if (params->workspace_size < qb + need)
+                return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, qb + need);
+            if ((uintptr_t)ws % 16) return fail(MI355X_ERR_WORKSPACE, "workspace must be 16-byte aligned");
+        } else {
+            rc = get_scratch(qb + need, &ws);
+            if (rc) return rc;
+        }
+        rc = qq_run(q, ws, (hipStream_t)stream);
+        if (rc) return rc;
+        mi355x_tensor qd;
+        qq_view(q, (char *)ws + qq_q8_bytes(q), &qd);
+        inner.workspace      = need ? (char *)ws + qb : nullptr;
+        inner.workspace_size = need;
+        return mi355x_flash_attn_ext(&qd, k, v, mask, dst, &inner, stream);
+    }
     FattnArgs a;
     fill_args(a, q, k, v, mask, (float *)dst->data, params);
     if ((int64_t)a.Nq * a.Hq * a.B == 0) return MI355X_OK;

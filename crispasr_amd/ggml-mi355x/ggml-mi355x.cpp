@@ -14,6 +14,7 @@
 
 #include "mi355x_fattn.h"
 
+#include <cstdlib>
 #include <cstring>
 #include <string>
 
@@ -34,6 +35,10 @@ static mi355x_fattn_params fa_params(const ggml_tensor * node) {
     std::memcpy(&p.max_bias,      (const float *)node->op_params + 1, sizeof(float));
     std::memcpy(&p.logit_softcap, (const float *)node->op_params + 2, sizeof(float));
     p.prec = ((const int32_t *)node->op_params)[3];
+    // GGML_MI355X_MATCH_CPU=1: quantise the query rows to Q8_0 when K is Q8_0, the arithmetic ggml-cpu is recalled to
+    // use there - for comparison runs (test-backend-ops, transcript diffs), not for production
+    static const bool match_cpu = getenv("GGML_MI355X_MATCH_CPU") != nullptr;
+    if (match_cpu && node->src[1]->type == GGML_TYPE_Q8_0 && node->src[0]->ne[0] % 32 == 0) p.q_quant = MI355X_TYPE_Q8_0;
     return p;
 }
 

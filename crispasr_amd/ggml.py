@@ -55,7 +55,7 @@ class CTensor(ctypes.Structure):
 class CParams(ctypes.Structure):
     _fields_ = [("scale", ctypes.c_float), ("max_bias", ctypes.c_float), ("logit_softcap", ctypes.c_float),
                 ("prec", ctypes.c_int32), ("kernel", ctypes.c_int32), ("n_splits", ctypes.c_int32),
-                ("workspace", ctypes.c_void_p), ("workspace_size", ctypes.c_size_t)]
+                ("workspace", ctypes.c_void_p), ("workspace_size", ctypes.c_size_t), ("q_quant", ctypes.c_int32)]
 
 
 class CDeviceInfo(ctypes.Structure):
@@ -289,8 +289,9 @@ def _stream_handle(stream) -> int:
     return int(stream.cuda_stream)
 
 
-def _params(scale, max_bias, logit_softcap, prec, kernel, n_splits, workspace) -> CParams:
+def _params(scale, max_bias, logit_softcap, prec, kernel, n_splits, workspace, q_quant=0) -> CParams:
     p = CParams()
+    p.q_quant = int(q_quant)
     p.scale, p.max_bias, p.logit_softcap = float(scale), float(max_bias), float(logit_softcap)
     p.prec, p.kernel, p.n_splits = int(prec), int(kernel), int(n_splits)
     if workspace is not None:
@@ -330,9 +331,9 @@ def flash_attn_plan(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor] = No
 
 def flash_attn_workspace_size(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor] = None, scale: float = 1.0,
                               max_bias: float = 0.0, logit_softcap: float = 0.0, kernel: int = KERNEL_AUTO,
-                              n_splits: int = 0) -> int:
+                              n_splits: int = 0, q_quant: int = 0) -> int:
     """Bytes of workspace the call would use (split-KV partials, f16 copies of F32 / Q8_0 K/V); 0 if none."""
-    p = _params(scale, max_bias, logit_softcap, PREC_DEFAULT, kernel, n_splits, None)
+    p = _params(scale, max_bias, logit_softcap, PREC_DEFAULT, kernel, n_splits, None, q_quant)
     n = ctypes.c_size_t(0)
     _check(lib().mi355x_fattn_workspace_size(q.ref(), k.ref(), v.ref(), mask.ref() if mask is not None else None,
                                              ctypes.byref(p), ctypes.byref(n)))
@@ -342,14 +343,15 @@ def flash_attn_workspace_size(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Te
 def flash_attn_ext(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor], scale: float,
                    max_bias: float = 0.0, logit_softcap: float = 0.0, *, prec: int = PREC_DEFAULT,
                    kernel: int = KERNEL_AUTO, n_splits: int = 0, out: Optional[Tensor] = None,
-                   workspace: Optional[torch.Tensor] = None, stream=None) -> Tensor:
+                   workspace: Optional[torch.Tensor] = None, stream=None, q_quant: int = 0) -> Tensor:
     """ggml_flash_attn_ext(ctx, q, k, v, mask, scale, max_bias, logit_softcap) computed on the GPU.
+    q_quant = Q8_0 rounds the query rows to Q8_0 blocks first (ggml-cpu's recalled arithmetic for Q8_0 K; comparison runs).
 
     Returns the F32 result tensor with ne = [DV, Hq, Nq, B] (what the reference's callers
     immediately reshape_2d to [DV*Hq, Nq])."""
     if out is None:
         out = Tensor.empty(F32, (v.ne[0], q.ne[2], q.ne[1], q.ne[3]), device=q.buf.device)
-    p = _params(scale, max_bias, logit_softcap, prec, kernel, n_splits, workspace)
+    p = _params(scale, max_bias, logit_softcap, prec, kernel, n_splits, workspace, q_quant)
     with _on_device(q.buf.device):
         _check(lib().mi355x_flash_attn_ext(q.ref(), k.ref(), v.ref(), mask.ref() if mask is not None else None,
                                            out.ref(), ctypes.byref(p), _stream_handle(stream)))

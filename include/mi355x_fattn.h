@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define MI355X_FATTN_API_VERSION 1
+#define MI355X_FATTN_API_VERSION 2
 
 /* ggml type ids of the storage types this path meets */
 enum mi355x_type {
@@ -81,6 +81,10 @@ typedef struct mi355x_fattn_params {
                               * With a caller's workspace of mi355x_fattn_workspace_size bytes the call allocates nothing
                               * and launches kernels only (no memset or copy nodes): it may be recorded into a HIP graph. */
     size_t  workspace_size;
+    int32_t q_quant;         /* 0 = the query rows as they are.  MI355X_TYPE_Q8_0 = round every query row to Q8_0 blocks first
+                              * (d = amax/127 per 32 values), which is what ggml-cpu is recalled to do when K is Q8_0 (the
+                              * vec_dot_type of Q8_0 is Q8_0): a comparison mode for runs against ggml-cpu, two small extra
+                              * launches and D % 32 == 0; never needed for correctness. */
 } mi355x_fattn_params;
 
 typedef struct mi355x_device_info {

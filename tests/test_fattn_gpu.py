@@ -99,3 +99,35 @@ def test_device_info_reports_a_gfx950():
     assert ggml.device_count() >= 1
     assert info["arch"].startswith("gfx950")
     assert info["wavefront_size"] == 64 and info["compute_units"] >= 64
+
+
+@pytest.mark.parametrize("spec,kernel", [
+    (dict(seed=971, D=128, Nq=1, Nkv=663, Hq=32, Hkv=8, ktype=ora.Q8_0), ggml.KERNEL_AUTO),                  # decode kernel
+    (dict(seed=972, D=128, Nq=160, Nkv=200, Hq=8, Hkv=2, ktype=ora.Q8_0, mask="causal", q_layout="thd"), ggml.KERNEL_MMA),
+    (dict(seed=973, D=96, Nq=3, Nkv=130, Hq=4, ktype=ora.Q8_0), ggml.KERNEL_VEC),
+    (dict(seed=974, D=64, Nq=40, Nkv=300, Hq=6, Hkv=3, B=2, ktype=ora.Q8_0, mask="random_inf_batched"), ggml.KERNEL_AUTO),
+])
+def test_query_rows_rounded_to_q8_0_follow_the_ggml_like_oracle(spec, kernel):
+    """q_quant = Q8_0: the comparison mode for runs against ggml-cpu, which is recalled to quantise each query row to
+    Q8_0 when K is Q8_0.  The oracle's ggml-like mode does the same, so this mode must sit within the path tolerance of
+    it, while the default (exact query rows) sits an order of magnitude further away from it - and on the exact oracle."""
+    import torch
+    case = make_case(**spec)
+    like = run_oracle(case, ora.MODE_GGML_LIKE)
+    exact = run_oracle(case)
+    q, k, v = upload(case["q"]), upload(case["k"]), upload(case["v"])
+    m = upload(case["mask"]) if case["mask"] is not None else None
+    print("q_quant", spec, flush=True)
+    got_qq = ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=kernel, q_quant=ggml.Q8_0).numpy_f32()
+    got = ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=kernel).numpy_f32()
+    assert_parity(got_qq, like, "q_quant vs ggml-like oracle")
+    assert_parity(got, exact, "default vs exact oracle")
+    from cases import errors
+    assert errors(got, like)[1] > 3 * errors(got_qq, like)[1]
+    # with a caller's workspace of the size the library names: the same bits
+    need = ggml.flash_attn_workspace_size(q, k, v, m, case["scale"], kernel=kernel, q_quant=ggml.Q8_0)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    again = ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=kernel, q_quant=ggml.Q8_0, workspace=ws).numpy_f32()
+    assert np.array_equal(again, got_qq)
+    with pytest.raises(ggml.Mi355xError):
+        ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=kernel, q_quant=ggml.Q8_0, workspace=ws[: need - 256])
