@@ -505,3 +505,45 @@ def test_reference_cross_attn_unit_test_shapes_and_fill(scaled):
         attn = ora.flash_attn_ext(q_t, k_t, v_t, None, float(scale), 0.0, 0.0, mode)      # [1, T_dec, n_heads, head_dim]
         got = o_proj.reshape(d_model, qd) @ attn.reshape(qd).astype(np.float32)          # reshape_2d(attn, n_heads*head_dim, T_dec)
         assert np.abs(got - ref).max() < 1e-4, (mode, np.abs(got - ref).max())
+
+
+# ---- the reference's query-tiled BD harness: same fill, same sizes, both of its formulations -----------------------
+
+def test_relpos_mask_matches_the_reference_tiled_bd_harness():
+    # tools/dev/tiledbd_parity.cpp:1-127 proves (max abs < 1e-4) that full rel-pos attention with the monolithic
+    # rel_shift, out[k,q] = a[k-q+(T-1), q] (:29-33, :61-67), equals a query-tiled form whose block b reads
+    # BDraw_b[k - i + (T-1) - b*BS, i] (:88-93).  Same deterministic fill (:27, :112-117) and sizes (:12-23) here:
+    # the oracle's mask must be the tiled form's BD (up to its f16 rounding), and attention on it the tool's result.
+    HD, NH, T, BS = 4, 2, 12, 3
+    D = HD * NH
+    frand = lambda n, s: (np.sin((np.arange(n) + s).astype(np.float32) * np.float32(0.37)) * np.float32(0.9)).astype(np.float32)  # noqa: E731
+    Q, K3, V3 = frand(D * T, 1).reshape(T, D), frand(D * T, 100).reshape(T, NH, HD), frand(D * T, 200).reshape(T, NH, HD)
+    R0 = frand(D * (2 * T - 1), 300).reshape(2 * T - 1, D)
+    pbu, pbv = frand(D, 400), frand(D, 500)
+    scale = 1.0 / math.sqrt(HD)
+    heads = lambda x: np.ascontiguousarray(x.reshape(x.shape[0], NH, HD).transpose(1, 0, 2))     # noqa: E731  (HD, rows, NH) in ggml order
+    Qu, Qv, Kh, Vh, Rh = heads(Q + pbu), heads(Q + pbv), heads(K3.reshape(T, D)), heads(V3.reshape(T, D)), heads(R0)
+    # graph B of the tool, block by block, in float64
+    bd_tiled = np.zeros((NH, T, T))                          # [h, i (query), k (key)]
+    for h in range(NH):
+        for b in range((T + BS - 1) // BS):
+            for ib in range(BS):
+                i = b * BS + ib
+                if i >= T:
+                    continue
+                raw_b = Qv[h, i].astype(np.float64) @ Rh[h].astype(np.float64).T          # BDraw_b[:, ib], 2T-1 rows
+                off = (T - 1) - b * BS
+                for k in range(T):
+                    bd_tiled[h, i, k] = raw_b[k - ib + off]
+    out_tool = np.zeros((T, NH, HD))
+    for h in range(NH):
+        s = scale * (Qu[h].astype(np.float64) @ Kh[h].astype(np.float64).T + bd_tiled[h])     # soft_max_ext scales the sum
+        p = np.exp(s - s.max(axis=1, keepdims=True))
+        out_tool[:, h] = (p / p.sum(axis=1, keepdims=True)) @ Vh[h].astype(np.float64)
+    # the oracle: the FastConformer graph chain (scale inside the mask), then FLASH_ATTN_EXT
+    as_t = lambda x: ora.from_f32(x[None])                                                 # noqa: E731  [1, NH, rows, HD]
+    mask = ora.relpos_bias(as_t(Qv), as_t(Rh), None, scale, T)
+    m = ora.fp16_to_fp32(mask.buf.view(np.uint16)).reshape(NH, T, T)
+    assert np.abs(m - scale * bd_tiled).max() <= 2.0 ** -11 * max(1.0, np.abs(scale * bd_tiled).max()) * 1.01
+    got = ora.flash_attn_ext(as_t(Qu), as_t(Kh), as_t(Vh), mask, scale)                    # [1, T, NH, HD]
+    assert np.abs(got[0] - out_tool).max() < 1e-3           # the tool's 1e-4 plus the f16 rounding of the mask
