@@ -77,3 +77,34 @@ def test_set_rows_into_quantised_cache(dtype):
         ca.set_rows(dst, upload(ora.from_f32(x, ora.F32)), torch.from_numpy(rows).to("cuda", idx_dtype))
         torch.cuda.synchronize()
         assert np.array_equal(dst.to_host(), expect)
+
+
+@pytest.mark.parametrize("dtype,tol", [(ora.F16, 1e-3), (ora.Q8_0, 0.02)])
+def test_reference_kv_quant_roundtrip_on_the_device(dtype, tol):
+    # tests/test-kv-quant-roundtrip.cpp:93-240: write 8 rows into a fresh [128, 64, 2] cache with set_rows (I64 indices
+    # 0..7) in one graph, read the layer back as F32 through a view in a second one; values in [-1, 1] from the test's own
+    # generator (seed 0x370) must survive within the test's per-type bound (f16 1e-3, q8_0 0.02).  Same sizes, same
+    # values, same bounds, both steps on the device.
+    hd, heads, max_ctx, n = 128, 2, 64, 8
+    s = [0x370]
+
+    def sym():                                   # the test's xorshift64 generator (:44-55)
+        m = (1 << 64) - 1
+        s[0] ^= (s[0] << 13) & m
+        s[0] ^= s[0] >> 7
+        s[0] ^= (s[0] << 17) & m
+        return np.float32((((s[0] >> 11) & 0xFFFFFFFF) % 20001) / 10000.0 - 1.0)
+
+    src = np.array([sym() for _ in range(hd * n * heads)], np.float32).reshape(1, heads, n, hd)    # ne [hd, n, heads]
+    rs = ora.row_size(dtype, hd)
+    cache = ca.Tensor.from_host(np.zeros(heads * max_ctx * rs, np.uint8), dtype, (hd, max_ctx, heads, 1))
+    print("kv round trip", dtype, flush=True)
+    ca.set_rows(cache, upload(ora.from_f32(src, ora.F32)), torch.arange(n, dtype=torch.int64, device="cuda"))
+    view = cache.view((hd, n, heads, 1), (ora.TYPE_SIZE[dtype], rs, max_ctx * rs, heads * max_ctx * rs))
+    back = ca.cpy(view, ca.Tensor.empty(ca.F32, (hd, n, heads, 1)))
+    torch.cuda.synchronize()
+    got = back.numpy_f32()
+    assert np.abs(got - src).max() <= tol
+    want = ora.from_f32(src, dtype)                                          # and exactly the oracle's stored values
+    from cases import to_f32
+    assert np.array_equal(got, to_f32(want))
