@@ -511,7 +511,18 @@ def scale_check(ca, torch, layer):
     t_full = _time_calls(torch, lambda: ca.flash_attn_ext(layer["q"], layer["k"], layer["v"], None, 0.125, out=layer["out"]), 10)
     t_half = _time_calls(torch, lambda: ca.flash_attn_ext(layer["q"], half["k"], half["v"], None, 0.125, out=layer["out"]), 10)
     log(f"[bench] scale check: {N} keys: {t_full:.1f} us, {N // 2} keys: {t_half:.1f} us, ratio {t_full / t_half:.2f}")
-    return {"us_n_kv_full": t_full, "us_n_kv_half": t_half, "ratio": t_full / t_half}
+    # the form the runtime really passes: K/V views of a cache padded to 1536 rows, the 36 pad rows zero and, with no
+    # mask, part of the softmax (src/crispasr.cpp:2733, 2806-2821)
+    NP, n_state = 1536, H * D
+    pad = {}
+    for n in ("k", "v"):
+        buf = torch.zeros(B * NP * n_state * 2, dtype=torch.uint8, device="cuda")
+        src = layer[n].buf.view(torch.float16).view(B, N, n_state)
+        buf.view(torch.float16).view(B, NP, n_state)[:, :N] = src
+        pad[n] = ca.Tensor(buf, ca.F16, (D, NP, H, B), (2, 2 * n_state, 2 * D, 2 * n_state * NP))
+    t_pad = _time_calls(torch, lambda: ca.flash_attn_ext(layer["q"], pad["k"], pad["v"], None, 0.125, out=layer["out"]), 10)
+    log(f"[bench] the same layer on 1536-row zero-padded K/V views: {t_pad:.1f} us")
+    return {"us_n_kv_full": t_full, "us_n_kv_half": t_half, "ratio": t_full / t_half, "us_n_kv_1536_zero_padded": t_pad}
 
 
 def bench_whisper_protocol(args, ca, ora, torch):
