@@ -266,6 +266,21 @@ def bench_decode(args, ca, ora, torch):
     run("voxtral_decode_q8_0_gqa4", layers, 128 ** -0.5, per_call, 10,
         "1 token, 32 q / 8 kv heads, Q8_0 K/V of 663 entries; 1.44 MB per call")
 
+    # the same step as the reference's Voxtral runtime reaches the op (src/voxtral.cpp:1062, GQA_MANUAL_CONT:
+    # src/core/attention.h:917-935): K/V expanded to the 32 q heads and contiguous, F16 - or F32 when the cache is
+    # quantised and read back through ggml_cast
+    for kt, nm, es in ((ca.F16, "f16", 2), (ca.F32, "f32", 4)):
+        layers = []
+        nbe = (es, es * D, es * D * Lk, es * D * Lk * Hq)
+        for l in range(120 if kt == ca.F16 else 60):
+            kv = [torch.randn(Hq * Lk * D, device="cuda") for _ in range(2)]
+            kv = [(t.half() if kt == ca.F16 else t).view(torch.uint8) for t in kv]
+            layers.append({"q": ca.Tensor(torch.randn(Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, 1)),
+                           "k": ca.Tensor(kv[0], kt, (D, Lk, Hq, 1), nbe), "v": ca.Tensor(kv[1], kt, (D, Lk, Hq, 1), nbe),
+                           "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 1))})
+        run(f"voxtral_decode_{nm}_expanded_heads", layers, 128 ** -0.5, 2 * Lk * Hq * D * es + 2 * Hq * D * 4, 10,
+            f"1 token, K/V repeated to 32 heads as the reference's graph does, {nm}; {2 * Lk * Hq * D * es / 1e6:.1f} MB per call")
+
     # saturating variants: the same kernels with many independent sequences per call (ne3), to show
     # the bandwidth ceiling that single calls of 1-8 MB cannot reach
     Bs = 64
