@@ -272,7 +272,7 @@ def bench_decode(args, ca, ora, torch):
     for kt, nm, es in ((ca.F16, "f16", 2), (ca.F32, "f32", 4)):
         layers = []
         nbe = (es, es * D, es * D * Lk, es * D * Lk * Hq)
-        for l in range(120 if kt == ca.F16 else 60):
+        for l in range(48 if kt == ca.F16 else 24):
             kv = [torch.randn(Hq * Lk * D, device="cuda") for _ in range(2)]
             kv = [(t.half() if kt == ca.F16 else t).view(torch.uint8) for t in kv]
             layers.append({"q": ca.Tensor(torch.randn(Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, 1)),
