@@ -137,3 +137,12 @@ def test_relpos_bias_supports_predicate():
     q80 = _t(ca.F32, (80, 16, 2, 1))
     assert sup(q80, _t(ca.F32, (80, 31, 2, 1)), None, _t(ca.F16, (16, 16, 2, 1))) == ggml.ERR_UNSUPPORTED   # head size
     assert sup(_t(ca.F16, (128, T, H, 1)), r, None, dst) == ggml.ERR_UNSUPPORTED         # Q_v must be F32
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stdout + r.stderr)
