@@ -75,6 +75,18 @@ int device_cus() {
     return g_dev[dev].cus;
 }
 
+// Extents a kernel can index: none negative, each below 2^31, their product below 2^62 (n = that product).
+bool sane_extents(const mi355x_tensor * t, int64_t * n) {
+    int64_t p = 1;
+    for (int i = 0; i < 4; i++) {
+        if (t->ne[i] < 0 || t->ne[i] > 0x7fffffff) return false;
+        if (t->ne[i] > 0 && p > ((int64_t)1 << 62) / t->ne[i]) return false;
+        p *= t->ne[i];
+    }
+    if (n) *n = p;
+    return true;
+}
+
 // Library-owned scratch for the split-KV partials: one growing allocation per device.
 // Outgrown blocks stay allocated until the process ends, so launches still in flight on
 // other streams keep valid memory.
@@ -117,6 +129,9 @@ struct Plan {
 int check(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
           const mi355x_tensor * mask, const mi355x_tensor * dst, const mi355x_fattn_params * p) {
     if (!q || !k || !v || !p) return fail(MI355X_ERR_INVALID, "null argument");
+    if (!sane_extents(q, nullptr) || !sane_extents(k, nullptr) || !sane_extents(v, nullptr) ||
+        (mask && !sane_extents(mask, nullptr)) || (dst && !sane_extents(dst, nullptr)))
+        return fail(MI355X_ERR_INVALID, "negative or oversized extent");
     if (q->type != MI355X_TYPE_F32) return fail(MI355X_ERR_UNSUPPORTED, "q must be F32 (type %d)", q->type);
     if (!type_size(k->type)) return fail(MI355X_ERR_UNSUPPORTED, "K type %d not covered", k->type);
     if (k->type != v->type) return fail(MI355X_ERR_UNSUPPORTED, "K and V types differ (%d, %d)", k->type, v->type);
@@ -582,7 +597,7 @@ static int cpy_check(const mi355x_tensor * src, const mi355x_tensor * dst) {
                     (s == MI355X_TYPE_Q8_0 && (d == MI355X_TYPE_F32 || d == MI355X_TYPE_Q8_0));
     if (!ok) return fail(MI355X_ERR_UNSUPPORTED, "copy %d -> %d not covered", s, d);
     int64_t ns = 1, nd = 1;
-    for (int i = 0; i < 4; i++) { ns *= src->ne[i]; nd *= dst->ne[i]; }
+    if (!sane_extents(src, &ns) || !sane_extents(dst, &nd)) return fail(MI355X_ERR_INVALID, "negative or oversized extent");
     if (ns != nd) return fail(MI355X_ERR_INVALID, "element counts differ (%lld vs %lld)", (long long)ns, (long long)nd);
     if (dst->nb[0] != type_size(d)) return fail(MI355X_ERR_UNSUPPORTED, "dst rows must be contiguous");
     if (s == MI355X_TYPE_Q8_0 && src->nb[0] != FATTN_Q8_0_BYTES) return fail(MI355X_ERR_UNSUPPORTED, "src blocks must be contiguous");
@@ -605,6 +620,8 @@ static bool aligned16_view(const mi355x_tensor * t) {
 static int relpos_check(const mi355x_tensor * qv, const mi355x_tensor * r, const mi355x_tensor * add,
                         const mi355x_tensor * dst) {
     if (!qv || !r || !dst) return fail(MI355X_ERR_INVALID, "null argument");
+    if (!sane_extents(qv, nullptr) || !sane_extents(r, nullptr) || !sane_extents(dst, nullptr) || (add && !sane_extents(add, nullptr)))
+        return fail(MI355X_ERR_INVALID, "negative or oversized extent");
     if (qv->type != MI355X_TYPE_F32 || qv->nb[0] != 4) return fail(MI355X_ERR_UNSUPPORTED, "q_v must be F32 with unit element stride");
     if (r->type != MI355X_TYPE_F32 && r->type != MI355X_TYPE_F16) return fail(MI355X_ERR_UNSUPPORTED, "r type %d not covered", r->type);
     if (r->nb[0] != type_size(r->type)) return fail(MI355X_ERR_UNSUPPORTED, "r rows must be contiguous");
@@ -810,6 +827,7 @@ int mi355x_set_rows(const mi355x_tensor * src, const void * idx, int32_t idx_typ
                     const int64_t idx_ne[3], const size_t idx_nb[3],
                     const mi355x_tensor * dst, void * stream) {
     if (!src || !dst || !idx_ne || !idx_nb) return fail(MI355X_ERR_INVALID, "null argument");
+    if (!sane_extents(src, nullptr) || !sane_extents(dst, nullptr)) return fail(MI355X_ERR_INVALID, "negative or oversized extent");
     if (src->type != MI355X_TYPE_F32) return fail(MI355X_ERR_UNSUPPORTED, "set_rows source must be F32");
     if (!type_size(dst->type)) return fail(MI355X_ERR_UNSUPPORTED, "set_rows destination type %d", dst->type);
     if (idx_type != 64 && idx_type != 32) return fail(MI355X_ERR_INVALID, "index type must be 32 or 64");
