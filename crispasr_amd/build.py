@@ -9,7 +9,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmi355x_fattn.so")
-SOURCES = ["api.hip", "fattn_vec.hip", "fattn_mma.hip", "fattn_mma_pipe.hip", "fattn_decode.hip", "cpy.hip", "relpos.hip"]
+SOURCES = ["api.hip", "fattn_vec.hip", "fattn_mma.hip", "fattn_decode.hip", "cpy.hip", "relpos.hip"]
 
 # packed-fp32 VALU ops are switched off for all device code of this library
 HIPCC_FLAGS = [
@@ -26,9 +26,7 @@ def _hipcc() -> str:
     return "hipcc"
 
 
-# per-file flags: the pipelined kernel wants its MFMA results in ordinary VGPRs (they feed v_exp_f32 directly;
-# accumulation registers would cost two moves per score)
-PER_FILE_FLAGS = {"fattn_mma_pipe.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+PER_FILE_FLAGS: dict = {}
 
 
 def _compile(src: str, extra) -> str:

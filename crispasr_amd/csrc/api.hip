@@ -219,6 +219,7 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
     }
     a.aligned16 = al16 ? 1 : 0;
     a.n_cus = device_cus();
+    a.tile_variant = p->tile_variant;
     a.softcap = p->logit_softcap;
     a.scale   = p->logit_softcap != 0.0f ? p->scale / p->logit_softcap : p->scale;
     a.max_bias = p->max_bias;
@@ -229,6 +230,18 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
     a.m1 = powf(2.0f, -(p->max_bias / 2.0f) / n2);
     a.n_splits = 1;
     a.keys_per_split = a.Nkv;
+}
+
+// the same call on the f16 copies of K and V that kv_to_f16_launch leaves at ws: contiguous [D, Nkv, Hkv, Bk], V behind K
+void use_f16_copies(FattnArgs & a, void * ws) {
+    const size_t half = (size_t)a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t);
+    a.k = (const char *)ws;
+    a.v = (const char *)ws + half;
+    a.nbk1 = a.nbv1 = (size_t)a.D * 2;
+    a.nbk2 = a.nbv2 = a.nbk1 * a.Nkv;
+    a.nbk3 = a.nbv3 = a.nbk2 * a.Hkv;
+    a.kv_aligned16 = a.kv_aligned4 = a.kv_aligned2 = 1;
+    a.aligned16 = a.q_aligned16;
 }
 
 void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Plan & plan) {
@@ -256,6 +269,9 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
     plan.keys_per_split = a.Nkv;
     plan.workspace = 0;
     plan.kv_to_f16 = false;
+    plan.ws_partials = 0;
+    // nothing to launch (no query rows) or nothing to read (no keys: the result is zeros): one range, no workspace
+    if ((int64_t)a.Nq * a.Hq * a.B == 0 || a.Nkv == 0) return;
     // The tile kernel rounds F32 and Q8_0 K/V to f16 on their way into LDS anyway.  With enough queries to share the work it
     // is cheaper to do that once, in a copy of its own, and let the f16 path (which moves tiles global->LDS without
     // touching registers) read the result: same values, same rounding.
@@ -274,7 +290,16 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
         // Whisper-base encoder, 96 workgroups x 24 key tiles, 25.0 -> 22.0 us in two ranges and slower again in three;
         // a 407-token prefill, 128 workgroups x 7 tiles, loses 2.5 us to any split).
         const int64_t rows    = (int64_t)a.Nq * a.Hq * a.B;
-        const int64_t wgs     = (int64_t)((a.Nq + 127) / 128) * a.Hq * a.B;
+        FattnArgs b  = a;
+        int       kt = ktype;
+        if (plan.kv_to_f16) {
+            use_f16_copies(b, nullptr);
+            kt = MI355X_TYPE_F16;
+        }
+        FattnMmaVariant var;
+        fattn_mma_variant(b, kt, var);
+        const int     qpw     = var.queries_per_workgroup < 128 ? var.queries_per_workgroup : 128;   // as measured: 128-query units
+        const int64_t wgs     = (int64_t)((a.Nq + qpw - 1) / qpw) * a.Hq * a.B;
         const int     n_tiles = (a.Nkv + 63) / 64;
         int ns = p->n_splits;
         if (ns <= 0) {
@@ -451,6 +476,41 @@ int mi355x_fattn_plan(const mi355x_tensor * q, const mi355x_tensor * k, const mi
     return MI355X_OK;
 }
 
+int mi355x_fattn_plan_details(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                              const mi355x_tensor * mask, const mi355x_fattn_params * params,
+                              mi355x_fattn_plan_info * info) {
+    if (!info) return fail(MI355X_ERR_INVALID, "null argument");
+    const int rc = check(q, k, v, mask, nullptr, params);
+    if (rc) return rc;
+    FattnArgs a;
+    fill_args(a, q, k, v, mask, nullptr, params);
+    Plan plan;
+    make_plan(a, k->type, params, plan);
+    memset(info, 0, sizeof(*info));
+    info->kernel         = plan.kernel;
+    info->n_splits       = plan.n_splits;
+    info->keys_per_split = plan.keys_per_split;
+    info->kv_to_f16      = plan.kv_to_f16 ? 1 : 0;
+    info->workspace      = plan.workspace;
+    if (plan.kernel == MI355X_FATTN_MMA && fattn_mma_supported(a, k->type)) {
+        int ktype = k->type;
+        if (plan.kv_to_f16) {
+            use_f16_copies(a, nullptr);
+            ktype = MI355X_TYPE_F16;
+        }
+        a.n_splits = plan.n_splits;
+        a.keys_per_split = plan.keys_per_split;
+        FattnMmaVariant var;
+        fattn_mma_variant(a, ktype, var);
+        info->queries_per_workgroup = var.queries_per_workgroup;
+        info->query_blocks = var.query_blocks;
+        info->key_split    = var.key_split;
+        info->direct       = var.direct ? 1 : 0;
+        info->mask_dma     = var.mask_dma ? 1 : 0;
+    }
+    return MI355X_OK;
+}
+
 int mi355x_fattn_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
                                 const mi355x_tensor * mask, const mi355x_fattn_params * params,
                                 size_t * bytes) {
@@ -506,12 +566,6 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     make_plan(a, k->type, params, plan);
     hipStream_t st = (hipStream_t)stream;
 
-    if (plan.kernel == MI355X_FATTN_MMA_PIPE) {
-        if (!fattn_mma_pipe_supported(a, k->type)) return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the pipelined MFMA kernel");
-        const int e = fattn_mma_pipe_launch(a, k->type, st);
-        if (e) return hip_fail((hipError_t)e, "fattn_mma_pipe launch");
-        return MI355X_OK;
-    }
     if (plan.kernel == MI355X_FATTN_MMA) {
         if (!fattn_mma_supported(a, k->type)) return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the MFMA kernel");
         int ktype = k->type;
@@ -528,17 +582,9 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
             }
         }
         if (plan.kv_to_f16) {
-            const size_t half = (size_t)a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t);
             const int e = kv_to_f16_launch(a, k->type, ws, st);
             if (e) return hip_fail((hipError_t)e, "K/V conversion launch");
-            // the same call on the f16 copies: contiguous [D, Nkv, Hkv, Bk]
-            a.k = (const char *)ws;
-            a.v = (const char *)ws + half;
-            a.nbk1 = a.nbv1 = (size_t)a.D * 2;
-            a.nbk2 = a.nbv2 = a.nbk1 * a.Nkv;
-            a.nbk3 = a.nbv3 = a.nbk2 * a.Hkv;
-            a.kv_aligned16 = a.kv_aligned4 = a.kv_aligned2 = 1;
-            a.aligned16 = a.q_aligned16;
+            use_f16_copies(a, ws);
             ktype = MI355X_TYPE_F16;
         }
         a.n_splits = plan.n_splits;

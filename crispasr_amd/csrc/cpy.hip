@@ -116,12 +116,15 @@ __global__ void __launch_bounds__(256) set_rows_kernel(const CpyArgs a) {
     const int64_t i3 = r / a.sne[2];
     const char * ip = a.idx + i1 * a.inb[0] + (i2 % a.ine[1]) * a.inb[1] + (i3 % a.ine[2]) * a.inb[2];
     const int64_t drow = a.idx_is_i64 ? *(const int64_t *)ip : (int64_t)*(const int32_t *)ip;
+    // A row index outside the destination writes nothing (ggml-cpu asserts 0 <= idx < ne1 instead): a stale or
+    // uninitialised index tensor must not become a write outside the cache.  The lanes stay in the block's reduction.
+    const bool inside = ok && drow >= 0 && drow < a.dne[1];
     const char * sp = a.src + (i0 * UNIT + e) * a.snb[0] + i1 * a.snb[1] + i2 * a.snb[2] + i3 * a.snb[3];
     const float  x  = ok ? *(const float *)sp : 0.0f;
-    char * dp = a.dst + i0 * a.dnb[0] + drow * a.dnb[1] + i2 * a.dnb[2] + i3 * a.dnb[3];
+    char * dp = a.dst + i0 * a.dnb[0] + (inside ? drow : 0) * a.dnb[1] + i2 * a.dnb[2] + i3 * a.dnb[3];
     if (DTYPE == MI355X_TYPE_Q8_0) {
-        quantize_block_store(x, dp, e, ok);
-    } else if (ok) {
+        quantize_block_store(x, dp, e, inside);
+    } else if (inside) {
         if (DTYPE == MI355X_TYPE_F16) *(_Float16 *)dp = (_Float16)x;
         else                          *(float *)dp = x;
     }
@@ -249,6 +252,7 @@ int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream) {
 
 int set_rows_launch(const CpyArgs & a, int dtype, hipStream_t stream) {
     if (a.n == 0) return 0;
+    if (a.n > ((int64_t)1 << 38)) return (int)hipErrorInvalidValue;
     if (dtype == MI355X_TYPE_Q8_0)
         hipLaunchKernelGGL((set_rows_kernel<MI355X_TYPE_Q8_0>), dim3((unsigned)((a.n + 7) / 8)), dim3(256), 0, stream, a);
     else if (dtype == MI355X_TYPE_F16)

@@ -41,6 +41,7 @@ struct FattnArgs {
     int32_t mask_al8;    // mask base and strides are multiples of 8 bytes
     int32_t mask_al4;    // ... of 4 bytes
     int32_t n_cus;       // compute units of the device
+    int32_t tile_variant; // 0, or 16 * key_split + query_blocks forced by the caller
 
     // split-KV
     int32_t n_splits;
@@ -123,9 +124,16 @@ struct RelposArgs {
 int fattn_vec_launch(const FattnArgs & a, int ktype, hipStream_t stream);
 int fattn_merge_launch(const FattnArgs & a, hipStream_t stream);
 int fattn_mma_launch(const FattnArgs & a, int ktype, hipStream_t stream);
+// the instantiation of the tile kernel a call takes
+struct FattnMmaVariant {
+    int  query_blocks;            // 32-query blocks per wave (1 or 2)
+    int  key_split;               // 2: the waves of a workgroup pair up over the two halves of every key tile
+    int  queries_per_workgroup;
+    bool direct;                  // K/V tiles move global -> LDS without passing registers
+    bool mask_dma;                // so does the mask
+};
+void fattn_mma_variant(const FattnArgs & a, int ktype, FattnMmaVariant & v);
 bool fattn_mma_supported(const FattnArgs & a, int ktype);
-int fattn_mma_pipe_launch(const FattnArgs & a, int ktype, hipStream_t stream);
-bool fattn_mma_pipe_supported(const FattnArgs & a, int ktype);
 int fattn_decode_launch(const FattnArgs & a, int ktype, hipStream_t stream);
 bool fattn_decode_supported(const FattnArgs & a, int ktype);
 int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream);

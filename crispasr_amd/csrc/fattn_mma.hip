@@ -31,6 +31,14 @@
 // every lane pull 8-byte pieces of 32 different rows through the vector cache.
 //
 // Softmax runs in base 2: scale*log2(e) is folded into Q when it is converted to f16.
+//
+// Grids that would leave CUs idle take the key-split form (KSP = 2): a workgroup owns half as many queries and its
+// waves pair up, the two waves of a pair walking the same queries over the first and the second 32 keys of every
+// tile; the pair's partial results meet in LDS once, after the last tile.  Same LDS traffic and MFMA count in all,
+// half the work per wave.
+//
+// A 32-key block whose mask excludes every key for all of the wave's queries is skipped outright (its probabilities
+// would all be exact zeros): the upper triangle of a causal prompt, the keys beyond a padded sequence's length.
 #include "fattn_common.h"
 
 #include <stdio.h>
@@ -134,10 +142,11 @@ template <int D> __device__ __forceinline__ int swz_v(int r) { return D == 64 ? 
 
 template <int D> __device__ __forceinline__ int swz_m(int r) { return (r >> 2) & 3; }     // mask half tile: 4 chunks per row
 
-template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA>
+template <int D, int NQB, int KSP, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA>
 __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnArgs a, const int n_qtiles) {
     static_assert(!DIRECT || TYPE == MI355X_TYPE_F16, "only f16 rows can go to LDS unconverted");
     static_assert(!MDMA || (DIRECT && MASK), "the mask goes through LDS only beside directly loaded K/V");
+    static_assert(KSP == 1 || (KSP == 2 && NQB == 1 && !MDMA), "key-split form: one query block per wave, mask through registers");
     constexpr int NMH   = NQB * 2;                 // MDMA: loads per wave and half tile (16 rows x 64 bytes each)
     constexpr int MHALF = NQB * 32 * 64;           //       bytes of a wave's half-tile block; a wave owns 2 of them
     constexpr int ROWB  = D * 2;                   // DIRECT: bytes per (unpadded) row
@@ -152,7 +161,12 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     constexpr int PK   = Pitch<D>::K;
     constexpr int PV   = Pitch<D>::V;
     constexpr int BMW  = 32 * NQB;                 // queries per wave
-    constexpr int BMG  = BMW * MMA_WAVES;          // queries per workgroup
+    constexpr int BMG  = BMW * MMA_WAVES / KSP;    // queries per workgroup
+    constexpr int NKB  = 2 / KSP;                  // 32-key blocks of a tile that one wave walks
+    // Skipping excluded blocks adds a branch round the block's body.  The instantiations that already fill the register
+    // file (two query blocks per wave, 128-wide heads without key split) answer it with spills inside the tile loop, so
+    // it is left to the others: the key-split form and one query block of 64-wide heads.
+    constexpr bool SKIP = MASK && (KSP == 2 || (D == 64 && NQB == 1));
 
     extern __shared__ __attribute__((aligned(16))) _Float16 lds_raw[];
     _Float16 (*k_lds)[BC * PK] = (_Float16 (*)[BC * PK])lds_raw;
@@ -184,7 +198,10 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     const int hk = h / a.gqa;
     const int bk = b / a.bq;
 
-    const int q0 = qt * BMG + wave * BMW;          // first query of this wave
+    // KSP == 2: waves w and w + 2 share their queries; wave w takes keys 0..31 of every tile, wave w + 2 keys 32..63
+    const int qgroup = KSP == 2 ? (wave & 1) : wave;
+    const int khalf  = KSP == 2 ? (wave >> 1) : 0;
+    const int q0 = qt * BMG + qgroup * BMW;        // first query of this wave
 
     // ---- Q -> f16 B operands, scaled so that the MFMA result is already in log2 units ----
     const float qscale = SOFTCAP ? a.scale : a.scale * LOG2E;   // a.scale is scale/softcap when capped
@@ -267,6 +284,8 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             vaddr[db] = (uint32_t)((kr0 * CH + (c ^ swz_v<D>(kr0))) * 16 + 8 * (i16 & 1));
         }
     }
+    typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+    typedef uint32_t u32x2_a2 __attribute__((ext_vector_type(2), aligned(2)));
     typedef __attribute__((address_space(3))) void * lds_vptr;
     typedef const __attribute__((address_space(1))) void * glb_vptr;
     // MDMA: slot (row, s) of a half-tile block holds the 8 keys of chunk s ^ swizzle(row) of query q0 + row
@@ -299,7 +318,6 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     // from the row's last 8 valid keys instead (Nkv is even and >= 64 here, so that address is dword-aligned and
     // in bounds) and shifted down by the difference: branch-free, all loads in flight together, nothing read past
     // Nkv; the positions shifted in from beyond belong to keys that the tail tile excludes.
-    typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
     auto stage_mask_tail = [&](int j0, char * mb) __attribute__((always_inline)) {
         u32x4_a4 raw[2][NMH];
         int      sh[2][NMH];
@@ -352,6 +370,21 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         }
     };
 
+    // Key-split form with the mask in registers: a wave is alone on its SIMD there, so the mask values of a full tile
+    // are requested a tile ahead and the check for excluded blocks does not wait on memory.
+    constexpr bool MPRE = MASK && DIRECT && !MDMA && KSP == 2;
+    uint2 mpre[MPRE ? NQB : 1][4];
+    auto load_mask_ahead = [&](int j0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int qb = 0; qb < NQB; qb++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const u32x2_a2 w = *(const u32x2_a2 *)(mrow[qb] + j0 + khalf * 32 + g * 8 + hh * 4);
+                mpre[MPRE ? qb : 0][g].x = w[0];
+                mpre[MPRE ? qb : 0][g].y = w[1];
+            }
+    };
+
     float16v oacc[NQB][DB];
     float16v negm[NQB];            // -m in all 16 slots: the C operand of the first Q.K^T MFMA
     RowState st[NQB];
@@ -382,30 +415,40 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         if (MLDS && !TAIL) load_mask_half(j0, 1, mb, 0.0f);
         if (DIRECT && jn >= 0) load_direct(jn, wk, wv, tn);
 
-        // additive mask values of this lane's 32 (key, query) pairs per query block, fetched early
-        uint2 mraw[MLDS ? 1 : NQB][2][4];
-        if (MASK && !MLDS) {
+        // additive mask values of this lane's 16 (key, query) pairs per query block and 32-key block, fetched early
+        uint2 mraw[MLDS ? 1 : NQB][NKB][4];
+        if (MPRE && !TAIL) {
 #pragma unroll
             for (int qb = 0; qb < NQB; qb++)
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++)
+                for (int g = 0; g < 4; g++) mraw[MLDS ? 0 : qb][0][g] = mpre[MPRE ? qb : 0][g];
+            if (mn) load_mask_ahead(j0 + BC);
+        } else if (MASK && !MLDS) {
+#pragma unroll
+            for (int qb = 0; qb < NQB; qb++)
+#pragma unroll
+                for (int kbi = 0; kbi < NKB; kbi++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        const int key = j0 + kb * 32 + g * 8 + hh * 4;
+                        const int key = j0 + (KSP == 2 ? khalf : kbi) * 32 + g * 8 + hh * 4;
                         // Past Nkv the loads are clamped to the row's last valid pair (or element): branch-free and in
                         // bounds; what they return belongs to keys that the tail tile excludes anyway.
-                        if (!TAIL && a.mask_al8) {
-                            mraw[qb][kb][g] = *(const uint2 *)(mrow[qb] + key);
+                        if (!TAIL) {
+                            // one 8-byte load whether the row starts on 8 bytes, on a dword or only on a halfword (an odd
+                            // Nkv): the memory pipeline takes it at any halfword
+                            const u32x2_a2 w = *(const u32x2_a2 *)(mrow[qb] + key);
+                            mraw[qb][kbi][g].x = w[0];
+                            mraw[qb][kbi][g].y = w[1];
                         } else if (a.mask_al4 && !(k_end & 1)) {
-                            const int k0 = TAIL ? min(key, k_end - 2) : key, k1 = TAIL ? min(key + 2, k_end - 2) : key + 2;
-                            mraw[qb][kb][g].x = *(const uint32_t *)(mrow[qb] + k0);
-                            mraw[qb][kb][g].y = *(const uint32_t *)(mrow[qb] + k1);
+                            const int k0 = min(key, k_end - 2), k1 = min(key + 2, k_end - 2);
+                            mraw[qb][kbi][g].x = *(const uint32_t *)(mrow[qb] + k0);
+                            mraw[qb][kbi][g].y = *(const uint32_t *)(mrow[qb] + k1);
                         } else {
                             uint16_t mv[4];
 #pragma unroll
-                            for (int e = 0; e < 4; e++) mv[e] = mrow[qb][TAIL ? min(key + e, k_end - 1) : key + e];
-                            mraw[qb][kb][g].x = (uint32_t)mv[0] | ((uint32_t)mv[1] << 16);
-                            mraw[qb][kb][g].y = (uint32_t)mv[2] | ((uint32_t)mv[3] << 16);
+                            for (int e = 0; e < 4; e++) mv[e] = mrow[qb][min(key + e, k_end - 1)];
+                            mraw[qb][kbi][g].x = (uint32_t)mv[0] | ((uint32_t)mv[1] << 16);
+                            mraw[qb][kbi][g].y = (uint32_t)mv[2] | ((uint32_t)mv[3] << 16);
                         }
                     }
         }
@@ -437,13 +480,40 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         };
 
         // with few reduction steps the next block's K operands are requested a block ahead
-        constexpr bool K_AHEAD = KS <= 4;
+        constexpr bool K_AHEAD = KS <= 4 && NKB == 2;
         half8 ka[K_AHEAD ? 2 : 1][KS];
-        load_k(0, ka[0]);
+        load_k(KSP == 2 ? khalf : 0, ka[0]);
 
-        // the tile is consumed in two blocks of 32 keys to keep the score registers few
+        // the tile is consumed in blocks of 32 keys to keep the score registers few
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
+        for (int kbi = 0; kbi < NKB; kbi++) {
+            const int kb = KSP == 2 ? khalf : kbi;         // which 32 keys of the tile
+            if (MLDS && kbi == 1 && !TAIL) {
+                // the second half was requested when the tile began; the only requests that can be younger than
+                // it are the next tile's first mask half (they follow block 0)
+                if (mn) __builtin_amdgcn_s_waitcnt(0x0F70 | NMH);
+                else    __builtin_amdgcn_s_waitcnt(0x0F70);
+            }
+            // A block that the mask excludes altogether for this wave's queries - every entry -inf - contributes exact
+            // zeros: it is skipped (wave-uniform), and the softmax state stays as it is.
+            bool     excluded = false;
+            uint32_t mdiff    = 0;
+            if (SKIP) {
+#pragma unroll
+                for (int qb = 0; qb < NQB; qb++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const uint2 mv = MLDS ? *(const uint2 *)(mb + wave * (2 * MHALF) + kb * MHALF + qb * 2048 + maddr[g])
+                                              : mraw[MLDS ? 0 : qb][kbi][g];
+                        mdiff |= (mv.x ^ 0xFC00FC00u) | (mv.y ^ 0xFC00FC00u);
+                    }
+                excluded = __builtin_amdgcn_ballot_w64(mdiff != 0) == 0;
+            }
+            if (excluded) {
+                if (NKB == 2 && kbi == 0) load_k(1, ka[K_AHEAD ? 1 : 0]);
+                if (MLDS && kbi == 0 && !TAIL && mn) load_mask_half(j0 + BC, 0, mb, __uint_as_float(mdiff));
+                continue;
+            }
             // ---- S^T = K . Q^T - m  (the reference m enters as the C operand of the first MFMA) ----
             float16v s[NQB];
 #pragma unroll
@@ -459,11 +529,11 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             for (int ks = 0; ks < KS; ks++)
 #pragma unroll
                 for (int qb = 0; qb < NQB; qb++)
-                    s[qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[K_AHEAD ? kb : 0][ks], qreg[qb][ks], s[qb], 0, 0, 0);
+                    s[qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[K_AHEAD ? kbi : 0][ks], qreg[qb][ks], s[qb], 0, 0, 0);
             // operands needed next are requested now, so their LDS latency hides behind the softmax
             half8 va[2][DB];
             load_v(kb, va);
-            if (kb == 0) load_k(1, ka[K_AHEAD ? 1 : 0]);
+            if (NKB == 2 && kbi == 0) load_k(1, ka[K_AHEAD ? 1 : 0]);
 
             // ---- soft cap (this path subtracts m explicitly), mask, key tail -----------------------------
             if (SOFTCAP) {
@@ -473,12 +543,6 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
 #pragma unroll
                     for (int r = 0; r < 16; r++) s[qb][r] = c2 * fast_tanh(s[qb][r]);
             }
-            if (MLDS && kb == 1 && !TAIL) {
-                // the second half was requested when the tile began; the only requests that can be younger than
-                // it are the next tile's first mask half (they follow block 0's exponentials)
-                if (mn) __builtin_amdgcn_s_waitcnt(0x0F70 | NMH);
-                else    __builtin_amdgcn_s_waitcnt(0x0F70);
-            }
             if (MASK) {
 #pragma unroll
                 for (int qb = 0; qb < NQB; qb++)
@@ -486,7 +550,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                     for (int g = 0; g < 4; g++) {
                         // f16 halves enter the FMA directly (mixed-precision FMA, no separate conversion)
                         const uint2 mv = MLDS ? *(const uint2 *)(mb + wave * (2 * MHALF) + kb * MHALF + qb * 2048 + maddr[g])
-                                              : mraw[MLDS ? 0 : qb][kb][g];
+                                              : mraw[MLDS ? 0 : qb][kbi][g];
                         const half2v w[2] = {__builtin_bit_cast(half2v, mv.x), __builtin_bit_cast(half2v, mv.y)};
 #pragma unroll
                         for (int e = 0; e < 4; e++)
@@ -579,7 +643,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             }
 #pragma unroll
             for (int qb = 0; qb < NQB; qb++) st[qb].l += lsum[qb];
-            if (MLDS && kb == 0 && !TAIL && mn) {
+            if (MLDS && kbi == 0 && !TAIL && mn) {
                 // block 0's mask has been consumed - the sums below depend on every value of it - so its LDS
                 // block can take the next tile's
                 load_mask_half(j0 + BC, 0, mb, lsum[0] + lsum[NQB - 1]);
@@ -603,6 +667,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         char * const mb = lb + 4 * TILEB;
         load_direct(k_begin, lb, lb + 2 * TILEB, n_full == 0);
         if (MDMA && n_full > 0) load_mask_half(k_begin, 0, mb, 0.0f);
+        if (MPRE && n_full > 0) load_mask_ahead(k_begin);
         load_q();
         __builtin_amdgcn_s_waitcnt(0x0F70);          // vmcnt(0): this wave's share of the tile is in LDS
         __syncthreads();
@@ -619,7 +684,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             }
             const int  cur = (t & 1) * TILEB, nxt = TILEB - cur;
             const int  jn  = t + 1 < n_tiles ? k_begin + (t + 1) * BC : -1;
-            const bool mn  = MDMA && t + 1 < n_full;
+            const bool mn  = (MDMA || MPRE) && t + 1 < n_full;     // the next tile's mask is requested during this one
             tile(k_begin + t * BC, 0, std::false_type{}, lb + cur, lb + 2 * TILEB + cur, lb + nxt, lb + 2 * TILEB + nxt, jn, t + 1 >= n_full, mb, mn);
             // everything requested during the tile has had at least half a tile to land
             __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -648,6 +713,35 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     }
     // at most one partial tile, already staged by the last iteration above (or the prologue)
     if (n_full < n_tiles) tile(k_begin + n_full * BC, n_full & 1, std::true_type{}, nullptr, nullptr, nullptr, nullptr, -1, false, nullptr, false);
+    }
+
+    // ---- key-split form: the pair's second wave hands its state to the first through LDS (free now) ---------------
+    if (KSP == 2) {
+        constexpr int XREGS = DB * 16 + 2;                 // accumulators, reference, sum: one dword per lane each
+        __syncthreads();                                   // every wave is done with the tile buffers
+        float * xs = (float *)lds_raw + qgroup * (XREGS * 64) + lane;
+        if (khalf == 1) {
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) xs[(db * 16 + r) * 64] = oacc[0][db][r];
+            xs[(DB * 16) * 64]     = st[0].have ? st[0].m : -INFINITY;
+            xs[(DB * 16 + 1) * 64] = st[0].l;
+        }
+        __syncthreads();
+        if (khalf == 1) return;
+        const float mo = xs[(DB * 16) * 64], lo = xs[(DB * 16 + 1) * 64];
+        const bool  ho = mo > -INFINITY;
+        const float mn = fmaxf(st[0].have ? st[0].m : -INFINITY, mo);
+        const float fa = st[0].have ? __builtin_amdgcn_exp2f(st[0].m - mn) : 0.0f;
+        const float fo = ho ? __builtin_amdgcn_exp2f(mo - mn) : 0.0f;
+        st[0].l = st[0].l * fa + lo * fo;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[0][db][r] = oacc[0][db][r] * fa + xs[(db * 16 + r) * 64] * fo;
+        st[0].have = st[0].have || ho;
+        st[0].m    = st[0].have ? mn : 0.0f;
     }
 
     // ---- normalise and write dst[D, Hq, Nq, B], or hand the unnormalised partial to the merge kernel --------------
@@ -680,16 +774,17 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     }
 }
 
-template <int D, int NQB, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA>
+template <int D, int NQB, int KSP, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA>
 int launch(const FattnArgs & a, hipStream_t stream) {
-    const int bmg = 32 * NQB * MMA_WAVES;
+    const int bmg = 32 * NQB * MMA_WAVES / KSP;
     const int n_qtiles = (a.Nq + bmg - 1) / bmg;
-    const dim3 grid((unsigned)(n_qtiles * a.Hq * a.B * a.n_splits));
+    if ((int64_t)n_qtiles * a.Hq * a.B * a.n_splits > 0x7fffffff) return (int)hipErrorInvalidValue;
+    const dim3 grid((unsigned)((int64_t)n_qtiles * a.Hq * a.B * a.n_splits));
     const size_t lds = DIRECT ? (size_t)4 * BC * D * sizeof(_Float16) + (MDMA ? (size_t)MMA_WAVES * NQB * 4096 : 0)
                               : (size_t)2 * BC * (Pitch<D>::K + Pitch<D>::V) * sizeof(_Float16);
     static bool attr_set = false;     // per instantiation; the attribute only matters above 64 KiB
     if (!attr_set && lds > 64 * 1024) {
-        const hipError_t e = hipFuncSetAttribute((const void *)fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP, DIRECT, MDMA>,
+        const hipError_t e = hipFuncSetAttribute((const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return (int)e;
         attr_set = true;
@@ -697,49 +792,75 @@ int launch(const FattnArgs & a, hipStream_t stream) {
     static const bool debug = getenv("MI355X_FATTN_DEBUG") != nullptr;
     if (debug) {
         int nb = -1;
-        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void *)fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP, DIRECT, MDMA>, MMA_THREADS, lds);
-        fprintf(stderr, "[mi355x] fattn_mma<%d,%d,%d,%d,%d,%d,%d> grid %u lds %zu B, resident workgroups per CU: %d\n",
-                D, NQB, TYPE, (int)MASK, (int)SOFTCAP, (int)DIRECT, (int)MDMA, grid.x, lds, nb);
+        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA>, MMA_THREADS, lds);
+        fprintf(stderr, "[mi355x] fattn_mma<%d,%d,%d,%d,%d,%d,%d,%d> grid %u lds %zu B, resident workgroups per CU: %d\n",
+                D, NQB, KSP, TYPE, (int)MASK, (int)SOFTCAP, (int)DIRECT, (int)MDMA, grid.x, lds, nb);
     }
-    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, TYPE, MASK, SOFTCAP, DIRECT, MDMA>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
+    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
     return (int)hipGetLastError();
 }
 
-template <int D, int NQB, int TYPE, bool DIRECT>
-int launch_mask(const FattnArgs & a, hipStream_t stream) {
+template <int D, int NQB, int KSP, int TYPE, bool DIRECT>
+int launch_mask(const FattnArgs & a, const FattnMmaVariant & v, hipStream_t stream) {
     const bool mask = a.mask != nullptr;
-    if (a.softcap != 0.0f) return mask ? launch<D, NQB, TYPE, true, true, DIRECT, false>(a, stream) : launch<D, NQB, TYPE, false, true, DIRECT, false>(a, stream);
-    if (!mask) return launch<D, NQB, TYPE, false, false, DIRECT, false>(a, stream);
-    // the mask follows K/V through LDS when its rows start on dwords, Nkv is even (the tail tile's dword-aligned
-    // stand-in chunk) and a wave's row offsets fit 32 bits
-    static const bool no_mdma = getenv("MI355X_FATTN_NO_MDMA") != nullptr;          // experiments only
-    if (DIRECT && !no_mdma && a.mask_al4 && a.Nkv >= 64 && !(a.Nkv & 1) && (uint64_t)a.Nq * a.nbm1 < (1ull << 31))
-        return launch<D, NQB, TYPE, true, false, DIRECT, DIRECT>(a, stream);
-    return launch<D, NQB, TYPE, true, false, DIRECT, false>(a, stream);
+    if (KSP == 1 && a.softcap != 0.0f)
+        return mask ? launch<D, NQB, 1, TYPE, true, true, DIRECT, false>(a, stream) : launch<D, NQB, 1, TYPE, false, true, DIRECT, false>(a, stream);
+    if (!mask) return launch<D, NQB, KSP, TYPE, false, false, DIRECT, false>(a, stream);
+    if (KSP == 1 && DIRECT && v.mask_dma) return launch<D, NQB, 1, TYPE, true, false, DIRECT, DIRECT>(a, stream);
+    return launch<D, NQB, KSP, TYPE, true, false, DIRECT, false>(a, stream);
 }
 
-template <int D, int NQB, int TYPE>
-int launch_flags(const FattnArgs & a, hipStream_t stream) {
-    // f16 rows go straight to LDS when a tile's row offsets fit 32 bits
-    static const bool no_direct = getenv("MI355X_FATTN_NO_DIRECT") != nullptr;       // experiments only
-    if (TYPE == MI355X_TYPE_F16 && !no_direct && a.nbk1 < (1u << 24) && a.nbv1 < (1u << 24))
-        return launch_mask<D, NQB, MI355X_TYPE_F16, true>(a, stream);
-    return launch_mask<D, NQB, TYPE, false>(a, stream);
+template <int D, int NQB, int KSP, int TYPE>
+int launch_flags(const FattnArgs & a, const FattnMmaVariant & v, hipStream_t stream) {
+    if (TYPE == MI355X_TYPE_F16 && v.direct) return launch_mask<D, NQB, KSP, MI355X_TYPE_F16, true>(a, v, stream);
+    return launch_mask<D, NQB, KSP, TYPE, false>(a, v, stream);
 }
 
 template <int TYPE>
-int launch_type(const FattnArgs & a, hipStream_t stream) {
-    // two query blocks per wave halve the LDS operand traffic per MFMA; one block keeps more
-    // workgroups in flight when there are few queries
-    const int64_t wg2 = (int64_t)((a.Nq + 255) / 256) * a.Hq * a.B;
-    static const char * force = getenv("MI355X_FATTN_NQB");          // experiments only
-    const bool two = force ? atoi(force) == 2 : wg2 >= 128;
-    if (a.D == 64)  return two ? launch_flags<64, 2, TYPE>(a, stream) : launch_flags<64, 1, TYPE>(a, stream);
-    if (a.D == 128) return launch_flags<128, 1, TYPE>(a, stream);
+int launch_type(const FattnArgs & a, const FattnMmaVariant & v, hipStream_t stream) {
+    // the key-split form exists for f16 K/V (what F32 and Q8_0 caches have become by now when there are >= 128 queries)
+    constexpr bool SPLITTABLE = TYPE == MI355X_TYPE_F16;
+    if (a.D == 64) {
+        if (v.query_blocks == 2) return launch_flags<64, 2, 1, TYPE>(a, v, stream);
+        if (SPLITTABLE && v.key_split == 2) return launch_flags<64, 1, SPLITTABLE ? 2 : 1, TYPE>(a, v, stream);
+        return launch_flags<64, 1, 1, TYPE>(a, v, stream);
+    }
+    if (a.D == 128) {
+        if (SPLITTABLE && v.key_split == 2) return launch_flags<128, 1, SPLITTABLE ? 2 : 1, TYPE>(a, v, stream);
+        return launch_flags<128, 1, 1, TYPE>(a, v, stream);
+    }
     return (int)hipErrorInvalidValue;
 }
 
 }  // namespace
+
+// Which instantiation a call takes (also what mi355x_fattn_plan_info reports):
+//  - two query blocks per wave (256 queries per workgroup) halve the LDS operand traffic per MFMA; one block keeps
+//    more workgroups in flight when there are few queries;
+//  - the key-split form (64 queries per workgroup) when even 128-query workgroups number no more than the CUs;
+//  - f16 rows go straight to LDS when a tile's row offsets fit 32 bits;
+//  - the mask follows K/V through LDS when its rows start on dwords, Nkv is even (the tail tile's dword-aligned
+//    stand-in chunk) and a wave's row offsets fit 32 bits.
+void fattn_mma_variant(const FattnArgs & a, int ktype, FattnMmaVariant & v) {
+    static const char * force_nqb = getenv("MI355X_FATTN_NQB");               // experiments only
+    static const char * force_ksp = getenv("MI355X_FATTN_KSP");
+    static const bool   no_direct = getenv("MI355X_FATTN_NO_DIRECT") != nullptr;
+    static const bool   no_mdma   = getenv("MI355X_FATTN_NO_MDMA") != nullptr;
+    const int64_t heads = (int64_t)a.Hq * a.B;
+    const int64_t wg2 = (int64_t)((a.Nq + 255) / 256) * heads;
+    const int64_t wg1 = (int64_t)((a.Nq + 127) / 128) * heads;
+    const int     cus = a.n_cus > 0 ? a.n_cus : 256;
+    const int want_nqb = a.tile_variant ? (a.tile_variant & 15) : force_nqb ? atoi(force_nqb) : 0;
+    const int want_ksp = a.tile_variant ? (a.tile_variant >> 4) : force_ksp ? atoi(force_ksp) : 0;
+    const bool two  = a.D == 64 && (want_nqb ? want_nqb == 2 : wg2 >= 128);
+    const bool ksp2 = !two && ktype == MI355X_TYPE_F16 && a.softcap == 0.0f && (want_ksp ? want_ksp == 2 : wg1 <= cus);
+    v.query_blocks = two ? 2 : 1;
+    v.key_split    = ksp2 ? 2 : 1;
+    v.queries_per_workgroup = 32 * v.query_blocks * MMA_WAVES / v.key_split;
+    v.direct   = ktype == MI355X_TYPE_F16 && !no_direct && a.nbk1 < (1u << 24) && a.nbv1 < (1u << 24);
+    v.mask_dma = a.mask != nullptr && a.softcap == 0.0f && v.direct && !ksp2 && !no_mdma && a.mask_al4 && a.Nkv >= 64 &&
+                 !(a.Nkv & 1) && (uint64_t)a.Nq * a.nbm1 < (1ull << 31);
+}
 
 bool fattn_mma_supported(const FattnArgs & a, int ktype) {
     if (a.D != 64 && a.D != 128) return false;
@@ -750,10 +871,12 @@ bool fattn_mma_supported(const FattnArgs & a, int ktype) {
 }
 
 int fattn_mma_launch(const FattnArgs & a, int ktype, hipStream_t stream) {
+    FattnMmaVariant v;
+    fattn_mma_variant(a, ktype, v);
     switch (ktype) {
-        case MI355X_TYPE_F16:  return launch_type<MI355X_TYPE_F16>(a, stream);
-        case MI355X_TYPE_F32:  return launch_type<MI355X_TYPE_F32>(a, stream);
-        case MI355X_TYPE_Q8_0: return launch_type<MI355X_TYPE_Q8_0>(a, stream);
+        case MI355X_TYPE_F16:  return launch_type<MI355X_TYPE_F16>(a, v, stream);
+        case MI355X_TYPE_F32:  return launch_type<MI355X_TYPE_F32>(a, v, stream);
+        case MI355X_TYPE_Q8_0: return launch_type<MI355X_TYPE_Q8_0>(a, v, stream);
         default:               return (int)hipErrorInvalidValue;
     }
 }

@@ -278,6 +278,7 @@ __global__ void __launch_bounds__(256) fattn_merge_kernel(const FattnArgs a, int
 template <int TYPE>
 int launch_typed(const FattnArgs & a, hipStream_t stream) {
     const int64_t rows = (int64_t)a.Nq * a.Hq * a.B;
+    if (rows * a.n_splits > 0x7fffffff) return (int)hipErrorInvalidValue;      // one workgroup per (row, split)
     const dim3 grid((unsigned)(rows * a.n_splits));
     const dim3 block(VEC_THREADS);
     const int  lanes = (a.D + 7) / 8;

@@ -23,8 +23,10 @@ QK8_0 = 32
 TYPE_SIZE = {F32: 4, F16: 2, Q8_0: 34}
 BLOCK_SIZE = {F32: 1, F16: 1, Q8_0: QK8_0}
 
-KERNEL_AUTO, KERNEL_VEC, KERNEL_MMA, KERNEL_DECODE_MMA, KERNEL_MMA_PIPE = 0, 1, 2, 3, 4
+KERNEL_AUTO, KERNEL_VEC, KERNEL_MMA, KERNEL_DECODE_MMA = 0, 1, 2, 3
 PREC_DEFAULT, PREC_F32 = 0, 10
+# tile_variant values: 16 * key_split + query_blocks
+TILE_Q256, TILE_Q128, TILE_Q64_KEYSPLIT = 16 + 2, 16 + 1, 32 + 1
 
 OK, ERR_UNSUPPORTED, ERR_INVALID, ERR_HIP, ERR_NO_DEVICE, ERR_WORKSPACE = range(6)
 
@@ -55,7 +57,15 @@ class CTensor(ctypes.Structure):
 class CParams(ctypes.Structure):
     _fields_ = [("scale", ctypes.c_float), ("max_bias", ctypes.c_float), ("logit_softcap", ctypes.c_float),
                 ("prec", ctypes.c_int32), ("kernel", ctypes.c_int32), ("n_splits", ctypes.c_int32),
-                ("workspace", ctypes.c_void_p), ("workspace_size", ctypes.c_size_t), ("q_quant", ctypes.c_int32)]
+                ("workspace", ctypes.c_void_p), ("workspace_size", ctypes.c_size_t), ("q_quant", ctypes.c_int32),
+                ("tile_variant", ctypes.c_int32)]
+
+
+class CPlanInfo(ctypes.Structure):
+    _fields_ = [("kernel", ctypes.c_int32), ("n_splits", ctypes.c_int32), ("keys_per_split", ctypes.c_int32),
+                ("kv_to_f16", ctypes.c_int32), ("workspace", ctypes.c_size_t),
+                ("queries_per_workgroup", ctypes.c_int32), ("query_blocks", ctypes.c_int32), ("key_split", ctypes.c_int32),
+                ("direct", ctypes.c_int32), ("mask_dma", ctypes.c_int32)]
 
 
 class CDeviceInfo(ctypes.Structure):
@@ -70,7 +80,7 @@ class CDeviceInfo(ctypes.Structure):
 EXPORTS = [
     "mi355x_api_version", "mi355x_status_string", "mi355x_last_error",
     "mi355x_device_count", "mi355x_device_get_info", "mi355x_set_device", "mi355x_stream_synchronize",
-    "mi355x_fattn_supports", "mi355x_flash_attn_ext", "mi355x_fattn_workspace_size", "mi355x_fattn_plan",
+    "mi355x_fattn_supports", "mi355x_flash_attn_ext", "mi355x_fattn_workspace_size", "mi355x_fattn_plan", "mi355x_fattn_plan_details",
     "mi355x_relpos_bias_supports", "mi355x_relpos_bias", "mi355x_flash_attn_relpos", "mi355x_fattn_relpos_workspace_size",
     "mi355x_cpy_supports", "mi355x_cpy", "mi355x_set_rows",
     "mi355x_buffer_alloc", "mi355x_buffer_free", "mi355x_host_buffer_alloc", "mi355x_host_buffer_free", "mi355x_buffer_memset", "mi355x_buffer_set",
@@ -102,6 +112,7 @@ def lib() -> ctypes.CDLL:
         L.mi355x_flash_attn_ext.argtypes = [PT, PT, PT, PT, PT, PP, ctypes.c_void_p]
         L.mi355x_fattn_workspace_size.argtypes = [PT, PT, PT, PT, PP, ctypes.POINTER(ctypes.c_size_t)]
         L.mi355x_fattn_plan.argtypes = [PT, PT, PT, PT, PP, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]
+        L.mi355x_fattn_plan_details.argtypes = [PT, PT, PT, PT, PP, ctypes.POINTER(CPlanInfo)]
         L.mi355x_relpos_bias_supports.argtypes = [PT, PT, PT, PT]
         L.mi355x_relpos_bias.argtypes = [PT, PT, PT, PT, ctypes.c_float, ctypes.c_void_p]
         L.mi355x_flash_attn_relpos.argtypes = [PT, PT, PT, PT, PT, PT, PT, PP, ctypes.c_void_p]
@@ -289,9 +300,10 @@ def _stream_handle(stream) -> int:
     return int(stream.cuda_stream)
 
 
-def _params(scale, max_bias, logit_softcap, prec, kernel, n_splits, workspace, q_quant=0) -> CParams:
+def _params(scale, max_bias, logit_softcap, prec, kernel, n_splits, workspace, q_quant=0, tile_variant=0) -> CParams:
     p = CParams()
     p.q_quant = int(q_quant)
+    p.tile_variant = int(tile_variant)
     p.scale, p.max_bias, p.logit_softcap = float(scale), float(max_bias), float(logit_softcap)
     p.prec, p.kernel, p.n_splits = int(prec), int(kernel), int(n_splits)
     if workspace is not None:
@@ -329,6 +341,17 @@ def flash_attn_plan(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor] = No
     return kern.value, ns.value
 
 
+def flash_attn_plan_details(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor] = None, scale: float = 1.0,
+                            max_bias: float = 0.0, logit_softcap: float = 0.0, kernel: int = KERNEL_AUTO,
+                            n_splits: int = 0, tile_variant: int = 0) -> dict:
+    """Kernel, split count and - for the tile kernel - the instantiation the call takes."""
+    p = _params(scale, max_bias, logit_softcap, PREC_DEFAULT, kernel, n_splits, None, 0, tile_variant)
+    info = CPlanInfo()
+    _check(lib().mi355x_fattn_plan_details(q.ref(), k.ref(), v.ref(), mask.ref() if mask is not None else None,
+                                           ctypes.byref(p), ctypes.byref(info)))
+    return {f: getattr(info, f) for f, _ in CPlanInfo._fields_}
+
+
 def flash_attn_workspace_size(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor] = None, scale: float = 1.0,
                               max_bias: float = 0.0, logit_softcap: float = 0.0, kernel: int = KERNEL_AUTO,
                               n_splits: int = 0, q_quant: int = 0) -> int:
@@ -343,7 +366,8 @@ def flash_attn_workspace_size(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Te
 def flash_attn_ext(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor], scale: float,
                    max_bias: float = 0.0, logit_softcap: float = 0.0, *, prec: int = PREC_DEFAULT,
                    kernel: int = KERNEL_AUTO, n_splits: int = 0, out: Optional[Tensor] = None,
-                   workspace: Optional[torch.Tensor] = None, stream=None, q_quant: int = 0) -> Tensor:
+                   workspace: Optional[torch.Tensor] = None, stream=None, q_quant: int = 0,
+                   tile_variant: int = 0) -> Tensor:
     """ggml_flash_attn_ext(ctx, q, k, v, mask, scale, max_bias, logit_softcap) computed on the GPU.
     q_quant = Q8_0 rounds the query rows to Q8_0 blocks first (ggml-cpu's recalled arithmetic for Q8_0 K; comparison runs).
 
@@ -351,7 +375,7 @@ def flash_attn_ext(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor], scal
     immediately reshape_2d to [DV*Hq, Nq])."""
     if out is None:
         out = Tensor.empty(F32, (v.ne[0], q.ne[2], q.ne[1], q.ne[3]), device=q.buf.device)
-    p = _params(scale, max_bias, logit_softcap, prec, kernel, n_splits, workspace, q_quant)
+    p = _params(scale, max_bias, logit_softcap, prec, kernel, n_splits, workspace, q_quant, tile_variant)
     with _on_device(q.buf.device):
         _check(lib().mi355x_flash_attn_ext(q.ref(), k.ref(), v.ref(), mask.ref() if mask is not None else None,
                                            out.ref(), ctypes.byref(p), _stream_handle(stream)))

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define MI355X_FATTN_API_VERSION 2
+#define MI355X_FATTN_API_VERSION 3
 
 /* ggml type ids of the storage types this path meets */
 enum mi355x_type {
@@ -64,8 +64,7 @@ enum mi355x_fattn_kernel {
     MI355X_FATTN_AUTO       = 0,
     MI355X_FATTN_VEC        = 1,  /* split-KV vector kernel: any supported shape */
     MI355X_FATTN_MMA        = 2,  /* f16 MFMA tile kernel: prefill / encoder shapes */
-    MI355X_FATTN_DECODE_MMA = 3,  /* split-KV MFMA kernel: the query rows of a KV head 16 at a time (decode steps, short prompts) */
-    MI355X_FATTN_MMA_PIPE   = 4   /* software-pipelined variant of the tile kernel (head size 64, no mask); never chosen by AUTO */
+    MI355X_FATTN_DECODE_MMA = 3   /* split-KV MFMA kernel: the query rows of a KV head 16 at a time (decode steps, short prompts) */
 };
 
 /* op_params of the node (scale, max_bias, logit_softcap as f32, prec as i32) plus
@@ -85,6 +84,8 @@ typedef struct mi355x_fattn_params {
                               * (d = amax/127 per 32 values), which is what ggml-cpu is recalled to do when K is Q8_0 (the
                               * vec_dot_type of Q8_0 is Q8_0): a comparison mode for runs against ggml-cpu, two small extra
                               * launches and D % 32 == 0; never needed for correctness. */
+    int32_t tile_variant;    /* 0 = choose.  Else 16 * key_split + query_blocks (see mi355x_fattn_plan_info) forces that
+                              * instantiation of the tile kernel where it exists (tests, tuning); otherwise ignored. */
 } mi355x_fattn_params;
 
 typedef struct mi355x_device_info {
@@ -148,6 +149,26 @@ int mi355x_fattn_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k
 int mi355x_fattn_plan(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
                       const mi355x_tensor * mask, const mi355x_fattn_params * params,
                       int32_t * kernel, int32_t * n_splits);
+
+/* The same, with the instantiation of the tile kernel the call takes: tests assert on it that a shape reaches the kernel
+ * it is meant to reach, the benchmark names the kernel it times.  (The variant depends on the mask's address too: plan
+ * with the data pointers the call will have.) */
+typedef struct mi355x_fattn_plan_info {
+    int32_t kernel;                  /* mi355x_fattn_kernel */
+    int32_t n_splits;
+    int32_t keys_per_split;
+    int32_t kv_to_f16;               /* 1: F32 / Q8_0 K and V are rounded to f16 copies in the workspace first */
+    size_t  workspace;               /* bytes, as mi355x_fattn_workspace_size reports (without the q_quant part) */
+    /* tile kernel only (0 otherwise) */
+    int32_t queries_per_workgroup;   /* 256, 128 or 64 */
+    int32_t query_blocks;            /* 32-query blocks per wave: 1 or 2 */
+    int32_t key_split;               /* 2: the waves of a workgroup pair up over the two halves of every 64-key tile */
+    int32_t direct;                  /* K/V tiles move global -> LDS without passing registers */
+    int32_t mask_dma;                /* the mask takes the same road */
+} mi355x_fattn_plan_info;
+int mi355x_fattn_plan_details(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                              const mi355x_tensor * mask, const mi355x_fattn_params * params,
+                              mi355x_fattn_plan_info * info);
 
 /* ---- FastConformer relative-position attention (src/core/fastconformer.h:876-935) ---------- */
 

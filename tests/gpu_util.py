@@ -12,12 +12,18 @@ def upload(t: ora.Tensor) -> ca.Tensor:
     return ca.Tensor.from_host(t.buf, t.type, t.ne, t.nb, t.offset)
 
 
-def run_gpu(case: dict, kernel: int = ca.ggml.KERNEL_AUTO, n_splits: int = 0) -> np.ndarray:
+def run_gpu(case: dict, kernel: int = ca.ggml.KERNEL_AUTO, n_splits: int = 0, tile_variant: int = 0) -> np.ndarray:
     q, k, v = upload(case["q"]), upload(case["k"]), upload(case["v"])
     m = upload(case["mask"]) if case["mask"] is not None else None
     out = ca.flash_attn_ext(q, k, v, m, case["scale"], case["max_bias"], case["softcap"],
-                            kernel=kernel, n_splits=n_splits)
+                            kernel=kernel, n_splits=n_splits, tile_variant=tile_variant)
     return out.numpy_f32()          # [B, Nq, Hq, DV]
+
+
+def plan_details(case: dict, **kw) -> dict:
+    q, k, v = upload(case["q"]), upload(case["k"]), upload(case["v"])
+    m = upload(case["mask"]) if case["mask"] is not None else None
+    return ca.ggml.flash_attn_plan_details(q, k, v, m, case["scale"], case["max_bias"], case["softcap"], **kw)
 
 
 def run_oracle(case: dict, mode: int = ora.MODE_EXACT) -> np.ndarray:
