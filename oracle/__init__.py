@@ -20,7 +20,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 F32, F16, Q8_0 = 0, 1, 8
-MODE_EXACT, MODE_GGML_LIKE = 0, 1
+MODE_EXACT, MODE_GGML_LIKE, MODE_GGML_LIKE_F16_ACC = 0, 1, 2
 ROUND_NEAREST_EVEN, ROUND_HALF_AWAY = 0, 1
 QK8_0 = 32
 BLOCK_Q8_0_BYTES = 34
@@ -131,6 +131,10 @@ def lib() -> ctypes.CDLL:
         L.ora_relpos_bias.restype = ctypes.c_int
         L.ora_relpos_bias.argtypes = [ctypes.POINTER(_CTensor), ctypes.POINTER(_CTensor), ctypes.POINTER(_CTensor),
                                       ctypes.c_float, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int]
+        L.ora_alibi_slope.restype = ctypes.c_float
+        L.ora_alibi_slope.argtypes = [ctypes.c_float, ctypes.c_int64, ctypes.c_int64]
+        L.ora_vec_dot_q8_0_q8_0.restype = ctypes.c_float
+        L.ora_vec_dot_q8_0_q8_0.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
         L.ora_max_threads.restype = ctypes.c_int
         _lib = L
     return _lib
@@ -236,6 +240,19 @@ def dequantize_q8_0(raw: np.ndarray) -> np.ndarray:
     out = np.empty(n, dtype=np.float32)
     lib().ora_dequantize_row_q8_0(raw.ctypes.data, out.ctypes.data, n)
     return out
+
+
+def alibi_slope(max_bias: float, h: int, n_head: int) -> float:
+    """the factor the oracle multiplies head h's mask by"""
+    return float(lib().ora_alibi_slope(float(max_bias), int(h), int(n_head)))
+
+
+def vec_dot_q8_0_q8_0(x_raw: np.ndarray, y_raw: np.ndarray) -> float:
+    """dot product of two rows of block_q8_0 (uint8[n/32*34] each), as ggml-like mode takes it for Q8_0 K"""
+    x_raw = np.ascontiguousarray(x_raw, dtype=np.uint8).reshape(-1)
+    y_raw = np.ascontiguousarray(y_raw, dtype=np.uint8).reshape(-1)
+    assert x_raw.size == y_raw.size and x_raw.size % BLOCK_Q8_0_BYTES == 0
+    return float(lib().ora_vec_dot_q8_0_q8_0(x_raw.ctypes.data, y_raw.ctypes.data, x_raw.size // BLOCK_Q8_0_BYTES * QK8_0))
 
 
 def randn(seed: int, shape) -> np.ndarray:

@@ -194,7 +194,9 @@ static void row_to_f32(const char * p, int type, int64_t n, float * out) {
 
 /* ALiBi slope of head h; 1 when max_bias == 0.  Every call site of the reference
  * passes max_bias = 0 (e.g. src/crispasr.cpp:2821, src/core/attention.h:992).
- * Formula recalled from ggml: PARITY UNPINNED. */
+ * The formula is ggml's as recalled; at max_bias = 8 it is the published ALiBi head-slope
+ * construction (slopes of the closest power of two, then every other slope of twice that set),
+ * which is what the tests hold it to for power-of-two and other head counts. */
 static float alibi_slope(float max_bias, int64_t h, int64_t n_head) {
     if (max_bias <= 0.0f) return 1.0f;
     const uint32_t n_head_log2 = 1u << (uint32_t)floor(log2((double)n_head));
@@ -202,6 +204,22 @@ static float alibi_slope(float max_bias, int64_t h, int64_t n_head) {
     const float m1 = powf(2.0f, -(max_bias / 2.0f) / n_head_log2);
     return h < (int64_t)n_head_log2 ? powf(m0, (float)(h + 1)) : powf(m1, (float)(2 * (h - n_head_log2) + 1));
 }
+
+float ora_alibi_slope(float max_bias, int64_t h, int64_t n_head) { return alibi_slope(max_bias, h, n_head); }
+
+/* Q8_0 x Q8_0 dot product of n values, as the reference's note on its bit-matching GPU kernels describes
+ * ggml_vec_dot_q8_0_q8_0_generic (tools/upstream-prs/09-metal-q8_0-bit-match.md:29-36): per block of 32 an
+ * int8 x int8 -> int32 sum, then sumf += sumi * (d_x * d_y) in f32, the scales being the stored f16 values. */
+static float vec_dot_q8_0_q8_0(const ora_block_q8_0 * x, const ora_block_q8_0 * y, int64_t n) {
+    float sumf = 0.0f;
+    for (int64_t ib = 0; ib < n / ORA_QK8_0; ib++) {
+        int sumi = 0;
+        for (int e = 0; e < ORA_QK8_0; e++) sumi += (int)x[ib].qs[e] * (int)y[ib].qs[e];
+        sumf += (float)sumi * (h2f(x[ib].d) * h2f(y[ib].d));
+    }
+    return sumf;
+}
+float ora_vec_dot_q8_0_q8_0(const ora_block_q8_0 * x, const ora_block_q8_0 * y, int64_t n) { return vec_dot_q8_0_q8_0(x, y, n); }
 
 typedef struct {
     const ora_tensor *q, *k, *v, *mask;
@@ -258,12 +276,15 @@ static void fa_row_exact(const fa_args * a, int64_t iq1, int64_t iq2, int64_t iq
 }
 
 /* f32 online softmax in key order, the way ggml-cpu walks one query row
- * (recurrence as in src/core/cpu_attention.h:53-83).  RECALLED details, PARITY UNPINNED:
- * the Q row is converted to K's vec_dot_type (F32 for F32/F16 K in the fork -
- * tools/upstream-prs/01-cpu-f16-saturation.md:17-23 - and Q8_0 for Q8_0 K), and the
- * P.V accumulator is fp16 when V is F16. */
+ * (recurrence as in src/core/cpu_attention.h:53-83).  The Q row is converted to K's vec_dot_type:
+ * F32 for F32/F16 K in the fork (tools/upstream-prs/01-cpu-f16-saturation.md:17-23), Q8_0 for Q8_0 K,
+ * the row quantiser and the block dot product being the ones the reference's note
+ * tools/upstream-prs/09-metal-q8_0-bit-match.md:24-36 writes down; that FLASH_ATTN_EXT routes a Q8_0 K
+ * through them is recalled.  f16_acc (ORA_MODE_GGML_LIKE_F16_ACC only): the P.V accumulator is kept in
+ * fp16 when V is F16 - recalled, held by nothing in the reference's tree: a diagnostic, PARITY UNPINNED,
+ * no test asserts against it. */
 static void fa_row_ggml_like(const fa_args * a, int64_t iq1, int64_t iq2, int64_t iq3,
-                             float * tmp, float * acc32, uint16_t * acc16, ora_block_q8_0 * qq) {
+                             float * tmp, float * acc32, uint16_t * acc16, ora_block_q8_0 * qq, int f16_acc) {
     const int64_t ik2 = iq2 / (a->Hq / a->Hkv);
     const int64_t ik3 = iq3 / (a->B / a->Bk);
     const float * qrow = (const float *)row_ptr(a->q, iq1, iq2, iq3);
@@ -279,7 +300,7 @@ static void fa_row_ggml_like(const fa_args * a, int64_t iq1, int64_t iq2, int64_
     const int     vtype  = a->v->type;
     const int64_t D      = a->D;
     const int64_t DV     = a->DV;
-    const int     v_f16  = vtype == ORA_TYPE_F16;
+    const int     v_f16  = f16_acc && vtype == ORA_TYPE_F16;
 
     if (ktype == ORA_TYPE_Q8_0) ora_quantize_row_q8_0(qrow, qq, D, ORA_ROUND_NEAREST_EVEN);
 
@@ -315,12 +336,7 @@ static void fa_row_ggml_like(const fa_args * a, int64_t iq1, int64_t iq2, int64_
             for (int64_t d = 0; d < D; d++) s += h2f(kh[d]) * qrow[d];
 #endif
         } else {
-            const ora_block_q8_0 * kb = (const ora_block_q8_0 *)kp;
-            for (int64_t ib = 0; ib < D / ORA_QK8_0; ib++) {
-                int sumi = 0;
-                for (int e = 0; e < ORA_QK8_0; e++) sumi += (int)kb[ib].qs[e] * (int)qq[ib].qs[e];
-                s += (float)sumi * (h2f(kb[ib].d) * h2f(qq[ib].d));
-            }
+            s = vec_dot_q8_0_q8_0((const ora_block_q8_0 *)kp, qq, D);
         }
         s *= scale;
         if (a->softcap != 0.0f) s = a->softcap * tanhf(s);
@@ -351,7 +367,7 @@ static void fa_row_ggml_like(const fa_args * a, int64_t iq1, int64_t iq2, int64_
             if (vtype == ORA_TYPE_F32) {
                 vf = (const float *)vp;
             } else {
-                ora_dequantize_row_q8_0((const ora_block_q8_0 *)vp, tmp, DV);
+                row_to_f32(vp, vtype, DV, tmp);
                 vf = tmp;
             }
             for (int64_t d = 0; d < DV; d++) acc32[d] += vf[d] * vs;
@@ -416,7 +432,7 @@ int ora_flash_attn_ext(const ora_tensor * q, const ora_tensor * k, const ora_ten
             if (mode == ORA_MODE_EXACT) {
                 fa_row_exact(&a, iq1, iq2, iq3, s, tmp, acc);
             } else {
-                fa_row_ggml_like(&a, iq1, iq2, iq3, tmp, acc32, acc16, qq);
+                fa_row_ggml_like(&a, iq1, iq2, iq3, tmp, acc32, acc16, qq, mode == ORA_MODE_GGML_LIKE_F16_ACC);
             }
         }
         free(s); free(acc); free(tmp); free(acc32); free(acc16); free(qq);

@@ -21,13 +21,19 @@
  *   ora_flash_attn_ext, mode ORA_MODE_EXACT : pinned by the mathematics (fp64
  *       textbook softmax(scale*QK^T + mask)V written independently in numpy, closed
  *       forms, brute force) and by the layouts the call sites fix.
- *   ora_flash_attn_ext, mode ORA_MODE_GGML_LIKE (f32 online softmax, Q row
- *       quantised to Q8_0 for Q8_0 K, f16 accumulator for F16 V), and the
- *       max_bias (ALiBi) slope formula : PARITY UNPINNED - recalled
- *       behaviour of ggml-cpu that no file, test or fixture of the reference
- *       holds.  logit_softcap is pinned by its closed form only.
- *       Exact and ggml-like mode with F32 K/V are also held against the reference's own compiled scalar attention
- *       (src/core/cpu_attention.h via oracle/ref_cpu_attention.cpp -> oracle/_ref/), where its tree is present.
+ *   ora_alibi_slope (max_bias) : pinned at max_bias = 8 by the published ALiBi head-slope construction, for
+ *       power-of-two and other head counts; other values of max_bias scale the exponent the same way.
+ *   ora_vec_dot_q8_0_q8_0 and the Q-row quantisation ggml-like mode uses for Q8_0 K : pinned by the reference's
+ *       description of ggml-cpu's arithmetic (tools/upstream-prs/09-metal-q8_0-bit-match.md:24-36: d = amax/127
+ *       kept in f32 for the division, q = rint(x/d), int8 x int8 -> int32 per block, sumf += sumi * d_k * d_q) on
+ *       hand-built blocks with integer answers.
+ *   ora_flash_attn_ext, mode ORA_MODE_GGML_LIKE (f32 online softmax in key order, Q row quantised to Q8_0 for
+ *       Q8_0 K, f32 accumulator) : the recurrence is the reference's own (src/core/cpu_attention.h:53-83, compiled
+ *       into oracle/_ref/ and compared where its tree is present); that the op quantises Q for a Q8_0 K is
+ *       recalled.  logit_softcap is pinned by its closed form only.
+ *   ora_flash_attn_ext, mode ORA_MODE_GGML_LIKE_F16_ACC (the same with the P.V accumulator rounded to fp16 at
+ *       every key when V is F16) : PARITY UNPINNED - recalled behaviour of ggml-cpu that no file, test or
+ *       fixture of the reference holds.  A diagnostic: reported by the benchmark, asserted by no test.
  *   ora_relpos_bias : pinned by the reference's own graph (src/core/fastconformer.h:98-102,
  *       876-918, every node of which is restated literally, the rel_shift view as byte strides)
  *       and by the mathematics: numpy matmul + numpy.lib.stride_tricks.as_strided with the
@@ -46,7 +52,7 @@ extern "C" {
 /* ggml type ids of the types this path meets */
 enum { ORA_TYPE_F32 = 0, ORA_TYPE_F16 = 1, ORA_TYPE_Q8_0 = 8 };
 
-enum { ORA_MODE_EXACT = 0, ORA_MODE_GGML_LIKE = 1 };
+enum { ORA_MODE_EXACT = 0, ORA_MODE_GGML_LIKE = 1, ORA_MODE_GGML_LIKE_F16_ACC = 2 };
 
 /* rounding of x/d in the Q8_0 quantiser */
 enum { ORA_ROUND_NEAREST_EVEN = 0, ORA_ROUND_HALF_AWAY = 1 };
@@ -97,6 +103,10 @@ int ora_cpy_f32(const ora_tensor * src, void * dst_data, int32_t dst_type, const
  * dst f16 [n_kv, Nq, H, B] contiguous. */
 int ora_relpos_bias(const ora_tensor * qv, const ora_tensor * r, const ora_tensor * add,
                     float scale, int64_t n_kv, uint16_t * dst, int n_threads);
+
+/* pieces of the above, exported so that tests can hold them to known answers */
+float ora_alibi_slope(float max_bias, int64_t h, int64_t n_head);
+float ora_vec_dot_q8_0_q8_0(const ora_block_q8_0 * x, const ora_block_q8_0 * y, int64_t n);
 
 int ora_max_threads(void);
 

@@ -131,3 +131,33 @@ def test_query_rows_rounded_to_q8_0_follow_the_ggml_like_oracle(spec, kernel):
     assert np.array_equal(again, got_qq)
     with pytest.raises(ggml.Mi355xError):
         ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=kernel, q_quant=ggml.Q8_0, workspace=ws[: need - 256])
+
+
+def _published_alibi_slopes(n: int):
+    """ALiBi head slopes as the paper's reference implementation builds them (get_slopes): geometric from 2^(-8/n) for a
+    power-of-two head count, else those of the closest smaller power of two followed by every other slope of twice that."""
+    import math
+
+    def power_of_two(m):
+        start = 2.0 ** (-(2.0 ** -(math.log2(m) - 3)))
+        return [start * start ** i for i in range(m)]
+    if math.log2(n).is_integer():
+        return power_of_two(n)
+    closest = 2 ** math.floor(math.log2(n))
+    return power_of_two(closest) + _published_alibi_slopes(2 * closest)[0::2][: n - closest]
+
+
+@pytest.mark.parametrize("kernel", [ggml.KERNEL_VEC, ggml.KERNEL_DECODE_MMA, ggml.KERNEL_MMA], ids=["vec", "decode", "tile"])
+@pytest.mark.parametrize("n_head", [6, 8, 12, 20])
+def test_alibi_slope_applied_by_each_kernel_is_the_published_one(kernel, n_head):
+    """Zero scores, mask[j] = -j, one-hot V rows: head h's output is softmax(-slope_h * j) and gives the slope the
+    kernel applied back, independently of the oracle's own formula - head counts that are not powers of two included."""
+    Nkv, D, Nq = 8, 64, 3
+    q = ora.from_f32(np.zeros((1, n_head, Nq, D), np.float32), ora.F32)
+    k = ora.from_f32(np.ones((1, n_head, Nkv, D), np.float32), ora.F16)
+    v = ora.from_f32(np.tile(np.eye(Nkv, D, dtype=np.float32), (1, n_head, 1, 1)), ora.F16)
+    m = ora.from_f32(np.tile(-np.arange(Nkv, dtype=np.float32), (1, 1, Nq, 1)), ora.F16)
+    out = ggml.flash_attn_ext(upload(q), upload(k), upload(v), upload(m), 1.0, 8.0, kernel=kernel).numpy_f32()   # [1, Nq, H, D]
+    slopes = np.log(out[0, :, :, 0] / out[0, :, :, 1])
+    want = np.array(_published_alibi_slopes(n_head))
+    assert np.allclose(slopes, want[None, :], rtol=2e-3, atol=2e-3), (n_head, slopes[0], want)   # p is an f16 ratio in the MFMA kernels

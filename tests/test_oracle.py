@@ -547,3 +547,106 @@ def test_relpos_mask_matches_the_reference_tiled_bd_harness():
     assert np.abs(m - scale * bd_tiled).max() <= 2.0 ** -11 * max(1.0, np.abs(scale * bd_tiled).max()) * 1.01
     got = ora.flash_attn_ext(as_t(Qu), as_t(Kh), as_t(Vh), mask, scale)                    # [1, T, NH, HD]
     assert np.abs(got[0] - out_tool).max() < 1e-3           # the tool's 1e-4 plus the f16 rounding of the mask
+
+
+# ----------------------------------------------------------------------------- ALiBi slopes, Q8_0 x Q8_0 dot: known answers
+
+def _published_alibi_slopes(n: int):
+    """Head slopes as the ALiBi paper's reference implementation builds them (Press et al., "Train Short, Test Long",
+    get_slopes): a geometric sequence starting at 2^(-8/n) for a power-of-two head count; otherwise the slopes of the
+    closest smaller power of two, followed by every other slope of twice that count."""
+    def power_of_two(m):
+        start = 2.0 ** (-(2.0 ** -(math.log2(m) - 3)))
+        return [start * start ** i for i in range(m)]
+    if math.log2(n).is_integer():
+        return power_of_two(n)
+    closest = 2 ** math.floor(math.log2(n))
+    return power_of_two(closest) + _published_alibi_slopes(2 * closest)[0::2][: n - closest]
+
+
+@pytest.mark.parametrize("n_head", [1, 2, 6, 8, 12, 16, 20, 28, 32])
+def test_alibi_slopes_follow_the_published_construction(n_head):
+    want = _published_alibi_slopes(n_head)
+    got = [ora.alibi_slope(8.0, h, n_head) for h in range(n_head)]
+    assert np.allclose(got, want, rtol=2e-6, atol=0.0), (n_head, got, want)
+    # no bias, no slope
+    assert all(ora.alibi_slope(0.0, h, n_head) == 1.0 for h in range(n_head))
+    # another max_bias scales the exponent: slope(b) = slope(8) ** (b / 8)
+    got4 = [ora.alibi_slope(4.0, h, n_head) for h in range(n_head)]
+    assert np.allclose(got4, np.sqrt(want), rtol=2e-6)
+
+
+def test_alibi_slope_reaches_the_attention_result():
+    """Zero scores, mask[j] = -j and one-hot V rows: head h's output is softmax(-slope_h * j), from which the slope
+    the attention really applied is read back - for head counts that are not powers of two as well."""
+    for n_head in (6, 12, 20):
+        Nkv, D = 8, 8
+        q = ora.from_f32(np.zeros((1, n_head, 1, D), np.float32), ora.F32)
+        k = ora.from_f32(np.ones((1, n_head, Nkv, D), np.float32), ora.F16)
+        v = ora.from_f32(np.tile(np.eye(Nkv, D, dtype=np.float32), (1, n_head, 1, 1)), ora.F16)
+        m = ora.from_f32(-np.arange(Nkv, dtype=np.float32).reshape(1, 1, 1, Nkv), ora.F16)
+        want = _published_alibi_slopes(n_head)
+        for mode in (ora.MODE_EXACT, ora.MODE_GGML_LIKE):
+            out = ora.flash_attn_ext(q, k, v, m, 1.0, 8.0, 0.0, mode)          # [1, 1, n_head, D]
+            slopes = np.log(out[0, 0, :, 0] / out[0, 0, :, 1])
+            assert np.allclose(slopes, want, rtol=1e-4), (n_head, mode)
+
+
+def _q8_block(d: float, qs) -> np.ndarray:
+    raw = np.zeros(34, np.uint8)
+    raw[0:2] = np.array([d], np.float16).view(np.uint8)
+    raw[2:] = np.asarray(qs, np.int8).view(np.uint8)
+    return raw
+
+
+def test_q8_0_dot_known_answers():
+    """tools/upstream-prs/09-metal-q8_0-bit-match.md:29-36: int8 x int8 -> int32 per block of 32, then
+    sumf += sumi * d_k * d_q in f32.  Hand-built blocks whose answers are integers (or dyadic)."""
+    ones = np.ones(32, np.int8)
+    ramp = np.arange(1, 33, dtype=np.int8)                     # 1..32, sum 528, sum of squares 11440
+    alt = np.where(np.arange(32) % 2 == 0, 1, -1).astype(np.int8)
+    # one block: sumi * d_k * d_q
+    assert ora.vec_dot_q8_0_q8_0(_q8_block(0.5, ramp), _q8_block(0.25, ones)) == 528 * 0.125
+    assert ora.vec_dot_q8_0_q8_0(_q8_block(2.0, ramp), _q8_block(0.5, ramp)) == 11440.0
+    assert ora.vec_dot_q8_0_q8_0(_q8_block(1.0, ramp), _q8_block(1.0, alt)) == -16.0       # (1-2)+(3-4)+... 16 pairs
+    # extremes: 32 * (-127 * 127) does not fit 16 bits, and the sign survives
+    lo, hi = np.full(32, -127, np.int8), np.full(32, 127, np.int8)
+    assert ora.vec_dot_q8_0_q8_0(_q8_block(1.0, lo), _q8_block(1.0, hi)) == -32.0 * 127 * 127
+    assert ora.vec_dot_q8_0_q8_0(_q8_block(1.0, np.full(32, -128, np.int8)), _q8_block(1.0, lo)) == 32.0 * 128 * 127
+    # several blocks, each with its own pair of scales: 528*0.125 + 11440*1 - 16*0.0625
+    x = np.concatenate([_q8_block(0.5, ramp), _q8_block(2.0, ramp), _q8_block(0.25, ramp)])
+    y = np.concatenate([_q8_block(0.25, ones), _q8_block(0.5, ramp), _q8_block(0.25, alt)])
+    assert ora.vec_dot_q8_0_q8_0(x, y) == 66.0 + 11440.0 - 1.0
+    # a zero scale silences its block whatever the quants
+    assert ora.vec_dot_q8_0_q8_0(_q8_block(0.0, hi), _q8_block(3.0, hi)) == 0.0
+    # the scales are the stored f16 values: 0.1 is stored as 0.0999755859375
+    d = float(np.float16(0.1))
+    assert ora.vec_dot_q8_0_q8_0(_q8_block(0.1, ones), _q8_block(1.0, ones)) == np.float32(32.0) * np.float32(d)
+
+
+def test_q8_0_row_quantisation_divides_by_the_unrounded_scale():
+    """tools/upstream-prs/09-metal-q8_0-bit-match.md:24-28: d = amax/127 in f32 is what x is divided by; only the
+    stored copy is rounded to f16.  amax = 1: d = 1/127, 1/d = 127 in f32; the stored scale is 0.0078735 (f16), whose
+    reciprocal would be 127.008.  x = 63.499/127 lands on 63.499 -> 63 with the former and on 63.503 -> 64 with the
+    latter."""
+    x = np.zeros(32, np.float32)
+    x[0] = 1.0
+    x[1] = np.float32(63.499 / 127.0)
+    x[2] = np.float32(-63.499 / 127.0)
+    x[3] = 0.5                                              # 63.5: a tie, to the even 64
+    x[4] = np.float32(62.5 / 127.0)                         # not a tie in f32 (62.5/127 is not representable): 62 or 63 by value
+    d, qs = _blocks(ora.quantize_q8_0(x))
+    assert d[0] == np.float32(np.float16(1.0 / 127.0))
+    assert qs[0][0] == 127 and qs[0][1] == 63 and qs[0][2] == -63 and qs[0][3] == 64
+    # and ggml-like attention on a Q8_0 K is that quantiser followed by that dot product
+    D, Nkv = 64, 5
+    q = ora.randn(910, (1, 1, 1, D))
+    k = ora.randn(911, (1, 1, Nkv, D))
+    kq = ora.quantize_q8_0(k.reshape(-1))
+    qq = ora.quantize_q8_0(q.reshape(-1))
+    scores = np.array([ora.vec_dot_q8_0_q8_0(kq[j * 68:(j + 1) * 68], qq) for j in range(Nkv)], np.float32)
+    v = np.eye(Nkv, D, dtype=np.float32).reshape(1, 1, Nkv, D)
+    out = ora.flash_attn_ext(ora.from_f32(q), ora.Tensor(kq, ora.Q8_0, (D, Nkv, 1, 1), ora.contiguous_nb(ora.Q8_0, (D, Nkv, 1, 1))),
+                             ora.from_f32(v, ora.F32), None, 0.125, mode=ora.MODE_GGML_LIKE)
+    p = np.exp((scores * np.float32(0.125)).astype(np.float64))
+    assert np.allclose(out[0, 0, 0, :Nkv], p / p.sum(), rtol=1e-5)
