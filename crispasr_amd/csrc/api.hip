@@ -9,6 +9,11 @@
 #include <mutex>
 #include <vector>
 
+// Scratch of the allocation-free entry point: one array per GPU, part of the library's code object, so that it exists
+// once the library is loaded on a device and no call ever has to allocate it.  Host code never uses the array's name as
+// an address (here it is only a handle for the lookup below): each device holds its own copy at its own address.
+static __device__ __align__(256) unsigned char scratch[MI355X_NOALLOC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -111,6 +116,25 @@ int get_scratch(size_t bytes, void ** out) {
         s.size = want;
     }
     *out = s.ptr;
+    return MI355X_OK;
+}
+
+void * g_noalloc_scratch[64];      // per device: the address hipGetSymbolAddress gave for `scratch`
+
+// the current device's copy of `scratch`, looked up once per device
+int noalloc_scratch(void ** out) {
+    int dev = 0;
+    HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return fail(MI355X_ERR_HIP, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_noalloc_scratch[dev]) {
+        void * ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+        if (!ptr) return fail(MI355X_ERR_HIP, "hipGetSymbolAddress(scratch) returned no address");
+        g_noalloc_scratch[dev] = ptr;
+    }
+    *out = g_noalloc_scratch[dev];
     return MI355X_OK;
 }
 
@@ -448,7 +472,8 @@ int mi355x_device_get_info(int device, mi355x_device_info * info) {
 
 int mi355x_set_device(int device) {
     HIP_TRY(hipSetDevice(device));
-    return MI355X_OK;
+    void * ptr = nullptr;
+    return noalloc_scratch(&ptr);      // set-up of mi355x_flash_attn_ext_noalloc for this device happens here when the caller comes this way
 }
 
 int mi355x_stream_synchronize(void * stream) {
@@ -631,6 +656,25 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
         if (e) return hip_fail((hipError_t)e, "fattn_merge launch");
     }
     return MI355X_OK;
+}
+
+int mi355x_flash_attn_ext_noalloc(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                                  const mi355x_tensor * mask, const mi355x_tensor * dst,
+                                  const mi355x_fattn_params * params, void * stream) {
+    if (!params) return fail(MI355X_ERR_INVALID, "null argument");
+    void * ptr = nullptr;
+    int rc = noalloc_scratch(&ptr);
+    if (rc) return rc;
+    size_t need = 0;
+    rc = mi355x_fattn_workspace_size(q, k, v, mask, params, &need);
+    if (rc) return rc;
+    if (need > (size_t)MI355X_NOALLOC_SCRATCH_BYTES)
+        return fail(MI355X_ERR_WORKSPACE, "this call needs %zu bytes of scratch; the allocation-free entry point holds %zu",
+                    need, (size_t)MI355X_NOALLOC_SCRATCH_BYTES);
+    mi355x_fattn_params inner = *params;
+    inner.workspace      = ptr;          // the kernels take the array's device address as they take any workspace
+    inner.workspace_size = (size_t)MI355X_NOALLOC_SCRATCH_BYTES;
+    return mi355x_flash_attn_ext(q, k, v, mask, dst, &inner, stream);
 }
 
 // ---- copies ------------------------------------------------------------------------------

@@ -29,6 +29,7 @@ PREC_DEFAULT, PREC_F32 = 0, 10
 TILE_Q256, TILE_Q128, TILE_Q64_KEYSPLIT = 16 + 2, 16 + 1, 32 + 1
 
 OK, ERR_UNSUPPORTED, ERR_INVALID, ERR_HIP, ERR_NO_DEVICE, ERR_WORKSPACE = range(6)
+NOALLOC_SCRATCH_BYTES = 32 << 20
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # MI355X_FATTN_LIB points at an alternative build of the same library (e.g. one compiled with other flags)
@@ -80,7 +81,7 @@ class CDeviceInfo(ctypes.Structure):
 EXPORTS = [
     "mi355x_api_version", "mi355x_status_string", "mi355x_last_error",
     "mi355x_device_count", "mi355x_device_get_info", "mi355x_set_device", "mi355x_stream_synchronize",
-    "mi355x_fattn_supports", "mi355x_flash_attn_ext", "mi355x_fattn_workspace_size", "mi355x_fattn_plan", "mi355x_fattn_plan_details",
+    "mi355x_fattn_supports", "mi355x_flash_attn_ext", "mi355x_flash_attn_ext_noalloc", "mi355x_fattn_workspace_size", "mi355x_fattn_plan", "mi355x_fattn_plan_details",
     "mi355x_relpos_bias_supports", "mi355x_relpos_bias", "mi355x_flash_attn_relpos", "mi355x_fattn_relpos_workspace_size",
     "mi355x_cpy_supports", "mi355x_cpy", "mi355x_set_rows",
     "mi355x_buffer_alloc", "mi355x_buffer_free", "mi355x_host_buffer_alloc", "mi355x_host_buffer_free", "mi355x_buffer_memset", "mi355x_buffer_set",
@@ -110,6 +111,7 @@ def lib() -> ctypes.CDLL:
         L.mi355x_stream_synchronize.argtypes = [ctypes.c_void_p]
         L.mi355x_fattn_supports.argtypes = [PT, PT, PT, PT, PT, PP]
         L.mi355x_flash_attn_ext.argtypes = [PT, PT, PT, PT, PT, PP, ctypes.c_void_p]
+        L.mi355x_flash_attn_ext_noalloc.argtypes = [PT, PT, PT, PT, PT, PP, ctypes.c_void_p]
         L.mi355x_fattn_workspace_size.argtypes = [PT, PT, PT, PT, PP, ctypes.POINTER(ctypes.c_size_t)]
         L.mi355x_fattn_plan.argtypes = [PT, PT, PT, PT, PP, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]
         L.mi355x_fattn_plan_details.argtypes = [PT, PT, PT, PT, PP, ctypes.POINTER(CPlanInfo)]
@@ -367,7 +369,7 @@ def flash_attn_ext(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor], scal
                    max_bias: float = 0.0, logit_softcap: float = 0.0, *, prec: int = PREC_DEFAULT,
                    kernel: int = KERNEL_AUTO, n_splits: int = 0, out: Optional[Tensor] = None,
                    workspace: Optional[torch.Tensor] = None, stream=None, q_quant: int = 0,
-                   tile_variant: int = 0) -> Tensor:
+                   tile_variant: int = 0, no_alloc: bool = False) -> Tensor:
     """ggml_flash_attn_ext(ctx, q, k, v, mask, scale, max_bias, logit_softcap) computed on the GPU.
     q_quant = Q8_0 rounds the query rows to Q8_0 blocks first (ggml-cpu's recalled arithmetic for Q8_0 K; comparison runs).
 
@@ -376,9 +378,12 @@ def flash_attn_ext(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor], scal
     if out is None:
         out = Tensor.empty(F32, (v.ne[0], q.ne[2], q.ne[1], q.ne[3]), device=q.buf.device)
     p = _params(scale, max_bias, logit_softcap, prec, kernel, n_splits, workspace, q_quant, tile_variant)
+    # no_alloc: the entry point that takes its scratch from the library's static device array (pass `out`: the result
+    # tensor is the caller's to provide there)
+    entry = lib().mi355x_flash_attn_ext_noalloc if no_alloc else lib().mi355x_flash_attn_ext
     with _on_device(q.buf.device):
-        _check(lib().mi355x_flash_attn_ext(q.ref(), k.ref(), v.ref(), mask.ref() if mask is not None else None,
-                                           out.ref(), ctypes.byref(p), _stream_handle(stream)))
+        _check(entry(q.ref(), k.ref(), v.ref(), mask.ref() if mask is not None else None,
+                     out.ref(), ctypes.byref(p), _stream_handle(stream)))
     return out
 
 

@@ -140,6 +140,24 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
                           const mi355x_tensor * mask, const mi355x_tensor * dst,
                           const mi355x_fattn_params * params, void * stream);
 
+/*
+ * The same call for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc).  No counterpart in the reference: ggml backends allocate their pools as they go.
+ * Whatever scratch the kernels need (split-KV partials, f16 copies of F32 / Q8_0 K and V, the q_quant staging) is taken
+ * from a static device array of MI355X_NOALLOC_SCRATCH_BYTES that is part of the library's image on every GPU it is
+ * loaded on; params->workspace and workspace_size are ignored.  The call itself never calls hipMalloc, hipFree or any
+ * allocating routine and launches kernels only; a call that would need more scratch than the array holds returns
+ * MI355X_ERR_WORKSPACE and launches nothing (mi355x_fattn_workspace_size tells beforehand).
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race -
+ * serialise them, or give the overlapping ones their own workspace through mi355x_flash_attn_ext.  Nothing in the array
+ * has to start at zero: every byte a call reads has been written by that call's own kernels before.
+ * The array's address is looked up once per device, on the first call there (or in mi355x_set_device).
+ */
+#define MI355X_NOALLOC_SCRATCH_BYTES (32u << 20)
+int mi355x_flash_attn_ext_noalloc(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                                  const mi355x_tensor * mask, const mi355x_tensor * dst,
+                                  const mi355x_fattn_params * params, void * stream);
+
 /* bytes of scratch the call above would use with these shapes (0 when none) */
 int mi355x_fattn_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
                                 const mi355x_tensor * mask, const mi355x_fattn_params * params,
