@@ -101,7 +101,13 @@ struct Scratch {
 };
 Scratch g_scratch[64];
 
-int get_scratch(size_t bytes, void ** out) {
+int get_scratch(size_t bytes, void ** out, hipStream_t st) {
+    // the block is shared by every call that brings no workspace and may have to grow: neither fits a call that is
+    // being recorded into a graph, whose replays would use it long after this call returned
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess) (void)hipGetLastError();
+    else if (cs != hipStreamCaptureStatusNone)
+        return fail(MI355X_ERR_WORKSPACE, "this call needs %zu bytes of workspace: pass one while the stream is capturing", bytes);
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= 64) return fail(MI355X_ERR_HIP, "device index %d out of range", dev);
@@ -572,7 +578,7 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
                 return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, qb + need);
             if ((uintptr_t)ws % 16) return fail(MI355X_ERR_WORKSPACE, "workspace must be 16-byte aligned");
         } else {
-            rc = get_scratch(qb + need, &ws);
+            rc = get_scratch(qb + need, &ws, (hipStream_t)stream);
             if (rc) return rc;
         }
         rc = qq_run(q, ws, (hipStream_t)stream);
@@ -602,7 +608,7 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
                     return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, plan.workspace);
                 if ((uintptr_t)ws % 16) return fail(MI355X_ERR_WORKSPACE, "workspace must be 16-byte aligned");
             } else {
-                rc = get_scratch(plan.workspace, &ws);
+                rc = get_scratch(plan.workspace, &ws, (hipStream_t)stream);
                 if (rc) return rc;
             }
         }
@@ -642,7 +648,7 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
                 return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, plan.workspace);
             if ((uintptr_t)ws % 16) return fail(MI355X_ERR_WORKSPACE, "workspace must be 16-byte aligned");
         } else {
-            rc = get_scratch(plan.workspace, &ws);
+            rc = get_scratch(plan.workspace, &ws, (hipStream_t)stream);
             if (rc) return rc;
         }
         const size_t rows = (size_t)a.Nq * a.Hq * a.B;
@@ -695,6 +701,11 @@ static int cpy_check(const mi355x_tensor * src, const mi355x_tensor * dst) {
         if (src->ne[0] % FATTN_QK8_0 || dst->ne[0] % FATTN_QK8_0)
             return fail(MI355X_ERR_INVALID, "Q8_0 copies need ne0 %% 32 == 0 on both sides");
     }
+    // every access is at least element-wide (Q8_0 blocks are read and written in 2-byte units)
+    const size_t sal = s == MI355X_TYPE_F32 ? 4 : 2, dal = d == MI355X_TYPE_F32 ? 4 : 2;
+    if ((uintptr_t)src->data % sal || (uintptr_t)dst->data % dal) return fail(MI355X_ERR_UNSUPPORTED, "misaligned data pointers");
+    for (int i = 0; i < 4; i++)
+        if (src->nb[i] % sal || dst->nb[i] % dal) return fail(MI355X_ERR_UNSUPPORTED, "misaligned strides");
     return MI355X_OK;
 }
 
@@ -766,7 +777,7 @@ static int relpos_run(const mi355x_tensor * qv, const mi355x_tensor * r, const m
     if (relpos_table_bytes(r)) {
         // the kernel multiplies f16 values anyway: round the table once, into a contiguous [D, NR, Hr, Br] copy
         if (!r16) {
-            const int rc = get_scratch(relpos_table_bytes(r), &r16);
+            const int rc = get_scratch(relpos_table_bytes(r), &r16, st);
             if (rc) return rc;
         }
         CpyArgs c;
@@ -807,11 +818,23 @@ int mi355x_relpos_bias_supports(const mi355x_tensor * q_v, const mi355x_tensor *
     return relpos_check(q_v, r, add, dst);
 }
 
+int mi355x_relpos_bias_workspace_size(const mi355x_tensor * r, size_t * bytes) {
+    if (!r || !bytes) return fail(MI355X_ERR_INVALID, "null argument");
+    if (!sane_extents(r, nullptr) || !type_size(r->type)) return fail(MI355X_ERR_INVALID, "bad table");
+    *bytes = relpos_table_bytes(r);
+    return MI355X_OK;
+}
+
 int mi355x_relpos_bias(const mi355x_tensor * q_v, const mi355x_tensor * r, const mi355x_tensor * add,
-                       const mi355x_tensor * dst, float scale, void * stream) {
+                       const mi355x_tensor * dst, float scale, void * workspace, size_t workspace_size, void * stream) {
     const int rc = relpos_check(q_v, r, add, dst);
     if (rc) return rc;
-    return relpos_run(q_v, r, add, dst, scale, nullptr, (hipStream_t)stream);
+    const size_t need = relpos_table_bytes(r);
+    if (workspace && need) {
+        if (workspace_size < need) return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", workspace_size, need);
+        if ((uintptr_t)workspace % 16) return fail(MI355X_ERR_WORKSPACE, "workspace must be 16-byte aligned");
+    }
+    return relpos_run(q_v, r, add, dst, scale, need ? workspace : nullptr, (hipStream_t)stream);
 }
 
 // the mask the fused call keeps in its workspace: [Nkv, Nq, H, B] with rows padded to whole 128-byte lines
@@ -876,7 +899,7 @@ int mi355x_flash_attn_relpos(const mi355x_tensor * q_u, const mi355x_tensor * q_
             return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, mb + ib);
         if ((uintptr_t)ws % 16) return fail(MI355X_ERR_WORKSPACE, "workspace must be 16-byte aligned");
     } else {
-        rc = get_scratch(mb + ib, &ws);
+        rc = get_scratch(mb + ib, &ws, (hipStream_t)stream);
         if (rc) return rc;
     }
     m.data = ws;
@@ -913,10 +936,8 @@ int mi355x_cpy(const mi355x_tensor * src, const mi355x_tensor * dst, void * stre
     return MI355X_OK;
 }
 
-int mi355x_set_rows(const mi355x_tensor * src, const void * idx, int32_t idx_type,
-                    const int64_t idx_ne[3], const size_t idx_nb[3],
-                    const mi355x_tensor * dst, void * stream) {
-    if (!src || !dst || !idx_ne || !idx_nb) return fail(MI355X_ERR_INVALID, "null argument");
+int mi355x_set_rows_supports(const mi355x_tensor * src, int32_t idx_type, const int64_t idx_ne[3], const mi355x_tensor * dst) {
+    if (!src || !dst || !idx_ne) return fail(MI355X_ERR_INVALID, "null argument");
     if (!sane_extents(src, nullptr) || !sane_extents(dst, nullptr)) return fail(MI355X_ERR_INVALID, "negative or oversized extent");
     if (src->type != MI355X_TYPE_F32) return fail(MI355X_ERR_UNSUPPORTED, "set_rows source must be F32");
     if (!type_size(dst->type)) return fail(MI355X_ERR_UNSUPPORTED, "set_rows destination type %d", dst->type);
@@ -925,8 +946,22 @@ int mi355x_set_rows(const mi355x_tensor * src, const void * idx, int32_t idx_typ
         return fail(MI355X_ERR_INVALID, "set_rows shapes do not match");
     if (idx_ne[0] != src->ne[1] || idx_ne[1] <= 0 || idx_ne[2] <= 0 || src->ne[2] % idx_ne[1] || src->ne[3] % idx_ne[2])
         return fail(MI355X_ERR_INVALID, "set_rows index shape does not match");
+    if (src->nb[0] % 4) return fail(MI355X_ERR_UNSUPPORTED, "misaligned strides");
     if (dst->nb[0] != type_size(dst->type)) return fail(MI355X_ERR_UNSUPPORTED, "dst rows must be contiguous");
-    if (dst->type == MI355X_TYPE_Q8_0 && src->ne[0] % FATTN_QK8_0) return fail(MI355X_ERR_INVALID, "Q8_0 rows need ne0 %% 32 == 0");
+    if (block_size(dst->type) > 1 && src->ne[0] % block_size(dst->type)) return fail(MI355X_ERR_INVALID, "quantised rows need ne0 %% 32 == 0");
+    const size_t dal = dst->type == MI355X_TYPE_F32 ? 4 : 2;
+    if ((uintptr_t)src->data % 4 || (uintptr_t)dst->data % dal) return fail(MI355X_ERR_UNSUPPORTED, "misaligned data pointers");
+    for (int i = 1; i < 4; i++)
+        if (src->nb[i] % 4 || dst->nb[i] % dal) return fail(MI355X_ERR_UNSUPPORTED, "misaligned strides");
+    return MI355X_OK;
+}
+
+int mi355x_set_rows(const mi355x_tensor * src, const void * idx, int32_t idx_type,
+                    const int64_t idx_ne[3], const size_t idx_nb[3],
+                    const mi355x_tensor * dst, void * stream) {
+    if (!idx_nb) return fail(MI355X_ERR_INVALID, "null argument");
+    const int rc = mi355x_set_rows_supports(src, idx_type, idx_ne, dst);
+    if (rc) return rc;
     CpyArgs a;
     memset(&a, 0, sizeof(a));
     a.src = (const char *)src->data;

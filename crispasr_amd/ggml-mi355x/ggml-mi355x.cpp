@@ -2,9 +2,10 @@
 // it through libmi355x_fattn.so; every other op stays on ggml-cpu, routed by ggml_backend_sched.
 //
 // NOT COMPILED IN THIS REPOSITORY: ggml's headers (ggml.h, ggml-backend.h, ggml-backend-impl.h) are an empty
-// submodule in the reference tree.  The vtable layouts below are written from the v0.17 API as recalled (the
-// buffer vtable's member order is the one the reference's own initialiser uses, src/core/gguf_loader.cpp:332-344)
-// and must be checked against the real headers before this file is trusted.  Build, once ggml is available:
+// submodule in the reference tree.  The vtables below are filled member by member, by name, from the v0.17 API as
+// recalled (the buffer vtable's members are the ones the reference's own initialiser names,
+// src/core/gguf_loader.cpp:332-344): a member that the real headers do not have, or spell differently, fails to
+// compile instead of shifting function pointers into the wrong slots.  Build, once ggml is available:
 //   g++ -std=c++17 -fPIC -shared -DGGML_BACKEND_DL -I$GGML/include -I$GGML/src -I../../include \
 //       ggml-mi355x.cpp -L.. -lmi355x_fattn -o libggml-mi355x.so
 // and let ggml_backend_load_all() pick it up (examples/cli/cli.cpp:2416).
@@ -25,6 +26,23 @@ static mi355x_tensor to_mi(const ggml_tensor * t) {
     m.data = t->data;
     m.type = (int32_t)t->type;                  // GGML_TYPE_F32 = 0, F16 = 1, Q8_0 = 8: the ids the library uses
     for (int i = 0; i < 4; i++) { m.ne[i] = t->ne[i]; m.nb[i] = t->nb[i]; }
+    return m;
+}
+
+// The same at planning time (supports_op runs before the graph is allocated, data may still be NULL): the library only
+// looks at the alignment of data pointers there, so it gets the low bits the address will have.  Buffers of this backend
+// start on 256 bytes (buft_align) and the allocator places tensors on that alignment; a view adds its offset into the
+// tensor it views.
+static mi355x_tensor to_mi_planning(const ggml_tensor * t) {
+    mi355x_tensor m = to_mi(t);
+    size_t low = 0;
+    if (t->data) {
+        low = (size_t)(uintptr_t)t->data % 256;
+    } else {
+        for (const ggml_tensor * v = t; v && v->view_src; v = v->view_src) low += v->view_offs;
+        low %= 256;
+    }
+    m.data = (void *)(uintptr_t)low;            // never dereferenced by mi355x_*_supports
     return m;
 }
 
@@ -79,19 +97,19 @@ static void buf_clear(ggml_backend_buffer_t b, uint8_t v) {
     mi355x_stream_synchronize(nullptr);
 }
 
-static const ggml_backend_buffer_i mi355x_buffer_iface = {
-    /* .free_buffer   = */ buf_free,
-    /* .get_base      = */ buf_base,
-    /* .init_tensor   = */ buf_init_tensor,
-    /* .memset_tensor = */ buf_memset,
-    /* .set_tensor    = */ buf_set,
-    /* .get_tensor    = */ buf_get,
-    /* .set_tensor_2d = */ nullptr,
-    /* .get_tensor_2d = */ nullptr,
-    /* .cpy_tensor    = */ buf_cpy,
-    /* .clear         = */ buf_clear,
-    /* .reset         = */ nullptr,
-};
+static ggml_backend_buffer_i make_buffer_iface() {
+    ggml_backend_buffer_i i = {};
+    i.free_buffer   = buf_free;
+    i.get_base      = buf_base;
+    i.init_tensor   = buf_init_tensor;
+    i.memset_tensor = buf_memset;
+    i.set_tensor    = buf_set;
+    i.get_tensor    = buf_get;
+    i.cpy_tensor    = buf_cpy;
+    i.clear         = buf_clear;
+    return i;                                   // set_tensor_2d, get_tensor_2d, reset: NULL (optional)
+}
+static const ggml_backend_buffer_i mi355x_buffer_iface = make_buffer_iface();
 
 template <bool DEVICE>
 static ggml_backend_buffer_t buft_alloc(ggml_backend_buffer_type_t buft, size_t size) {
@@ -109,14 +127,25 @@ static bool   buft_is_host(ggml_backend_buffer_type_t)  { return true; }
 static bool   buft_not_host(ggml_backend_buffer_type_t) { return false; }
 
 static ggml_backend_dev_t g_dev();
+template <bool DEVICE>
+static ggml_backend_buffer_type make_buft() {
+    ggml_backend_buffer_type t = {};
+    t.iface.get_name       = DEVICE ? buft_dev_name : buft_host_name;
+    t.iface.alloc_buffer   = buft_alloc<DEVICE>;
+    t.iface.get_alignment  = buft_align;
+    t.iface.get_max_size   = buft_max;
+    t.iface.get_alloc_size = buft_alloc_size;
+    t.iface.is_host        = DEVICE ? buft_not_host : buft_is_host;
+    t.device  = g_dev();
+    t.context = nullptr;
+    return t;
+}
 static ggml_backend_buffer_type_t mi355x_host_buft() {
-    static ggml_backend_buffer_type t = {
-        { buft_host_name, buft_alloc<false>, buft_align, buft_max, buft_alloc_size, buft_is_host }, g_dev(), nullptr };
+    static ggml_backend_buffer_type t = make_buft<false>();
     return &t;
 }
 static ggml_backend_buffer_type_t mi355x_dev_buft() {
-    static ggml_backend_buffer_type t = {
-        { buft_dev_name, buft_alloc<true>, buft_align, buft_max, buft_alloc_size, buft_not_host }, g_dev(), nullptr };
+    static ggml_backend_buffer_type t = make_buft<true>();
     return &t;
 }
 
@@ -126,22 +155,25 @@ static bool dev_supports_op(ggml_backend_dev_t, const ggml_tensor * op) {
     switch (op->op) {
         case GGML_OP_FLASH_ATTN_EXT: {
             if (op->src[4]) return false;                      // sinks
-            mi355x_tensor q = to_mi(op->src[0]), k = to_mi(op->src[1]), v = to_mi(op->src[2]), d = to_mi(op);
+            // a view that would fail the library's alignment checks at launch is refused here, so that the scheduler
+            // leaves the node on the CPU instead of getting GGML_STATUS_FAILED from graph_compute
+            const mi355x_tensor q = to_mi_planning(op->src[0]), k = to_mi_planning(op->src[1]), v = to_mi_planning(op->src[2]),
+                                d = to_mi_planning(op);
             mi355x_tensor m;
-            if (op->src[3]) m = to_mi(op->src[3]);
+            if (op->src[3]) m = to_mi_planning(op->src[3]);
             const mi355x_fattn_params p = fa_params(op);
-            q.data = k.data = v.data = d.data = nullptr;        // planning happens before allocation
             return mi355x_fattn_supports(&q, &k, &v, op->src[3] ? &m : nullptr, &d, &p) == MI355X_OK;
         }
         case GGML_OP_CPY: case GGML_OP_CONT: case GGML_OP_DUP: {
-            mi355x_tensor s = to_mi(op->src[0]), d = to_mi(op);
+            const mi355x_tensor s = to_mi_planning(op->src[0]), d = to_mi_planning(op);
             return mi355x_cpy_supports(&s, &d) == MI355X_OK;
         }
         case GGML_OP_SET_ROWS: {                                // the write into a quantised KV cache (src/core/attention.h:366-376)
             const ggml_tensor * src = op->src[0], * idx = op->src[1];
-            if (src->type != GGML_TYPE_F32 || (idx->type != GGML_TYPE_I64 && idx->type != GGML_TYPE_I32)) return false;
-            if (op->type != GGML_TYPE_F32 && op->type != GGML_TYPE_F16 && op->type != GGML_TYPE_Q8_0) return false;
-            return src->nb[0] == sizeof(float) && op->nb[0] == ggml_type_size(op->type);
+            if (idx->type != GGML_TYPE_I64 && idx->type != GGML_TYPE_I32) return false;
+            const mi355x_tensor s = to_mi_planning(src), d = to_mi_planning(op);
+            const int64_t ine[3] = {idx->ne[0], idx->ne[1], idx->ne[2]};
+            return mi355x_set_rows_supports(&s, idx->type == GGML_TYPE_I64 ? 64 : 32, ine, &d) == MI355X_OK;   // the library's own shape checks
         }
         case GGML_OP_NONE: case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE:
             return true;                                        // no-ops on any backend
@@ -199,22 +231,15 @@ static enum ggml_status be_graph_compute(ggml_backend_t, ggml_cgraph * g) {
     return mi355x_stream_synchronize(nullptr) == MI355X_OK ? GGML_STATUS_SUCCESS : GGML_STATUS_FAILED;
 }
 
-static const ggml_backend_i mi355x_backend_iface = {
-    /* .get_name           = */ be_name,
-    /* .free               = */ be_free,
-    /* .set_tensor_async   = */ nullptr,
-    /* .get_tensor_async   = */ nullptr,
-    /* .cpy_tensor_async   = */ nullptr,
-    /* .synchronize        = */ be_sync,
-    /* .graph_plan_create  = */ nullptr,
-    /* .graph_plan_free    = */ nullptr,
-    /* .graph_plan_update  = */ nullptr,
-    /* .graph_plan_compute = */ nullptr,
-    /* .graph_compute      = */ be_graph_compute,
-    /* .event_record       = */ nullptr,
-    /* .event_wait         = */ nullptr,
-    /* .graph_optimize     = */ nullptr,
-};
+static ggml_backend_i make_backend_iface() {
+    ggml_backend_i i = {};                      // every optional member (async copies, graph plans, events, graph_optimize) stays NULL
+    i.get_name      = be_name;
+    i.free          = be_free;
+    i.synchronize   = be_sync;
+    i.graph_compute = be_graph_compute;
+    return i;
+}
+static const ggml_backend_i mi355x_backend_iface = make_backend_iface();
 
 static ggml_guid_t mi355x_guid() {
     static ggml_guid guid = {0x6d, 0x69, 0x33, 0x35, 0x35, 0x78, 0x2d, 0x66, 0x61, 0x74, 0x74, 0x6e, 0x00, 0x00, 0x00, 0x01};
@@ -239,20 +264,40 @@ static enum ggml_backend_dev_type dev_type(ggml_backend_dev_t) { return GGML_BAC
 static void dev_props(ggml_backend_dev_t d, ggml_backend_dev_props * p) {
     p->name = dev_name(d); p->description = dev_desc(d); p->type = dev_type(d);
     dev_memory(d, &p->memory_free, &p->memory_total);
-    p->caps = { /* async */ false, /* host_buffer */ true, /* buffer_from_host_ptr */ false, /* events */ false };
+    p->caps = {};
+    p->caps.async                = false;
+    p->caps.host_buffer          = true;
+    p->caps.buffer_from_host_ptr = false;
+    p->caps.events               = false;
 }
 static ggml_backend_t dev_init(ggml_backend_dev_t d, const char *) {
     if (mi355x_set_device(0) != MI355X_OK) return nullptr;     // callers fall back to the CPU backend (src/voxtral.cpp:842-845)
-    return new ggml_backend{ mi355x_guid(), mi355x_backend_iface, d, nullptr };
+    ggml_backend * be = new ggml_backend();
+    be->guid    = mi355x_guid();
+    be->iface   = mi355x_backend_iface;
+    be->device  = d;
+    be->context = nullptr;
+    return be;
 }
 static ggml_backend_buffer_type_t dev_buft(ggml_backend_dev_t)      { return mi355x_host_buft(); }
 static ggml_backend_buffer_type_t dev_host_buft(ggml_backend_dev_t) { return mi355x_host_buft(); }
 
-static const ggml_backend_device_i mi355x_device_iface = {
-    dev_name, dev_desc, dev_memory, dev_type, dev_props, dev_init, dev_buft, dev_host_buft,
-    /* buffer_from_host_ptr */ nullptr, dev_supports_op, dev_supports_buft, dev_offload_op,
-    /* event_new */ nullptr, /* event_free */ nullptr, /* event_synchronize */ nullptr,
-};
+static ggml_backend_device_i make_device_iface() {
+    ggml_backend_device_i i = {};               // buffer_from_host_ptr and the event members stay NULL
+    i.get_name             = dev_name;
+    i.get_description      = dev_desc;
+    i.get_memory           = dev_memory;
+    i.get_type             = dev_type;
+    i.get_props            = dev_props;
+    i.init_backend         = dev_init;
+    i.get_buffer_type      = dev_buft;
+    i.get_host_buffer_type = dev_host_buft;
+    i.supports_op          = dev_supports_op;
+    i.supports_buft        = dev_supports_buft;
+    i.offload_op           = dev_offload_op;
+    return i;
+}
+static const ggml_backend_device_i mi355x_device_iface = make_device_iface();
 
 static const char * reg_name(ggml_backend_reg_t) { return "MI355X"; }
 static size_t reg_count(ggml_backend_reg_t) { int n = 0; mi355x_device_count(&n); return n > 0 ? 1 : 0; }
@@ -260,11 +305,26 @@ static ggml_backend_dev_t reg_dev(ggml_backend_reg_t, size_t) { return g_dev(); 
 static void * reg_proc(ggml_backend_reg_t, const char *) { return nullptr; }
 
 extern "C" ggml_backend_reg_t ggml_backend_mi355x_reg(void) {
-    static ggml_backend_reg reg = { GGML_BACKEND_API_VERSION, { reg_name, reg_count, reg_dev, reg_proc }, nullptr };
+    static ggml_backend_reg reg = [] {
+        ggml_backend_reg r = {};
+        r.api_version            = GGML_BACKEND_API_VERSION;
+        r.iface.get_name         = reg_name;
+        r.iface.get_device_count = reg_count;
+        r.iface.get_device       = reg_dev;
+        r.iface.get_proc_address = reg_proc;
+        r.context                = nullptr;
+        return r;
+    }();
     return &reg;
 }
 static ggml_backend_dev_t g_dev() {
-    static ggml_backend_device dev = { mi355x_device_iface, ggml_backend_mi355x_reg(), nullptr };
+    static ggml_backend_device dev = [] {
+        ggml_backend_device d = {};
+        d.iface   = mi355x_device_iface;
+        d.reg     = ggml_backend_mi355x_reg();
+        d.context = nullptr;
+        return d;
+    }();
     return &dev;
 }
 

@@ -82,8 +82,8 @@ EXPORTS = [
     "mi355x_api_version", "mi355x_status_string", "mi355x_last_error",
     "mi355x_device_count", "mi355x_device_get_info", "mi355x_set_device", "mi355x_stream_synchronize",
     "mi355x_fattn_supports", "mi355x_flash_attn_ext", "mi355x_flash_attn_ext_noalloc", "mi355x_fattn_workspace_size", "mi355x_fattn_plan", "mi355x_fattn_plan_details",
-    "mi355x_relpos_bias_supports", "mi355x_relpos_bias", "mi355x_flash_attn_relpos", "mi355x_fattn_relpos_workspace_size",
-    "mi355x_cpy_supports", "mi355x_cpy", "mi355x_set_rows",
+    "mi355x_relpos_bias_supports", "mi355x_relpos_bias", "mi355x_relpos_bias_workspace_size", "mi355x_flash_attn_relpos", "mi355x_fattn_relpos_workspace_size",
+    "mi355x_cpy_supports", "mi355x_cpy", "mi355x_set_rows", "mi355x_set_rows_supports",
     "mi355x_buffer_alloc", "mi355x_buffer_free", "mi355x_host_buffer_alloc", "mi355x_host_buffer_free", "mi355x_buffer_memset", "mi355x_buffer_set",
     "mi355x_buffer_get", "mi355x_buffer_copy",
 ]
@@ -116,7 +116,9 @@ def lib() -> ctypes.CDLL:
         L.mi355x_fattn_plan.argtypes = [PT, PT, PT, PT, PP, ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int32)]
         L.mi355x_fattn_plan_details.argtypes = [PT, PT, PT, PT, PP, ctypes.POINTER(CPlanInfo)]
         L.mi355x_relpos_bias_supports.argtypes = [PT, PT, PT, PT]
-        L.mi355x_relpos_bias.argtypes = [PT, PT, PT, PT, ctypes.c_float, ctypes.c_void_p]
+        L.mi355x_relpos_bias.argtypes = [PT, PT, PT, PT, ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+        L.mi355x_relpos_bias_workspace_size.argtypes = [PT, ctypes.POINTER(ctypes.c_size_t)]
+        L.mi355x_set_rows_supports.argtypes = [PT, ctypes.c_int32, ctypes.POINTER(ctypes.c_int64), PT]
         L.mi355x_flash_attn_relpos.argtypes = [PT, PT, PT, PT, PT, PT, PT, PP, ctypes.c_void_p]
         L.mi355x_fattn_relpos_workspace_size.argtypes = [PT, PT, PT, PT, PT, PT, PP, ctypes.POINTER(ctypes.c_size_t)]
         L.mi355x_cpy_supports.argtypes = [PT, PT]
@@ -240,7 +242,9 @@ class Tensor:
 
     def data_ptr(self) -> int:
         if self.buf is None:
-            return 0
+            # planning before allocation: the predicates never dereference, they only look at the address's low bits
+            # (buffers start on 256 bytes, so the view's offset modulo 256 stands for them)
+            return self.offset % 256
         if self.offset + self.span() > self.buf.numel():
             raise InvalidError(ERR_INVALID, "tensor view exceeds its buffer")
         return self.buf.data_ptr() + self.offset
@@ -387,8 +391,15 @@ def flash_attn_ext(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor], scal
     return out
 
 
+def relpos_bias_workspace_size(r: Tensor) -> int:
+    """Bytes of workspace relpos_bias uses for this table (0: an F16 table with contiguous rows is read in place)."""
+    n = ctypes.c_size_t(0)
+    _check(lib().mi355x_relpos_bias_workspace_size(r.ref(), ctypes.byref(n)))
+    return n.value
+
+
 def relpos_bias(q_v: Tensor, r: Tensor, add: Optional[Tensor], scale: float, n_kv: Optional[int] = None, *,
-                out: Optional[Tensor] = None, stream=None) -> Tensor:
+                out: Optional[Tensor] = None, workspace: Optional[torch.Tensor] = None, stream=None) -> Tensor:
     """The F16 mask core_conformer::build_block builds for its flash-attention call (src/core/fastconformer.h:880-918):
     cast_f16(scale * rel_shift(mul_mat(cont(R), Q_v)) [+ add]).  Returns it with ne = [n_kv, Nq, H, B]."""
     if out is None:
@@ -397,7 +408,9 @@ def relpos_bias(q_v: Tensor, r: Tensor, add: Optional[Tensor], scale: float, n_k
         out = Tensor.empty(F16, (n_kv, q_v.ne[1], q_v.ne[2], q_v.ne[3]), device=q_v.buf.device)
     with _on_device(q_v.buf.device):
         _check(lib().mi355x_relpos_bias(q_v.ref(), r.ref(), add.ref() if add is not None else None, out.ref(),
-                                        float(scale), _stream_handle(stream)))
+                                        float(scale), workspace.data_ptr() if workspace is not None else None,
+                                        workspace.numel() * workspace.element_size() if workspace is not None else 0,
+                                        _stream_handle(stream)))
     return out
 
 
@@ -431,6 +444,12 @@ def cpy(src: Tensor, dst: Tensor, stream=None) -> Tensor:
     with torch.cuda.device(dst.buf.device):
         _check(lib().mi355x_cpy(ctypes.byref(cs), ctypes.byref(cd), _stream_handle(stream)))
     return dst
+
+
+def set_rows_supports(dst: Tensor, src: Tensor, n_idx: Sequence[int], idx_bits: int = 64) -> int:
+    """planning predicate of set_rows: idx extents [n_rows, I1, I2] in ggml order, idx type 64 or 32"""
+    ine3 = tuple(int(x) for x in n_idx) + (1,) * (3 - len(n_idx))
+    return lib().mi355x_set_rows_supports(src.ref(), idx_bits, (ctypes.c_int64 * 3)(*ine3), dst.ref())
 
 
 def set_rows(dst: Tensor, src: Tensor, idx: torch.Tensor, stream=None) -> Tensor:

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define MI355X_FATTN_API_VERSION 3
+#define MI355X_FATTN_API_VERSION 4
 
 /* ggml type ids of the storage types this path meets */
 enum mi355x_type {
@@ -76,8 +76,10 @@ typedef struct mi355x_fattn_params {
     int32_t prec;            /* GGML_PREC_DEFAULT = 0, GGML_PREC_F32 = 10; accumulation is f32 either way */
     int32_t kernel;          /* mi355x_fattn_kernel */
     int32_t n_splits;        /* 0 = choose; forces the KV split count of the split-KV kernels */
-    void *  workspace;       /* NULL = library-owned scratch (grown with hipMalloc when needed); else 16-byte aligned.
-                              * With a caller's workspace of mi355x_fattn_workspace_size bytes the call allocates nothing
+    void *  workspace;       /* NULL = library-owned scratch: one block per device, grown with hipMalloc when needed and
+                              * shared by every call that passes NULL, so such calls belong on one stream at a time; a
+                              * call that needs scratch is refused (MI355X_ERR_WORKSPACE) while its stream is capturing.
+                              * Else 16-byte aligned.  With a caller's workspace of mi355x_fattn_workspace_size bytes the call allocates nothing
                               * and launches kernels only (no memset or copy nodes): it may be recorded into a HIP graph. */
     size_t  workspace_size;
     int32_t q_quant;         /* 0 = the query rows as they are.  MI355X_TYPE_Q8_0 = round every query row to Q8_0 blocks first
@@ -130,7 +132,10 @@ int mi355x_stream_synchronize(void * stream);
  *
  * mi355x_fattn_supports is the predicate the backend's supports_op mirrors: it returns
  * MI355X_OK, MI355X_ERR_UNSUPPORTED or MI355X_ERR_INVALID without touching the device.
- * Data pointers may be NULL there (graph planning happens before allocation).
+ * Data pointers are never dereferenced there: they may be NULL (graph planning happens before allocation), or carry
+ * just the low bits the address will have (say offset-into-buffer modulo 256 for buffers that start on 256 bytes), so
+ * that a view whose address would fail the alignment rules above at launch is answered MI355X_ERR_UNSUPPORTED at
+ * planning already (the strides are always checked).  The same holds for the other *_supports predicates.
  */
 int mi355x_fattn_supports(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
                           const mi355x_tensor * mask, const mi355x_tensor * dst,
@@ -212,8 +217,12 @@ int mi355x_fattn_plan_details(const mi355x_tensor * q, const mi355x_tensor * k, 
  */
 int mi355x_relpos_bias_supports(const mi355x_tensor * q_v, const mi355x_tensor * r, const mi355x_tensor * add,
                                 const mi355x_tensor * dst);
+/* workspace: room for the f16 copy of an F32 or strided table (mi355x_relpos_bias_workspace_size bytes, 16-byte aligned;
+ * 0 for an F16 table with contiguous rows), or NULL to use the library's per-device scratch block under the rules of
+ * mi355x_fattn_params.workspace (one stream at a time, refused while the stream is capturing). */
+int mi355x_relpos_bias_workspace_size(const mi355x_tensor * r, size_t * bytes);
 int mi355x_relpos_bias(const mi355x_tensor * q_v, const mi355x_tensor * r, const mi355x_tensor * add,
-                       const mi355x_tensor * dst, float scale, void * stream);
+                       const mi355x_tensor * dst, float scale, void * workspace, size_t workspace_size, void * stream);
 
 /*
  * The whole flash branch of that block (fastconformer.h:915-934) in one call:
@@ -236,7 +245,11 @@ int mi355x_fattn_relpos_workspace_size(const mi355x_tensor * q_u, const mi355x_t
  * dst[i] = convert(src[i]) for tensors of equal ne.  Supported: F32 -> F32 | F16 | Q8_0,
  * F16 -> F16 | F32, Q8_0 -> F32 | Q8_0.  F32 -> F16 rounds to nearest even; F32 -> Q8_0
  * uses d = amax/127, q = round-to-nearest-even(x * (1/d)) per block of 32 along
- * dimension 0.  src may have any strides; dst rows (dimension 0) must be contiguous.
+ * dimension 0: the rounding of ggml-cpu's vectorised quantiser as the reference describes it
+ * (tools/upstream-prs/09-metal-q8_0-bit-match.md:24-28, rint / vcvtnq); ggml's scalar reference quantiser is recalled to
+ * round halves away from zero instead, so a value that lands exactly on a tie (x/d = k + 0.5) may differ by one step from
+ * a cache written by a backend that follows the scalar code - tie behaviour is not pinned by anything in the reference.
+ * src may have any strides; dst rows (dimension 0) must be contiguous.
  */
 int mi355x_cpy_supports(const mi355x_tensor * src, const mi355x_tensor * dst);
 int mi355x_cpy(const mi355x_tensor * src, const mi355x_tensor * dst, void * stream);
@@ -247,6 +260,10 @@ int mi355x_cpy(const mi355x_tensor * src, const mi355x_tensor * dst, void * stre
  * src F32 [n0, n_rows, n2, n3]; idx I64 (idx_type 64) or I32 (idx_type 32) with
  * ne = {n_rows, I1, I2} and byte strides idx_nb; dst F32 | F16 | Q8_0 [n0, rows, n2, n3].
  */
+/* Rows whose index lies outside [0, rows) are not written (ggml-cpu asserts on them): a stale or uninitialised index
+ * tensor cannot become a write outside the cache.  mi355x_set_rows_supports is the planning predicate (shapes, types,
+ * alignment; data pointers as for mi355x_fattn_supports). */
+int mi355x_set_rows_supports(const mi355x_tensor * src, int32_t idx_type, const int64_t idx_ne[3], const mi355x_tensor * dst);
 int mi355x_set_rows(const mi355x_tensor * src, const void * idx, int32_t idx_type,
                     const int64_t idx_ne[3], const size_t idx_nb[3],
                     const mi355x_tensor * dst, void * stream);

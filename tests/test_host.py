@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(L, n), f"{n} declared in include/mi355x_fattn.h but not exported"
     assert sorted(ggml.EXPORTS) == names
-    assert L.mi355x_api_version() == 3
+    assert L.mi355x_api_version() == 4
     assert L.mi355x_status_string(0) == b"ok"
 
 
@@ -146,3 +146,78 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode != 0
     assert "one GPU" in (r.stdout + r.stderr)
+
+
+def test_planning_sees_the_alignment_a_view_will_have():
+    """supports_op runs before allocation: the predicates take the low bits of the future address in the data
+    field (never dereferenced), so a view that would be refused at launch is refused at planning already."""
+    H, D = 8, 64
+    q = _t(ca.F32, (D, 4, H, 1))
+    k = _t(ca.F16, (D, 32, H, 1))
+    assert ggml.flash_attn_supports(q, k, k, None) == ggml.OK
+    for off, want in ((0, ggml.OK), (256, ggml.OK), (16, ggml.OK), (2, ggml.OK), (1, ggml.ERR_UNSUPPORTED), (7, ggml.ERR_UNSUPPORTED)):
+        kv = ca.Tensor(None, ca.F16, (D, 32, H, 1), offset=off)
+        assert ggml.flash_attn_supports(q, kv, kv, None) == want, off
+    assert ggml.flash_attn_supports(ca.Tensor(None, ca.F32, (D, 4, H, 1), offset=4), k, k, None) == ggml.OK
+    assert ggml.flash_attn_supports(ca.Tensor(None, ca.F32, (D, 4, H, 1), offset=2), k, k, None) == ggml.ERR_UNSUPPORTED
+    # the plan follows the alignment too: the tile kernel's direct-to-LDS loads need 16-byte rows
+    qb = _t(ca.F32, (D, 256, H, 1))
+    kb = _t(ca.F16, (D, 512, H, 1))
+    assert ggml.flash_attn_plan_details(qb, kb, kb, None, kernel=ggml.KERNEL_MMA)["direct"] == 1
+    ko = ca.Tensor(None, ca.F16, (D, 512, H, 1), offset=2)
+    assert ggml.flash_attn_plan_details(qb, ko, ko, None, kernel=ggml.KERNEL_MMA)["direct"] == 0
+    # Q8_0 blocks are 34 bytes: the kernels read them in 2-byte units
+    kq = ca.Tensor(None, ca.Q8_0, (D, 32, H, 1), offset=34)
+    assert ggml.flash_attn_supports(q, kq, kq, None) == ggml.OK
+    kq = ca.Tensor(None, ca.Q8_0, (D, 32, H, 1), offset=35)
+    assert ggml.flash_attn_supports(q, kq, kq, None) == ggml.ERR_UNSUPPORTED
+    # the copies
+    cpy_supports = lambda a, b: ggml.lib().mi355x_cpy_supports(a.ref(), b.ref())
+    src = _t(ca.F32, (D, 4, H, 1))
+    assert cpy_supports(src, ca.Tensor(None, ca.F16, (D, 4, H, 1), offset=2)) == ggml.OK
+    assert cpy_supports(src, ca.Tensor(None, ca.F16, (D, 4, H, 1), offset=1)) == ggml.ERR_UNSUPPORTED
+    assert cpy_supports(ca.Tensor(None, ca.F32, (D, 4, H, 1), offset=2), _t(ca.F16, (D, 4, H, 1))) == ggml.ERR_UNSUPPORTED
+
+
+def test_set_rows_supports_checks_shapes_types_and_alignment():
+    D, rows = 128, 64
+    dst = _t(ca.Q8_0, (D, rows, 8, 1))
+    src = _t(ca.F32, (D, 3, 8, 1))
+    assert ggml.set_rows_supports(dst, src, (3,)) == ggml.OK
+    assert ggml.set_rows_supports(dst, src, (3,), 32) == ggml.OK
+    assert ggml.set_rows_supports(dst, src, (3,), 16) != ggml.OK                               # no such index type
+    assert ggml.set_rows_supports(dst, src, (4,)) == ggml.ERR_INVALID                          # one index per source row
+    assert ggml.set_rows_supports(dst, _t(ca.F32, (64, 3, 8, 1)), (3,)) == ggml.ERR_INVALID    # row length
+    assert ggml.set_rows_supports(dst, _t(ca.F32, (D, 3, 4, 1)), (3,)) == ggml.ERR_INVALID     # planes
+    assert ggml.set_rows_supports(dst, src, (3, 3)) == ggml.ERR_INVALID                        # 8 % 3: index planes must divide
+    assert ggml.set_rows_supports(dst, src, (3, 2)) == ggml.OK
+    assert ggml.set_rows_supports(dst, _t(ca.F16, (D, 3, 8, 1)), (3,)) == ggml.ERR_UNSUPPORTED # source must be F32
+    assert ggml.set_rows_supports(_t(ca.F16, (D, rows, 8, 1)), src, (3,)) == ggml.OK
+    assert ggml.set_rows_supports(_t(ca.F32, (D, rows, 8, 1)), src, (3,)) == ggml.OK
+    assert ggml.set_rows_supports(ca.Tensor(None, ca.Q8_0, (D, rows, 8, 1), offset=1), src, (3,)) == ggml.ERR_UNSUPPORTED
+    assert ggml.set_rows_supports(dst, ca.Tensor(None, ca.F32, (D, 3, 8, 1), offset=2), (3,)) == ggml.ERR_UNSUPPORTED
+    # zero rows: nothing to do, still a supported node
+    assert ggml.set_rows_supports(dst, _t(ca.F32, (D, 0, 8, 1)), (0,)) == ggml.OK
+
+
+@pytest.mark.parametrize("kernel", [ggml.KERNEL_AUTO, ggml.KERNEL_VEC, ggml.KERNEL_MMA, ggml.KERNEL_DECODE_MMA])
+@pytest.mark.parametrize("nq,nkv", [(0, 32), (4, 0), (0, 0)])
+def test_planning_an_empty_op_with_any_forced_kernel(kernel, nq, nkv):
+    """a forced kernel on a shape with no queries or no keys used to divide by zero while planning"""
+    q = _t(ca.F32, (64, nq, 8, 1))
+    k = _t(ca.F16, (64, nkv, 8, 1))
+    for ns in (0, 1, 4):
+        try:
+            kern, n = ggml.flash_attn_plan(q, k, k, None, kernel=kernel, n_splits=ns)
+            assert n >= 1
+            assert ggml.flash_attn_workspace_size(q, k, k, None, kernel=kernel, n_splits=ns) >= 0
+        except ggml.Mi355xError:
+            pass            # a refusal is fine; the process must survive
+
+
+def test_relpos_workspace_size_is_the_f16_copy_of_the_table():
+    D, NR = 128, 149
+    r32 = _t(ca.F32, (D, NR, 8, 1))
+    assert ggml.relpos_bias_workspace_size(r32) == (D * NR * 8 * 2 + 255) // 256 * 256
+    assert ggml.relpos_bias_workspace_size(_t(ca.F16, (D, NR, 8, 1))) == 0
+    assert ggml.relpos_bias_workspace_size(_t(ca.F16, (D, NR, 8, 1), (2, 512, 512 * NR, 512 * NR * 8))) > 0     # padded rows

@@ -189,3 +189,35 @@ def test_fused_relpos_attention_matches_the_reference_relpos_attention(T, n_head
     out = ggml.flash_attn_relpos(heads(qu), heads(qv), heads(k), heads(v), heads(p), None, 1.0 / math.sqrt(hd))
     got = out.numpy_f32()                                  # [1, T, n_heads, hd]
     assert_parity(got.reshape(T, d), want, "fused rel-pos attention vs reference helpers")
+
+
+def test_relpos_mask_with_a_caller_workspace_for_the_f32_table():
+    """An F32 table is rounded to f16 once, into the caller's workspace when one is passed (needed under graph
+    capture, where the library may not allocate); the result is the same bits as with the library's own block."""
+    import torch
+    c = make(seed=331, D=128, Nq=75, Nkv=75, H=2, B=1)
+    dqv, dr = upload(c["qv"]), upload(c["r"])
+    need = ggml.relpos_bias_workspace_size(dr)
+    assert need == (128 * 149 * 2 * 2 + 255) // 256 * 256
+    plain = ggml.relpos_bias(dqv, dr, None, c["scale"], 75).to_host()
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    got = ggml.relpos_bias(dqv, dr, None, c["scale"], 75, workspace=ws).to_host()
+    assert np.array_equal(plain, got)
+    with pytest.raises(ggml.Mi355xError, match="workspace"):
+        ggml.relpos_bias(dqv, dr, None, c["scale"], 75, workspace=ws[: need - 256])
+    # while a stream is capturing, a call that would have to use the library's block is refused before it launches
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    out = ggml.Tensor.empty(ggml.F16, (75, 75, 2, 1))
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            with pytest.raises(ggml.Mi355xError, match="capturing"):
+                ggml.relpos_bias(dqv, dr, None, c["scale"], 75, out=out, stream=side)
+            ggml.relpos_bias(dqv, dr, None, c["scale"], 75, out=out, workspace=ws, stream=side)
+    torch.cuda.synchronize()
+    for _ in range(2):
+        out.buf.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out.to_host()[: plain.size], plain)
