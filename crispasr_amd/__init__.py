@@ -6,6 +6,6 @@ benchmark drive it through: ``ggml`` mirrors the reference's operator interface 
 path (``ggml_flash_attn_ext``, ``ggml_cpy``, ``ggml_set_rows`` on strided tensor views).
 """
 from . import ggml  # noqa: F401
-from .ggml import (F16, F32, Q8_0, HostBuffer, Tensor, cpy, flash_attn_ext, set_rows)  # noqa: F401
+from .ggml import (F16, F32, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, HostBuffer, Tensor, cpy, flash_attn_ext, set_rows)  # noqa: F401
 
-__all__ = ["ggml", "Tensor", "HostBuffer", "F32", "F16", "Q8_0", "flash_attn_ext", "cpy", "set_rows"]
+__all__ = ["ggml", "Tensor", "HostBuffer", "F32", "F16", "Q8_0", "Q4_0", "Q4_1", "Q5_0", "Q5_1", "flash_attn_ext", "cpy", "set_rows"]

@@ -41,11 +41,12 @@ size_t type_size(int t) {
     switch (t) {
         case MI355X_TYPE_F32:  return 4;
         case MI355X_TYPE_F16:  return 2;
-        case MI355X_TYPE_Q8_0: return FATTN_Q8_0_BYTES;
-        default:               return 0;
+        default:               return (size_t)fattn_block_bytes(t);      // 0 for a type this library does not know
     }
 }
-int64_t block_size(int t) { return t == MI355X_TYPE_Q8_0 ? FATTN_QK8_0 : 1; }
+int64_t block_size(int t) { return FATTN_IS_BLOCK_TYPE(t) ? FATTN_QK8_0 : 1; }
+// Q4_0, Q4_1, Q5_0, Q5_1: read natively by the vector kernel, through f16 copies by the tile kernel
+bool narrow_quant(int t) { return FATTN_IS_BLOCK_TYPE(t) && t != MI355X_TYPE_Q8_0; }
 
 bool is_contiguous(const mi355x_tensor * t) {
     const size_t ts = type_size(t->type);
@@ -173,7 +174,7 @@ int check(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor 
     if (Hkv <= 0 || Bk <= 0 || Hq % Hkv || B % Bk) return fail(MI355X_ERR_INVALID, "q heads/batch not a multiple of kv heads/batch");
     if (v->ne[0] != D) return fail(MI355X_ERR_UNSUPPORTED, "DV %lld != DK %lld", (long long)v->ne[0], (long long)D);
     if (D <= 0 || D % 8 || D > 256) return fail(MI355X_ERR_UNSUPPORTED, "head size %lld (need a multiple of 8, <= 256)", (long long)D);
-    if (k->type == MI355X_TYPE_Q8_0 && D % FATTN_QK8_0) return fail(MI355X_ERR_INVALID, "Q8_0 rows need D %% 32 == 0");
+    if (FATTN_IS_BLOCK_TYPE(k->type) && D % FATTN_QK8_0) return fail(MI355X_ERR_INVALID, "quantised rows need D %% 32 == 0");
     if (Nq < 0 || Nkv < 0 || Hq <= 0 || B <= 0) return fail(MI355X_ERR_INVALID, "negative or zero extent");
     if (q->nb[0] != 4) return fail(MI355X_ERR_UNSUPPORTED, "q rows must be contiguous (nb0 = %zu)", q->nb[0]);
     if (k->nb[0] != type_size(k->type) || v->nb[0] != type_size(v->type))
@@ -290,6 +291,8 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
         // such calls go to the vector kernel, which works on the exact values - and has nothing to gain from MFMA there.
         const bool few_keys = a.Nkv <= 16 && ktype != MI355X_TYPE_F16;
         if (few_keys)                                                              kernel = MI355X_FATTN_VEC;
+        else if (narrow_quant(ktype))     // no decode kernel for these: rows of queries share one conversion to f16, single rows read the blocks
+            kernel = a.Nq >= 16 && (a.D == 64 || a.D == 128) && a.q_aligned16 ? MI355X_FATTN_MMA : MI355X_FATTN_VEC;
         else if (fattn_decode_supported(a, ktype) && (a.q_chunks <= 1 || chunked)) kernel = MI355X_FATTN_DECODE_MMA;
         else if (a.Nq >= 16 && fattn_mma_supported(a, ktype)) kernel = MI355X_FATTN_MMA;
         else                                                  kernel = MI355X_FATTN_VEC;
@@ -307,7 +310,7 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
     // touching registers) read the result: same values, same rounding.
     plan.ws_partials = 0;
     const bool convertible = (ktype == MI355X_TYPE_F32 && a.kv_aligned16) || (ktype == MI355X_TYPE_Q8_0 && a.kv_aligned2);
-    if (kernel == MI355X_FATTN_MMA && convertible && a.Nq >= 128) {
+    if (kernel == MI355X_FATTN_MMA && ((convertible && a.Nq >= 128) || narrow_quant(ktype))) {
         plan.kv_to_f16 = true;
         plan.workspace = ((size_t)2 * a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t) + 255) / 256 * 256;
         plan.ws_partials = plan.workspace;
@@ -598,7 +601,12 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     hipStream_t st = (hipStream_t)stream;
 
     if (plan.kernel == MI355X_FATTN_MMA) {
-        if (!fattn_mma_supported(a, k->type)) return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the MFMA kernel");
+        {
+            FattnArgs b = a;
+            if (plan.kv_to_f16) use_f16_copies(b, nullptr);
+            if (!fattn_mma_supported(b, plan.kv_to_f16 ? MI355X_TYPE_F16 : k->type))
+                return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the MFMA kernel");
+        }
         int ktype = k->type;
         void * ws = nullptr;
         if (plan.workspace) {
@@ -688,18 +696,19 @@ int mi355x_flash_attn_ext_noalloc(const mi355x_tensor * q, const mi355x_tensor *
 static int cpy_check(const mi355x_tensor * src, const mi355x_tensor * dst) {
     if (!src || !dst) return fail(MI355X_ERR_INVALID, "null argument");
     const int s = src->type, d = dst->type;
-    const bool ok = (s == MI355X_TYPE_F32 && (d == MI355X_TYPE_F32 || d == MI355X_TYPE_F16 || d == MI355X_TYPE_Q8_0)) ||
+    const bool sb = FATTN_IS_BLOCK_TYPE(s), db = FATTN_IS_BLOCK_TYPE(d);
+    const bool ok = (s == MI355X_TYPE_F32 && (d == MI355X_TYPE_F32 || d == MI355X_TYPE_F16 || db)) ||
                     (s == MI355X_TYPE_F16 && (d == MI355X_TYPE_F16 || d == MI355X_TYPE_F32)) ||
-                    (s == MI355X_TYPE_Q8_0 && (d == MI355X_TYPE_F32 || d == MI355X_TYPE_Q8_0));
+                    (sb && (d == MI355X_TYPE_F32 || d == s));
     if (!ok) return fail(MI355X_ERR_UNSUPPORTED, "copy %d -> %d not covered", s, d);
     int64_t ns = 1, nd = 1;
     if (!sane_extents(src, &ns) || !sane_extents(dst, &nd)) return fail(MI355X_ERR_INVALID, "negative or oversized extent");
     if (ns != nd) return fail(MI355X_ERR_INVALID, "element counts differ (%lld vs %lld)", (long long)ns, (long long)nd);
     if (dst->nb[0] != type_size(d)) return fail(MI355X_ERR_UNSUPPORTED, "dst rows must be contiguous");
-    if (s == MI355X_TYPE_Q8_0 && src->nb[0] != FATTN_Q8_0_BYTES) return fail(MI355X_ERR_UNSUPPORTED, "src blocks must be contiguous");
-    if (s == MI355X_TYPE_Q8_0 || d == MI355X_TYPE_Q8_0) {
+    if (sb && src->nb[0] != type_size(s)) return fail(MI355X_ERR_UNSUPPORTED, "src blocks must be contiguous");
+    if (sb || db) {
         if (src->ne[0] % FATTN_QK8_0 || dst->ne[0] % FATTN_QK8_0)
-            return fail(MI355X_ERR_INVALID, "Q8_0 copies need ne0 %% 32 == 0 on both sides");
+            return fail(MI355X_ERR_INVALID, "quantised copies need ne0 %% 32 == 0 on both sides");
     }
     // every access is at least element-wide (Q8_0 blocks are read and written in 2-byte units)
     const size_t sal = s == MI355X_TYPE_F32 ? 4 : 2, dal = d == MI355X_TYPE_F32 ? 4 : 2;
@@ -926,7 +935,7 @@ int mi355x_cpy(const mi355x_tensor * src, const mi355x_tensor * dst, void * stre
         a.snb[i] = (int64_t)src->nb[i]; a.dnb[i] = (int64_t)dst->nb[i];
         n *= src->ne[i];
     }
-    const bool blocks = src->type == MI355X_TYPE_Q8_0 || dst->type == MI355X_TYPE_Q8_0;
+    const bool blocks = FATTN_IS_BLOCK_TYPE(src->type) || FATTN_IS_BLOCK_TYPE(dst->type);
     a.n = blocks ? n / FATTN_QK8_0 : n;
     if (a.n == 0) return MI355X_OK;
     if (!a.src || !a.dst) return fail(MI355X_ERR_INVALID, "null data pointer");
@@ -975,7 +984,7 @@ int mi355x_set_rows(const mi355x_tensor * src, const void * idx, int32_t idx_typ
         n *= src->ne[i];
     }
     for (int i = 0; i < 3; i++) { a.ine[i] = idx_ne[i]; a.inb[i] = (int64_t)idx_nb[i]; }
-    a.n = dst->type == MI355X_TYPE_Q8_0 ? n / FATTN_QK8_0 : n;
+    a.n = FATTN_IS_BLOCK_TYPE(dst->type) ? n / FATTN_QK8_0 : n;
     if (a.n == 0) return MI355X_OK;
     if (!a.src || !a.dst || !a.idx) return fail(MI355X_ERR_INVALID, "null data pointer");
     const int e = set_rows_launch(a, dst->type, (hipStream_t)stream);

@@ -1,7 +1,7 @@
 // GGML_OP_CPY / CONT / DUP / SET_ROWS with the destination in device memory: the KV-cache
 // writes that feed FLASH_ATTN_EXT (src/crispasr.cpp:2810-2811, 3185-3203, 2956-2973;
 // src/core/attention.h:342-378) and the dequantising reads (src/core/attention.h:917-920).
-// HBM-bound byte work: one element (or one Q8_0 block of 32) per lane, coalesced along
+// HBM-bound byte work: one element (or one element of a block of 32) per lane, coalesced along
 // dimension 0.  Source and destination may have different shapes with equal element
 // counts (the reference copies a [n_state, n_ctx] tensor into a 1-D cache view).
 #include "fattn_common.h"
@@ -45,49 +45,92 @@ __global__ void __launch_bounds__(256) cpy_vec8_kernel(const CpyArgs a) {
     *(vd8 *)dp = y;
 }
 
-// quantise one block of 32 held one element per lane (32 consecutive lanes):
-// d = amax/127 (f32), q = rne(x * (1/d)), d stored as fp16
-// (called by every lane of the wave: the reduction runs before any divergence)
+// quantise one block of 32 held one element per lane (32 consecutive lanes) and store it
+// (called by every lane of the wave: the reductions run before any divergence).
+//   Q8_0: d = amax/127 (f32), q = rne(x * (1/d)), d stored as fp16
+//   Q4_0 / Q5_0: d = (signed value of largest magnitude, the first one) / -8 (-16), q = min(15 (31), trunc(x/d + 8.5 (16.5)))
+//   Q4_1 / Q5_1: d = (max - min) / 15 (31), m = min, q = min(15 (31), trunc((x - min)/d + 0.5))
+// every product and sum is a single f32 operation, none fused.
+template <int TYPE>
 __device__ __forceinline__ void quantize_block_store(float x, char * blk, int e, bool ok) {
-    const float amax = group_max<32>(fabsf(x));
-    const float d    = amax / 127.0f;
-    const float id   = d != 0.0f ? 1.0f / d : 0.0f;
-    const int   qi   = (int)rintf(x * id);
+    typedef BlockFormat<TYPE> F;
+    if (TYPE == MI355X_TYPE_Q8_0) {
+        const float amax = group_max<32>(fabsf(x));
+        const float d    = amax / 127.0f;
+        const float id   = d != 0.0f ? 1.0f / d : 0.0f;
+        const int   qi   = (int)rintf(x * id);
+        if (ok) {
+            ((int8_t *)(blk + 2))[e] = (int8_t)qi;
+            if (e == 0) *(_Float16 *)blk = (_Float16)d;
+        }
+        return;
+    }
+    const int half = (threadIdx.x & 32);                 // which 32 lanes of the wave hold this block
+    float d, m = 0.0f;
+    int   qi;
+    if (!F::HAS_M) {
+        const float    amax  = group_max<32>(fabsf(x));
+        const uint32_t who   = (uint32_t)(__ballot(fabsf(x) == amax) >> half);
+        const int      first = who ? __ffs(who) - 1 : 0;
+        float ext = __shfl(x, half + first, 64);
+        if (!(amax > 0.0f)) ext = 0.0f;
+        d = ext / (float)(-(F::LEVELS / 2));
+        const float id = d != 0.0f ? 1.0f / d : 0.0f;
+        qi = (int)(int8_t)(int)__fadd_rn(__fmul_rn(x, id), (float)(F::LEVELS / 2) + 0.5f);
+    } else {
+        m = group_min<32>(x);
+        const float mx = group_max<32>(x);
+        d = __fsub_rn(mx, m) / (float)(F::LEVELS - 1);
+        const float id = d != 0.0f ? 1.0f / d : 0.0f;
+        qi = (int)(uint8_t)(int)__fadd_rn(__fmul_rn(__fsub_rn(x, m), id), 0.5f);
+    }
+    qi = qi < F::LEVELS - 1 ? qi : F::LEVELS - 1;
+    const int      hi = __shfl(qi, half + (e & 15) + 16, 64);       // the element that shares this lane's byte
+    const uint32_t qh = (uint32_t)(__ballot((qi & 0x10) != 0) >> half);
     if (ok) {
-        ((int8_t *)(blk + 2))[e] = (int8_t)qi;
-        if (e == 0) *(_Float16 *)blk = (_Float16)d;
+        if (e < 16) ((uint8_t *)(blk + F::QS))[e] = (uint8_t)((qi & 15) | ((hi & 15) << 4));
+        if (e == 16) *(_Float16 *)blk = (_Float16)d;
+        if (F::HAS_M && e == 17) *(_Float16 *)(blk + 2) = (_Float16)m;
+        if (F::QH && e == 18) *(uint16_t *)(blk + F::QH) = (uint16_t)qh;
+        if (F::QH && e == 19) *(uint16_t *)(blk + F::QH + 2) = (uint16_t)(qh >> 16);
     }
 }
 
-// F32 -> Q8_0; one block per 32 lanes
-__global__ void __launch_bounds__(256) cpy_f32_q8_0_kernel(const CpyArgs a) {
+// F32 -> block type; one block per 32 lanes
+template <int TYPE>
+__global__ void __launch_bounds__(256) cpy_f32_block_kernel(const CpyArgs a) {
     const int64_t blk = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
     const int     e   = threadIdx.x & 31;
     const bool    ok  = blk < a.n;
-    const int64_t bc  = ok ? blk : 0;                       // keep all lanes in the reduction
+    const int64_t bc  = ok ? blk : 0;                       // keep all lanes in the reductions
     const char *  sp  = a.src + offset_of(bc, a.sne, a.snb, FATTN_QK8_0) + e * a.snb[0];
     const float   x   = ok ? *(const float *)sp : 0.0f;
     char * dp = a.dst + offset_of(bc, a.dne, a.dnb, FATTN_QK8_0, FATTN_QK8_0);
-    quantize_block_store(x, dp, e, ok);
+    quantize_block_store<TYPE>(x, dp, e, ok);
 }
 
-// Q8_0 -> F32; one block per 32 lanes
-__global__ void __launch_bounds__(256) cpy_q8_0_f32_kernel(const CpyArgs a) {
-    const int64_t blk = (int64_t)blockIdx.x * 8 + (threadIdx.x >> 5);
-    const int     e   = threadIdx.x & 31;
+// block type -> F32; 8 elements per lane, four lanes per block
+template <int TYPE>
+__global__ void __launch_bounds__(256) cpy_block_f32_kernel(const CpyArgs a) {
+    const int64_t t   = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t blk = t >> 2;
+    const int     j0  = (int)(t & 3) * 8;
     if (blk >= a.n) return;
     const char * sp = a.src + offset_of(blk, a.sne, a.snb, FATTN_QK8_0, FATTN_QK8_0);
-    const float  d  = h2f_bits(*(const uint16_t *)sp);
-    const float  x  = (float)((const int8_t *)(sp + 2))[e] * d;
-    char * dp = a.dst + offset_of(blk, a.dne, a.dnb, FATTN_QK8_0) + e * a.dnb[0];
-    *(float *)dp = x;
+    float y[8];
+    dequant8<TYPE>(sp, j0, y);
+    char * dp = a.dst + offset_of(blk, a.dne, a.dnb, FATTN_QK8_0) + j0 * a.dnb[0];
+#pragma unroll
+    for (int i = 0; i < 8; i++) *(float *)(dp + i * a.dnb[0]) = y[i];
 }
 
-// Q8_0 -> Q8_0: move 34-byte blocks as 17 halfwords
-__global__ void __launch_bounds__(256) cpy_q8_0_q8_0_kernel(const CpyArgs a) {
+// same block type on both sides: move the blocks as halfwords
+template <int TYPE>
+__global__ void __launch_bounds__(256) cpy_block_block_kernel(const CpyArgs a) {
+    constexpr int HW = BlockFormat<TYPE>::BYTES / 2;
     const int64_t t   = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t blk = t / 17;
-    const int     w   = (int)(t % 17);
+    const int64_t blk = t / HW;
+    const int     w   = (int)(t % HW);
     if (blk >= a.n) return;
     const uint16_t * sp = (const uint16_t *)(a.src + offset_of(blk, a.sne, a.snb, FATTN_QK8_0, FATTN_QK8_0));
     uint16_t *       dp = (uint16_t *)(a.dst + offset_of(blk, a.dne, a.dnb, FATTN_QK8_0, FATTN_QK8_0));
@@ -97,8 +140,9 @@ __global__ void __launch_bounds__(256) cpy_q8_0_q8_0_kernel(const CpyArgs a) {
 // SET_ROWS: dst[:, idx[i1, i2 % ine1, i3 % ine2], i2, i3] = convert(src[:, i1, i2, i3]), src F32
 template <int DTYPE>
 __global__ void __launch_bounds__(256) set_rows_kernel(const CpyArgs a) {
-    // one unit = 32 elements of a source row (Q8_0) or 1 element (F16/F32)
-    constexpr int UNIT = DTYPE == MI355X_TYPE_Q8_0 ? FATTN_QK8_0 : 1;
+    // one unit = 32 elements of a source row (block types) or 1 element (F16/F32)
+    constexpr bool BLOCKS = FATTN_IS_BLOCK_TYPE(DTYPE);
+    constexpr int  UNIT   = BLOCKS ? FATTN_QK8_0 : 1;
     int64_t u;
     int     e = 0;
     if (UNIT == 1) {
@@ -122,8 +166,8 @@ __global__ void __launch_bounds__(256) set_rows_kernel(const CpyArgs a) {
     const char * sp = a.src + (i0 * UNIT + e) * a.snb[0] + i1 * a.snb[1] + i2 * a.snb[2] + i3 * a.snb[3];
     const float  x  = ok ? *(const float *)sp : 0.0f;
     char * dp = a.dst + i0 * a.dnb[0] + (inside ? drow : 0) * a.dnb[1] + i2 * a.dnb[2] + i3 * a.dnb[3];
-    if (DTYPE == MI355X_TYPE_Q8_0) {
-        quantize_block_store(x, dp, e, inside);
+    if constexpr (BLOCKS) {
+        quantize_block_store<DTYPE>(x, dp, e, inside);
     } else if (inside) {
         if (DTYPE == MI355X_TYPE_F16) *(_Float16 *)dp = (_Float16)x;
         else                          *(float *)dp = x;
@@ -151,21 +195,16 @@ __global__ void __launch_bounds__(256) kv_to_f16_kernel(const FattnArgs a, char 
                             : a.k + j * a.nbk1 + h * a.nbk2 + b * a.nbk3;
     typedef _Float16 h8 __attribute__((ext_vector_type(8)));
     h8 y;
-    if (TYPE == MI355X_TYPE_F32) {
+    if constexpr (TYPE == MI355X_TYPE_F32) {
         const float4 x0 = *(const float4 *)(row + c * 32);
         const float4 x1 = *(const float4 *)(row + c * 32 + 16);
         y[0] = (_Float16)x0.x; y[1] = (_Float16)x0.y; y[2] = (_Float16)x0.z; y[3] = (_Float16)x0.w;
         y[4] = (_Float16)x1.x; y[5] = (_Float16)x1.y; y[6] = (_Float16)x1.z; y[7] = (_Float16)x1.w;
     } else {
-        const char *     blk = row + (c >> 2) * FATTN_Q8_0_BYTES;
-        const uint16_t * qs  = (const uint16_t *)(blk + 2 + (c & 3) * 8);      // blocks are only 2-byte aligned
-        const float      d   = h2f_bits(*(const uint16_t *)blk);
+        float f[8];
+        dequant8<TYPE>(row + (c >> 2) * fattn_block_bytes(TYPE), (c & 3) * 8, f);
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const uint32_t w = qs[e];
-            y[2 * e]     = (_Float16)((float)(int8_t)(w & 0xff) * d);
-            y[2 * e + 1] = (_Float16)((float)(int8_t)(w >> 8) * d);
-        }
+        for (int e = 0; e < 8; e++) y[e] = (_Float16)f[e];
     }
     *(h8 *)(dst + ((is_v ? half : 0) + i) * 16) = y;
 }
@@ -200,14 +239,22 @@ int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t str
     const int64_t n = 2 * (int64_t)(a.D / 8) * a.Nkv * a.Hkv * a.Bk;
     if (n == 0) return 0;
     const unsigned g = (unsigned)((n + 255) / 256);
-    if (ktype == MI355X_TYPE_F32)       hipLaunchKernelGGL((kv_to_f16_kernel<MI355X_TYPE_F32>), dim3(g), dim3(256), 0, stream, a, (char *)dst);
-    else if (ktype == MI355X_TYPE_Q8_0) hipLaunchKernelGGL((kv_to_f16_kernel<MI355X_TYPE_Q8_0>), dim3(g), dim3(256), 0, stream, a, (char *)dst);
-    else return (int)hipErrorInvalidValue;
+    switch (ktype) {
+#define KV16(T) case T: hipLaunchKernelGGL((kv_to_f16_kernel<T>), dim3(g), dim3(256), 0, stream, a, (char *)dst); break
+        KV16(MI355X_TYPE_F32);
+        KV16(MI355X_TYPE_Q8_0);
+        KV16(MI355X_TYPE_Q4_0);
+        KV16(MI355X_TYPE_Q4_1);
+        KV16(MI355X_TYPE_Q5_0);
+        KV16(MI355X_TYPE_Q5_1);
+#undef KV16
+        default: return (int)hipErrorInvalidValue;
+    }
     return (int)hipGetLastError();
 }
 
 static bool vec8_ok(const CpyArgs & a, int stype, int dtype) {
-    if (stype == MI355X_TYPE_Q8_0 || dtype == MI355X_TYPE_Q8_0) return false;
+    if (FATTN_IS_BLOCK_TYPE(stype) || FATTN_IS_BLOCK_TYPE(dtype)) return false;
     const int64_t ss = stype == MI355X_TYPE_F32 ? 4 : 2, ds = dtype == MI355X_TYPE_F32 ? 4 : 2;
     if (a.sne[0] % 8 || a.dne[0] % 8 || a.snb[0] != ss || a.dnb[0] != ds) return false;
     if (((uintptr_t)a.src % (8 * ss)) || ((uintptr_t)a.dst % (8 * ds))) return false;
@@ -239,12 +286,19 @@ int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream) {
         hipLaunchKernelGGL((cpy_scalar_kernel<_Float16, _Float16>), dim3(g256), dim3(256), 0, stream, a);
     else if (stype == MI355X_TYPE_F16 && dtype == MI355X_TYPE_F32)
         hipLaunchKernelGGL((cpy_scalar_kernel<_Float16, float>), dim3(g256), dim3(256), 0, stream, a);
-    else if (stype == MI355X_TYPE_F32 && dtype == MI355X_TYPE_Q8_0)
-        hipLaunchKernelGGL(cpy_f32_q8_0_kernel, dim3(g8), dim3(256), 0, stream, a);
-    else if (stype == MI355X_TYPE_Q8_0 && dtype == MI355X_TYPE_F32)
-        hipLaunchKernelGGL(cpy_q8_0_f32_kernel, dim3(g8), dim3(256), 0, stream, a);
-    else if (stype == MI355X_TYPE_Q8_0 && dtype == MI355X_TYPE_Q8_0)
-        hipLaunchKernelGGL(cpy_q8_0_q8_0_kernel, dim3((unsigned)((a.n * 17 + 255) / 256)), dim3(256), 0, stream, a);
+#define BLOCK_CASES(T)                                                                                                    \
+    else if (stype == MI355X_TYPE_F32 && dtype == T)                                                                       \
+        hipLaunchKernelGGL((cpy_f32_block_kernel<T>), dim3(g8), dim3(256), 0, stream, a);                                 \
+    else if (stype == T && dtype == MI355X_TYPE_F32)                                                                       \
+        hipLaunchKernelGGL((cpy_block_f32_kernel<T>), dim3((unsigned)((a.n * 4 + 255) / 256)), dim3(256), 0, stream, a);  \
+    else if (stype == T && dtype == T)                                                                                     \
+        hipLaunchKernelGGL((cpy_block_block_kernel<T>), dim3((unsigned)((a.n * (BlockFormat<T>::BYTES / 2) + 255) / 256)), dim3(256), 0, stream, a);
+    BLOCK_CASES(MI355X_TYPE_Q8_0)
+    BLOCK_CASES(MI355X_TYPE_Q4_0)
+    BLOCK_CASES(MI355X_TYPE_Q4_1)
+    BLOCK_CASES(MI355X_TYPE_Q5_0)
+    BLOCK_CASES(MI355X_TYPE_Q5_1)
+#undef BLOCK_CASES
     else
         return (int)hipErrorInvalidValue;
     return (int)hipGetLastError();
@@ -253,8 +307,12 @@ int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream) {
 int set_rows_launch(const CpyArgs & a, int dtype, hipStream_t stream) {
     if (a.n == 0) return 0;
     if (a.n > ((int64_t)1 << 38)) return (int)hipErrorInvalidValue;
-    if (dtype == MI355X_TYPE_Q8_0)
-        hipLaunchKernelGGL((set_rows_kernel<MI355X_TYPE_Q8_0>), dim3((unsigned)((a.n + 7) / 8)), dim3(256), 0, stream, a);
+    const dim3 gb((unsigned)((a.n + 7) / 8));
+    if (dtype == MI355X_TYPE_Q8_0)      hipLaunchKernelGGL((set_rows_kernel<MI355X_TYPE_Q8_0>), gb, dim3(256), 0, stream, a);
+    else if (dtype == MI355X_TYPE_Q4_0) hipLaunchKernelGGL((set_rows_kernel<MI355X_TYPE_Q4_0>), gb, dim3(256), 0, stream, a);
+    else if (dtype == MI355X_TYPE_Q4_1) hipLaunchKernelGGL((set_rows_kernel<MI355X_TYPE_Q4_1>), gb, dim3(256), 0, stream, a);
+    else if (dtype == MI355X_TYPE_Q5_0) hipLaunchKernelGGL((set_rows_kernel<MI355X_TYPE_Q5_0>), gb, dim3(256), 0, stream, a);
+    else if (dtype == MI355X_TYPE_Q5_1) hipLaunchKernelGGL((set_rows_kernel<MI355X_TYPE_Q5_1>), gb, dim3(256), 0, stream, a);
     else if (dtype == MI355X_TYPE_F16)
         hipLaunchKernelGGL((set_rows_kernel<MI355X_TYPE_F16>), dim3((unsigned)((a.n + 255) / 256)), dim3(256), 0, stream, a);
     else if (dtype == MI355X_TYPE_F32)

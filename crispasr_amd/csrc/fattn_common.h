@@ -8,6 +8,7 @@
 
 #define FATTN_QK8_0 32
 #define FATTN_Q8_0_BYTES 34
+#define FATTN_IS_BLOCK_TYPE(t) ((t) == MI355X_TYPE_Q8_0 || (t) == MI355X_TYPE_Q4_0 || (t) == MI355X_TYPE_Q4_1 || (t) == MI355X_TYPE_Q5_0 || (t) == MI355X_TYPE_Q5_1)
 
 // Everything a kernel needs about one FLASH_ATTN_EXT node, by value.
 struct FattnArgs {
@@ -93,13 +94,75 @@ static __device__ __forceinline__ float group_max(float x) {
     return x;
 }
 
+template <int GROUP>
+static __device__ __forceinline__ float group_min(float x) { return -group_max<GROUP>(-x); }
+
+// ---- block-32 storage types ------------------------------------------------------------
+// BYTES per block, offsets of the quants (QS), of the fifth bits (QH, 0 = none) and whether a minimum follows the scale
+template <int TYPE> struct BlockFormat;
+template <> struct BlockFormat<MI355X_TYPE_Q4_0> { static constexpr int BYTES = 18, QS = 2, QH = 0, LEVELS = 16; static constexpr bool HAS_M = false; };
+template <> struct BlockFormat<MI355X_TYPE_Q4_1> { static constexpr int BYTES = 20, QS = 4, QH = 0, LEVELS = 16; static constexpr bool HAS_M = true;  };
+template <> struct BlockFormat<MI355X_TYPE_Q5_0> { static constexpr int BYTES = 22, QS = 6, QH = 2, LEVELS = 32; static constexpr bool HAS_M = false; };
+template <> struct BlockFormat<MI355X_TYPE_Q5_1> { static constexpr int BYTES = 24, QS = 8, QH = 4, LEVELS = 32; static constexpr bool HAS_M = true;  };
+template <> struct BlockFormat<MI355X_TYPE_Q8_0> { static constexpr int BYTES = 34, QS = 2, QH = 0, LEVELS = 256; static constexpr bool HAS_M = false; };
+
+static inline __host__ __device__ int fattn_block_bytes(int type) {
+    switch (type) {
+        case MI355X_TYPE_Q4_0: return 18;
+        case MI355X_TYPE_Q4_1: return 20;
+        case MI355X_TYPE_Q5_0: return 22;
+        case MI355X_TYPE_Q5_1: return 24;
+        case MI355X_TYPE_Q8_0: return 34;
+        default:               return 0;
+    }
+}
+
+// elements j0 .. j0+7 (j0 = 0, 8, 16 or 24) of one block as f32: q*d is exact, q*d + m is one product and one sum,
+// each rounded to f32 (not fused).  Blocks are only 2-byte aligned: halfword reads.
+template <int TYPE>
+static __device__ __forceinline__ void dequant8(const char * blk, int j0, float (&out)[8]) {
+    typedef BlockFormat<TYPE> F;
+    const float d = h2f_bits(*(const uint16_t *)blk);
+    if (TYPE == MI355X_TYPE_Q8_0) {
+        const uint16_t * qs = (const uint16_t *)(blk + 2 + j0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint16_t w = qs[i];
+            out[2 * i]     = (float)(int8_t)(w & 0xff) * d;
+            out[2 * i + 1] = (float)(int8_t)(w >> 8) * d;
+        }
+        return;
+    }
+    const float m = F::HAS_M ? h2f_bits(*(const uint16_t *)(blk + 2)) : 0.0f;
+    const uint16_t * qs = (const uint16_t *)(blk + F::QS + (j0 & 8));       // elements j and j + 16 share a byte
+    const int sh = (j0 & 16) ? 4 : 0;
+    uint32_t hb = 0;
+    if (F::QH) {
+        const uint16_t * qh = (const uint16_t *)(blk + F::QH);
+        hb = (((uint32_t)qh[0] | (uint32_t)qh[1] << 16) >> j0) & 0xffu;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t w  = qs[i];
+        const int      q0 = (int)(((w >> sh) & 15u) | (((hb >> (2 * i)) & 1u) << 4));
+        const int      q1 = (int)(((w >> (8 + sh)) & 15u) | (((hb >> (2 * i + 1)) & 1u) << 4));
+        if (F::HAS_M) {
+            out[2 * i]     = __fadd_rn(__fmul_rn((float)q0, d), m);
+            out[2 * i + 1] = __fadd_rn(__fmul_rn((float)q1, d), m);
+        } else {
+            out[2 * i]     = (float)(q0 - F::LEVELS / 2) * d;
+            out[2 * i + 1] = (float)(q1 - F::LEVELS / 2) * d;
+        }
+    }
+}
+
 // One CPY / SET_ROWS node.
 struct CpyArgs {
     const char * src;
     char *       dst;
     int64_t sne[4], dne[4];
     int64_t snb[4], dnb[4];
-    int64_t n;                 // elements (or blocks of 32 when a side is Q8_0)
+    int64_t n;                 // elements (or blocks of 32 when a side is a block type)
     // SET_ROWS only
     const char * idx;
     int32_t idx_is_i64;

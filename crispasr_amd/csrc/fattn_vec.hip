@@ -23,7 +23,7 @@ constexpr int VEC_UNROLL  = 4;
 // 8 consecutive elements of a K/V row starting at element d0, as f32 (exact for all types)
 template <int TYPE>
 __device__ __forceinline__ void load8(const char * row, int d0, bool aligned16, float (&out)[8]) {
-    if (TYPE == MI355X_TYPE_F16) {
+    if constexpr (TYPE == MI355X_TYPE_F16) {
         const char * p = row + (size_t)d0 * 2;
         if (aligned16) {
             const uint4 u = *(const uint4 *)p;
@@ -38,7 +38,7 @@ __device__ __forceinline__ void load8(const char * row, int d0, bool aligned16, 
 #pragma unroll
             for (int i = 0; i < 8; i++) out[i] = h2f_bits(h[i]);
         }
-    } else if (TYPE == MI355X_TYPE_F32) {
+    } else if constexpr (TYPE == MI355X_TYPE_F32) {
         const char * p = row + (size_t)d0 * 4;
         if (aligned16) {
             const float4 a = *(const float4 *)p;
@@ -50,16 +50,8 @@ __device__ __forceinline__ void load8(const char * row, int d0, bool aligned16, 
 #pragma unroll
             for (int i = 0; i < 8; i++) out[i] = f[i];
         }
-    } else {  // Q8_0: block = fp16 d + 32 int8; blocks are only 2-byte aligned
-        const char * blk = row + (size_t)(d0 / FATTN_QK8_0) * FATTN_Q8_0_BYTES;
-        const float  d   = h2f_bits(*(const uint16_t *)blk);
-        const uint16_t * qs = (const uint16_t *)(blk + 2 + (d0 % FATTN_QK8_0));
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint16_t w = qs[i];
-            out[2 * i]     = (float)(int8_t)(w & 0xff) * d;
-            out[2 * i + 1] = (float)(int8_t)(w >> 8) * d;
-        }
+    } else {  // block-32 types: blocks are only 2-byte aligned
+        dequant8<TYPE>(row + (size_t)(d0 / FATTN_QK8_0) * fattn_block_bytes(TYPE), d0 % FATTN_QK8_0, out);
     }
 }
 
@@ -296,6 +288,10 @@ int fattn_vec_launch(const FattnArgs & a, int ktype, hipStream_t stream) {
         case MI355X_TYPE_F16:  return launch_typed<MI355X_TYPE_F16>(a, stream);
         case MI355X_TYPE_F32:  return launch_typed<MI355X_TYPE_F32>(a, stream);
         case MI355X_TYPE_Q8_0: return launch_typed<MI355X_TYPE_Q8_0>(a, stream);
+        case MI355X_TYPE_Q4_0: return launch_typed<MI355X_TYPE_Q4_0>(a, stream);
+        case MI355X_TYPE_Q4_1: return launch_typed<MI355X_TYPE_Q4_1>(a, stream);
+        case MI355X_TYPE_Q5_0: return launch_typed<MI355X_TYPE_Q5_0>(a, stream);
+        case MI355X_TYPE_Q5_1: return launch_typed<MI355X_TYPE_Q5_1>(a, stream);
         default:               return (int)hipErrorInvalidValue;
     }
 }

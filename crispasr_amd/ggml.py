@@ -18,10 +18,10 @@ from typing import Optional, Sequence
 import numpy as np
 import torch
 
-F32, F16, Q8_0 = 0, 1, 8
+F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 = 0, 1, 2, 3, 6, 7, 8
 QK8_0 = 32
-TYPE_SIZE = {F32: 4, F16: 2, Q8_0: 34}
-BLOCK_SIZE = {F32: 1, F16: 1, Q8_0: QK8_0}
+TYPE_SIZE = {F32: 4, F16: 2, Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: 34}
+BLOCK_SIZE = {F32: 1, F16: 1, Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: QK8_0}
 
 KERNEL_AUTO, KERNEL_VEC, KERNEL_MMA, KERNEL_DECODE_MMA = 0, 1, 2, 3
 PREC_DEFAULT, PREC_F32 = 0, 10

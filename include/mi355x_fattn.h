@@ -39,7 +39,15 @@ extern "C" {
 enum mi355x_type {
     MI355X_TYPE_F32  = 0,
     MI355X_TYPE_F16  = 1,
-    MI355X_TYPE_Q8_0 = 8   /* blocks of 32: fp16 scale d + 32 x int8, 34 bytes, x = q*d */
+    /* the block-32 cache types CRISPASR_KV_QUANT can name (src/core/attention.h:79-105).  Element j < 16 of a block is the
+     * low nibble of qs[j], element j + 16 the high nibble; qh holds the fifth bit of element e in bit e (little-endian).
+     * ggml itself is not part of the reference's tree: the four narrow layouts and their scalar quantisers are ggml's as
+     * recalled (scale from the signed value of largest magnitude, q = min(15, trunc(x/d + 8.5)) and siblings). */
+    MI355X_TYPE_Q4_0 = 2,  /* fp16 d, qs[16]: 18 bytes, x = (q - 8) * d */
+    MI355X_TYPE_Q4_1 = 3,  /* fp16 d, fp16 m, qs[16]: 20 bytes, x = q * d + m */
+    MI355X_TYPE_Q5_0 = 6,  /* fp16 d, qh[4], qs[16]: 22 bytes, x = (q - 16) * d */
+    MI355X_TYPE_Q5_1 = 7,  /* fp16 d, fp16 m, qh[4], qs[16]: 24 bytes, x = q * d + m */
+    MI355X_TYPE_Q8_0 = 8   /* fp16 scale d + 32 x int8, 34 bytes, x = q*d */
 };
 
 enum mi355x_status {
@@ -122,8 +130,10 @@ int mi355x_stream_synchronize(void * stream);
  * dst[DV, Hq, Nq, B] (f32, contiguous, 16-byte aligned) = softmax(scale * q.k^T [soft-capped] + slope(h) * mask) . v
  *
  *   q    F32  [D,  Nq,  Hq,  B ]   any strides with nb[0] == 4
- *   k    F16 | F32 | Q8_0 [D,  Nkv, Hkv, Bk]   rows contiguous (nb[0] == type size)
+ *   k    F16 | F32 | Q8_0 | Q4_0 | Q4_1 | Q5_0 | Q5_1 [D,  Nkv, Hkv, Bk]   rows contiguous (nb[0] == type size)
  *   v    same type as k   [DV, Nkv, Hkv, Bk]   DV == D
+ *        (Q4_0 .. Q5_1: read block by block by the vector kernel for a few query rows; 16 query rows or more go through
+ *         one conversion of K and V to f16 in the workspace and the tile kernel; the decode kernel does not take them)
  *   mask NULL, or F16 [>=Nkv, >=Nq, Hm, Bm], rows contiguous; head h reads h % Hm,
  *        batch b reads b % Bm; -inf entries exclude the key
  *   Hq % Hkv == 0 (query head h reads KV head h / (Hq/Hkv)), B % Bk == 0.
@@ -180,7 +190,7 @@ typedef struct mi355x_fattn_plan_info {
     int32_t kernel;                  /* mi355x_fattn_kernel */
     int32_t n_splits;
     int32_t keys_per_split;
-    int32_t kv_to_f16;               /* 1: F32 / Q8_0 K and V are rounded to f16 copies in the workspace first */
+    int32_t kv_to_f16;               /* 1: F32 / quantised K and V are rounded to f16 copies in the workspace first */
     size_t  workspace;               /* bytes, as mi355x_fattn_workspace_size reports (without the q_quant part) */
     /* tile kernel only (0 otherwise) */
     int32_t queries_per_workgroup;   /* 256, 128 or 64 */
@@ -242,13 +252,15 @@ int mi355x_fattn_relpos_workspace_size(const mi355x_tensor * q_u, const mi355x_t
 /* ---- GGML_OP_CPY / CONT / DUP with the destination in a device buffer --------------------- */
 
 /*
- * dst[i] = convert(src[i]) for tensors of equal ne.  Supported: F32 -> F32 | F16 | Q8_0,
- * F16 -> F16 | F32, Q8_0 -> F32 | Q8_0.  F32 -> F16 rounds to nearest even; F32 -> Q8_0
+ * dst[i] = convert(src[i]) for tensors of equal ne.  Supported: F32 -> F32 | F16 | any block type,
+ * F16 -> F16 | F32, block type -> F32 | the same block type.  F32 -> F16 rounds to nearest even; F32 -> Q8_0
  * uses d = amax/127, q = round-to-nearest-even(x * (1/d)) per block of 32 along
  * dimension 0: the rounding of ggml-cpu's vectorised quantiser as the reference describes it
  * (tools/upstream-prs/09-metal-q8_0-bit-match.md:24-28, rint / vcvtnq); ggml's scalar reference quantiser is recalled to
  * round halves away from zero instead, so a value that lands exactly on a tie (x/d = k + 0.5) may differ by one step from
  * a cache written by a backend that follows the scalar code - tie behaviour is not pinned by anything in the reference.
+ * F32 -> Q4_0 | Q4_1 | Q5_0 | Q5_1 follow ggml's scalar quantisers as recalled (see mi355x_type), every product and sum a
+ * single f32 operation; dequantisation is q*d (exact) or q*d + m (product, then sum, each rounded to f32).
  * src may have any strides; dst rows (dimension 0) must be contiguous.
  */
 int mi355x_cpy_supports(const mi355x_tensor * src, const mi355x_tensor * dst);
@@ -258,7 +270,7 @@ int mi355x_cpy(const mi355x_tensor * src, const mi355x_tensor * dst, void * stre
  * GGML_OP_SET_ROWS, the write into a quantised KV cache (src/core/attention.h:366-376):
  * dst[:, idx[i1, i2 % I1, i3 % I2], i2, i3] = convert(src[:, i1, i2, i3]).
  * src F32 [n0, n_rows, n2, n3]; idx I64 (idx_type 64) or I32 (idx_type 32) with
- * ne = {n_rows, I1, I2} and byte strides idx_nb; dst F32 | F16 | Q8_0 [n0, rows, n2, n3].
+ * ne = {n_rows, I1, I2} and byte strides idx_nb; dst F32 | F16 | any block type [n0, rows, n2, n3].
  */
 /* Rows whose index lies outside [0, rows) are not written (ggml-cpu asserts on them): a stale or uninitialised index
  * tensor cannot become a write outside the cache.  mi355x_set_rows_supports is the planning predicate (shapes, types,

@@ -19,14 +19,15 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
-F32, F16, Q8_0 = 0, 1, 8
+F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 = 0, 1, 2, 3, 6, 7, 8
+BLOCK_TYPES = (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0)
 MODE_EXACT, MODE_GGML_LIKE, MODE_GGML_LIKE_F16_ACC = 0, 1, 2
 ROUND_NEAREST_EVEN, ROUND_HALF_AWAY = 0, 1
 QK8_0 = 32
 BLOCK_Q8_0_BYTES = 34
 
-TYPE_SIZE = {F32: 4, F16: 2, Q8_0: BLOCK_Q8_0_BYTES}
-BLOCK_SIZE = {F32: 1, F16: 1, Q8_0: QK8_0}
+TYPE_SIZE = {F32: 4, F16: 2, Q4_0: 18, Q4_1: 20, Q5_0: 22, Q5_1: 24, Q8_0: BLOCK_Q8_0_BYTES}
+BLOCK_SIZE = {F32: 1, F16: 1, Q4_0: 32, Q4_1: 32, Q5_0: 32, Q5_1: 32, Q8_0: QK8_0}
 
 
 def build() -> str:
@@ -114,6 +115,10 @@ def lib() -> ctypes.CDLL:
         L.ora_quantize_row_q8_0.restype = None
         L.ora_quantize_row_q8_0.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int]
         L.ora_dequantize_row_q8_0.restype = None
+        L.ora_quantize_row.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+        L.ora_dequantize_row.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+        L.ora_block_bytes.restype = ctypes.c_size_t
+        L.ora_block_bytes.argtypes = [ctypes.c_int]
         L.ora_dequantize_row_q8_0.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
         L.ora_randn.restype = None
         L.ora_randn.argtypes = [ctypes.c_uint64, ctypes.c_int64, ctypes.c_void_p]
@@ -197,6 +202,8 @@ def from_f32(x: np.ndarray, type_: int = F32, rounding: int = ROUND_NEAREST_EVEN
         raw = fp32_to_fp16(x).view(np.uint8).reshape(-1).copy()
     elif type_ == Q8_0:
         raw = quantize_q8_0(x.reshape(-1), rounding)
+    elif type_ in BLOCK_TYPES:
+        raw = quantize(type_, x.reshape(-1))
     else:
         raise ValueError(type_)
     return Tensor(raw, type_, ne)
@@ -239,6 +246,24 @@ def dequantize_q8_0(raw: np.ndarray) -> np.ndarray:
     n = raw.size // BLOCK_Q8_0_BYTES * QK8_0
     out = np.empty(n, dtype=np.float32)
     lib().ora_dequantize_row_q8_0(raw.ctypes.data, out.ctypes.data, n)
+    return out
+
+
+def quantize(type_: int, x: np.ndarray) -> np.ndarray:
+    """f32[n] (n % 32 == 0) -> the bytes of n/32 blocks of a block-32 type (Q8_0: round to nearest even)"""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    assert x.size % 32 == 0 and type_ in BLOCK_TYPES
+    out = np.empty(x.size // 32 * TYPE_SIZE[type_], dtype=np.uint8)
+    assert lib().ora_quantize_row(type_, x.ctypes.data, out.ctypes.data, x.size) == 0
+    return out
+
+
+def dequantize(type_: int, raw: np.ndarray) -> np.ndarray:
+    raw = np.ascontiguousarray(raw, dtype=np.uint8).reshape(-1)
+    assert type_ in BLOCK_TYPES and raw.size % TYPE_SIZE[type_] == 0
+    n = raw.size // TYPE_SIZE[type_] * 32
+    out = np.empty(n, dtype=np.float32)
+    assert lib().ora_dequantize_row(type_, raw.ctypes.data, out.ctypes.data, n) == 0
     return out
 
 

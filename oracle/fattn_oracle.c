@@ -4,6 +4,7 @@
  */
 #include "fattn_oracle.h"
 
+#include <float.h>
 #include <math.h>
 #include <stdlib.h>
 #include <string.h>
@@ -138,6 +139,134 @@ void ora_dequantize_row_q8_0(const ora_block_q8_0 * x, float * y, int64_t n) {
     }
 }
 
+/* --------------------------------------------------- Q4_0 Q4_1 Q5_0 Q5_1 -- */
+
+/* ggml's scalar quantisers as recalled (quantize_row_q4_0_ref and siblings; the types are the ones
+ * src/core/attention.h:79-105 lets CRISPASR_KV_QUANT name).  Symmetric types: the scale comes from the value of
+ * largest magnitude WITH its sign (the first such value in the block), d = max / -8 (or -16), so that value maps to
+ * quant 0 and the other end of the range clips at 15 (31); q = min(15, trunc(x/d + 8.5)).  Types with a minimum:
+ * d = (max - min) / 15 (or 31), q = trunc((x - min)/d + 0.5).  The products and sums are single f32 operations in
+ * that order (this file is built without contraction into fused multiply-adds). */
+static void quantize_block_sym(const float * x, int levels, uint16_t * d_out, uint8_t * q) {
+    float amax = 0.0f, max = 0.0f;
+    for (int j = 0; j < 32; j++) {
+        const float v = x[j];
+        if (amax < fabsf(v)) { amax = fabsf(v); max = v; }
+    }
+    const float d  = max / (float)(-(levels / 2));
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    *d_out = fp32_to_fp16_soft(d);
+    for (int j = 0; j < 32; j++) {
+        const float x0 = x[j] * id;
+        const int   qi = (int)(int8_t)(x0 + ((float)(levels / 2) + 0.5f));
+        q[j] = (uint8_t)(qi < levels - 1 ? qi : levels - 1);
+    }
+}
+
+static void quantize_block_min(const float * x, int levels, uint16_t * d_out, uint16_t * m_out, uint8_t * q) {
+    float min = FLT_MAX, max = -FLT_MAX;
+    for (int j = 0; j < 32; j++) {
+        if (x[j] < min) min = x[j];
+        if (x[j] > max) max = x[j];
+    }
+    const float d  = (max - min) / (float)(levels - 1);
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    *d_out = fp32_to_fp16_soft(d);
+    *m_out = fp32_to_fp16_soft(min);
+    for (int j = 0; j < 32; j++) {
+        const float x0 = (x[j] - min) * id;
+        const int   qi = (int)(uint8_t)(x0 + 0.5f);
+        q[j] = (uint8_t)(qi < levels - 1 ? qi : levels - 1);
+    }
+}
+
+static void pack_nibbles(const uint8_t * q, uint8_t * qs, uint8_t * qh) {
+    uint32_t h = 0;
+    for (int j = 0; j < 16; j++) {
+        qs[j] = (uint8_t)((q[j] & 0x0F) | ((q[j + 16] & 0x0F) << 4));
+        h |= (uint32_t)((q[j] & 0x10) >> 4) << j;
+        h |= (uint32_t)((q[j + 16] & 0x10) >> 4) << (j + 16);
+    }
+    if (qh) { qh[0] = (uint8_t)h; qh[1] = (uint8_t)(h >> 8); qh[2] = (uint8_t)(h >> 16); qh[3] = (uint8_t)(h >> 24); }
+}
+
+static void unpack_nibbles(const uint8_t * qs, const uint8_t * qh, uint8_t * q) {
+    const uint32_t h = qh ? (uint32_t)qh[0] | (uint32_t)qh[1] << 8 | (uint32_t)qh[2] << 16 | (uint32_t)qh[3] << 24 : 0;
+    for (int j = 0; j < 16; j++) {
+        q[j]      = (uint8_t)((qs[j] & 0x0F) | (((h >> j) & 1) << 4));
+        q[j + 16] = (uint8_t)((qs[j] >> 4) | (((h >> (j + 16)) & 1) << 4));
+    }
+}
+
+size_t ora_block_bytes(int type) {
+    switch (type) {
+        case ORA_TYPE_Q4_0: return sizeof(ora_block_q4_0);
+        case ORA_TYPE_Q4_1: return sizeof(ora_block_q4_1);
+        case ORA_TYPE_Q5_0: return sizeof(ora_block_q5_0);
+        case ORA_TYPE_Q5_1: return sizeof(ora_block_q5_1);
+        case ORA_TYPE_Q8_0: return sizeof(ora_block_q8_0);
+        default:            return 0;
+    }
+}
+
+int ora_quantize_row(int type, const float * x, void * y, int64_t n) {
+    if (type == ORA_TYPE_Q8_0) { ora_quantize_row_q8_0(x, (ora_block_q8_0 *)y, n, ORA_ROUND_NEAREST_EVEN); return 0; }
+    if (!ora_block_bytes(type)) return -2;
+    uint8_t q[32];
+    for (int64_t i = 0; i < n / 32; i++) {
+        const float * xb = x + i * 32;
+        if (type == ORA_TYPE_Q4_0) {
+            ora_block_q4_0 * b = (ora_block_q4_0 *)y + i;
+            quantize_block_sym(xb, 16, &b->d, q);
+            pack_nibbles(q, b->qs, NULL);
+        } else if (type == ORA_TYPE_Q4_1) {
+            ora_block_q4_1 * b = (ora_block_q4_1 *)y + i;
+            quantize_block_min(xb, 16, &b->d, &b->m, q);
+            pack_nibbles(q, b->qs, NULL);
+        } else if (type == ORA_TYPE_Q5_0) {
+            ora_block_q5_0 * b = (ora_block_q5_0 *)y + i;
+            quantize_block_sym(xb, 32, &b->d, q);
+            pack_nibbles(q, b->qs, b->qh);
+        } else {
+            ora_block_q5_1 * b = (ora_block_q5_1 *)y + i;
+            quantize_block_min(xb, 32, &b->d, &b->m, q);
+            pack_nibbles(q, b->qs, b->qh);
+        }
+    }
+    return 0;
+}
+
+int ora_dequantize_row(int type, const void * x, float * y, int64_t n) {
+    if (type == ORA_TYPE_Q8_0) { ora_dequantize_row_q8_0((const ora_block_q8_0 *)x, y, n); return 0; }
+    if (!ora_block_bytes(type)) return -2;
+    uint8_t q[32];
+    for (int64_t i = 0; i < n / 32; i++) {
+        float * yb = y + i * 32;
+        if (type == ORA_TYPE_Q4_0) {
+            const ora_block_q4_0 * b = (const ora_block_q4_0 *)x + i;
+            const float d = fp16_to_fp32_soft(b->d);
+            unpack_nibbles(b->qs, NULL, q);
+            for (int j = 0; j < 32; j++) yb[j] = (float)((int)q[j] - 8) * d;
+        } else if (type == ORA_TYPE_Q4_1) {
+            const ora_block_q4_1 * b = (const ora_block_q4_1 *)x + i;
+            const float d = fp16_to_fp32_soft(b->d), m = fp16_to_fp32_soft(b->m);
+            unpack_nibbles(b->qs, NULL, q);
+            for (int j = 0; j < 32; j++) yb[j] = (float)q[j] * d + m;
+        } else if (type == ORA_TYPE_Q5_0) {
+            const ora_block_q5_0 * b = (const ora_block_q5_0 *)x + i;
+            const float d = fp16_to_fp32_soft(b->d);
+            unpack_nibbles(b->qs, b->qh, q);
+            for (int j = 0; j < 32; j++) yb[j] = (float)((int)q[j] - 16) * d;
+        } else {
+            const ora_block_q5_1 * b = (const ora_block_q5_1 *)x + i;
+            const float d = fp16_to_fp32_soft(b->d), m = fp16_to_fp32_soft(b->m);
+            unpack_nibbles(b->qs, b->qh, q);
+            for (int j = 0; j < 32; j++) yb[j] = (float)q[j] * d + m;
+        }
+    }
+    return 0;
+}
+
 /* ------------------------------------------------------------------- RNG -- */
 
 static inline uint64_t splitmix64_at(uint64_t seed, uint64_t idx) {
@@ -178,7 +307,7 @@ static inline const char * row_ptr(const ora_tensor * t, int64_t i1, int64_t i2,
     return (const char *)t->data + i1 * t->nb[1] + i2 * t->nb[2] + i3 * t->nb[3];
 }
 
-static int type_ok(int t) { return t == ORA_TYPE_F32 || t == ORA_TYPE_F16 || t == ORA_TYPE_Q8_0; }
+static int type_ok(int t) { return t == ORA_TYPE_F32 || t == ORA_TYPE_F16 || ora_block_bytes(t) != 0; }
 
 /* one K or V row -> f32 (exact for every storage type) */
 static void row_to_f32(const char * p, int type, int64_t n, float * out) {
@@ -188,7 +317,7 @@ static void row_to_f32(const char * p, int type, int64_t n, float * out) {
         const uint16_t * h = (const uint16_t *)p;
         for (int64_t i = 0; i < n; i++) out[i] = h2f(h[i]);
     } else {
-        ora_dequantize_row_q8_0((const ora_block_q8_0 *)p, out, n);
+        ora_dequantize_row(type, p, out, n);
     }
 }
 
@@ -302,7 +431,11 @@ static void fa_row_ggml_like(const fa_args * a, int64_t iq1, int64_t iq2, int64_
     const int64_t DV     = a->DV;
     const int     v_f16  = f16_acc && vtype == ORA_TYPE_F16;
 
-    if (ktype == ORA_TYPE_Q8_0) ora_quantize_row_q8_0(qrow, qq, D, ORA_ROUND_NEAREST_EVEN);
+    float qdq[512];
+    if (ktype == ORA_TYPE_Q8_0 || ora_block_bytes(ktype)) {
+        ora_quantize_row_q8_0(qrow, qq, D, ORA_ROUND_NEAREST_EVEN);
+        ora_dequantize_row_q8_0(qq, qdq, D);
+    }
 
     float S = 0.0f;
     float M = -INFINITY;
@@ -335,8 +468,15 @@ static void fa_row_ggml_like(const fa_args * a, int64_t iq1, int64_t iq2, int64_
 #else
             for (int64_t d = 0; d < D; d++) s += h2f(kh[d]) * qrow[d];
 #endif
-        } else {
+        } else if (ktype == ORA_TYPE_Q8_0) {
             s = vec_dot_q8_0_q8_0((const ora_block_q8_0 *)kp, qq, D);
+        } else {
+            /* Q4_0 .. Q5_1: the rounded query row against the dequantised key row, summed in f32 in element order.
+             * ggml-cpu's integer block dot products for these types are not written down anywhere in the reference's
+             * tree: this stands in for them as a diagnostic, PARITY UNPINNED. */
+            float kf[512];
+            ora_dequantize_row(ktype, kp, kf, D);
+            for (int64_t d = 0; d < D; d++) s += kf[d] * qdq[d];
         }
         s *= scale;
         if (a->softcap != 0.0f) s = a->softcap * tanhf(s);
@@ -400,7 +540,8 @@ int ora_flash_attn_ext(const ora_tensor * q, const ora_tensor * k, const ora_ten
     /* contract of the constructor (ggml_flash_attn_ext), as the call sites use it */
     if (k->ne[0] != a.D || v->ne[1] != a.Nkv || v->ne[2] != a.Hkv || v->ne[3] != a.Bk) return -3;
     if (a.Hkv <= 0 || a.Bk <= 0 || a.Hq % a.Hkv != 0 || a.B % a.Bk != 0) return -3;
-    if ((k->type == ORA_TYPE_Q8_0 && a.D % ORA_QK8_0) || (v->type == ORA_TYPE_Q8_0 && a.DV % ORA_QK8_0)) return -3;
+    if ((ora_block_bytes(k->type) && a.D % ORA_QK8_0) || (ora_block_bytes(v->type) && a.DV % ORA_QK8_0)) return -3;
+    if (a.D > 512) return -3;
     if (mask) {
         if (mask->ne[0] < a.Nkv || mask->ne[1] < a.Nq) return -4;
         if (a.Hq % mask->ne[2] != 0 || a.B % mask->ne[3] != 0) return -4;
@@ -448,7 +589,7 @@ int ora_flash_attn_ext(const ora_tensor * q, const ora_tensor * k, const ora_ten
 int ora_cpy_f32(const ora_tensor * src, void * dst_data, int32_t dst_type, const int64_t dst_nb[4],
                 int rounding) {
     if (!src || src->type != ORA_TYPE_F32 || !type_ok(dst_type)) return -2;
-    if (dst_type == ORA_TYPE_Q8_0 && src->ne[0] % ORA_QK8_0) return -3;
+    if (ora_block_bytes(dst_type) && src->ne[0] % ORA_QK8_0) return -3;
     const int64_t n0 = src->ne[0];
     float * tmp = (float *)malloc((size_t)(n0 > 0 ? n0 : 1) * 4);
     for (int64_t i3 = 0; i3 < src->ne[3]; i3++)
@@ -461,8 +602,10 @@ int ora_cpy_f32(const ora_tensor * src, void * dst_data, int32_t dst_type, const
             for (int64_t i0 = 0; i0 < n0; i0++) *(float *)(dp + i0 * dst_nb[0]) = tmp[i0];
         } else if (dst_type == ORA_TYPE_F16) {
             for (int64_t i0 = 0; i0 < n0; i0++) *(uint16_t *)(dp + i0 * dst_nb[0]) = fp32_to_fp16_soft(tmp[i0]);
-        } else {
+        } else if (dst_type == ORA_TYPE_Q8_0) {
             ora_quantize_row_q8_0(tmp, (ora_block_q8_0 *)dp, n0, rounding);
+        } else {
+            ora_quantize_row(dst_type, tmp, dp, n0);
         }
     }
     free(tmp);

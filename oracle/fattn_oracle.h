@@ -50,7 +50,7 @@ extern "C" {
 #endif
 
 /* ggml type ids of the types this path meets */
-enum { ORA_TYPE_F32 = 0, ORA_TYPE_F16 = 1, ORA_TYPE_Q8_0 = 8 };
+enum { ORA_TYPE_F32 = 0, ORA_TYPE_F16 = 1, ORA_TYPE_Q4_0 = 2, ORA_TYPE_Q4_1 = 3, ORA_TYPE_Q5_0 = 6, ORA_TYPE_Q5_1 = 7, ORA_TYPE_Q8_0 = 8 };
 
 enum { ORA_MODE_EXACT = 0, ORA_MODE_GGML_LIKE = 1, ORA_MODE_GGML_LIKE_F16_ACC = 2 };
 
@@ -63,6 +63,17 @@ typedef struct {
     uint16_t d;               /* fp16 scale */
     int8_t   qs[ORA_QK8_0];   /* quants */
 } ora_block_q8_0;             /* 34 bytes, no padding */
+
+/* The narrower block-32 cache types the reference's CRISPASR_KV_QUANT accepts (src/core/attention.h:79-105).  ggml is
+ * absent from the reference's tree: layouts and arithmetic are ggml's as recalled (quantize_row_q*_ref /
+ * dequantize_row_q*), held by the tests to known-answer blocks worked out by hand from these definitions and to the
+ * reference's own round-trip bounds (tests/test-kv-quant-roundtrip.cpp:184-199).
+ * Element j (< 16) of a block sits in the low nibble of qs[j], element j + 16 in the high nibble; the fifth bit of
+ * element e (0..31) is bit e of qh (little-endian 32-bit). */
+typedef struct { uint16_t d; uint8_t qs[16]; } ora_block_q4_0;                       /* 18 bytes: x = (q - 8) * d   */
+typedef struct { uint16_t d, m; uint8_t qs[16]; } ora_block_q4_1;                    /* 20 bytes: x = q * d + m     */
+typedef struct { uint16_t d; uint8_t qh[4]; uint8_t qs[16]; } ora_block_q5_0;        /* 22 bytes: x = (q - 16) * d  */
+typedef struct { uint16_t d, m; uint8_t qh[4]; uint8_t qs[16]; } ora_block_q5_1;     /* 24 bytes: x = q * d + m     */
 
 /* a ggml tensor view: ne = elements per dim, nb = byte strides, dim 0 fastest */
 typedef struct {
@@ -80,6 +91,11 @@ void     ora_fp16_to_fp32_row(const uint16_t * x, float * y, int64_t n);
 void ora_quantize_row_q8_0(const float * x, ora_block_q8_0 * y, int64_t n, int rounding);
 void ora_dequantize_row_q8_0(const ora_block_q8_0 * x, float * y, int64_t n);
 
+/* any block-32 type (Q8_0 with round-to-nearest-even): n values <-> n/32 blocks; 0, or -2 for a type without blocks */
+int    ora_quantize_row(int type, const float * x, void * y, int64_t n);
+int    ora_dequantize_row(int type, const void * x, float * y, int64_t n);
+size_t ora_block_bytes(int type);      /* bytes of one block of 32 (0: not a block type) */
+
 /* deterministic N(0,1): splitmix64 counter -> Box-Muller in fp64 -> float.
  * element i of stream `seed` depends only on (seed, i). */
 void ora_randn(uint64_t seed, int64_t n, float * out);
@@ -93,8 +109,8 @@ int ora_flash_attn_ext(const ora_tensor * q, const ora_tensor * k, const ora_ten
                        float scale, float max_bias, float logit_softcap,
                        int mode, int n_threads);
 
-/* KV-cache writes (ggml_cpy F32 -> F16/F32/Q8_0 into a strided view whose rows
- * are contiguous): src and dst have equal ne, src is F32. */
+/* KV-cache writes (ggml_cpy F32 -> F16/F32/block-32 type into a strided view whose rows
+ * are contiguous): src and dst have equal ne, src is F32.  rounding applies to Q8_0 only. */
 int ora_cpy_f32(const ora_tensor * src, void * dst_data, int32_t dst_type, const int64_t dst_nb[4],
                 int rounding);
 

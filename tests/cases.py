@@ -122,7 +122,7 @@ def to_f32(t: ora.Tensor) -> np.ndarray:
                 elif t.type == ora.F16:
                     out[i3, i2, i1] = raw.view(np.float16).astype(np.float32)
                 else:
-                    out[i3, i2, i1] = ora.dequantize_q8_0(raw)
+                    out[i3, i2, i1] = ora.dequantize(t.type, raw)
     return out
 
 

@@ -73,7 +73,13 @@ def test_supports_rejects_contract_violations_and_uncovered_ops():
     # valid for ggml, outside these kernels: goes to the CPU backend
     assert ggml.flash_attn_supports(q, k, _t(ca.F32, (64, 16, 8, 1)), None) == ggml.ERR_UNSUPPORTED      # mixed K/V types
     assert ggml.flash_attn_supports(_t(ca.F16, (64, 4, 8, 1)), k, k, None) == ggml.ERR_UNSUPPORTED       # q not F32
-    assert ggml.flash_attn_supports(q, _t(2, (64, 16, 8, 1), (18, 36, 576, 4608)), _t(2, (64, 16, 8, 1), (18, 36, 576, 4608)), None) == ggml.ERR_UNSUPPORTED  # Q4_0
+    k4 = _t(ca.Q4_0, (64, 16, 8, 1), (18, 36, 576, 4608))
+    assert ggml.flash_attn_supports(q, k4, k4, None) == ggml.OK                                          # Q4_0 cache view
+    assert ggml.flash_attn_supports(q, k4, _t(ca.Q5_1, (64, 16, 8, 1)), None) == ggml.ERR_UNSUPPORTED    # mixed K/V types
+    assert ggml.flash_attn_supports(_t(ca.F32, (48, 4, 8, 1)), _t(ca.Q4_0, (32, 16, 8, 1), (18, 18, 288, 2304)),
+                                    _t(ca.Q4_0, (32, 16, 8, 1), (18, 18, 288, 2304)), None) == ggml.ERR_INVALID
+    k12 = ca.Tensor.__new__(ca.Tensor); k12.__dict__.update(_t(ca.F16, (64, 16, 8, 1)).__dict__); k12.type = 12   # a k-quant
+    assert ggml.flash_attn_supports(q, k12, k12, None) == ggml.ERR_UNSUPPORTED
     assert ggml.flash_attn_supports(q, k, k, _t(ca.F32, (16, 4, 1, 1))) == ggml.ERR_UNSUPPORTED          # F32 mask
     q72 = _t(ca.F32, (36, 4, 8, 1))
     assert ggml.flash_attn_supports(q72, _t(ca.F16, (36, 16, 8, 1)), _t(ca.F16, (36, 16, 8, 1)), None) == ggml.ERR_UNSUPPORTED
@@ -96,6 +102,9 @@ def test_cpy_supports_matrix():
     assert ok(ca.F32, ca.F16) == ok(ca.F32, ca.Q8_0) == ok(ca.F32, ca.F32) == ggml.OK
     assert ok(ca.F16, ca.F32) == ok(ca.Q8_0, ca.F32) == ok(ca.Q8_0, ca.Q8_0) == ggml.OK
     assert ok(ca.F16, ca.Q8_0) == ggml.ERR_UNSUPPORTED
+    for t in (ca.Q4_0, ca.Q4_1, ca.Q5_0, ca.Q5_1):
+        assert ok(ca.F32, t) == ok(t, ca.F32) == ok(t, t) == ggml.OK
+        assert ok(t, ca.F16) == ok(t, ca.Q8_0) == ok(ca.F16, t) == ggml.ERR_UNSUPPORTED
     assert ok(ca.F32, ca.F16, (64, 4, 2, 1), (512, 1, 1, 1)) == ggml.OK          # reshape with equal counts
     assert ok(ca.F32, ca.F16, (64, 4, 2, 1), (64, 5, 2, 1)) == ggml.ERR_INVALID
     assert ok(ca.F32, ca.Q8_0, (48, 4, 2, 1)) == ggml.ERR_INVALID
