@@ -220,7 +220,14 @@ def bench_decode(args, ca, ora, torch):
         return torch.randn(n, device="cuda").half().view(torch.uint8)
 
     def q8_buf(seed, n):
-        return torch.from_numpy(ora.quantize_q8_0(ora.randn(seed, (n,)))).cuda()
+        # N(0,1) values quantised by the library's own CPY F32 -> Q8_0 (bit-exact against the oracle in the tests)
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(seed)
+        src = ca.Tensor(torch.randn(n, device="cuda", generator=gen).view(torch.uint8), ca.F32, (n,))
+        dst = ca.Tensor.empty(ca.Q8_0, (n,))
+        ca.cpy(src, dst)
+        torch.cuda.synchronize()
+        return dst.buf
 
     # Whisper large-v3 decoder step, beam 5, 20 heads x 64 (strides of the [token][head][dim] cache)
     D, H = 64, 20
@@ -312,6 +319,17 @@ def bench_decode(args, ca, ora, torch):
                        "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 64))})
     run("llm_decode_q8_0_gqa4_4096x64seq", layers, 128 ** -0.5, 64 * (2 * Lk * Hkv * rs + 2 * Hq * D * 4), 10,
         "64 sequences x 4096-entry Q8_0 cache per call")
+    del layers
+    # twice the sequences: the same loop with the launch's fixed cost (first loads, last step, merge of the waves) spread
+    # over twice the bytes
+    layers = []
+    for l in range(2):
+        layers.append({"q": ca.Tensor(torch.randn(128 * Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, 128)),
+                       "k": ca.Tensor(q8_buf(1200 + 2 * l, 128 * Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, 128), nbk),
+                       "v": ca.Tensor(q8_buf(1201 + 2 * l, 128 * Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, 128), nbk),
+                       "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 128))})
+    run("llm_decode_q8_0_gqa4_4096x128seq", layers, 128 ** -0.5, 128 * (2 * Lk * Hkv * rs + 2 * Hq * D * 4), 10,
+        "128 sequences x 4096-entry Q8_0 cache per call")
     return out
 
 

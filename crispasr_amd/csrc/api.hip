@@ -103,18 +103,18 @@ struct Scratch {
 Scratch g_scratch[64];
 
 int get_scratch(size_t bytes, void ** out, hipStream_t st) {
-    // the block is shared by every call that brings no workspace and may have to grow: neither fits a call that is
-    // being recorded into a graph, whose replays would use it long after this call returned
-    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(st, &cs) != hipSuccess) (void)hipGetLastError();
-    else if (cs != hipStreamCaptureStatusNone)
-        return fail(MI355X_ERR_WORKSPACE, "this call needs %zu bytes of workspace: pass one while the stream is capturing", bytes);
     int dev = 0;
     HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= 64) return fail(MI355X_ERR_HIP, "device index %d out of range", dev);
     std::lock_guard<std::mutex> lk(g_mu);
     Scratch & s = g_scratch[dev];
     if (s.size < bytes) {
+        // growing means hipMalloc: not while the stream is being recorded into a graph
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &cs) != hipSuccess) (void)hipGetLastError();
+        else if (cs != hipStreamCaptureStatusNone)
+            return fail(MI355X_ERR_WORKSPACE, "this call needs %zu bytes of workspace and the library holds %zu: pass one, or make the call "
+                        "once before capturing", bytes, s.size);
         size_t want = s.size ? s.size : (size_t)(8u << 20);
         while (want < bytes) want *= 2;
         void * p = nullptr;

@@ -18,11 +18,17 @@
 // aligned dword loads and a byte funnel shift (blocks are 34 bytes, so chunks sit at 2 mod 4),
 // widened to exact f16 integers with v_perm_b32 + one packed add, and scaled by the block's f16 d
 // with one packed multiply (one rounding, = f16(q*d)).  When the rows of a Q8_0 cache are contiguous the
-// bytes of a step are fetched as one coalesced stream of 8- (or 4-)byte units into a wave-private raw
+// K bytes of a step are fetched as one coalesced stream of 8- (or 4-)byte units into a wave-private raw
 // stage in LDS and the chunks are cut out of LDS instead - three times fewer global load instructions.
+// V then skips the f16 stage: its quants are stored to LDS as bytes (one 8-byte load per chunk, from its
+// 2-byte aligned address, and one aligned 8-byte LDS store) and read back through ds_read_b64_tr_b8,
+// which hands every lane eight consecutive keys of one column - the A operand of the second product -
+// to be widened and multiplied by those keys' scales in registers: same values, a third of the LDS
+// instructions, half the LDS bytes, one register stage instead of two.
 // Loads of the next step are in flight while the current one is consumed.  Waves are merged through LDS, splits by fattn_merge_kernel.
 #include "fattn_common.h"
 
+#include <stdlib.h>
 #include <type_traits>
 
 namespace {
@@ -100,6 +106,17 @@ __device__ __forceinline__ half8 q8_dequant(uint2 q, uint16_t dbits) {
     return r;
 }
 
+// 8 quants of 8 different keys (one column of V) times those keys' scales
+__device__ __forceinline__ half8 q8_dequant_keys(uint32_t q0, uint32_t q1, half8 d) {
+    half2v h0, h1, h2, h3;
+    q8_widen(q0, h0, h1);
+    q8_widen(q1, h2, h3);
+    half8 r;
+    r[0] = h0[0]; r[1] = h0[1]; r[2] = h1[0]; r[3] = h1[1];
+    r[4] = h2[0]; r[5] = h2[1]; r[6] = h3[0]; r[7] = h3[1];
+    return r * d;
+}
+
 // raw global data of one 8-element chunk
 struct Chunk {
     uint4 v;         // f16: the 8 halves; q8_0: x,y = quants, z = scale bits
@@ -126,18 +143,29 @@ __device__ __forceinline__ half8 chunk_to_half8(const Chunk & r) {
     return q8_dequant(make_uint2(r.v.x, r.v.y), (uint16_t)r.v.z);
 }
 
-// LDS bytes per workgroup: the per-wave f16 V stages, plus per-wave raw K and V stages when RAW
-template <int D, bool RAW>
+// row pitch in bytes of the int8 V stage: the 16 rows one half of a transpose read touches start 4 banks apart
+template <int D> constexpr int v8_pitch() { return D == 128 ? 136 : 80; }
+
+// LDS bytes per workgroup: the per-wave f16 V stages, plus per-wave raw K and V stages when RAW; with V8 the V side is
+// one int8 stage and the scales of its 32 x D/32 blocks instead
+template <int D, bool RAW, bool V8>
 constexpr int decode_lds_bytes() {
     constexpr int RS     = D / 32 * FATTN_Q8_0_BYTES;
-    constexpr int RAWB   = RAW ? 2 * ((STEP * RS + 511) / 512 * 512 + 64) : 0;      // 9 x 64 units each, padded
-    constexpr int stage  = DEC_WAVES * (STEP * (D + 32) * 2 + RAWB);
+    constexpr int RAWSZ  = (STEP * RS + 511) / 512 * 512 + 64;                      // 9 x 64 units, padded
+    constexpr int wave   = V8 ? RAWSZ + STEP * v8_pitch<D>() + D / 32 * STEP * 2
+                              : STEP * (D + 32) * 2 + (RAW ? 2 * RAWSZ : 0);
+    constexpr int stage  = DEC_WAVES * wave;
     constexpr int red    = DEC_WAVES * 16 * (D + 1 + 2) * 4;
     return stage > red ? stage : red;
 }
 
-template <int D, int TYPE, bool MASK, bool RAW>
-__global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const FattnArgs a) {
+// V8 (with RAW): V's quants go to LDS as bytes and come back through ds_read_b64_tr_b8 already in operand layout
+// (8 consecutive keys of one column per lane); the transposing read ignores the low three address bits, and the quants
+// of block b start at byte 34 b + 2 of a row, so V is not taken from the coalesced stream: each lane fetches the 8
+// quants of one chunk with one 8-byte load from its 2-byte aligned address, and the scales with halfword loads.
+template <int D, int TYPE, bool MASK, bool RAW, bool V8>
+__global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode_kernel(const FattnArgs a) {
+    static_assert(!V8 || RAW, "the int8 V stage belongs to the streamed Q8_0 path");
     constexpr int KS  = D / 32;                    // reduction steps of Q.K^T (one Q8_0 block each)
     constexpr int DBK = D / 16;                    // 16-wide blocks of the output's d
     constexpr int CH  = D / 8;                     // chunks per row
@@ -154,10 +182,16 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
 
     // the per-wave stages; after the key loop the same memory carries the cross-wave reduction
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    constexpr int WAVE_BYTES = STEP * PV * 2 + (RAW ? 2 * RAWSZ : 0);
-    _Float16 * v_stage = (_Float16 *)(smem + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * WAVE_BYTES);
-    char * k_rawst     = smem + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * WAVE_BYTES + STEP * PV * 2;
-    char * v_rawst     = k_rawst + RAWSZ;
+    constexpr int VP8 = v8_pitch<D>();
+    constexpr int NV8 = STEP * (D / 8) / 64;       // 8-quant chunks of V per lane and step
+    constexpr int NSC = STEP * KS / 64;            // V scales per lane and step
+    constexpr int WAVE_BYTES = V8 ? RAWSZ + STEP * VP8 + KS * STEP * 2 : STEP * PV * 2 + (RAW ? 2 * RAWSZ : 0);
+    char * const wave_mem = smem + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * WAVE_BYTES;
+    _Float16 * v_stage = (_Float16 *)wave_mem;                          // (!V8)
+    char * k_rawst     = V8 ? wave_mem : wave_mem + STEP * PV * 2;
+    char * v_rawst     = k_rawst + RAWSZ;                               // (!V8)
+    char * v8_stage    = wave_mem + RAWSZ;                              // (V8) [32 keys][VP8]
+    char * vsc_stage   = v8_stage + STEP * VP8;                         // (V8) f16 [KS][32 keys]
     float (*red_o)[16][D + 1]      = (float (*)[16][D + 1])smem;
     float (*red_ml)[16][2]         = (float (*)[16][2])(smem + DEC_WAVES * 16 * (D + 1) * 4);
 
@@ -203,7 +237,10 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     Chunk kraw[2][RAW ? 1 : 2][RAW ? 1 : KS];
     Chunk vraw[2][RAW ? 1 : NV];
     typedef typename std::conditional<UNIT == 8, uint2, uint32_t>::type unit_t;
-    unit_t kun[2][RAW ? NU : 1], vun[2][RAW ? NU : 1];
+    unit_t kun[V8 ? 1 : 2][RAW ? NU : 1], vun[2][RAW && !V8 ? NU : 1];
+    typedef uint32_t u32x2_a2 __attribute__((ext_vector_type(2), aligned(2)));
+    u32x2_a2 v8q[1][V8 ? NV8 : 1];
+    uint16_t v8d[1][V8 ? NSC : 1];
     // a partial last step: its loads are clamped to the last valid row or unit (branch-free, in bounds) and the
     // keys they stand for are excluded in the step
     auto issue = [&](int it, auto stage) __attribute__((always_inline)) {
@@ -218,7 +255,22 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
             for (int i = 0; i < NU; i++) {
                 const uint32_t off = (uint32_t)min(i * 64 + lane, last) * UNIT;
                 kun[s][i] = *(const unit_t *)(kp + off);
-                vun[s][i] = *(const unit_t *)(vp + off);
+                if (!V8) vun[s][i] = *(const unit_t *)(vp + off);
+            }
+            if (V8) {
+                const int last_row = min(STEP, k_end - j0) - 1;
+#pragma unroll
+                for (int i = 0; i < NV8; i++) {
+                    const int flat = i * 64 + lane;
+                    const int row  = min(flat / CH, last_row), c = flat % CH;
+                    v8q[s][i] = *(const u32x2_a2 *)(vp + row * RS + (c >> 2) * FATTN_Q8_0_BYTES + 2 + (c & 3) * 8);
+                }
+#pragma unroll
+                for (int i = 0; i < NSC; i++) {
+                    const int flat = i * 64 + lane;
+                    const int row  = min(flat / KS, last_row);
+                    v8d[s][i] = *(const uint16_t *)(vp + row * RS + (flat % KS) * FATTN_Q8_0_BYTES);
+                }
             }
             return;
         }
@@ -246,15 +298,31 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
         constexpr int s = decltype(stage)::value;
         const int  j0   = k_begin + it * STEP;
         const bool tail = j0 + STEP > k_end;                  // wave-uniform
-        if (it + DEC_WAVES < n_steps) issue(it + DEC_WAVES, std::integral_constant<int, 1 - s>{});
+        // the following step's loads: into the other register stage, or (V8) into this one as soon as it is in LDS
+        if (!V8 && it + DEC_WAVES < n_steps) issue(it + DEC_WAVES, std::integral_constant<int, 1 - s>{});
 
         if (RAW) {
 #pragma unroll
             for (int i = 0; i < NU; i++) {
                 *(unit_t *)(k_rawst + (i * 64 + lane) * UNIT) = kun[s][i];
-                *(unit_t *)(v_rawst + (i * 64 + lane) * UNIT) = vun[s][i];
+                if (!V8) *(unit_t *)(v_rawst + (i * 64 + lane) * UNIT) = vun[s][i];
             }
-            if (tail) {
+            if (V8) {
+#pragma unroll
+                for (int i = 0; i < NV8; i++) {
+                    const int flat = i * 64 + lane;
+                    *(uint2 *)(v8_stage + (flat / CH) * VP8 + (flat % CH) * 8) = make_uint2(v8q[s][i][0], v8q[s][i][1]);
+                }
+                // rows past k_end repeat the last row's bytes: a zero scale makes exact zeros of them
+#pragma unroll
+                for (int i = 0; i < NSC; i++) {
+                    const int flat = i * 64 + lane;
+                    const int row  = flat / KS;
+                    *(uint16_t *)(vsc_stage + ((flat % KS) * STEP + row) * 2) = (tail && j0 + row >= k_end) ? (uint16_t)0 : v8d[s][i];
+                }
+            }
+            if (V8 && it + DEC_WAVES < n_steps) issue(it + DEC_WAVES, stage);
+            if (!V8 && tail) {
                 // rows past k_end hold bytes of no row: a zero scale keeps what is made of them finite
 #pragma unroll
                 for (int t = 0; t < STEP * KS / 64; t++) {
@@ -272,14 +340,16 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
 #pragma unroll
             for (int ks = 0; ks < KS; ks++) {
                 Chunk c;
-                if (RAW) c.v = q8_lds_chunk<true>(k_rawst, (kb * 16 + j) * RS, ks, g4);
+                // (V8: row i of tile kb is key (i / 4) * 8 + kb * 4 + i % 4, so that a lane's eight scores are eight
+                //  consecutive keys, the order in which the transposing read hands out V)
+                if (RAW) c.v = q8_lds_chunk<true>(k_rawst, (V8 ? (j >> 2) * 8 + kb * 4 + (j & 3) : kb * 16 + j) * RS, ks, g4);
                 else     c = kraw[s][kb][ks];
                 sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_to_half8<TYPE>(c), qreg[ks], sc[kb], 0, 0, 0);
             }
         }
         // V rows into this wave's LDS stage (f16, dequantised when the cache is Q8_0)
 #pragma unroll
-        for (int i = 0; i < NV; i++) {
+        for (int i = 0; i < (V8 ? 0 : NV); i++) {
             const int flat = i * 64 + lane;
             Chunk c;
             if (RAW) {
@@ -291,13 +361,13 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
         }
         __builtin_amdgcn_wave_barrier();      // LDS runs a wave's instructions in order; keep the compiler from reordering
 
-        // lane holds keys j0 + kb*16 + g4*4 + r of column j
+        // lane holds keys j0 + kb*16 + g4*4 + r of column j (V8: j0 + g4*8 + kb*4 + r)
         float sv[8];
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const int key = j0 + kb * 16 + g4 * 4 + r;
+                const int key = V8 ? j0 + g4 * 8 + kb * 4 + r : j0 + kb * 16 + g4 * 4 + r;
                 float x = sc[kb][r];
                 if (MASK) x = fmaf(mslope, h2f_bits(mrow[min(key, k_end - 1)]), x);
                 if (tail && key >= k_end) x = -INFINITY;
@@ -346,7 +416,20 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
         l += lsum;
 
         // ---- O^T += V^T . P^T: transpose reads of the stage, 16 d at a time --------------------------
-        {
+        if (V8) {
+            half8 vsc[KS];
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) vsc[ks] = *(const half8 *)(vsc_stage + (ks * STEP + g4 * 8) * 2);
+            // lane r of a group of 16 addresses key r / 2, columns 8 (r % 2) ..: the group receives keys g4*8 .. +7 x 16 columns
+            const char * p0 = v8_stage + (g4 * 8 + (j >> 1)) * VP8 + (j & 1) * 8;
+#pragma unroll
+            for (int db = 0; db < DBK; db++) {
+                typedef int int2v __attribute__((ext_vector_type(2)));
+                const int2v q = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) int2v *)(p0 + db * 16));
+                const half8 va = q8_dequant_keys((uint32_t)q[0], (uint32_t)q[1], vsc[db >> 1]);
+                oacc[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, preg, oacc[db], 0, 0, 0);
+            }
+        } else {
             const int kr = g4 * 4 + (j >> 2);
 #pragma unroll
             for (int db = 0; db < DBK; db++) {
@@ -376,7 +459,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     }
     for (int it = wave; it < n_steps; it += 2 * DEC_WAVES) {
         step(it, S0{});
-        if (it + DEC_WAVES < n_steps) step(it + DEC_WAVES, S1{});
+        if (it + DEC_WAVES < n_steps) step(it + DEC_WAVES, std::integral_constant<int, V8 ? 0 : 1>{});
     }
 
     // ---- column totals, then the four waves through LDS ----------------------------------------------
@@ -430,20 +513,20 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     }
 }
 
-template <int D, int TYPE, bool MASK, bool RAW>
+template <int D, int TYPE, bool MASK, bool RAW, bool V8 = false>
 int launch_one(const FattnArgs & a, hipStream_t stream) {
     const int64_t wgs = (int64_t)a.n_splits * a.q_chunks * a.Hkv * a.B;
     if (wgs > 0x7fffffff || a.q_chunks != (a.Nq * a.gqa + 15) / 16) return (int)hipErrorInvalidValue;
     const dim3 grid((unsigned)wgs);
-    constexpr int lds = decode_lds_bytes<D, RAW>();
+    constexpr int lds = decode_lds_bytes<D, RAW, V8>();
     static bool attr_set = false;
     if (!attr_set && lds > 64 * 1024) {
-        const hipError_t e = hipFuncSetAttribute((const void *)fattn_decode_kernel<D, TYPE, MASK, RAW>,
+        const hipError_t e = hipFuncSetAttribute((const void *)fattn_decode_kernel<D, TYPE, MASK, RAW, V8>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, lds);
         if (e != hipSuccess) return (int)e;
         attr_set = true;
     }
-    hipLaunchKernelGGL((fattn_decode_kernel<D, TYPE, MASK, RAW>), grid, dim3(DEC_THREADS), lds, stream, a);
+    hipLaunchKernelGGL((fattn_decode_kernel<D, TYPE, MASK, RAW, V8>), grid, dim3(DEC_THREADS), lds, stream, a);
     return (int)hipGetLastError();
 }
 
@@ -458,7 +541,9 @@ int launch(const FattnArgs & a, hipStream_t stream) {
                          !(a.nbk2 % UNIT) && !(a.nbk3 % UNIT) && !(a.nbv2 % UNIT) && !(a.nbv3 % UNIT);
         if (raw) {
             constexpr int T = MI355X_TYPE_Q8_0;     // (TYPE itself, spelled so that the f16 instantiation never names a RAW kernel)
-            return a.mask ? launch_one<D, T, true, true>(a, stream) : launch_one<D, T, false, true>(a, stream);
+            static const bool f16_stage = getenv("MI355X_FATTN_DECODE_F16_STAGE") != nullptr;     // the earlier V path, for comparison runs
+            if (f16_stage) return a.mask ? launch_one<D, T, true, true>(a, stream) : launch_one<D, T, false, true>(a, stream);
+            return a.mask ? launch_one<D, T, true, true, true>(a, stream) : launch_one<D, T, false, true, true>(a, stream);
         }
     }
     return a.mask ? launch_one<D, TYPE, true, false>(a, stream) : launch_one<D, TYPE, false, false>(a, stream);

@@ -24,7 +24,7 @@
 static mi355x_tensor to_mi(const ggml_tensor * t) {
     mi355x_tensor m;
     m.data = t->data;
-    m.type = (int32_t)t->type;                  // GGML_TYPE_F32 = 0, F16 = 1, Q8_0 = 8: the ids the library uses
+    m.type = (int32_t)t->type;                  // GGML_TYPE_F32 = 0, F16 = 1, Q4_0 = 2, Q4_1 = 3, Q5_0 = 6, Q5_1 = 7, Q8_0 = 8: the ids the library uses
     for (int i = 0; i < 4; i++) { m.ne[i] = t->ne[i]; m.nb[i] = t->nb[i]; }
     return m;
 }

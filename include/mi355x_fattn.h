@@ -85,8 +85,9 @@ typedef struct mi355x_fattn_params {
     int32_t kernel;          /* mi355x_fattn_kernel */
     int32_t n_splits;        /* 0 = choose; forces the KV split count of the split-KV kernels */
     void *  workspace;       /* NULL = library-owned scratch: one block per device, grown with hipMalloc when needed and
-                              * shared by every call that passes NULL, so such calls belong on one stream at a time; a
-                              * call that needs scratch is refused (MI355X_ERR_WORKSPACE) while its stream is capturing.
+                              * shared by every call that passes NULL, so such calls (and replays of graphs that recorded
+                              * them) belong on one stream at a time; while its stream is capturing, a call that would
+                              * have to grow the block is refused with MI355X_ERR_WORKSPACE instead.
                               * Else 16-byte aligned.  With a caller's workspace of mi355x_fattn_workspace_size bytes the call allocates nothing
                               * and launches kernels only (no memset or copy nodes): it may be recorded into a HIP graph. */
     size_t  workspace_size;
@@ -229,7 +230,7 @@ int mi355x_relpos_bias_supports(const mi355x_tensor * q_v, const mi355x_tensor *
                                 const mi355x_tensor * dst);
 /* workspace: room for the f16 copy of an F32 or strided table (mi355x_relpos_bias_workspace_size bytes, 16-byte aligned;
  * 0 for an F16 table with contiguous rows), or NULL to use the library's per-device scratch block under the rules of
- * mi355x_fattn_params.workspace (one stream at a time, refused while the stream is capturing). */
+ * mi355x_fattn_params.workspace (one stream at a time, never grown while the stream is capturing). */
 int mi355x_relpos_bias_workspace_size(const mi355x_tensor * r, size_t * bytes);
 int mi355x_relpos_bias(const mi355x_tensor * q_v, const mi355x_tensor * r, const mi355x_tensor * add,
                        const mi355x_tensor * dst, float scale, void * workspace, size_t workspace_size, void * stream);
