@@ -9,7 +9,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmi355x_fattn.so")
-SOURCES = ["api.hip", "fattn_vec.hip", "fattn_mma.hip", "fattn_decode.hip", "cpy.hip", "relpos.hip"]
+SOURCES = ["api.hip", "fattn_vec.hip", "fattn_mma.hip", "fattn_decode.hip", "cpy.hip", "relpos.hip", "fattn_relpos.hip"]
 
 # packed-fp32 VALU ops are switched off for all device code of this library
 HIPCC_FLAGS = [

@@ -881,6 +881,98 @@ static int relpos_fused_check(const mi355x_tensor * q_u, const mi355x_tensor * q
     return MI355X_OK;
 }
 
+// The one-kernel form: taken when no kernel is asked for by name and the shape fits it.  Workspace: f16 copies of K and V
+// (unless they are f16 with 16-byte rows already), then the f16 table (unless it is read in place).
+struct RelposFused {
+    bool   ok;
+    bool   kv_copy;
+    size_t kv_bytes, table_bytes;
+};
+static RelposFused relpos_fused_plan(const mi355x_tensor * q_u, const mi355x_tensor * q_v, const mi355x_tensor * k,
+                                     const mi355x_tensor * v, const mi355x_tensor * r, const mi355x_tensor * add,
+                                     const mi355x_fattn_params * params) {
+    RelposFused f = {false, false, 0, 0};
+    static const bool off = getenv("MI355X_RELPOS_TWO_LAUNCHES") != nullptr;        // comparison runs
+    if (off || params->kernel != MI355X_FATTN_AUTO || params->n_splits > 1 || params->q_quant) return f;
+    const int64_t D = q_u->ne[0];
+    if ((D != 64 && D != 128) || q_u->ne[1] < 1 || k->ne[1] < 1) return f;
+    FattnArgs a;
+    fill_args(a, q_u, k, v, nullptr, nullptr, params);
+    if (!a.q_aligned16 || !aligned16_view(q_v)) return f;
+    if (add && add->ne[0] > 0) {
+        const size_t es = type_size(add->type);
+        if (add->nb[0] != es) return f;
+    }
+    if (k->type == MI355X_TYPE_F16 && a.kv_aligned16) {
+        f.kv_copy = false;
+    } else if ((k->type == MI355X_TYPE_F32 && a.kv_aligned16) || (FATTN_IS_BLOCK_TYPE(k->type) && a.kv_aligned2)) {
+        f.kv_copy  = true;
+        f.kv_bytes = ((size_t)2 * a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t) + 255) / 256 * 256;
+    } else {
+        return f;
+    }
+    f.table_bytes = relpos_table_bytes(r);
+    if (!f.table_bytes && !aligned16_view(r)) return f;
+    f.ok = true;
+    return f;
+}
+
+static int relpos_fused_run(const mi355x_tensor * q_u, const mi355x_tensor * q_v, const mi355x_tensor * k,
+                            const mi355x_tensor * v, const mi355x_tensor * r, const mi355x_tensor * add,
+                            const mi355x_tensor * dst, const mi355x_fattn_params * params, const RelposFused & f,
+                            void * ws, hipStream_t st) {
+    FattnArgs a;
+    fill_args(a, q_u, k, v, nullptr, (float *)dst->data, params);
+    if (!q_v->data || !r->data) return fail(MI355X_ERR_INVALID, "null data pointer");
+    if (f.kv_copy) {
+        const int e = kv_to_f16_launch(a, k->type, ws, st);
+        if (e) return hip_fail((hipError_t)e, "K/V conversion launch");
+        use_f16_copies(a, ws);
+    }
+    FattnRelposArgs g;
+    memset(&g, 0, sizeof(g));
+    g.qu = a.q; g.nbu1 = a.nbq1; g.nbu2 = a.nbq2; g.nbu3 = a.nbq3;
+    g.qv = (const char *)q_v->data; g.nbw1 = (int64_t)q_v->nb[1]; g.nbw2 = (int64_t)q_v->nb[2]; g.nbw3 = (int64_t)q_v->nb[3];
+    g.k = a.k; g.nbk1 = a.nbk1; g.nbk2 = a.nbk2; g.nbk3 = a.nbk3;
+    g.v = a.v; g.nbv1 = a.nbv1; g.nbv2 = a.nbv2; g.nbv3 = a.nbv3;
+    g.r = (const char *)r->data; g.nbr1 = (int64_t)r->nb[1]; g.nbr2 = (int64_t)r->nb[2]; g.nbr3 = (int64_t)r->nb[3];
+    g.Hr = (int)r->ne[2]; g.Br = (int)r->ne[3];
+    if (f.table_bytes) {
+        char * r16 = (char *)ws + f.kv_bytes;
+        CpyArgs c;
+        memset(&c, 0, sizeof(c));
+        c.src = (const char *)r->data;
+        c.dst = r16;
+        int64_t nb = 2;
+        c.n = 1;
+        for (int i = 0; i < 4; i++) {
+            c.sne[i] = c.dne[i] = r->ne[i];
+            c.snb[i] = (int64_t)r->nb[i];
+            c.dnb[i] = nb;
+            nb *= r->ne[i];
+            c.n *= r->ne[i];
+        }
+        const int e = cpy_launch(c, r->type, MI355X_TYPE_F16, st);
+        if (e) return hip_fail((hipError_t)e, "table conversion launch");
+        g.r = r16;
+        g.nbr1 = (int64_t)a.D * 2; g.nbr2 = g.nbr1 * r->ne[1]; g.nbr3 = g.nbr2 * r->ne[2];
+    }
+    g.Ha = g.Ba = 1;
+    if (add && add->ne[0] > 0) {
+        if (!add->data) return fail(MI355X_ERR_INVALID, "null data pointer");
+        g.add = (const char *)add->data; g.nba1 = (int64_t)add->nb[1]; g.nba2 = (int64_t)add->nb[2]; g.nba3 = (int64_t)add->nb[3];
+        g.Ha = (int)add->ne[2]; g.Ba = (int)add->ne[3];
+        g.add_f16 = add->type == MI355X_TYPE_F16;
+    }
+    g.dst = (float *)dst->data;
+    g.D = a.D; g.Nq = a.Nq; g.Nkv = a.Nkv; g.H = a.Hq; g.B = a.B; g.gqa = a.gqa; g.bq = a.bq;
+    g.scale = params->scale;
+    if (!fattn_relpos_supported(g)) return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the one-kernel form");
+    const int e = fattn_relpos_launch(g, st);
+    if (e) return hip_fail((hipError_t)e, "relative-position attention launch");
+    return MI355X_OK;
+}
+
 int mi355x_fattn_relpos_workspace_size(const mi355x_tensor * q_u, const mi355x_tensor * q_v, const mi355x_tensor * k,
                                        const mi355x_tensor * v, const mi355x_tensor * r, const mi355x_tensor * add,
                                        const mi355x_fattn_params * params, size_t * bytes) {
@@ -889,7 +981,8 @@ int mi355x_fattn_relpos_workspace_size(const mi355x_tensor * q_u, const mi355x_t
     size_t mb = 0, ib = 0;
     const int rc = relpos_fused_check(q_u, q_v, k, v, r, add, nullptr, params, &m, &mb, &ib);
     if (rc) return rc;
-    *bytes = mb + ib;
+    const RelposFused f = relpos_fused_plan(q_u, q_v, k, v, r, add, params);
+    *bytes = f.ok ? f.kv_bytes + f.table_bytes : mb + ib;
     return MI355X_OK;
 }
 
@@ -902,6 +995,22 @@ int mi355x_flash_attn_relpos(const mi355x_tensor * q_u, const mi355x_tensor * q_
     int rc = relpos_fused_check(q_u, q_v, k, v, r, add, dst, params, &m, &mb, &ib);
     if (rc) return rc;
     if ((int64_t)q_u->ne[1] * q_u->ne[2] * q_u->ne[3] == 0) return MI355X_OK;
+    const RelposFused f = relpos_fused_plan(q_u, q_v, k, v, r, add, params);
+    if (f.ok) {
+        if (!q_u->data || !k->data || !v->data || !dst->data) return fail(MI355X_ERR_INVALID, "null data pointer");
+        const size_t need = f.kv_bytes + f.table_bytes;
+        void * ws = params->workspace;
+        if (need) {
+            if (ws) {
+                if (params->workspace_size < need) return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, need);
+                if ((uintptr_t)ws % 16) return fail(MI355X_ERR_WORKSPACE, "workspace must be 16-byte aligned");
+            } else {
+                rc = get_scratch(need, &ws, (hipStream_t)stream);
+                if (rc) return rc;
+            }
+        }
+        return relpos_fused_run(q_u, q_v, k, v, r, add, dst, params, f, ws, (hipStream_t)stream);
+    }
     void * ws = params->workspace;
     if (ws) {
         if (params->workspace_size < mb + ib)

@@ -183,6 +183,20 @@ struct RelposArgs {
     int32_t n_qblocks, n_chunks, chunk_tiles;                   // filled in by the launcher
 };
 
+// FastConformer's relative-position attention in one kernel (fattn_relpos.hip): K, V and the table are f16
+struct FattnRelposArgs {
+    const char * qu;  int64_t nbu1, nbu2, nbu3;                  // F32 [D, Nq, H, B]: q + pos_bias_u
+    const char * qv;  int64_t nbw1, nbw2, nbw3;                  // F32 [D, Nq, H, B]: q + pos_bias_v
+    const char * k;   int64_t nbk1, nbk2, nbk3;                  // F16 [D, Nkv, H / gqa, B / bq]
+    const char * v;   int64_t nbv1, nbv2, nbv3;
+    const char * r;   int64_t nbr1, nbr2, nbr3; int32_t Hr, Br;   // F16 [D, Nq+Nkv-1, Hr, Br]
+    const char * add; int64_t nba1, nba2, nba3; int32_t Ha, Ba;   // optional F32 | F16 [>=Nkv, >=Nq, Ha, Ba]
+    int32_t add_f16;
+    float *      dst;                                            // F32 [D, H, Nq, B] contiguous
+    int32_t D, Nq, Nkv, H, B, gqa, bq;
+    float   scale;
+};
+
 // Launchers implemented next to their kernels; all return hipError_t as int.
 int fattn_vec_launch(const FattnArgs & a, int ktype, hipStream_t stream);
 int fattn_merge_launch(const FattnArgs & a, hipStream_t stream);
@@ -204,4 +218,6 @@ int set_rows_launch(const CpyArgs & a, int dtype, hipStream_t stream);
 int fill_launch(void * ptr, int value, size_t size, hipStream_t stream);      // memset by a kernel
 // K and V (F32 or Q8_0, any strides) -> contiguous f16 [D, Nkv, Hkv, Bk] at dst and right behind it
 int relpos_bias_launch(RelposArgs a, int rtype, hipStream_t stream);
+int fattn_relpos_launch(const FattnRelposArgs & a, hipStream_t stream);
+bool fattn_relpos_supported(const FattnRelposArgs & a);
 int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t stream);

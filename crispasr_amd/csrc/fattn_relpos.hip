@@ -1,0 +1,347 @@
+// FastConformer's relative-position attention in one kernel (the flash branch of core_conformer::build_block,
+// src/core/fastconformer.h:876-934):
+//
+//   dst[:, h, i, b] = softmax_j( scale * <q_u[i], k[j]> + mask[j, i] ) . v[j]
+//   mask[j, i]      = f16( scale * <q_v[i], r[Nq-1+j-i]> + add[j, i] )         (the graph's rel_shift view, scale, add, cast)
+//
+// The reference materialises `mask` as an F16 [T, T, H] tensor per sequence and hands it to ggml_flash_attn_ext; here
+// the position term is produced tile by tile inside the attention loop and never leaves the CU.
+//
+// A workgroup of 4 waves owns 128 consecutive queries of one (head, batch), 32 per wave (the N columns of
+// v_mfma_f32_32x32x16_f16 accumulators), and walks the keys 32 at a time.  Per step and wave:
+//   S^T  = K tile . Q_u^T                       8 (D = 128) MFMAs, A = K rows from LDS, B = Q_u in registers
+//   BD   = R block . Q_v^T                      8 MFMAs, A = 32 rows of the table from LDS, B = Q_v in registers.
+//          Block n x the wave's 32 queries is one accumulator whose element (row, il) belongs to key
+//          j = 32 n + row + il - 31: tile t is the lower-right triangle (row + il >= 31) of block t and the upper-left
+//          one of block t + 1, and for one accumulator slot exactly one of the two owns the slot's place in the tile -
+//          so the previous block stays in registers, one new block is computed per step and a select per slot gives
+//          the tile, each product computed once.
+//   un-skew: the selected values sit at key (row + il + 1) mod 32 of their query; they go through a wave-private
+//          32 x 32 f32 square in LDS (pitch 36: writes and the 16-byte row reads are both conflict-free) and come back
+//          in the layout of S^T.
+//   mask = f16(scale * BD + add), s = S + mask in log2 units, exact online softmax (the accumulators are rescaled
+//          only on steps where some row's maximum rises), P -> f16
+//   O^T += V^T . P^T                            8 MFMAs, A = V tile through ds_read_b64_tr_b16, B = P from registers
+// The four waves need the same table rows one step apart, so the table is staged once per workgroup in a ring of five
+// 32-row blocks; K, V and the next table block are fetched one step ahead into registers and written to LDS behind the
+// two barriers of a step.  K, V and the table are f16 with 16-byte aligned rows (the caller rounds F32 ones first, as
+// the reference's own graph does for the mask product's operands).
+#include "fattn_common.h"
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float    float16v __attribute__((ext_vector_type(16)));
+typedef float    float4v __attribute__((ext_vector_type(4)));
+typedef short    short4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float    float4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef _Float16 half4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+
+constexpr int   FR_WAVES = 4;
+constexpr int   FR_SLOTS = 5;                       // table blocks resident: four in use, one being written
+constexpr int   FR_SQP   = 36;                      // pitch of the un-skew square in floats
+constexpr float FR_LOG2E = 1.4426950408889634f;
+
+template <int D> constexpr int fr_kp() { return 2 * D + 16; }     // bytes per K / table row in LDS
+template <int D> constexpr int fr_vp() { return 2 * D + 64; }     // bytes per V row in LDS
+template <int D> constexpr int fr_lds_bytes() {
+    return 32 * fr_kp<D>() + 32 * fr_vp<D>() + FR_SLOTS * 32 * fr_kp<D>() + FR_WAVES * 32 * FR_SQP * 4;
+}
+
+template <int D, bool ADD, bool ADD_F16>
+__global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const FattnRelposArgs a) {
+    constexpr int KS  = D / 16;                     // reduction steps of the two Q products
+    constexpr int DBO = D / 32;                     // 32-wide blocks of the output's d
+    constexpr int CH  = D / 8;                      // 16-byte chunks per row
+    constexpr int NLD = 32 * CH / (FR_WAVES * 64);  // chunks per thread and 32-row tile
+    constexpr int KP  = fr_kp<D>();
+    constexpr int VP  = fr_vp<D>();
+
+    extern __shared__ __attribute__((aligned(16))) char fr_lds[];
+    char * const kt   = fr_lds;
+    char * const vt   = kt + 32 * KP;
+    char * const ring = vt + 32 * VP;
+    const int tid  = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lane = tid & 63;
+    const int il   = lane & 31;
+    const int hh   = lane >> 5;
+    float * const sq = (float *)(ring + FR_SLOTS * 32 * KP) + wave * 32 * FR_SQP;
+
+    // Workgroups go to the 8 XCDs round-robin, each with its own L2: the query blocks of one (head, batch) are given to
+    // one XCD, so that K, V and the table rows they share come from that L2.
+    const int     n_qb = (a.Nq + 127) / 128;
+    const int64_t G    = (int64_t)n_qb * a.H * a.B;
+    const int64_t per  = (G + 7) / 8;
+    const int64_t L    = (int64_t)(blockIdx.x & 7) * per + (blockIdx.x >> 3);
+    if ((blockIdx.x >> 3) >= per || L >= G) return;
+    const int qb = (int)(L % n_qb);
+    const int h  = (int)((L / n_qb) % a.H);
+    const int b  = (int)(L / ((int64_t)n_qb * a.H));
+    const int hk = h / a.gqa, bk = b / a.bq;
+
+    const int q0  = qb * 128;
+    const int i0w = q0 + wave * 32;
+    const int iq  = min(i0w + il, a.Nq - 1);        // rows past Nq repeat the last one and are not stored
+    const int NT  = (a.Nkv + 31) / 32;
+    const int NR  = a.Nq + a.Nkv - 1;
+    const int p_base0 = a.Nq - 1 - q0 - 31;         // table row of (block 0, row 0) in wave 0's numbering; wave w's block n is block n - w
+
+    const char * kbase = a.k + (int64_t)hk * a.nbk2 + (int64_t)bk * a.nbk3;
+    const char * vbase = a.v + (int64_t)hk * a.nbv2 + (int64_t)bk * a.nbv3;
+    const char * rbase = a.r + (int64_t)(h % a.Hr) * a.nbr2 + (int64_t)(b % a.Br) * a.nbr3;
+
+    // ---- staging: thread -> (row, chunk) of a 32-row tile ------------------------------------------------------
+    u32x4 kraw[NLD], vraw[NLD], rraw[NLD];
+    auto load_k = [&](int t) __attribute__((always_inline)) {
+#pragma unroll
+        for (int n = 0; n < NLD; n++) {
+            const int idx = n * 256 + tid, row = idx / CH, c = idx % CH;
+            const int key = min(32 * t + row, a.Nkv - 1);
+            kraw[n] = *(const u32x4 *)(kbase + (int64_t)key * a.nbk1 + c * 16);
+        }
+    };
+    auto load_v = [&](int t) __attribute__((always_inline)) {
+#pragma unroll
+        for (int n = 0; n < NLD; n++) {
+            const int idx = n * 256 + tid, row = idx / CH, c = idx % CH;
+            const int key = min(32 * t + row, a.Nkv - 1);
+            vraw[n] = *(const u32x4 *)(vbase + (int64_t)key * a.nbv1 + c * 16);
+        }
+    };
+    auto load_r = [&](int beta) __attribute__((always_inline)) {
+#pragma unroll
+        for (int n = 0; n < NLD; n++) {
+            const int idx = n * 256 + tid, row = idx / CH, c = idx % CH;
+            const int rho = min(max(p_base0 + 32 * beta + row, 0), NR - 1);       // rows outside the table belong to no key
+            rraw[n] = *(const u32x4 *)(rbase + (int64_t)rho * a.nbr1 + c * 16);
+        }
+    };
+    auto store_tile = [&](char * dst, int pitch, const u32x4 (&raw)[NLD]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int n = 0; n < NLD; n++) {
+            const int idx = n * 256 + tid, row = idx / CH, c = idx % CH;
+            *(u32x4 *)(dst + row * pitch + c * 16) = raw[n];
+        }
+    };
+    auto slot_of = [&](int beta) { return ring + ((beta + 3) % FR_SLOTS) * 32 * KP; };   // beta >= -3
+
+    // ---- prologue: table blocks -3 .. 1, the first K and V tiles, Q_u and Q_v as B operands ------------------------
+#pragma unroll 1
+    for (int beta = -3; beta <= 1; beta++) {
+        load_r(beta);
+        store_tile(slot_of(beta), KP, rraw);
+    }
+    load_k(0);
+    load_v(0);
+    half8 qu[KS], qv[KS];
+    {
+        const float * pu = (const float *)(a.qu + (int64_t)iq * a.nbu1 + (int64_t)h * a.nbu2 + (int64_t)b * a.nbu3);
+        const float * pv = (const float *)(a.qv + (int64_t)iq * a.nbw1 + (int64_t)h * a.nbw2 + (int64_t)b * a.nbw3);
+        const float   qs = a.scale * FR_LOG2E;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const float4v u0 = *(const float4v *)(pu + ks * 16 + hh * 8), u1 = *(const float4v *)(pu + ks * 16 + hh * 8 + 4);
+            const float4v w0 = *(const float4v *)(pv + ks * 16 + hh * 8), w1 = *(const float4v *)(pv + ks * 16 + hh * 8 + 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                qu[ks][e] = (_Float16)(u0[e] * qs); qu[ks][e + 4] = (_Float16)(u1[e] * qs);
+                qv[ks][e] = (_Float16)w0[e];        qv[ks][e + 4] = (_Float16)w1[e];
+            }
+        }
+    }
+    store_tile(kt, KP, kraw);
+    store_tile(vt, VP, vraw);
+    __syncthreads();
+    if (NT > 1) { load_k(1); load_v(1); }
+    load_r(2);
+
+    // operand fetch of a K or table row block: lane (il, hh) takes d = 16 ks + 8 hh .. +7 of row il
+    auto block_times_q = [&](const char * blk, const half8 (&q)[KS]) __attribute__((always_inline)) {
+        float16v acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const half8 av = *(const half8 *)(blk + il * KP + (ks * 2 + hh) * 16);
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, q[ks], acc, 0, 0, 0);
+        }
+        return acc;
+    };
+
+    // the wave's block 0 (= block -wave in wave 0's numbering): its lower-right triangle is the first tile's
+    float16v bd_prev = block_times_q(slot_of(-wave), qv);
+
+    float16v oacc[DBO];
+#pragma unroll
+    for (int db = 0; db < DBO; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[db][r] = 0.0f;
+    float m = -INFINITY, l = 0.0f;
+
+    const char * addrow = nullptr;
+    if (ADD) addrow = a.add + (int64_t)iq * a.nba1 + (int64_t)(h % a.Ha) * a.nba2 + (int64_t)(b % a.Ba) * a.nba3;
+
+#pragma unroll 1
+    for (int t = 0; t < NT; t++) {
+        // ---- the two products against this step's K tile and table block --------------------------------------------
+        float16v s      = block_times_q(kt, qu);
+        float16v bd_new = block_times_q(slot_of(t + 1 - wave), qv);
+        __syncthreads();                                  // every wave has read the K tile and its table block
+        if (t + 1 < NT) store_tile(kt, KP, kraw);
+        store_tile(slot_of(t + 2), KP, rraw);
+        if (t + 2 < NT) load_k(t + 2);
+        load_r(t + 3);
+
+        // ---- select per slot, un-skew through the square ---------------------------------------------------------
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int   row = 8 * (r >> 2) + 4 * hh + (r & 3);
+            const float val = row + il >= 31 ? bd_prev[r] : bd_new[r];
+            sq[il * FR_SQP + ((row + il + 1) & 31)] = val;
+        }
+        bd_prev = bd_new;
+        __builtin_amdgcn_wave_barrier();
+        float bd[16];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const float4v x = *(const float4v *)&sq[il * FR_SQP + 8 * g + 4 * hh];
+            bd[4 * g] = x[0]; bd[4 * g + 1] = x[1]; bd[4 * g + 2] = x[2]; bd[4 * g + 3] = x[3];
+        }
+        __builtin_amdgcn_wave_barrier();
+
+        // ---- mask = f16(scale * BD + add); scores in log2 units ------------------------------------------------------
+        const bool tail = 32 * t + 32 > a.Nkv;             // uniform
+        float s2[16];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const int key0 = 32 * t + 8 * g + 4 * hh;
+            float av[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (ADD) {
+                if (!tail) {
+                    if (ADD_F16) {
+                        const half4_a2 x = *(const half4_a2 *)(addrow + (int64_t)key0 * 2);
+                        av[0] = (float)x[0]; av[1] = (float)x[1]; av[2] = (float)x[2]; av[3] = (float)x[3];
+                    } else {
+                        const float4_a4 x = *(const float4_a4 *)(addrow + (int64_t)key0 * 4);
+                        av[0] = x[0]; av[1] = x[1]; av[2] = x[2]; av[3] = x[3];
+                    }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        const int key = min(key0 + c, a.Nkv - 1);
+                        av[c] = ADD_F16 ? (float)*(const _Float16 *)(addrow + (int64_t)key * 2) : *(const float *)(addrow + (int64_t)key * 4);
+                    }
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const float    mk = __fadd_rn(__fmul_rn(bd[4 * g + c], a.scale), av[c]);     // as the graph: scale, then add
+                const _Float16 mh = (_Float16)mk;
+                float x = fmaf((float)mh, FR_LOG2E, s[4 * g + c]);
+                if (tail && key0 + c >= a.Nkv) x = -INFINITY;
+                s2[4 * g + c] = x;
+            }
+        }
+
+        // ---- online softmax ----------------------------------------------------------------------------------------------
+        float tmax = s2[0];
+#pragma unroll
+        for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, s2[r]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        if (__builtin_amdgcn_ballot_w64(tmax > m) != 0) {
+            const float mn = fmaxf(m, tmax);
+            const float f  = mn == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m - mn);     // m = -inf: nothing accumulated yet, f = 0
+            l *= f;
+#pragma unroll
+            for (int db = 0; db < DBO; db++) oacc[db] *= f;
+            m = mn;
+        }
+        const float ms = m == -INFINITY ? 0.0f : m;
+        half8 p[2];
+        float lsum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const float e = __builtin_amdgcn_exp2f(s2[r] - ms);
+            lsum += e;
+            p[r >> 3][r & 7] = (_Float16)e;
+        }
+        l += lsum;
+
+        // ---- O^T += V^T . P^T -------------------------------------------------------------------------------------------
+        {
+            const int j16 = lane & 15, G16 = lane >> 4;
+#pragma unroll
+            for (int db = 0; db < DBO; db++) {
+#pragma unroll
+                for (int ks = 0; ks < 2; ks++) {
+                    const char * p0 = vt + (16 * ks + 4 * (G16 >> 1) + (j16 >> 2)) * VP + (32 * db + 16 * (G16 & 1) + 4 * (j16 & 3)) * 2;
+                    const half4 lo = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p0));
+                    const half4 hi = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(p0 + 8 * VP)));
+                    const half8 va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, p[ks], oacc[db], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();                                  // every wave has read the V tile (the next one is read behind the next step's first barrier)
+        if (t + 1 < NT) store_tile(vt, VP, vraw);
+        if (t + 2 < NT) load_v(t + 2);
+    }
+
+    // ---- normalise and store: lane (il, hh) holds d = 32 db + 8 g + 4 hh + c of its query -------------------------------
+    l += __shfl_xor(l, 32, 64);
+    if (i0w + il < a.Nq) {
+        const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+        float * orow = a.dst + (((int64_t)b * a.Nq + (i0w + il)) * a.H + h) * D;
+#pragma unroll
+        for (int db = 0; db < DBO; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                float4v o;
+#pragma unroll
+                for (int c = 0; c < 4; c++) o[c] = oacc[db][4 * g + c] * inv;
+                *(float4v *)(orow + 32 * db + 8 * g + 4 * hh) = o;
+            }
+    }
+}
+
+template <int D>
+int launch_d(const FattnRelposArgs & a, hipStream_t stream) {
+    const int64_t G = (int64_t)((a.Nq + 127) / 128) * a.H * a.B;
+    const int64_t grid = (G + 7) / 8 * 8;
+    if (grid > 0x7fffffff) return (int)hipErrorInvalidValue;
+    constexpr int lds = fr_lds_bytes<D>();
+#define FR_LAUNCH(ADD, F16)                                                                                                   \
+    do {                                                                                                                      \
+        static bool attr_set = false;                                                                                         \
+        if (!attr_set && lds > 64 * 1024) {                                                                                   \
+            const hipError_t e = hipFuncSetAttribute((const void *)fattn_relpos_kernel<D, ADD, F16>,                          \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, lds);                      \
+            if (e != hipSuccess) return (int)e;                                                                               \
+            attr_set = true;                                                                                                  \
+        }                                                                                                                     \
+        hipLaunchKernelGGL((fattn_relpos_kernel<D, ADD, F16>), dim3((unsigned)grid), dim3(FR_WAVES * 64), lds, stream, a);    \
+    } while (0)
+    if (!a.add)          FR_LAUNCH(false, false);
+    else if (a.add_f16)  FR_LAUNCH(true, true);
+    else                 FR_LAUNCH(true, false);
+#undef FR_LAUNCH
+    return (int)hipGetLastError();
+}
+
+}  // namespace
+
+bool fattn_relpos_supported(const FattnRelposArgs & a) {
+    if (a.D != 64 && a.D != 128) return false;
+    if (a.Nq < 1 || a.Nkv < 1 || a.H < 1 || a.B < 1) return false;
+    // 32-bit tile indices; the table's rows Nq-1+j-i must exist
+    if ((int64_t)a.Nq + a.Nkv > (1 << 24)) return false;
+    return true;
+}
+
+int fattn_relpos_launch(const FattnRelposArgs & a, hipStream_t stream) {
+    if (!fattn_relpos_supported(a)) return (int)hipErrorInvalidValue;
+    return a.D == 64 ? launch_d<64>(a, stream) : launch_d<128>(a, stream);
+}
