@@ -23,8 +23,9 @@
 //          only on steps where some row's maximum rises), P -> f16
 //   O^T += V^T . P^T                            8 MFMAs, A = V tile through ds_read_b64_tr_b16, B = P from registers
 // The four waves need the same table rows one step apart, so the table is staged once per workgroup in a ring of five
-// 32-row blocks; K, V and the next table block are fetched one step ahead into registers and written to LDS behind the
-// two barriers of a step.  K, V and the table are f16 with 16-byte aligned rows (the caller rounds F32 ones first, as
+// 32-row blocks.  K tiles and table blocks move global -> LDS without passing registers (global_load_lds_dwordx4, the
+// 16-byte chunks of a row XOR-swizzled so that the operand reads are conflict-free), requested behind the first barrier
+// of a step and waited for before the second; V is fetched one step ahead into registers and written behind the second.  K, V and the table are f16 with 16-byte aligned rows (the caller rounds F32 ones first, as
 // the reference's own graph does for the mask product's operands).
 #include "fattn_common.h"
 
@@ -44,7 +45,8 @@ constexpr int   FR_SLOTS = 5;                       // table blocks resident: fo
 constexpr int   FR_SQP   = 36;                      // pitch of the un-skew square in floats
 constexpr float FR_LOG2E = 1.4426950408889634f;
 
-template <int D> constexpr int fr_kp() { return 2 * D + 16; }     // bytes per K / table row in LDS
+template <int D> constexpr int fr_kp() { return 2 * D; }          // bytes per K / table row in LDS (chunks swizzled, no padding)
+template <int D> __device__ __forceinline__ int fr_swz(int r) { return D == 64 ? (r >> 1) & 7 : r & 15; }
 template <int D> constexpr int fr_vp() { return 2 * D + 64; }     // bytes per V row in LDS
 template <int D> constexpr int fr_lds_bytes() {
     return 32 * fr_kp<D>() + 32 * fr_vp<D>() + FR_SLOTS * 32 * fr_kp<D>() + FR_WAVES * 32 * FR_SQP * 4;
@@ -93,48 +95,52 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
     const char * vbase = a.v + (int64_t)hk * a.nbv2 + (int64_t)bk * a.nbv3;
     const char * rbase = a.r + (int64_t)(h % a.Hr) * a.nbr2 + (int64_t)(b % a.Br) * a.nbr3;
 
-    // ---- staging: thread -> (row, chunk) of a 32-row tile ------------------------------------------------------
-    u32x4 kraw[NLD], vraw[NLD], rraw[NLD];
-    auto load_k = [&](int t) __attribute__((always_inline)) {
+    // ---- staging ------------------------------------------------------------------------------------------------
+    // K tiles and table blocks: each wave moves its quarter, 64 x 16 bytes per instruction; LDS slot
+    // L = (wave * NDM + j) * 64 + lane holds chunk (L % CH) ^ swizzle of row L / CH.  Rows that stick out (the last key
+    // tile, the ends of the table) repeat the nearest valid row: they belong to excluded keys or to no key at all.
+    constexpr int NDM = 32 * CH * 16 / 1024 / FR_WAVES;
+    typedef __attribute__((address_space(3))) void * lds_vptr;
+    typedef const __attribute__((address_space(1))) void * glb_vptr;
+    auto dma_rows = [&](char * dst, const char * base, int64_t nb1, int row0, int last_row) __attribute__((always_inline)) {
+        const bool inside = row0 >= 0 && row0 + 31 <= last_row;      // uniform
+        const char * p = base + (int64_t)(inside ? row0 : 0) * nb1;
 #pragma unroll
-        for (int n = 0; n < NLD; n++) {
-            const int idx = n * 256 + tid, row = idx / CH, c = idx % CH;
-            const int key = min(32 * t + row, a.Nkv - 1);
-            kraw[n] = *(const u32x4 *)(kbase + (int64_t)key * a.nbk1 + c * 16);
+        for (int j = 0; j < NDM; j++) {
+            const int L = (wave * NDM + j) * 64 + lane, r = L / CH, c = (L % CH) ^ fr_swz<D>(r);
+            const int rr = inside ? r : min(max(row0 + r, 0), last_row);
+            __builtin_amdgcn_global_load_lds((glb_vptr)(p + ((uint32_t)rr * (uint32_t)nb1 + (uint32_t)c * 16u)),
+                                             (lds_vptr)(dst + (wave * NDM + j) * 1024), 16, 0, 0);
         }
     };
-    auto load_v = [&](int t) __attribute__((always_inline)) {
-#pragma unroll
-        for (int n = 0; n < NLD; n++) {
-            const int idx = n * 256 + tid, row = idx / CH, c = idx % CH;
-            const int key = min(32 * t + row, a.Nkv - 1);
-            vraw[n] = *(const u32x4 *)(vbase + (int64_t)key * a.nbv1 + c * 16);
-        }
-    };
-    auto load_r = [&](int beta) __attribute__((always_inline)) {
-#pragma unroll
-        for (int n = 0; n < NLD; n++) {
-            const int idx = n * 256 + tid, row = idx / CH, c = idx % CH;
-            const int rho = min(max(p_base0 + 32 * beta + row, 0), NR - 1);       // rows outside the table belong to no key
-            rraw[n] = *(const u32x4 *)(rbase + (int64_t)rho * a.nbr1 + c * 16);
-        }
-    };
-    auto store_tile = [&](char * dst, int pitch, const u32x4 (&raw)[NLD]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int n = 0; n < NLD; n++) {
-            const int idx = n * 256 + tid, row = idx / CH, c = idx % CH;
-            *(u32x4 *)(dst + row * pitch + c * 16) = raw[n];
-        }
-    };
+    auto dma_k = [&](int t) __attribute__((always_inline)) { dma_rows(kt, kbase, a.nbk1, 32 * t, a.Nkv - 1); };
     auto slot_of = [&](int beta) { return ring + ((beta + 3) % FR_SLOTS) * 32 * KP; };   // beta >= -3
+    auto dma_r = [&](int beta) __attribute__((always_inline)) { dma_rows(slot_of(beta), rbase, a.nbr1, p_base0 + 32 * beta, NR - 1); };
+    // V: thread -> (row, chunk), one step ahead through registers
+    u32x4 vraw[NLD];
+    auto load_v = [&](int t) __attribute__((always_inline)) {
+        const int  row0   = 32 * t;
+        const bool inside = row0 + 31 <= a.Nkv - 1;
+        const char * p = vbase + (int64_t)(inside ? row0 : 0) * a.nbv1;
+#pragma unroll
+        for (int n = 0; n < NLD; n++) {
+            const int idx = n * 256 + tid, row = idx / CH, c = idx % CH;
+            const int rr  = inside ? row : min(row0 + row, a.Nkv - 1);
+            vraw[n] = *(const u32x4 *)(p + ((uint32_t)rr * (uint32_t)a.nbv1 + (uint32_t)c * 16u));
+        }
+    };
+    auto store_v = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int n = 0; n < NLD; n++) {
+            const int idx = n * 256 + tid, row = idx / CH, c = idx % CH;
+            *(u32x4 *)(vt + row * VP + c * 16) = vraw[n];
+        }
+    };
 
     // ---- prologue: table blocks -3 .. 1, the first K and V tiles, Q_u and Q_v as B operands ------------------------
 #pragma unroll 1
-    for (int beta = -3; beta <= 1; beta++) {
-        load_r(beta);
-        store_tile(slot_of(beta), KP, rraw);
-    }
-    load_k(0);
+    for (int beta = -3; beta <= 1; beta++) dma_r(beta);
+    dma_k(0);
     load_v(0);
     half8 qu[KS], qv[KS];
     {
@@ -152,20 +158,23 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
             }
         }
     }
-    store_tile(kt, KP, kraw);
-    store_tile(vt, VP, vraw);
+    store_v();
+    __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): this wave's share of the blocks is in LDS
     __syncthreads();
-    if (NT > 1) { load_k(1); load_v(1); }
-    load_r(2);
+    if (NT > 1) load_v(1);
 
-    // operand fetch of a K or table row block: lane (il, hh) takes d = 16 ks + 8 hh .. +7 of row il
+    // operand reads of a K or table block: lane (il, hh) takes d = 16 ks + 8 hh .. +7 of row il
+    uint32_t opaddr[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) opaddr[ks] = (uint32_t)((il * CH + ((ks * 2 + hh) ^ fr_swz<D>(il))) * 16);
+
     auto block_times_q = [&](const char * blk, const half8 (&q)[KS]) __attribute__((always_inline)) {
         float16v acc;
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[r] = 0.0f;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-            const half8 av = *(const half8 *)(blk + il * KP + (ks * 2 + hh) * 16);
+            const half8 av = *(const half8 *)(blk + opaddr[ks]);
             acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, q[ks], acc, 0, 0, 0);
         }
         return acc;
@@ -184,67 +193,74 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
     const char * addrow = nullptr;
     if (ADD) addrow = a.add + (int64_t)iq * a.nba1 + (int64_t)(h % a.Ha) * a.nba2 + (int64_t)(b % a.Ba) * a.nba3;
 
+    // un-skew constants: slot r of a lane sits at row k_r + 4 hh of its block, i.e. at key (x + k_r) mod 32 with
+    // x = il + 4 hh + 1, and belongs to the previous block exactly when that sum reaches 32
+    const int x_lane = il + 4 * hh + 1;
+    const int sq_new = il * FR_SQP + x_lane, sq_prev = sq_new - 32;
+
 #pragma unroll 1
     for (int t = 0; t < NT; t++) {
-        // ---- the two products against this step's K tile and table block --------------------------------------------
-        float16v s      = block_times_q(kt, qu);
-        float16v bd_new = block_times_q(slot_of(t + 1 - wave), qv);
-        __syncthreads();                                  // every wave has read the K tile and its table block
-        if (t + 1 < NT) store_tile(kt, KP, kraw);
-        store_tile(slot_of(t + 2), KP, rraw);
-        if (t + 2 < NT) load_k(t + 2);
-        load_r(t + 3);
-
-        // ---- select per slot, un-skew through the square ---------------------------------------------------------
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int   row = 8 * (r >> 2) + 4 * hh + (r & 3);
-            const float val = row + il >= 31 ? bd_prev[r] : bd_new[r];
-            sq[il * FR_SQP + ((row + il + 1) & 31)] = val;
-        }
-        bd_prev = bd_new;
-        __builtin_amdgcn_wave_barrier();
-        float bd[16];
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const float4v x = *(const float4v *)&sq[il * FR_SQP + 8 * g + 4 * hh];
-            bd[4 * g] = x[0]; bd[4 * g + 1] = x[1]; bd[4 * g + 2] = x[2]; bd[4 * g + 3] = x[3];
-        }
-        __builtin_amdgcn_wave_barrier();
-
-        // ---- mask = f16(scale * BD + add); scores in log2 units ------------------------------------------------------
         const bool tail = 32 * t + 32 > a.Nkv;             // uniform
-        float s2[16];
+        // the additive mask of this tile: requested first, used after the products
+        float av[16];
+        if (ADD) {
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const int key0 = 32 * t + 8 * g + 4 * hh;
-            float av[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (ADD) {
+            for (int g = 0; g < 4; g++) {
+                const int key0 = 32 * t + 8 * g + 4 * hh;
                 if (!tail) {
                     if (ADD_F16) {
                         const half4_a2 x = *(const half4_a2 *)(addrow + (int64_t)key0 * 2);
-                        av[0] = (float)x[0]; av[1] = (float)x[1]; av[2] = (float)x[2]; av[3] = (float)x[3];
+#pragma unroll
+                        for (int c = 0; c < 4; c++) av[4 * g + c] = (float)x[c];
                     } else {
                         const float4_a4 x = *(const float4_a4 *)(addrow + (int64_t)key0 * 4);
-                        av[0] = x[0]; av[1] = x[1]; av[2] = x[2]; av[3] = x[3];
+#pragma unroll
+                        for (int c = 0; c < 4; c++) av[4 * g + c] = x[c];
                     }
                 } else {
 #pragma unroll
                     for (int c = 0; c < 4; c++) {
                         const int key = min(key0 + c, a.Nkv - 1);
-                        av[c] = ADD_F16 ? (float)*(const _Float16 *)(addrow + (int64_t)key * 2) : *(const float *)(addrow + (int64_t)key * 4);
+                        av[4 * g + c] = ADD_F16 ? (float)*(const _Float16 *)(addrow + (int64_t)key * 2) : *(const float *)(addrow + (int64_t)key * 4);
                     }
                 }
             }
+        }
+        // ---- the position product against this step's table block; select per slot, un-skew through the square ------
+        {
+            const float16v bd_new = block_times_q(slot_of(t + 1 - wave), qv);
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int  k_r  = 8 * (r >> 2) + (r & 3);
+                const bool prev = x_lane + k_r >= 32;
+                sq[(prev ? sq_prev : sq_new) + k_r] = prev ? bd_prev[r] : bd_new[r];
+            }
+            bd_prev = bd_new;
+        }
+        // ---- the content product against this step's K tile -------------------------------------------------------------
+        const float16v s = block_times_q(kt, qu);
+        __syncthreads();                                  // every wave has read the K tile and its table block
+        if (t + 1 < NT) {
+            dma_k(t + 1);
+            dma_r(t + 2);
+        }
+
+        // ---- mask = f16(scale * BD + add); scores in log2 units ------------------------------------------------------
+        float s2[16];
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const float4v bd = *(const float4v *)&sq[il * FR_SQP + 8 * g + 4 * hh];
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                const float    mk = __fadd_rn(__fmul_rn(bd[4 * g + c], a.scale), av[c]);     // as the graph: scale, then add
+                float mk = __fmul_rn(bd[c], a.scale);                                        // as the graph: scale, then add
+                if (ADD) mk = __fadd_rn(mk, av[4 * g + c]);
                 const _Float16 mh = (_Float16)mk;
                 float x = fmaf((float)mh, FR_LOG2E, s[4 * g + c]);
-                if (tail && key0 + c >= a.Nkv) x = -INFINITY;
+                if (tail && 32 * t + 8 * g + 4 * hh + c >= a.Nkv) x = -INFINITY;
                 s2[4 * g + c] = x;
             }
         }
+        __builtin_amdgcn_wave_barrier();
 
         // ---- online softmax ----------------------------------------------------------------------------------------------
         float tmax = s2[0];
@@ -285,8 +301,9 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
                 }
             }
         }
+        __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): the next K tile and table block (and V in registers) have arrived
         __syncthreads();                                  // every wave has read the V tile (the next one is read behind the next step's first barrier)
-        if (t + 1 < NT) store_tile(vt, VP, vraw);
+        if (t + 1 < NT) store_v();
         if (t + 2 < NT) load_v(t + 2);
     }
 
