@@ -924,8 +924,20 @@ static int relpos_fused_run(const mi355x_tensor * q_u, const mi355x_tensor * q_v
     FattnArgs a;
     fill_args(a, q_u, k, v, nullptr, (float *)dst->data, params);
     if (!q_v->data || !r->data) return fail(MI355X_ERR_INVALID, "null data pointer");
+    // an F32 table with aligned rows is rounded by the launch that rounds K and V
+    bool table_done = false;
     if (f.kv_copy) {
-        const int e = kv_to_f16_launch(a, k->type, ws, st);
+        F32Rider x;
+        memset(&x, 0, sizeof(x));
+        if (f.table_bytes && r->type == MI355X_TYPE_F32 && aligned16_view(r)) {
+            x.src = (const char *)r->data;
+            x.dst = (char *)ws + f.kv_bytes;
+            x.ne1 = r->ne[1]; x.ne2 = r->ne[2];
+            x.nb1 = (int64_t)r->nb[1]; x.nb2 = (int64_t)r->nb[2]; x.nb3 = (int64_t)r->nb[3];
+            x.n   = (int64_t)(a.D / 8) * r->ne[1] * r->ne[2] * r->ne[3];
+            table_done = true;
+        }
+        const int e = kv_to_f16_launch(a, k->type, ws, st, table_done ? &x : nullptr);
         if (e) return hip_fail((hipError_t)e, "K/V conversion launch");
         use_f16_copies(a, ws);
     }
@@ -940,6 +952,7 @@ static int relpos_fused_run(const mi355x_tensor * q_u, const mi355x_tensor * q_v
     if (f.table_bytes) {
         char * r16 = (char *)ws + f.kv_bytes;
         CpyArgs c;
+        if (!table_done) {
         memset(&c, 0, sizeof(c));
         c.src = (const char *)r->data;
         c.dst = r16;
@@ -954,6 +967,7 @@ static int relpos_fused_run(const mi355x_tensor * q_u, const mi355x_tensor * q_v
         }
         const int e = cpy_launch(c, r->type, MI355X_TYPE_F16, st);
         if (e) return hip_fail((hipError_t)e, "table conversion launch");
+        }
         g.r = r16;
         g.nbr1 = (int64_t)a.D * 2; g.nbr2 = g.nbr1 * r->ne[1]; g.nbr3 = g.nbr2 * r->ne[2];
     }
@@ -967,6 +981,7 @@ static int relpos_fused_run(const mi355x_tensor * q_u, const mi355x_tensor * q_v
     g.dst = (float *)dst->data;
     g.D = a.D; g.Nq = a.Nq; g.Nkv = a.Nkv; g.H = a.Hq; g.B = a.B; g.gqa = a.gqa; g.bq = a.bq;
     g.scale = params->scale;
+    g.n_cus = a.n_cus;
     if (!fattn_relpos_supported(g)) return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the one-kernel form");
     const int e = fattn_relpos_launch(g, st);
     if (e) return hip_fail((hipError_t)e, "relative-position attention launch");

@@ -6,6 +6,8 @@
 // counts (the reference copies a [n_state, n_ctx] tensor into a 1-D cache view).
 #include "fattn_common.h"
 
+#include <string.h>
+
 namespace {
 
 // byte offset of unit i, where a unit is `unit0` elements along dimension 0 and one step of
@@ -178,12 +180,31 @@ __global__ void __launch_bounds__(256) set_rows_kernel(const CpyArgs a) {
 // launch for both.  One lane per 8 elements of a row: two 128-bit loads (F32) or 8 quants and the block's scale
 // (Q8_0), one 128-bit store.  Rounding is the tile kernel's own: f32 -> f16 round-to-nearest-even, q*d exact in f32
 // and then rounded once.
+// An F32 table [D, n1, n2, n3] with 16-byte aligned rows may ride along (the relative-position table of a FastConformer
+// block, rounded for the same call): the threads behind K's and V's write its contiguous f16 copy.
 template <int TYPE>
-__global__ void __launch_bounds__(256) kv_to_f16_kernel(const FattnArgs a, char * dst) {
+__global__ void __launch_bounds__(256) kv_to_f16_kernel(const FattnArgs a, char * dst, const F32Rider x) {
     const int     cpr  = a.D / 8;                                  // chunks per row
     const int64_t half = (int64_t)cpr * a.Nkv * a.Hkv * a.Bk;      // chunks per tensor
     int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= 2 * half) return;
+    if (i >= 2 * half) {
+        i -= 2 * half;
+        if (i >= x.n) return;
+        const int c = (int)(i % cpr);
+        int64_t   r = i / cpr;
+        const int64_t i1 = r % x.ne1;  r /= x.ne1;
+        const int64_t i2 = r % x.ne2;
+        const int64_t i3 = r / x.ne2;
+        const char * row = x.src + i1 * x.nb1 + i2 * x.nb2 + i3 * x.nb3;
+        const float4 x0 = *(const float4 *)(row + c * 32);
+        const float4 x1 = *(const float4 *)(row + c * 32 + 16);
+        typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+        h8 y;
+        y[0] = (_Float16)x0.x; y[1] = (_Float16)x0.y; y[2] = (_Float16)x0.z; y[3] = (_Float16)x0.w;
+        y[4] = (_Float16)x1.x; y[5] = (_Float16)x1.y; y[6] = (_Float16)x1.z; y[7] = (_Float16)x1.w;
+        *(h8 *)(x.dst + i * 16) = y;
+        return;
+    }
     const bool is_v = i >= half;
     if (is_v) i -= half;
     const int     c = (int)(i % cpr);
@@ -235,12 +256,16 @@ int fill_launch(void * ptr, int value, size_t size, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
-int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t stream) {
-    const int64_t n = 2 * (int64_t)(a.D / 8) * a.Nkv * a.Hkv * a.Bk;
+int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t stream, const F32Rider * rider) {
+    F32Rider x;
+    memset(&x, 0, sizeof(x));
+    if (rider) x = *rider;
+    const int64_t n = 2 * (int64_t)(a.D / 8) * a.Nkv * a.Hkv * a.Bk + x.n;
     if (n == 0) return 0;
+    if ((n + 255) / 256 > 0x7fffffff) return (int)hipErrorInvalidValue;
     const unsigned g = (unsigned)((n + 255) / 256);
     switch (ktype) {
-#define KV16(T) case T: hipLaunchKernelGGL((kv_to_f16_kernel<T>), dim3(g), dim3(256), 0, stream, a, (char *)dst); break
+#define KV16(T) case T: hipLaunchKernelGGL((kv_to_f16_kernel<T>), dim3(g), dim3(256), 0, stream, a, (char *)dst, x); break
         KV16(MI355X_TYPE_F32);
         KV16(MI355X_TYPE_Q8_0);
         KV16(MI355X_TYPE_Q4_0);

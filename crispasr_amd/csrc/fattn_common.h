@@ -194,6 +194,7 @@ struct FattnRelposArgs {
     int32_t add_f16;
     float *      dst;                                            // F32 [D, H, Nq, B] contiguous
     int32_t D, Nq, Nkv, H, B, gqa, bq;
+    int32_t n_cus;
     float   scale;
 };
 
@@ -220,4 +221,11 @@ int fill_launch(void * ptr, int value, size_t size, hipStream_t stream);      //
 int relpos_bias_launch(RelposArgs a, int rtype, hipStream_t stream);
 int fattn_relpos_launch(const FattnRelposArgs & a, hipStream_t stream);
 bool fattn_relpos_supported(const FattnRelposArgs & a);
-int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t stream);
+// an F32 tensor [D, ne1, ne2, ne3] (D = the attention call's head size, rows 16-byte aligned) converted to a contiguous f16
+// copy by the same launch; n = its 8-element chunks
+struct F32Rider {
+    const char * src;
+    char *       dst;
+    int64_t ne1, ne2, nb1, nb2, nb3, n;
+};
+int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t stream, const F32Rider * rider = nullptr);

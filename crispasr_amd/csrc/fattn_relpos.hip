@@ -19,8 +19,8 @@
 //   un-skew: the selected values sit at key (row + il + 1) mod 32 of their query; they go through a wave-private
 //          32 x 32 f32 square in LDS (pitch 36: writes and the 16-byte row reads are both conflict-free) and come back
 //          in the layout of S^T.
-//   mask = f16(scale * BD + add), s = S + mask in log2 units, exact online softmax (the accumulators are rescaled
-//          only on steps where some row's maximum rises), P -> f16
+//   mask = f16(scale * BD + add), s = S + mask in log2 units, online softmax against a reference that is raised
+//          only when a row's maximum outgrows it by a factor 256, P -> f16
 //   O^T += V^T . P^T                            8 MFMAs, A = V tile through ds_read_b64_tr_b16, B = P from registers
 // The four waves need the same table rows one step apart, so the table is staged once per workgroup in a ring of five
 // 32-row blocks.  K tiles and table blocks move global -> LDS without passing registers (global_load_lds_dwordx4, the
@@ -28,6 +28,9 @@
 // of a step and waited for before the second; V is fetched one step ahead into registers and written behind the second.  K, V and the table are f16 with 16-byte aligned rows (the caller rounds F32 ones first, as
 // the reference's own graph does for the mask product's operands).
 #include "fattn_common.h"
+
+#include <stdlib.h>
+#include <type_traits>
 
 namespace {
 
@@ -40,31 +43,29 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float    float4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 typedef _Float16 half4_a2 __attribute__((ext_vector_type(4), aligned(2)));
 
-constexpr int   FR_WAVES = 4;
-constexpr int   FR_SLOTS = 5;                       // table blocks resident: four in use, one being written
 constexpr int   FR_SQP   = 36;                      // pitch of the un-skew square in floats
 constexpr float FR_LOG2E = 1.4426950408889634f;
+constexpr float FR_SLACK = 8.0f;                    // log2 of the largest probability kept before the reference is raised
 
 template <int D> constexpr int fr_kp() { return 2 * D; }          // bytes per K / table row in LDS (chunks swizzled, no padding)
 template <int D> __device__ __forceinline__ int fr_swz(int r) { return D == 64 ? (r >> 1) & 7 : r & 15; }
-template <int D> constexpr int fr_vp() { return 2 * D + 64; }     // bytes per V row in LDS
-template <int D> constexpr int fr_lds_bytes() {
-    return 32 * fr_kp<D>() + 32 * fr_vp<D>() + FR_SLOTS * 32 * fr_kp<D>() + FR_WAVES * 32 * FR_SQP * 4;
-}
+template <int D> __device__ __forceinline__ int fr_swz_v(int r) { return D == 64 ? r & 7 : (r & 3) << 2; }
+// K tile, V tile, NW + 1 table blocks (NW in use, one being written), one un-skew square per wave
+template <int D, int NW> constexpr int fr_lds_bytes() { return (2 + NW + 1) * 32 * fr_kp<D>() + NW * 32 * FR_SQP * 4; }
 
-template <int D, bool ADD, bool ADD_F16>
-__global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const FattnRelposArgs a) {
+template <int D, int NW, bool ADD, bool ADD_F16>
+__global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) fattn_relpos_kernel(const FattnRelposArgs a) {
+    constexpr int FR_WAVES = NW;
+    constexpr int FR_SLOTS = NW + 1;
     constexpr int KS  = D / 16;                     // reduction steps of the two Q products
     constexpr int DBO = D / 32;                     // 32-wide blocks of the output's d
     constexpr int CH  = D / 8;                      // 16-byte chunks per row
-    constexpr int NLD = 32 * CH / (FR_WAVES * 64);  // chunks per thread and 32-row tile
     constexpr int KP  = fr_kp<D>();
-    constexpr int VP  = fr_vp<D>();
 
     extern __shared__ __attribute__((aligned(16))) char fr_lds[];
     char * const kt   = fr_lds;
     char * const vt   = kt + 32 * KP;
-    char * const ring = vt + 32 * VP;
+    char * const ring = vt + 32 * KP;
     const int tid  = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
@@ -74,7 +75,7 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
 
     // Workgroups go to the 8 XCDs round-robin, each with its own L2: the query blocks of one (head, batch) are given to
     // one XCD, so that K, V and the table rows they share come from that L2.
-    const int     n_qb = (a.Nq + 127) / 128;
+    const int     n_qb = (a.Nq + 32 * NW - 1) / (32 * NW);
     const int64_t G    = (int64_t)n_qb * a.H * a.B;
     const int64_t per  = (G + 7) / 8;
     const int64_t L    = (int64_t)(blockIdx.x & 7) * per + (blockIdx.x >> 3);
@@ -84,7 +85,7 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
     const int b  = (int)(L / ((int64_t)n_qb * a.H));
     const int hk = h / a.gqa, bk = b / a.bq;
 
-    const int q0  = qb * 128;
+    const int q0  = qb * 32 * NW;
     const int i0w = q0 + wave * 32;
     const int iq  = min(i0w + il, a.Nq - 1);        // rows past Nq repeat the last one and are not stored
     const int NT  = (a.Nkv + 31) / 32;
@@ -99,49 +100,36 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
     // K tiles and table blocks: each wave moves its quarter, 64 x 16 bytes per instruction; LDS slot
     // L = (wave * NDM + j) * 64 + lane holds chunk (L % CH) ^ swizzle of row L / CH.  Rows that stick out (the last key
     // tile, the ends of the table) repeat the nearest valid row: they belong to excluded keys or to no key at all.
-    constexpr int NDM = 32 * CH * 16 / 1024 / FR_WAVES;
+    constexpr int TI  = 32 * CH * 16 / 1024;                  // 64-lane instructions per tile
+    constexpr int NDM = (TI + NW - 1) / NW;                   // ... per wave: instruction j of wave w is number j * NW + w
     typedef __attribute__((address_space(3))) void * lds_vptr;
     typedef const __attribute__((address_space(1))) void * glb_vptr;
-    auto dma_rows = [&](char * dst, const char * base, int64_t nb1, int row0, int last_row) __attribute__((always_inline)) {
+    auto dma_rows = [&](char * dst, const char * base, int64_t nb1, int row0, int last_row, auto is_v) __attribute__((always_inline)) {
         const bool inside = row0 >= 0 && row0 + 31 <= last_row;      // uniform
         const char * p = base + (int64_t)(inside ? row0 : 0) * nb1;
 #pragma unroll
         for (int j = 0; j < NDM; j++) {
-            const int L = (wave * NDM + j) * 64 + lane, r = L / CH, c = (L % CH) ^ fr_swz<D>(r);
+            const int ins = j * NW + wave;                            // uniform
+            if (TI % NW != 0 && ins >= TI) break;
+            const int L = ins * 64 + lane, r = L / CH;
+            const int c = (L % CH) ^ (decltype(is_v)::value ? fr_swz_v<D>(r) : fr_swz<D>(r));
             const int rr = inside ? r : min(max(row0 + r, 0), last_row);
             __builtin_amdgcn_global_load_lds((glb_vptr)(p + ((uint32_t)rr * (uint32_t)nb1 + (uint32_t)c * 16u)),
-                                             (lds_vptr)(dst + (wave * NDM + j) * 1024), 16, 0, 0);
+                                             (lds_vptr)(dst + ins * 1024), 16, 0, 0);
         }
     };
-    auto dma_k = [&](int t) __attribute__((always_inline)) { dma_rows(kt, kbase, a.nbk1, 32 * t, a.Nkv - 1); };
-    auto slot_of = [&](int beta) { return ring + ((beta + 3) % FR_SLOTS) * 32 * KP; };   // beta >= -3
-    auto dma_r = [&](int beta) __attribute__((always_inline)) { dma_rows(slot_of(beta), rbase, a.nbr1, p_base0 + 32 * beta, NR - 1); };
-    // V: thread -> (row, chunk), one step ahead through registers
-    u32x4 vraw[NLD];
-    auto load_v = [&](int t) __attribute__((always_inline)) {
-        const int  row0   = 32 * t;
-        const bool inside = row0 + 31 <= a.Nkv - 1;
-        const char * p = vbase + (int64_t)(inside ? row0 : 0) * a.nbv1;
-#pragma unroll
-        for (int n = 0; n < NLD; n++) {
-            const int idx = n * 256 + tid, row = idx / CH, c = idx % CH;
-            const int rr  = inside ? row : min(row0 + row, a.Nkv - 1);
-            vraw[n] = *(const u32x4 *)(p + ((uint32_t)rr * (uint32_t)a.nbv1 + (uint32_t)c * 16u));
-        }
-    };
-    auto store_v = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int n = 0; n < NLD; n++) {
-            const int idx = n * 256 + tid, row = idx / CH, c = idx % CH;
-            *(u32x4 *)(vt + row * VP + c * 16) = vraw[n];
-        }
-    };
+    typedef std::integral_constant<bool, false> KLayout;
+    typedef std::integral_constant<bool, true>  VLayout;
+    auto dma_k = [&](int t) __attribute__((always_inline)) { dma_rows(kt, kbase, a.nbk1, 32 * t, a.Nkv - 1, KLayout{}); };
+    auto dma_v = [&](int t) __attribute__((always_inline)) { dma_rows(vt, vbase, a.nbv1, 32 * t, a.Nkv - 1, VLayout{}); };
+    auto slot_of = [&](int beta) { return ring + ((beta + NW - 1) % FR_SLOTS) * 32 * KP; };   // beta >= 1 - NW
+    auto dma_r = [&](int beta) __attribute__((always_inline)) { dma_rows(slot_of(beta), rbase, a.nbr1, p_base0 + 32 * beta, NR - 1, KLayout{}); };
 
-    // ---- prologue: table blocks -3 .. 1, the first K and V tiles, Q_u and Q_v as B operands ------------------------
+    // ---- prologue: table blocks 1 - NW .. 1, the first K and V tiles, Q_u and Q_v as B operands ---------------------
 #pragma unroll 1
-    for (int beta = -3; beta <= 1; beta++) dma_r(beta);
+    for (int beta = 1 - NW; beta <= 1; beta++) dma_r(beta);
     dma_k(0);
-    load_v(0);
+    dma_v(0);
     half8 qu[KS], qv[KS];
     {
         const float * pu = (const float *)(a.qu + (int64_t)iq * a.nbu1 + (int64_t)h * a.nbu2 + (int64_t)b * a.nbu3);
@@ -158,15 +146,24 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
             }
         }
     }
-    store_v();
     __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): this wave's share of the blocks is in LDS
     __syncthreads();
-    if (NT > 1) load_v(1);
 
     // operand reads of a K or table block: lane (il, hh) takes d = 16 ks + 8 hh .. +7 of row il
     uint32_t opaddr[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) opaddr[ks] = (uint32_t)((il * CH + ((ks * 2 + hh) ^ fr_swz<D>(il))) * 16);
+    // transposing reads of the V tile: lane j16 of a group of 16 addresses key 4 hh + j16 / 4 (+ 8, + 16 ks) and four
+    // values of d from 32 db + 16 (group % 2) + 4 (j16 % 4) on; the swizzle depends on key % 8 only
+    uint32_t vaddr[DBO];
+    {
+        const int j16 = lane & 15, G16 = lane >> 4, kr0 = 4 * (G16 >> 1) + (j16 >> 2);
+#pragma unroll
+        for (int db = 0; db < DBO; db++) {
+            const int c = 4 * db + 2 * (G16 & 1) + ((j16 & 3) >> 1);
+            vaddr[db] = (uint32_t)((kr0 * CH + (c ^ fr_swz_v<D>(kr0))) * 16 + 8 * (j16 & 1));
+        }
+    }
 
     auto block_times_q = [&](const char * blk, const half8 (&q)[KS]) __attribute__((always_inline)) {
         float16v acc;
@@ -190,8 +187,10 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
         for (int r = 0; r < 16; r++) oacc[db][r] = 0.0f;
     float m = -INFINITY, l = 0.0f;
 
-    const char * addrow = nullptr;
+    constexpr int AES = ADD_F16 ? 2 : 4;
+    const char * addrow = nullptr;                  // the query's row of the additive mask; addp walks it, 32 keys a step
     if (ADD) addrow = a.add + (int64_t)iq * a.nba1 + (int64_t)(h % a.Ha) * a.nba2 + (int64_t)(b % a.Ba) * a.nba3;
+    const char * addp = addrow + 4 * hh * AES;
 
     // un-skew constants: slot r of a lane sits at row k_r + 4 hh of its block, i.e. at key (x + k_r) mod 32 with
     // x = il + 4 hh + 1, and belongs to the previous block exactly when that sum reaches 32
@@ -209,11 +208,11 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
                 const int key0 = 32 * t + 8 * g + 4 * hh;
                 if (!tail) {
                     if (ADD_F16) {
-                        const half4_a2 x = *(const half4_a2 *)(addrow + (int64_t)key0 * 2);
+                        const half4_a2 x = *(const half4_a2 *)(addp + 8 * g * AES);
 #pragma unroll
                         for (int c = 0; c < 4; c++) av[4 * g + c] = (float)x[c];
                     } else {
-                        const float4_a4 x = *(const float4_a4 *)(addrow + (int64_t)key0 * 4);
+                        const float4_a4 x = *(const float4_a4 *)(addp + 8 * g * AES);
 #pragma unroll
                         for (int c = 0; c < 4; c++) av[4 * g + c] = x[c];
                     }
@@ -226,6 +225,7 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
                 }
             }
         }
+        if (ADD) addp += 32 * AES;
         // ---- the position product against this step's table block; select per slot, un-skew through the square ------
         {
             const float16v bd_new = block_times_q(slot_of(t + 1 - wave), qv);
@@ -239,7 +239,8 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
         }
         // ---- the content product against this step's K tile -------------------------------------------------------------
         const float16v s = block_times_q(kt, qu);
-        __syncthreads();                                  // every wave has read the K tile and its table block
+        __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): this wave's share of the V tile is in LDS
+        __syncthreads();                                  // every wave has read the K tile and its table block; the V tile is complete
         if (t + 1 < NT) {
             dma_k(t + 1);
             dma_r(t + 2);
@@ -263,12 +264,15 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
         __builtin_amdgcn_wave_barrier();
 
         // ---- online softmax ----------------------------------------------------------------------------------------------
+        // The reference m of a row is raised only when the tile's maximum exceeds it by more than FR_SLACK (a factor 256):
+        // probabilities stay below 2^8 in f16, sums and accumulators are f32, and the accumulators are rescaled on a
+        // handful of steps instead of on most.
         float tmax = s2[0];
 #pragma unroll
         for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, s2[r]);
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        if (__builtin_amdgcn_ballot_w64(tmax > m) != 0) {
-            const float mn = fmaxf(m, tmax);
+        if (__builtin_amdgcn_ballot_w64(tmax > m + FR_SLACK) != 0) {
+            const float mn = tmax > m + FR_SLACK ? tmax : m;
             const float f  = mn == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m - mn);     // m = -inf: nothing accumulated yet, f = 0
             l *= f;
 #pragma unroll
@@ -288,23 +292,21 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
 
         // ---- O^T += V^T . P^T -------------------------------------------------------------------------------------------
         {
-            const int j16 = lane & 15, G16 = lane >> 4;
 #pragma unroll
             for (int db = 0; db < DBO; db++) {
 #pragma unroll
                 for (int ks = 0; ks < 2; ks++) {
-                    const char * p0 = vt + (16 * ks + 4 * (G16 >> 1) + (j16 >> 2)) * VP + (32 * db + 16 * (G16 & 1) + 4 * (j16 & 3)) * 2;
+                    const char * p0 = vt + vaddr[db] + 16 * ks * KP;
                     const half4 lo = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p0));
-                    const half4 hi = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(p0 + 8 * VP)));
+                    const half4 hi = __builtin_bit_cast(half4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)(p0 + 8 * KP)));
                     const half8 va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                     oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, p[ks], oacc[db], 0, 0, 0);
                 }
             }
         }
-        __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): the next K tile and table block (and V in registers) have arrived
-        __syncthreads();                                  // every wave has read the V tile (the next one is read behind the next step's first barrier)
-        if (t + 1 < NT) store_v();
-        if (t + 2 < NT) load_v(t + 2);
+        __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): this wave's share of the next K tile and table block is in LDS
+        __syncthreads();                                  // every wave has read the V tile; the next K tile and table block are complete
+        if (t + 1 < NT) dma_v(t + 1);
     }
 
     // ---- normalise and store: lane (il, hh) holds d = 32 db + 8 g + 4 hh + c of its query -------------------------------
@@ -324,22 +326,22 @@ __global__ void __launch_bounds__(FR_WAVES * 64, 2) fattn_relpos_kernel(const Fa
     }
 }
 
-template <int D>
+template <int D, int NW>
 int launch_d(const FattnRelposArgs & a, hipStream_t stream) {
-    const int64_t G = (int64_t)((a.Nq + 127) / 128) * a.H * a.B;
+    const int64_t G = (int64_t)((a.Nq + 32 * NW - 1) / (32 * NW)) * a.H * a.B;
     const int64_t grid = (G + 7) / 8 * 8;
     if (grid > 0x7fffffff) return (int)hipErrorInvalidValue;
-    constexpr int lds = fr_lds_bytes<D>();
+    constexpr int lds = fr_lds_bytes<D, NW>();
 #define FR_LAUNCH(ADD, F16)                                                                                                   \
     do {                                                                                                                      \
         static bool attr_set = false;                                                                                         \
         if (!attr_set && lds > 64 * 1024) {                                                                                   \
-            const hipError_t e = hipFuncSetAttribute((const void *)fattn_relpos_kernel<D, ADD, F16>,                          \
+            const hipError_t e = hipFuncSetAttribute((const void *)fattn_relpos_kernel<D, NW, ADD, F16>,                          \
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, lds);                      \
             if (e != hipSuccess) return (int)e;                                                                               \
             attr_set = true;                                                                                                  \
         }                                                                                                                     \
-        hipLaunchKernelGGL((fattn_relpos_kernel<D, ADD, F16>), dim3((unsigned)grid), dim3(FR_WAVES * 64), lds, stream, a);    \
+        hipLaunchKernelGGL((fattn_relpos_kernel<D, NW, ADD, F16>), dim3((unsigned)grid), dim3(NW * 64), lds, stream, a);    \
     } while (0)
     if (!a.add)          FR_LAUNCH(false, false);
     else if (a.add_f16)  FR_LAUNCH(true, true);
@@ -360,5 +362,16 @@ bool fattn_relpos_supported(const FattnRelposArgs & a) {
 
 int fattn_relpos_launch(const FattnRelposArgs & a, hipStream_t stream) {
     if (!fattn_relpos_supported(a)) return (int)hipErrorInvalidValue;
-    return a.D == 64 ? launch_d<64>(a, stream) : launch_d<128>(a, stream);
+    // Workgroups of 2, 3 or 4 waves (32 queries each).  Every workgroup stages all K, V and table tiles of its head and pays
+    // a step's barriers and waits whatever its width, so the widest one that the queries fill is taken (measured at
+    // 8 heads x 128, T = 750, batch 8: 4 waves, 384 workgroups: 74 us; 3 waves, 512 workgroups: 80 us; 2 waves, 768: 81 us).
+    int best = (a.Nq + 31) / 32;
+    best = best < 2 ? 2 : best > 4 ? 4 : best;
+    static const char * force = getenv("MI355X_RELPOS_WAVES");            // experiments only
+    if (force && atoi(force) >= 2 && atoi(force) <= 4) best = atoi(force);
+    switch (best) {
+        case 2:  return a.D == 64 ? launch_d<64, 2>(a, stream) : launch_d<128, 2>(a, stream);
+        case 3:  return a.D == 64 ? launch_d<64, 3>(a, stream) : launch_d<128, 3>(a, stream);
+        default: return a.D == 64 ? launch_d<64, 4>(a, stream) : launch_d<128, 4>(a, stream);
+    }
 }
