@@ -146,8 +146,69 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
             }
         }
     }
+    constexpr int AES = ADD_F16 ? 2 : 4;
+    const char * addrow = nullptr;                  // the query's row of the additive mask; addp walks it, 32 keys a step
+    if (ADD) addrow = a.add + (int64_t)iq * a.nba1 + (int64_t)(h % a.Ha) * a.nba2 + (int64_t)(b % a.Ba) * a.nba3;
+    const char * addp = addrow + 4 * hh * AES;
+    // Keys beyond the length of a padded sequence carry -inf in the additive mask for every query: tiles that are masked
+    // out entirely at the END of the key range add nothing and are not walked at all.  Each wave looks at its queries'
+    // last tile while the first blocks are on their way (that is all an unpadded sequence costs) and, if that one is
+    // masked, scans backwards four tiles per round trip; the workgroup takes the largest count.
+    int NTL = NT;
+    if (ADD) {
+        auto tile_max = [&](int tt) __attribute__((always_inline)) {
+            float v = -INFINITY;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int key0 = 32 * tt + 8 * g + 4 * hh;
+                if (32 * tt + 32 <= a.Nkv) {
+                    if (ADD_F16) {
+                        const half4_a2 x = *(const half4_a2 *)(addrow + (int64_t)key0 * 2);
+                        v = fmaxf(fmaxf(v, fmaxf((float)x[0], (float)x[1])), fmaxf((float)x[2], (float)x[3]));
+                    } else {
+                        const float4_a4 x = *(const float4_a4 *)(addrow + (int64_t)key0 * 4);
+                        v = fmaxf(fmaxf(v, fmaxf(x[0], x[1])), fmaxf(x[2], x[3]));
+                    }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        const int key = min(key0 + c, a.Nkv - 1);
+                        v = fmaxf(v, ADD_F16 ? (float)*(const _Float16 *)(addrow + (int64_t)key * 2) : *(const float *)(addrow + (int64_t)key * 4));
+                    }
+                }
+            }
+            return v;
+        };
+        auto any_live = [&](float v) { return __builtin_amdgcn_ballot_w64(v > -INFINITY || v != v) != 0; };
+        int live = NT;
+        if (!any_live(tile_max(NT - 1))) {
+            live = NT - 1;
+            while (live > 0) {
+                const int t0 = max(live - 4, 0);
+                float mx[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) mx[u] = tile_max(min(t0 + u, live - 1));
+                unsigned bits = 0;
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+                    if (any_live(mx[u])) bits |= 1u << u;
+                if (bits) {
+                    live = min(t0 + (32 - __builtin_clz(bits)), live);
+                    break;
+                }
+                live = t0;
+            }
+        }
+        // (the four floats behind each row of a square are padding that nothing else writes)
+        if (lane == 0) ((int *)(ring + FR_SLOTS * 32 * KP))[32 + wave] = live;
+    }
     __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): this wave's share of the blocks is in LDS
     __syncthreads();
+    if (ADD) {
+        NTL = 0;
+#pragma unroll
+        for (int w = 0; w < NW; w++) NTL = max(NTL, ((const int *)(ring + FR_SLOTS * 32 * KP))[32 + w]);
+    }
 
     // operand reads of a K or table block: lane (il, hh) takes d = 16 ks + 8 hh .. +7 of row il
     uint32_t opaddr[KS];
@@ -187,10 +248,6 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
         for (int r = 0; r < 16; r++) oacc[db][r] = 0.0f;
     float m = -INFINITY, l = 0.0f;
 
-    constexpr int AES = ADD_F16 ? 2 : 4;
-    const char * addrow = nullptr;                  // the query's row of the additive mask; addp walks it, 32 keys a step
-    if (ADD) addrow = a.add + (int64_t)iq * a.nba1 + (int64_t)(h % a.Ha) * a.nba2 + (int64_t)(b % a.Ba) * a.nba3;
-    const char * addp = addrow + 4 * hh * AES;
 
     // un-skew constants: slot r of a lane sits at row k_r + 4 hh of its block, i.e. at key (x + k_r) mod 32 with
     // x = il + 4 hh + 1, and belongs to the previous block exactly when that sum reaches 32
@@ -198,7 +255,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
     const int sq_new = il * FR_SQP + x_lane, sq_prev = sq_new - 32;
 
 #pragma unroll 1
-    for (int t = 0; t < NT; t++) {
+    for (int t = 0; t < NTL; t++) {
         const bool tail = 32 * t + 32 > a.Nkv;             // uniform
         // the additive mask of this tile: requested first, used after the products
         float av[16];
@@ -241,7 +298,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
         const float16v s = block_times_q(kt, qu);
         __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): this wave's share of the V tile is in LDS
         __syncthreads();                                  // every wave has read the K tile and its table block; the V tile is complete
-        if (t + 1 < NT) {
+        if (t + 1 < NTL) {
             dma_k(t + 1);
             dma_r(t + 2);
         }
@@ -306,7 +363,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
         }
         __builtin_amdgcn_s_waitcnt(0x0F70);               // vmcnt(0): this wave's share of the next K tile and table block is in LDS
         __syncthreads();                                  // every wave has read the V tile; the next K tile and table block are complete
-        if (t + 1 < NT) dma_v(t + 1);
+        if (t + 1 < NTL) dma_v(t + 1);
     }
 
     // ---- normalise and store: lane (il, hh) holds d = 32 db + 8 g + 4 hh + c of its query -------------------------------

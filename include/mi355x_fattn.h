@@ -237,10 +237,15 @@ int mi355x_relpos_bias(const mi355x_tensor * q_v, const mi355x_tensor * r, const
 
 /*
  * The whole flash branch of that block (fastconformer.h:915-934) in one call:
- *   dst = softmax(scale * (q_u.k^T + BD) + add) . v,   BD[j, i] = <q_v[i], r[Nq-1+j-i]>
- * computed as mi355x_relpos_bias into the workspace (rows padded to whole 128-byte lines) followed by mi355x_flash_attn_ext
- * with that mask: same values as the two calls made separately.  q_u, k, v, dst, params as for
- * mi355x_flash_attn_ext (max_bias and logit_softcap must be 0); Nkv = k->ne[1].
+ *   dst = softmax(scale * q_u.k^T + mask) . v,   mask[j, i] = f16(scale * <q_v[i], r[Nq-1+j-i]> + add[j, i])
+ * q_u, k, v, dst, params as for mi355x_flash_attn_ext (max_bias and logit_softcap must be 0); Nkv = k->ne[1].
+ * With params->kernel = MI355X_FATTN_AUTO and head size 64 or 128 the position term is computed inside the attention
+ * kernel, tile by tile, and never written out: the workspace then holds only f16 copies of K and V (unless they are F16
+ * with 16-byte aligned rows already) and of the table (unless it is read in place); key tiles at the end of the range whose
+ * additive mask is -inf for every query (a padded batch) are not walked.  With a kernel asked for by name - or a shape
+ * the one-kernel form does not cover - the call is mi355x_relpos_bias into the workspace (rows padded to whole 128-byte
+ * lines) followed by mi355x_flash_attn_ext with that mask: the same bits as the two calls made separately.  The two
+ * forms round the same mask values and differ by the summation order of their matrix products only.
  */
 int mi355x_flash_attn_relpos(const mi355x_tensor * q_u, const mi355x_tensor * q_v, const mi355x_tensor * k,
                              const mi355x_tensor * v, const mi355x_tensor * r, const mi355x_tensor * add,

@@ -33,6 +33,10 @@ def make(seed, D, Nq, Nkv, H, B, Br=1, rtype=ora.F32, add=None, layout="cont", a
         a = np.zeros((B, 1, Nq, Nkv), np.float32)
         for b in range(B):
             a[b, :, :, Nkv - 1 - (7 * b + 3) % max(1, Nkv // 2):] = -np.inf
+    elif add == "padlong":                             # whole tiles of keys beyond a sequence's length, one sequence empty
+        a = np.zeros((B, 1, Nq, Nkv), np.float32)
+        for b in range(B):
+            a[b, :, :, [Nkv, max(1, Nkv // 3), 40, 0, Nkv - 33][b % 5]:] = -np.inf
     elif add == "local":                               # window mask with the finite -1e9 (src/core/fastconformer.h:139-163)
         a = np.full((1, 1, Nq, Nkv), -1e9, np.float32)
         for i in range(Nq):
@@ -102,6 +106,8 @@ ATTN = [
     dict(seed=326, D=128, Nq=1, Nkv=1, H=2, B=1, ktype=ora.F16),
     dict(seed=327, D=64, Nq=33, Nkv=31, H=1, B=3, add="pad", ktype=ora.F32),                       # one partial tile
     dict(seed=328, D=128, Nq=300, Nkv=289, H=2, B=1, add="perhead", ktype=ora.F16),                # 9 full tiles + 1 key
+    dict(seed=329, D=128, Nq=200, Nkv=200, H=2, B=5, add="padlong", layout="thd", ktype=ora.F32),  # padded batch: masked tiles are not walked
+    dict(seed=330, D=64, Nq=97, Nkv=300, H=1, B=5, add="padlong", add_type=ora.F16, ktype=ora.F16),
 ]
 
 
@@ -150,6 +156,86 @@ def test_relpos_attention_in_one_kernel_and_as_two_launches_matches_oracle(spec)
     # the two forms round the same mask values (f16 of scale * BD + add): they agree far inside the tolerance
     from cases import errors
     assert errors(got, got2)[0] <= 1e-3
+
+
+def test_relpos_contract_violations_are_reported():
+    c = make(seed=331, D=64, Nq=10, Nkv=10, H=1, B=1)
+    qv, r = upload(c["qv"]), upload(c["r"])
+    short = ggml.Tensor(r.buf, ggml.F32, (64, 18, 1, 1))                               # needs Nq+Nkv-1 = 19 rows
+    with pytest.raises(ggml.InvalidError):
+        ggml.relpos_bias(qv, short, None, 0.125, 10)
+    c80 = dict(qv=ora.from_f32(ora.randn(1, (1, 1, 4, 80))), r=ora.from_f32(ora.randn(2, (1, 1, 7, 80))))
+    with pytest.raises(ggml.UnsupportedError):
+        ggml.relpos_bias(upload(c80["qv"]), upload(c80["r"]), None, 0.1, 4)
+
+
+def _draw(seed: int) -> dict:
+    """a seeded random rel-pos case: sizes off the tile grid, broadcast tables, both table and add types, layouts"""
+    r = lambda i, lo, hi: ora.randint(9000 + seed, i, lo, hi)
+    H = r(0, 1, 4)
+    B = r(1, 1, 3)
+    return dict(seed=400 + seed, D=(64, 128)[r(2, 0, 1)], Nq=r(3, 1, 150), Nkv=r(4, 1, 330), H=H, B=B,
+                Br=(1, B)[r(5, 0, 1)], rtype=(ora.F32, ora.F16)[r(6, 0, 1)],
+                add=(None, "pad", "local", "perhead")[r(7, 0, 3)], layout=("cont", "thd")[r(8, 0, 1)],
+                add_type=(ora.F32, ora.F16)[r(9, 0, 1)])
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("RELPOS_RANDOM_CASES", "24"))))
+def test_relpos_mask_random_shapes(seed):
+    spec = _draw(seed)
+    c = make(**spec)
+    ref = ora.relpos_bias(c["qv"], c["r"], c["add"], c["scale"], c["Nkv"])
+    got = ggml.relpos_bias(upload(c["qv"]), upload(c["r"]), upload(c["add"]) if c["add"] is not None else None,
+                           c["scale"], c["Nkv"])
+    n = c["Nkv"] * c["Nq"] * c["H"] * c["B"]
+    check_mask(got.to_host()[: 2 * n].view(np.uint16), ref.buf.view(np.uint16), str(spec))
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("RELPOS_ATTN_RANDOM_CASES", "20"))))
+def test_relpos_attention_random_shapes(seed):
+    """the one-kernel form on seeded random shapes off the tile grid: broadcast tables, every K/V type, both mask types"""
+    spec = _draw(100 + seed)
+    ktype = (ora.F32, ora.F16, ora.Q8_0, ora.F32)[ora.randint(9100 + seed, 0, 0, 3)]
+    c = make(qgain=0.7, **spec)
+    D, Nq, Nkv, H, B = c["D"], c["Nq"], c["Nkv"], c["H"], c["B"]
+    qu = strided(np.float32(0.7) * ora.randn(spec["seed"] + 10, (B, H, Nq, D)), spec.get("layout", "cont"))
+    k = ora.from_f32(ora.randn(spec["seed"] + 11, (B, H, Nkv, D)), ktype)
+    v = ora.from_f32(ora.randn(spec["seed"] + 12, (B, H, Nkv, D)), ktype)
+    mask = ora.relpos_bias(c["qv"], c["r"], c["add"], c["scale"], Nkv)
+    ref = ora.flash_attn_ext(qu, k, v, mask, c["scale"])
+    print("relpos attention, random shape", spec, ktype, flush=True)
+    got = ggml.flash_attn_relpos(upload(qu), upload(c["qv"]), upload(k), upload(v), upload(c["r"]),
+                                 upload(c["add"]) if c["add"] is not None else None, c["scale"]).numpy_f32()
+    # The mask is an f16 tensor by the reference's own construction, and the device's value may sit one f16 step
+    # (2^-10 .. 2^-8 at magnitudes 1 .. 4) from the oracle's where scale * BD lands next to a rounding boundary
+    # (check_mask above).  Over many keys such steps average out; a row that sees a handful keeps them.
+    few = Nkv <= 32
+    assert_parity(got, ref, str(spec), max_abs_tol=5e-3 if few else 2e-3, rel_l2_tol=2e-3 if few else 1e-3)
+
+
+@pytest.mark.skipif(ora.ref_lib() is None, reason="oracle/_ref not built (needs the reference tree)")
+@pytest.mark.parametrize("T,n_heads,hd", [(150, 2, 128), (97, 3, 64)])
+def test_fused_relpos_attention_matches_the_reference_relpos_attention(T, n_heads, hd):
+    # the device path end to end against compiled reference code: FireRed's conformer attention
+    # (src/firered_asr.cpp:1525-1577 over src/core/cpu_attention.h), score = ((q+bu).k + (q+bv).p[T-1-tq+tk]) / sqrt(hd)
+    d = n_heads * hd
+    q, k, v = (0.7 * ora.randn(9300 + i, (T, d)) for i in range(3))
+    p = 0.7 * ora.randn(9303, (2 * T - 1, d))
+    bu, bv = 0.3 * ora.randn(9304, (n_heads, hd)), 0.3 * ora.randn(9305, (n_heads, hd))
+    want = ora.ref_relpos_mha(q, k, v, p, bu, bv, n_heads)
+
+    def heads(x):          # [rows, d] row-major -> ggml view ne [hd, rows, n_heads, 1] over the same bytes
+        rows = x.shape[0]
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        return upload(ora.Tensor(x.view(np.uint8).reshape(-1).copy(), ora.F32, (hd, rows, n_heads, 1),
+                                 (4, 4 * d, 4 * hd, 4 * d * rows)))
+
+    qu = (q.reshape(T, n_heads, hd) + bu[None]).reshape(T, d)
+    qv = (q.reshape(T, n_heads, hd) + bv[None]).reshape(T, d)
+    print("fused rel-pos attention vs reference helpers", T, n_heads, hd, flush=True)
+    out = ggml.flash_attn_relpos(heads(qu), heads(qv), heads(k), heads(v), heads(p), None, 1.0 / math.sqrt(hd))
+    got = out.numpy_f32()                                  # [1, T, n_heads, hd]
+    assert_parity(got.reshape(T, d), want, "fused rel-pos attention vs reference helpers")
 
 
 def test_relpos_mask_with_a_caller_workspace_for_the_f32_table():
