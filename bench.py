@@ -127,12 +127,18 @@ def bench_encoder(args, ca, ora, torch):
                 traffic = float(ln.split()[1])
     except OSError:
         pass
+    pd = ca.ggml.flash_attn_plan_details(layers[0]["q"], layers[0]["k"], layers[0]["v"], None, scale)
+    kname = (f"fattn_mma_kernel<D={D}, query_blocks={pd['query_blocks']}, key_split={pd['key_split']}, F16, "
+             f"direct={pd['direct']}>" if pd["kernel"] == ca.ggml.KERNEL_MMA else f"kernel {pd['kernel']}")
     res = {
         "value": value, "ms_per_step": ms_per_step,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_F16_TFLOPS, "traffic": traffic,
-                     "kernel": "fattn_mma_kernel<64,2,F16,direct>", "us_per_launch": kernel_ms * 1e3,
-                     "flops_per_launch": flops_layer},
+                     "traffic_source": "profiles/fattn_mma_whisper_large_v3_encoder.txt: rocprofv3 FETCH_SIZE + WRITE_SIZE of this "
+                                       "command in runs of their own, scaled by a plain copy; a constant of that profile, not "
+                                       "measured by this run",
+                     "kernel": kname, "queries_per_workgroup": pd["queries_per_workgroup"], "n_splits": pd["n_splits"],
+                     "us_per_launch": kernel_ms * 1e3, "flops_per_launch": flops_layer},
         "parity": {"max_abs": max_abs, "rel_l2": rel, "ok": bool(parity_ok), "rows_checked": 50,
                    "oracle": "oracle/fattn_oracle.c exact mode"},
     }
@@ -487,8 +493,9 @@ def bench_configs(args, ca, ora, torch):
 def bench_relpos(ca, ora, torch, lengths):
     """The flash branch of a FastConformer block as the reference builds it (src/core/fastconformer.h:876-934) at the
     Parakeet / Canary-CTC shape: Q_u, Q_v, K, V F32 views [128, 750, 8] of [1024, 750] activations, R F32 [128, 1499, 8],
-    F32 pad mask [750, 750] per sequence with -inf beyond its length, batch 8.  Times the mask kernel alone and the
-    fused call (mask kernel + attention).  Content and position terms are drawn with std 0.7 each (unit-variance
+    F32 pad mask [750, 750] per sequence with -inf beyond its length, batch 8.  Times the mask kernel alone, the call in its
+    one-kernel form (the position term computed inside the attention loop) and in its two-launch form (mask written out,
+    then the plain attention call).  Content and position terms are drawn with std 0.7 each (unit-variance
     scores).  Parity: the oracle's node-by-node mask and exact attention, on the first and the last sequence."""
     import numpy as np
     from cases import errors, MAX_ABS_TOL, REL_L2_TOL
@@ -514,7 +521,10 @@ def bench_relpos(ca, ora, torch, lengths):
     mbuf = torch.empty(pitch * T * H * B, dtype=torch.uint8, device="cuda")
     dm_t = ca.Tensor(mbuf, ca.F16, (T, T, H, B), (2, pitch, pitch * T, pitch * T * H))
     us_mask = _time_calls(torch, lambda: ca.ggml.relpos_bias(dqv, dr, da, scale, out=dm_t), 20)
+    us_two = _time_calls(torch, lambda: ca.ggml.flash_attn_relpos(dqu, dqv, dk, dv, dr, da, scale, out=out,
+                                                                   kernel=ca.ggml.KERNEL_MMA), 20)
     us_all = _time_calls(torch, lambda: ca.ggml.flash_attn_relpos(dqu, dqv, dk, dv, dr, da, scale, out=out), 20)
+    ws_one = ca.ggml.flash_attn_relpos_workspace_size(dqu, dqv, dk, dv, dr, da, scale)
     got = out.numpy_f32()
     worst = [0.0, 0.0]
     for b in (0, B - 1):
@@ -526,15 +536,17 @@ def bench_relpos(ca, ora, torch, lengths):
     ok = bool(worst[0] <= MAX_ABS_TOL and worst[1] <= REL_L2_TOL)
     flops = attn_flops(D, T, T, H, B) * 1.5                     # + one 2*D-flop dot per (query, key) for the position term
     nbytes = (4 * T + 2 * T - 1) * dm * 4 + 4 * T * dm * 4 * (B - 1) + T * T * 4 * B + T * dm * 4 * B
-    log(f"[bench] C5_fastconformer_relpos_f32: mask kernel {us_mask:.1f} us, fused call {us_all:.1f} us, "
+    log(f"[bench] C5_fastconformer_relpos_f32: mask kernel {us_mask:.1f} us, two launches {us_two:.1f} us, one kernel {us_all:.1f} us, "
         f"{flops / us_all / 1e6:.1f} TFLOP/s, parity (2 of 8 sequences) max_abs={worst[0]:.2e} rel_l2={worst[1]:.2e} "
         f"{'ok' if ok else 'FAIL: timing withheld'}")
     return {"us_per_call": us_all if ok else None, "us_mask_kernel": us_mask if ok else None,
+            "us_per_call_two_launches": us_two if ok else None,
             "TFLOP/s": flops / us_all / 1e6 if ok else None, "GB/s": nbytes / us_all / 1e3 if ok else None,
-            "flops": flops, "bytes": nbytes, "mask_workspace_bytes": pitch * T * H * B,
+            "flops": flops, "bytes": nbytes, "workspace_bytes": ws_one, "mask_bytes_of_the_two_launch_form": pitch * T * H * B,
             "parity": {"max_abs": worst[0], "rel_l2": worst[1], "ok": ok, "sequences_checked": 2},
             "note": "8 heads x 128, T=750, batch 8: Q_u/Q_v/K/V F32 strided views, R F32 [128,1499,8], F32 pad mask; "
-                    "mask kernel + attention in one call, nothing computed on the host"}
+                    "position term computed inside the attention kernel (K, V and the table rounded to f16 by one launch "
+                    "before it), nothing computed on the host; us_per_call_two_launches = mask written out, then plain attention"}
 
 
 def scale_check(ca, torch, layer):

@@ -313,10 +313,13 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
                 float mk = __fmul_rn(bd[c], a.scale);                                        // as the graph: scale, then add
                 if (ADD) mk = __fadd_rn(mk, av[4 * g + c]);
                 const _Float16 mh = (_Float16)mk;
-                float x = fmaf((float)mh, FR_LOG2E, s[4 * g + c]);
-                if (tail && 32 * t + 8 * g + 4 * hh + c >= a.Nkv) x = -INFINITY;
-                s2[4 * g + c] = x;
+                s2[4 * g + c] = fmaf((float)mh, FR_LOG2E, s[4 * g + c]);
             }
+        }
+        if (tail) {                                        // keys past the end of the last tile
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                if (32 * t + 8 * (r >> 2) + 4 * hh + (r & 3) >= a.Nkv) s2[r] = -INFINITY;
         }
         __builtin_amdgcn_wave_barrier();
 
@@ -338,14 +341,14 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
         }
         const float ms = m == -INFINITY ? 0.0f : m;
         half8 p[2];
-        float lsum = 0.0f;
+        float ls[4] = {0.0f, 0.0f, 0.0f, 0.0f};           // four chains instead of one of sixteen dependent additions
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const float e = __builtin_amdgcn_exp2f(s2[r] - ms);
-            lsum += e;
+            ls[r & 3] += e;
             p[r >> 3][r & 7] = (_Float16)e;
         }
-        l += lsum;
+        l += (ls[0] + ls[1]) + (ls[2] + ls[3]);
 
         // ---- O^T += V^T . P^T -------------------------------------------------------------------------------------------
         {
