@@ -41,6 +41,10 @@ def draw(seed: int) -> dict:
         spec["max_bias"] = 8.0
     if r.random() < 0.1:
         spec["softcap"] = 20.0
+    # (drawn last, so that the cases above are the ones earlier sweeps ran) the narrower cache types, one case in five
+    if r.random() < 0.2:
+        spec["ktype"] = int(r.choice([ora.Q4_0, ora.Q4_1, ora.Q5_0, ora.Q5_1]))
+    spec["variant"] = int(r.choice([ggml.TILE_Q128, ggml.TILE_Q256, ggml.TILE_Q64_KEYSPLIT]))
     return spec
 
 
@@ -50,7 +54,8 @@ N_CASES = int(os.environ.get("FATTN_RANDOM_CASES", "150"))        # more for a l
 @pytest.mark.parametrize("seed", range(N_CASES))
 def test_random_shape_matches_oracle_on_every_kernel(seed):
     spec = draw(seed)
-    print("case", spec, flush=True)
+    variant = spec.pop("variant")
+    print("case", spec, "variant", variant, flush=True)
     case = make_case(**spec)
     ref = run_oracle(case)
     # The tolerance is quoted at unit-variance scores.  The MFMA kernels round q * scale to f16, an error in a score
@@ -69,5 +74,11 @@ def test_random_shape_matches_oracle_on_every_kernel(seed):
         # onto such a call rounds K/V to f16 with nothing to average the rounding over (2.01e-3 at 7 keys, seed 1932)
         few = spec["Nkv"] <= 16 and spec["ktype"] != ora.F16 and kern != ggml.KERNEL_VEC
         assert_parity(got, ref, "kernel %d %s" % (kern, spec), **(dict(max_abs_tol=3e-3) if few else tol))
+        if kern == ggml.KERNEL_MMA:                             # one of the instantiations by name (refused where it does not exist)
+            try:
+                assert_parity(run_gpu(case, kernel=kern, tile_variant=variant), ref, "tile kernel variant %d %s" % (variant, spec),
+                              **(dict(max_abs_tol=3e-3) if few else tol))
+            except (ggml.UnsupportedError, ggml.InvalidError):
+                pass
         if kern == ggml.KERNEL_MMA and spec["Nkv"] > 64:       # key ranges of whole tiles + merge pass
             assert_parity(run_gpu(case, kernel=kern, n_splits=2 + seed % 3), ref, "tile kernel, split keys %s" % spec, **tol)
