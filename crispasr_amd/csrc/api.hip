@@ -913,6 +913,11 @@ static RelposFused relpos_fused_plan(const mi355x_tensor * q_u, const mi355x_ten
     }
     f.table_bytes = relpos_table_bytes(r);
     if (!f.table_bytes && !aligned16_view(r)) return f;
+    // the kernel keeps 32-bit byte offsets inside a (head, batch) plane of K, V and the table
+    const uint64_t lim = (uint64_t)1 << 31;
+    const uint64_t kpitch = f.kv_copy ? (uint64_t)a.D * 2 : (uint64_t)k->nb[1], vpitch = f.kv_copy ? (uint64_t)a.D * 2 : (uint64_t)v->nb[1];
+    const uint64_t rpitch = f.table_bytes ? (uint64_t)a.D * 2 : (uint64_t)r->nb[1];
+    if ((uint64_t)a.Nkv * kpitch >= lim || (uint64_t)a.Nkv * vpitch >= lim || (uint64_t)r->ne[1] * rpitch >= lim) return f;
     f.ok = true;
     return f;
 }

@@ -230,3 +230,19 @@ def test_relpos_workspace_size_is_the_f16_copy_of_the_table():
     assert ggml.relpos_bias_workspace_size(r32) == (D * NR * 8 * 2 + 255) // 256 * 256
     assert ggml.relpos_bias_workspace_size(_t(ca.F16, (D, NR, 8, 1))) == 0
     assert ggml.relpos_bias_workspace_size(_t(ca.F16, (D, NR, 8, 1), (2, 512, 512 * NR, 512 * NR * 8))) > 0     # padded rows
+
+
+def test_public_header_is_plain_c(tmp_path):
+    """the boundary is a C ABI: the header must compile as C99 and as C++11 with nothing but itself"""
+    import shutil
+    import subprocess
+    src = tmp_path / "chk.c"
+    src.write_text('#include "mi355x_fattn.h"\nint main(void) { mi355x_fattn_params p; mi355x_fattn_plan_info i; (void)p; (void)i; '
+                   'return MI355X_FATTN_API_VERSION > 0 ? 0 : 1; }\n')
+    inc = os.path.join(ROOT, "include")
+    for cc, std, extra in (("gcc", "-std=c99", []), ("g++", "-std=c++11", ["-x", "c++"])):
+        if shutil.which(cc) is None:
+            pytest.skip(cc + " not installed")
+        res = subprocess.run([cc, std, "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc, *extra, "-c", str(src), "-o", str(tmp_path / "chk.o")],
+                             capture_output=True, text=True)
+        assert res.returncode == 0, res.stderr
