@@ -237,7 +237,8 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
     Chunk kraw[2][RAW ? 1 : 2][RAW ? 1 : KS];
     Chunk vraw[2][RAW ? 1 : NV];
     typedef typename std::conditional<UNIT == 8, uint2, uint32_t>::type unit_t;
-    unit_t kun[V8 ? 1 : 2][RAW ? NU : 1], vun[2][RAW && !V8 ? NU : 1];
+    // (V8 keeps one register stage: index 0 whatever the step's stage number)
+    unit_t kun[2][RAW ? NU : 1], vun[2][RAW && !V8 ? NU : 1];
     typedef uint32_t u32x2_a2 __attribute__((ext_vector_type(2), aligned(2)));
     u32x2_a2 v8q[1][V8 ? NV8 : 1];
     uint16_t v8d[1][V8 ? NSC : 1];
@@ -254,7 +255,7 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
 #pragma unroll
             for (int i = 0; i < NU; i++) {
                 const uint32_t off = (uint32_t)min(i * 64 + lane, last) * UNIT;
-                kun[s][i] = *(const unit_t *)(kp + off);
+                kun[V8 ? 0 : s][i] = *(const unit_t *)(kp + off);
                 if (!V8) vun[s][i] = *(const unit_t *)(vp + off);
             }
             if (V8) {
@@ -263,13 +264,13 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
                 for (int i = 0; i < NV8; i++) {
                     const int flat = i * 64 + lane;
                     const int row  = min(flat / CH, last_row), c = flat % CH;
-                    v8q[s][i] = *(const u32x2_a2 *)(vp + row * RS + (c >> 2) * FATTN_Q8_0_BYTES + 2 + (c & 3) * 8);
+                    v8q[0][i] = *(const u32x2_a2 *)(vp + row * RS + (c >> 2) * FATTN_Q8_0_BYTES + 2 + (c & 3) * 8);
                 }
 #pragma unroll
                 for (int i = 0; i < NSC; i++) {
                     const int flat = i * 64 + lane;
                     const int row  = min(flat / KS, last_row);
-                    v8d[s][i] = *(const uint16_t *)(vp + row * RS + (flat % KS) * FATTN_Q8_0_BYTES);
+                    v8d[0][i] = *(const uint16_t *)(vp + row * RS + (flat % KS) * FATTN_Q8_0_BYTES);
                 }
             }
             return;
@@ -291,7 +292,6 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
 
     const int n_steps = k_end > k_begin ? (k_end - k_begin + STEP - 1) / STEP : 0;
     typedef std::integral_constant<int, 0> S0;
-    typedef std::integral_constant<int, 1> S1;
 
     // one step of 32 keys out of register stage s; the following step is requested into the other stage
     auto step = [&](const int it, auto stage) __attribute__((always_inline)) {
@@ -304,21 +304,21 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
         if (RAW) {
 #pragma unroll
             for (int i = 0; i < NU; i++) {
-                *(unit_t *)(k_rawst + (i * 64 + lane) * UNIT) = kun[s][i];
+                *(unit_t *)(k_rawst + (i * 64 + lane) * UNIT) = kun[V8 ? 0 : s][i];
                 if (!V8) *(unit_t *)(v_rawst + (i * 64 + lane) * UNIT) = vun[s][i];
             }
             if (V8) {
 #pragma unroll
                 for (int i = 0; i < NV8; i++) {
                     const int flat = i * 64 + lane;
-                    *(uint2 *)(v8_stage + (flat / CH) * VP8 + (flat % CH) * 8) = make_uint2(v8q[s][i][0], v8q[s][i][1]);
+                    *(uint2 *)(v8_stage + (flat / CH) * VP8 + (flat % CH) * 8) = make_uint2(v8q[0][i][0], v8q[0][i][1]);
                 }
                 // rows past k_end repeat the last row's bytes: a zero scale makes exact zeros of them
 #pragma unroll
                 for (int i = 0; i < NSC; i++) {
                     const int flat = i * 64 + lane;
                     const int row  = flat / KS;
-                    *(uint16_t *)(vsc_stage + ((flat % KS) * STEP + row) * 2) = (tail && j0 + row >= k_end) ? (uint16_t)0 : v8d[s][i];
+                    *(uint16_t *)(vsc_stage + ((flat % KS) * STEP + row) * 2) = (tail && j0 + row >= k_end) ? (uint16_t)0 : v8d[0][i];
                 }
             }
             if (V8 && it + DEC_WAVES < n_steps) issue(it + DEC_WAVES, stage);
