@@ -291,8 +291,10 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
         // such calls go to the vector kernel, which works on the exact values - and has nothing to gain from MFMA there.
         const bool few_keys = a.Nkv <= 16 && ktype != MI355X_TYPE_F16;
         if (few_keys)                                                              kernel = MI355X_FATTN_VEC;
-        else if (narrow_quant(ktype))     // no decode kernel for these: rows of queries share one conversion to f16, single rows read the blocks
-            kernel = a.Nq >= 16 && (a.D == 64 || a.D == 128) && a.q_aligned16 ? MI355X_FATTN_MMA : MI355X_FATTN_VEC;
+        else if (narrow_quant(ktype))     // up to 16 rows per KV head read the blocks in the decode kernel; more rows share one conversion to f16
+            kernel = fattn_decode_supported(a, ktype) && a.q_chunks <= 1                  ? MI355X_FATTN_DECODE_MMA
+                     : a.Nq >= 16 && (a.D == 64 || a.D == 128) && a.q_aligned16 ? MI355X_FATTN_MMA
+                                                                                : MI355X_FATTN_VEC;
         else if (fattn_decode_supported(a, ktype) && (a.q_chunks <= 1 || chunked)) kernel = MI355X_FATTN_DECODE_MMA;
         else if (a.Nq >= 16 && fattn_mma_supported(a, ktype)) kernel = MI355X_FATTN_MMA;
         else                                                  kernel = MI355X_FATTN_VEC;

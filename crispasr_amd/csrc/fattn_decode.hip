@@ -122,25 +122,77 @@ struct Chunk {
     uint4 v;         // f16: the 8 halves; q8_0: x,y = quants, z = scale bits
 };
 
+// Q4_0 / Q4_1 / Q5_0 / Q5_1: x, y = the 8 bytes that hold the chunk's nibbles, shifted so that they sit in the low halves;
+// z = d (low) and m (high halfword); w = the chunk's 8 fifth bits.  Blocks are 2-byte aligned: loads at natural alignment.
 template <int TYPE>
 __device__ __forceinline__ Chunk load_chunk(const char * row, int c) {
     Chunk r;
-    if (TYPE == MI355X_TYPE_F16) {
+    if constexpr (TYPE == MI355X_TYPE_F16) {
         r.v = *(const uint4 *)(row + c * 16);
-    } else {
+    } else if constexpr (TYPE == MI355X_TYPE_Q8_0) {
         const uint2 q = q8_load_chunk(row, c >> 2, c & 3);
         r.v.x = q.x;
         r.v.y = q.y;
         r.v.z = *(const uint16_t *)(row + (c >> 2) * FATTN_Q8_0_BYTES);
         r.v.w = 0;
+    } else {
+        typedef BlockFormat<TYPE> F;
+        typedef uint32_t u32_a2 __attribute__((aligned(2)));
+        typedef uint32_t u32x2_a2 __attribute__((ext_vector_type(2), aligned(2)));
+        const char * blk = row + (c >> 2) * F::BYTES;
+        const int    j0  = (c & 3) * 8;                                   // first element of the chunk inside its block
+        const u32x2_a2 q = *(const u32x2_a2 *)(blk + F::QS + (j0 & 8));     // elements j and j + 16 share a byte
+        const int sh = (j0 & 16) ? 4 : 0;
+        r.v.x = (q[0] >> sh) & 0x0F0F0F0Fu;
+        r.v.y = (q[1] >> sh) & 0x0F0F0F0Fu;
+        r.v.z = F::HAS_M ? *(const u32_a2 *)blk : (uint32_t)*(const uint16_t *)blk;
+        r.v.w = F::QH ? (*(const u32_a2 *)(blk + F::QH) >> j0) & 0xFFu : 0u;
     }
     return r;
 }
 
+// 4 unsigned bytes -> 4 exact f16 integers minus `off`: a byte becomes the low mantissa bits of 1024 + b
+__device__ __forceinline__ void u8_widen(uint32_t w, float off, half2v & lo, half2v & hi) {
+    const uint32_t a = __builtin_amdgcn_perm(w, 0x64646464u, 0x00050004u);   // {0x64, b1, 0x64, b0}
+    const uint32_t b = __builtin_amdgcn_perm(w, 0x64646464u, 0x00070006u);   // {0x64, b3, 0x64, b2}
+    const _Float16 o = (_Float16)(1024.0f + off);
+    const half2v   o2 = {o, o};
+    lo = __builtin_bit_cast(half2v, a) - o2;
+    hi = __builtin_bit_cast(half2v, b) - o2;
+}
+
 template <int TYPE>
 __device__ __forceinline__ half8 chunk_to_half8(const Chunk & r) {
-    if (TYPE == MI355X_TYPE_F16) return __builtin_bit_cast(half8, r.v);
-    return q8_dequant(make_uint2(r.v.x, r.v.y), (uint16_t)r.v.z);
+    if constexpr (TYPE == MI355X_TYPE_F16) {
+        return __builtin_bit_cast(half8, r.v);
+    } else if constexpr (TYPE == MI355X_TYPE_Q8_0) {
+        return q8_dequant(make_uint2(r.v.x, r.v.y), (uint16_t)r.v.z);
+    } else {
+        typedef BlockFormat<TYPE> F;
+        uint32_t x = r.v.x, y = r.v.y;
+        if (F::QH) {       // bit i of the byte of fifth bits -> bit 4 of byte i
+            x |= (((r.v.w & 0xFu) * 0x00204081u) & 0x01010101u) << 4;
+            y |= (((r.v.w >> 4) * 0x00204081u) & 0x01010101u) << 4;
+        }
+        half2v h0, h1, h2, h3;
+        const float off = F::HAS_M ? 0.0f : (float)(F::LEVELS / 2);
+        u8_widen(x, off, h0, h1);
+        u8_widen(y, off, h2, h3);
+        const _Float16 d = __builtin_bit_cast(_Float16, (uint16_t)(r.v.z & 0xFFFFu));
+        const half2v   d2 = {d, d};
+        if (F::HAS_M) {    // f16(q * d + m), one rounding
+            const _Float16 m = __builtin_bit_cast(_Float16, (uint16_t)(r.v.z >> 16));
+            const half2v   m2 = {m, m};
+            h0 = __builtin_elementwise_fma(h0, d2, m2); h1 = __builtin_elementwise_fma(h1, d2, m2);
+            h2 = __builtin_elementwise_fma(h2, d2, m2); h3 = __builtin_elementwise_fma(h3, d2, m2);
+        } else {
+            h0 *= d2; h1 *= d2; h2 *= d2; h3 *= d2;
+        }
+        half8 o;
+        o[0] = h0[0]; o[1] = h0[1]; o[2] = h1[0]; o[3] = h1[1];
+        o[4] = h2[0]; o[5] = h2[1]; o[6] = h3[0]; o[7] = h3[1];
+        return o;
+    }
 }
 
 // row pitch in bytes of the int8 V stage: the 16 rows one half of a transpose read touches start 4 banks apart
@@ -558,11 +610,20 @@ bool fattn_decode_supported(const FattnArgs & a, int ktype) {
     if (a.softcap != 0.0f) return false;
     if (ktype == MI355X_TYPE_F16) return a.kv_aligned16 != 0;
     if (ktype == MI355X_TYPE_Q8_0) return a.kv_aligned4 != 0;
+    if (FATTN_IS_BLOCK_TYPE(ktype)) return a.kv_aligned2 != 0;
     return false;
 }
 
 int fattn_decode_launch(const FattnArgs & a, int ktype, hipStream_t stream) {
     if (ktype == MI355X_TYPE_F16) return a.D == 64 ? launch<64, MI355X_TYPE_F16>(a, stream) : launch<128, MI355X_TYPE_F16>(a, stream);
-    if (ktype == MI355X_TYPE_Q8_0) return a.D == 64 ? launch<64, MI355X_TYPE_Q8_0>(a, stream) : launch<128, MI355X_TYPE_Q8_0>(a, stream);
-    return (int)hipErrorInvalidValue;
+    switch (ktype) {
+#define DEC(T) case T: return a.D == 64 ? launch<64, T>(a, stream) : launch<128, T>(a, stream)
+        DEC(MI355X_TYPE_Q8_0);
+        DEC(MI355X_TYPE_Q4_0);
+        DEC(MI355X_TYPE_Q4_1);
+        DEC(MI355X_TYPE_Q5_0);
+        DEC(MI355X_TYPE_Q5_1);
+#undef DEC
+        default: return (int)hipErrorInvalidValue;
+    }
 }

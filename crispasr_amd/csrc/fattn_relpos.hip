@@ -55,7 +55,6 @@ template <int D, int NW> constexpr int fr_lds_bytes() { return (2 + NW + 1) * 32
 
 template <int D, int NW, bool ADD, bool ADD_F16>
 __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) fattn_relpos_kernel(const FattnRelposArgs a) {
-    constexpr int FR_WAVES = NW;
     constexpr int FR_SLOTS = NW + 1;
     constexpr int KS  = D / 16;                     // reduction steps of the two Q products
     constexpr int DBO = D / 32;                     // 32-wide blocks of the output's d

@@ -133,8 +133,9 @@ int mi355x_stream_synchronize(void * stream);
  *   q    F32  [D,  Nq,  Hq,  B ]   any strides with nb[0] == 4
  *   k    F16 | F32 | Q8_0 | Q4_0 | Q4_1 | Q5_0 | Q5_1 [D,  Nkv, Hkv, Bk]   rows contiguous (nb[0] == type size)
  *   v    same type as k   [DV, Nkv, Hkv, Bk]   DV == D
- *        (Q4_0 .. Q5_1: read block by block by the vector kernel for a few query rows; 16 query rows or more go through
- *         one conversion of K and V to f16 in the workspace and the tile kernel; the decode kernel does not take them)
+ *        (Q4_0 .. Q5_1: up to 16 query rows per KV head read the blocks in the decode kernel (head sizes 64 and 128, no
+ *         soft cap; other shapes in the vector kernel); more rows go through one conversion of K and V to f16 in the
+ *         workspace and the tile kernel)
  *   mask NULL, or F16 [>=Nkv, >=Nq, Hm, Bm], rows contiguous; head h reads h % Hm,
  *        batch b reads b % Bm; -inf entries exclude the key
  *   Hq % Hkv == 0 (query head h reads KV head h / (Hq/Hkv)), B % Bk == 0.

@@ -129,8 +129,10 @@ def test_reference_kv_quant_roundtrip_with_an_appended_row(dtype):
 
 ATTN = [
     # single-token decode against a strided cache view, GQA 4 (the decoder of src/canary.cpp:953-972 with a narrow cache)
-    (dict(seed=4411, D=128, Nq=1, Nkv=300, Hq=8, Hkv=2, kv_layout="gap"), ggml.KERNEL_VEC),
-    (dict(seed=4412, D=64, Nq=3, Nkv=77, Hq=6, Hkv=3, B=2, mask="random_inf_batched"), ggml.KERNEL_VEC),
+    (dict(seed=4411, D=128, Nq=1, Nkv=300, Hq=8, Hkv=2, kv_layout="gap"), ggml.KERNEL_DECODE_MMA),
+    (dict(seed=4412, D=64, Nq=3, Nkv=77, Hq=6, Hkv=3, B=2, mask="random_inf_batched"), ggml.KERNEL_DECODE_MMA),
+    (dict(seed=4417, D=128, Nq=1, Nkv=2999, Hq=16, Hkv=4), ggml.KERNEL_DECODE_MMA),       # split over key ranges
+    (dict(seed=4418, D=64, Nq=2, Nkv=1111, Hq=8, Hkv=1, B=3, mask="causal"), ggml.KERNEL_DECODE_MMA),
     (dict(seed=4413, D=96, Nq=5, Nkv=130, Hq=4, softcap=30.0), ggml.KERNEL_VEC),
     # prefill: one conversion to f16, then the tile kernel
     (dict(seed=4414, D=128, Nq=160, Nkv=200, Hq=8, Hkv=2, mask="causal", q_layout="thd"), ggml.KERNEL_MMA),
@@ -159,9 +161,16 @@ def test_attention_over_a_narrow_cache_matches_the_exact_oracle(spec, want_kerne
         ws = torch.empty(need, dtype=torch.uint8, device="cuda")
         again = ggml.flash_attn_ext(q, k, v, m, case["scale"], workspace=ws, **kw).numpy_f32()
         assert np.array_equal(again, got)
-    # the decode kernel does not read these types: asked for by name, the call is refused, nothing is launched
-    with pytest.raises(ggml.Mi355xError):
-        ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA, **kw)
+    # the decode kernel by name: it dequantises the blocks itself, whatever the number of query rows; shapes it does not
+    # cover (other head sizes, a soft cap) are refused and nothing is launched
+    if spec["D"] in (64, 128) and not case["softcap"] and spec["Nkv"] > 16:     # (f16 rounding of K/V shows over a handful of keys)
+        forced = ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA, **kw).numpy_f32()
+        assert_parity(forced, ref, f"decode kernel {NAMES[ktype]} {spec}")
+        if want_kernel == ggml.KERNEL_DECODE_MMA:
+            assert np.array_equal(forced, got)
+    elif spec["Nkv"] > 16:
+        with pytest.raises(ggml.Mi355xError):
+            ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA, **kw)
 
 
 def test_mixed_cache_types_are_left_to_the_cpu_backend():
