@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 
 #include "../../include/mi355x_fattn.h"
 
@@ -50,6 +51,21 @@ struct FattnArgs {
     float * part_acc;    // [rows, n_splits, D]  unnormalised accumulators
     float * part_ml;     // [rows, n_splits, 2]  running max, running sum
 };
+
+// Workgroups that use more than 64 KiB of dynamic LDS need hipFuncAttributeMaxDynamicSharedMemorySize raised, and that
+// attribute belongs to the (kernel, device) pair: `done` is the launcher's own record per kernel instantiation, one bit
+// per device.  Racing callers at worst set the attribute twice.
+static inline hipError_t fattn_allow_lds(const void * kernel, int lds_bytes, std::atomic<uint64_t> & done) {
+    if (lds_bytes <= 64 * 1024) return hipSuccess;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = dev >= 0 && dev < 64 ? (uint64_t)1 << dev : 0;      // devices past 63: set on every launch
+    if (bit && (done.load(std::memory_order_relaxed) & bit)) return hipSuccess;
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e == hipSuccess && bit) done.fetch_or(bit, std::memory_order_relaxed);
+    return e;
+}
 
 static __device__ __forceinline__ float fattn_slope(const FattnArgs & a, int h) {
     if (a.max_bias <= 0.0f) return 1.0f;

@@ -571,13 +571,9 @@ int launch_one(const FattnArgs & a, hipStream_t stream) {
     if (wgs > 0x7fffffff || a.q_chunks != (a.Nq * a.gqa + 15) / 16) return (int)hipErrorInvalidValue;
     const dim3 grid((unsigned)wgs);
     constexpr int lds = decode_lds_bytes<D, RAW, V8>();
-    static bool attr_set = false;
-    if (!attr_set && lds > 64 * 1024) {
-        const hipError_t e = hipFuncSetAttribute((const void *)fattn_decode_kernel<D, TYPE, MASK, RAW, V8>,
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    const hipError_t e = fattn_allow_lds((const void *)fattn_decode_kernel<D, TYPE, MASK, RAW, V8>, lds, lds_allowed);
+    if (e != hipSuccess) return (int)e;
     hipLaunchKernelGGL((fattn_decode_kernel<D, TYPE, MASK, RAW, V8>), grid, dim3(DEC_THREADS), lds, stream, a);
     return (int)hipGetLastError();
 }

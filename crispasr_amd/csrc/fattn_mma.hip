@@ -782,13 +782,9 @@ int launch(const FattnArgs & a, hipStream_t stream) {
     const dim3 grid((unsigned)((int64_t)n_qtiles * a.Hq * a.B * a.n_splits));
     const size_t lds = DIRECT ? (size_t)4 * BC * D * sizeof(_Float16) + (MDMA ? (size_t)MMA_WAVES * NQB * 4096 : 0)
                               : (size_t)2 * BC * (Pitch<D>::K + Pitch<D>::V) * sizeof(_Float16);
-    static bool attr_set = false;     // per instantiation; the attribute only matters above 64 KiB
-    if (!attr_set && lds > 64 * 1024) {
-        const hipError_t e = hipFuncSetAttribute((const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA>,
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};     // per instantiation
+    const hipError_t ea = fattn_allow_lds((const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA>, (int)lds, lds_allowed);
+    if (ea != hipSuccess) return (int)ea;
     static const bool debug = getenv("MI355X_FATTN_DEBUG") != nullptr;
     if (debug) {
         int nb = -1;

@@ -393,13 +393,9 @@ int launch_d(const FattnRelposArgs & a, hipStream_t stream) {
     constexpr int lds = fr_lds_bytes<D, NW>();
 #define FR_LAUNCH(ADD, F16)                                                                                                   \
     do {                                                                                                                      \
-        static bool attr_set = false;                                                                                         \
-        if (!attr_set && lds > 64 * 1024) {                                                                                   \
-            const hipError_t e = hipFuncSetAttribute((const void *)fattn_relpos_kernel<D, NW, ADD, F16>,                          \
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, lds);                      \
-            if (e != hipSuccess) return (int)e;                                                                               \
-            attr_set = true;                                                                                                  \
-        }                                                                                                                     \
+        static std::atomic<uint64_t> lds_allowed{0};                                                                          \
+        const hipError_t e = fattn_allow_lds((const void *)fattn_relpos_kernel<D, NW, ADD, F16>, lds, lds_allowed);           \
+        if (e != hipSuccess) return (int)e;                                                                                   \
         hipLaunchKernelGGL((fattn_relpos_kernel<D, NW, ADD, F16>), dim3((unsigned)grid), dim3(NW * 64), lds, stream, a);    \
     } while (0)
     if (!a.add)          FR_LAUNCH(false, false);

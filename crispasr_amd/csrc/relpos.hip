@@ -324,13 +324,9 @@ __global__ void __launch_bounds__(RP_WAVES * 64, 2) relpos_bias_kernel(const Rel
 template <int D, int RTYPE>
 int launch_dt(const RelposArgs & a, hipStream_t stream) {
     constexpr int LDS = RP_SLOTS * (D / 64) * RP_SLAB_BYTES + RP_WAVES * 2 * RP_TILE_BYTES;
-    static bool attr_set = false;     // per instantiation; the attribute only matters above 64 KiB
-    if (!attr_set && LDS > 64 * 1024) {
-        const hipError_t e = hipFuncSetAttribute((const void *)relpos_bias_kernel<D, RTYPE>,
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};     // per instantiation
+    const hipError_t ea = fattn_allow_lds((const void *)relpos_bias_kernel<D, RTYPE>, LDS, lds_allowed);
+    if (ea != hipSuccess) return (int)ea;
     const int64_t groups = (int64_t)((a.n_qblocks + RP_WAVES - 1) / RP_WAVES) * a.B;
     const dim3 grid((unsigned)((groups + 7) / 8 * 8 * a.n_chunks * a.H));
     hipLaunchKernelGGL((relpos_bias_kernel<D, RTYPE>), grid, dim3(RP_WAVES * 64), LDS, stream, a);
