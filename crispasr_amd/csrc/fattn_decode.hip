@@ -123,7 +123,44 @@ struct Chunk {
 };
 
 // Q4_0 / Q4_1 / Q5_0 / Q5_1: x, y = the 8 bytes that hold the chunk's nibbles, shifted so that they sit in the low halves;
-// z = d (low) and m (high halfword); w = the chunk's 8 fifth bits.  Blocks are 2-byte aligned: loads at natural alignment.
+// z = d (low) and m (high halfword); w = the chunk's 8 fifth bits.  q0, q1: the 8 bytes at QS + 8 (c % 2) of the block,
+// h0, h1: the block's first 8 bytes, c: which 8 of the block's 32 elements.
+template <int TYPE>
+__device__ __forceinline__ Chunk narrow_chunk(uint32_t q0, uint32_t q1, uint32_t h0, uint32_t h1, int c) {
+    typedef BlockFormat<TYPE> F;
+    Chunk r;
+    const int sh = (c & 2) ? 4 : 0;
+    r.v.x = (q0 >> sh) & 0x0F0F0F0Fu;
+    r.v.y = (q1 >> sh) & 0x0F0F0F0Fu;
+    r.v.z = F::HAS_M ? h0 : h0 & 0xFFFFu;
+    const uint32_t qh = !F::QH ? 0u : F::QH == 4 ? h1 : __builtin_amdgcn_alignbyte(h1, h0, 2);
+    r.v.w = (qh >> (c * 8)) & 0xFFu;
+    return r;
+}
+
+// the same chunk cut out of a raw copy of the rows in LDS (row_off: byte offset of the row inside the stage, a multiple
+// of 4; blocks and their quants start on even bytes): aligned dword reads, shifted by two bytes where needed.  The
+// stage is padded, so the third dword of a pair is always inside it.
+template <int TYPE>
+__device__ __forceinline__ Chunk narrow_lds_chunk(const char * stage, int row_off, int blk, int c) {
+    typedef BlockFormat<TYPE> F;
+    const int oh = row_off + blk * F::BYTES;
+    const int oq = oh + F::QS + (c & 1) * 8;
+    const uint32_t * ph = (const uint32_t *)(stage + (oh & ~3));
+    const uint32_t * pq = (const uint32_t *)(stage + (oq & ~3));
+    const uint32_t a0 = ph[0], a1 = ph[1], a2 = ph[2];
+    const uint32_t b0 = pq[0], b1 = pq[1], b2 = pq[2];
+    const uint32_t sa = oh & 2, sb = oq & 2;
+    return narrow_chunk<TYPE>(__builtin_amdgcn_alignbyte(b1, b0, sb), __builtin_amdgcn_alignbyte(b2, b1, sb),
+                              __builtin_amdgcn_alignbyte(a1, a0, sa), __builtin_amdgcn_alignbyte(a2, a1, sa), c);
+}
+
+// bytes per block of the types the raw stream carries (Q8_0 for the others: they never instantiate it)
+template <int TYPE> constexpr int raw_block_bytes() {
+    if constexpr (FATTN_IS_BLOCK_TYPE(TYPE)) return BlockFormat<TYPE>::BYTES;
+    else return FATTN_Q8_0_BYTES;
+}
+
 template <int TYPE>
 __device__ __forceinline__ Chunk load_chunk(const char * row, int c) {
     Chunk r;
@@ -137,16 +174,12 @@ __device__ __forceinline__ Chunk load_chunk(const char * row, int c) {
         r.v.w = 0;
     } else {
         typedef BlockFormat<TYPE> F;
-        typedef uint32_t u32_a2 __attribute__((aligned(2)));
         typedef uint32_t u32x2_a2 __attribute__((ext_vector_type(2), aligned(2)));
         const char * blk = row + (c >> 2) * F::BYTES;
         const int    j0  = (c & 3) * 8;                                   // first element of the chunk inside its block
         const u32x2_a2 q = *(const u32x2_a2 *)(blk + F::QS + (j0 & 8));     // elements j and j + 16 share a byte
-        const int sh = (j0 & 16) ? 4 : 0;
-        r.v.x = (q[0] >> sh) & 0x0F0F0F0Fu;
-        r.v.y = (q[1] >> sh) & 0x0F0F0F0Fu;
-        r.v.z = F::HAS_M ? *(const u32_a2 *)blk : (uint32_t)*(const uint16_t *)blk;
-        r.v.w = F::QH ? (*(const u32_a2 *)(blk + F::QH) >> j0) & 0xFFu : 0u;
+        const u32x2_a2 h = *(const u32x2_a2 *)blk;                          // the block's first 8 bytes: d [, m] [, fifth bits]
+        r = narrow_chunk<TYPE>(q[0], q[1], h[0], h[1], c & 3);
     }
     return r;
 }
@@ -200,9 +233,9 @@ template <int D> constexpr int v8_pitch() { return D == 128 ? 136 : 80; }
 
 // LDS bytes per workgroup: the per-wave f16 V stages, plus per-wave raw K and V stages when RAW; with V8 the V side is
 // one int8 stage and the scales of its 32 x D/32 blocks instead
-template <int D, bool RAW, bool V8>
+template <int D, int TYPE, bool RAW, bool V8>
 constexpr int decode_lds_bytes() {
-    constexpr int RS     = D / 32 * FATTN_Q8_0_BYTES;
+    constexpr int RS     = D / 32 * raw_block_bytes<TYPE>();
     constexpr int RAWSZ  = (STEP * RS + 511) / 512 * 512 + 64;                      // 9 x 64 units, padded
     constexpr int wave   = V8 ? RAWSZ + STEP * v8_pitch<D>() + D / 32 * STEP * 2
                               : STEP * (D + 32) * 2 + (RAW ? 2 * RAWSZ : 0);
@@ -223,13 +256,15 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
     constexpr int CH  = D / 8;                     // chunks per row
     constexpr int NV  = STEP * CH / 64;            // V chunks per lane and step
     constexpr int PV  = D + 32;                    // LDS pitch in halves: 64 mod 128 bytes
-    // raw streaming of contiguous Q8_0 rows: UNIT-byte loads, NU per lane and tensor and step
-    constexpr int RS    = D / 32 * FATTN_Q8_0_BYTES;
+    // raw streaming of contiguous rows of blocks: UNIT-byte loads, NU per lane and tensor and step
+    constexpr int BB    = raw_block_bytes<TYPE>();
+    constexpr int RS    = D / 32 * BB;
     constexpr int UNIT  = RS % 8 == 0 ? 8 : 4;
     constexpr int UPS   = STEP * RS / UNIT;        // units per full step
     constexpr int NU    = (UPS + 63) / 64;
     constexpr int RAWSZ = (STEP * RS + 511) / 512 * 512 + 64;
-    static_assert(!RAW || TYPE == MI355X_TYPE_Q8_0, "raw streaming is the Q8_0 path");
+    static_assert(!RAW || FATTN_IS_BLOCK_TYPE(TYPE), "raw streaming is for rows of blocks");
+    static_assert(!V8 || TYPE == MI355X_TYPE_Q8_0, "the int8 V stage holds Q8_0 quants");
     static_assert(NU * 64 * UNIT <= RAWSZ, "raw stage too small");
 
     // the per-wave stages; after the key loop the same memory carries the cross-wave reduction
@@ -379,7 +414,10 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
 #pragma unroll
                 for (int t = 0; t < STEP * KS / 64; t++) {
                     const int idx = t * 64 + lane;
-                    if (j0 + idx / KS >= k_end) *(uint16_t *)(v_rawst + (idx / KS) * RS + (idx % KS) * FATTN_Q8_0_BYTES) = 0;
+                    if (j0 + idx / KS >= k_end) {
+                        *(uint16_t *)(v_rawst + (idx / KS) * RS + (idx % KS) * BB) = 0;
+                        if (TYPE == MI355X_TYPE_Q4_1 || TYPE == MI355X_TYPE_Q5_1) *(uint16_t *)(v_rawst + (idx / KS) * RS + (idx % KS) * BB + 2) = 0;
+                    }
                 }
             }
             __builtin_amdgcn_wave_barrier();
@@ -394,7 +432,8 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
                 Chunk c;
                 // (V8: row i of tile kb is key (i / 4) * 8 + kb * 4 + i % 4, so that a lane's eight scores are eight
                 //  consecutive keys, the order in which the transposing read hands out V)
-                if (RAW) c.v = q8_lds_chunk<true>(k_rawst, (V8 ? (j >> 2) * 8 + kb * 4 + (j & 3) : kb * 16 + j) * RS, ks, g4);
+                if (RAW && TYPE == MI355X_TYPE_Q8_0) c.v = q8_lds_chunk<true>(k_rawst, (V8 ? (j >> 2) * 8 + kb * 4 + (j & 3) : kb * 16 + j) * RS, ks, g4);
+                else if (RAW) c = narrow_lds_chunk<RAW ? TYPE : MI355X_TYPE_Q4_0>(k_rawst, (kb * 16 + j) * RS, ks, g4);
                 else     c = kraw[s][kb][ks];
                 sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_to_half8<TYPE>(c), qreg[ks], sc[kb], 0, 0, 0);
             }
@@ -405,7 +444,8 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
             const int flat = i * 64 + lane;
             Chunk c;
             if (RAW) {
-                c.v = q8_lds_chunk<false>(v_rawst, (flat / CH) * RS, (flat % CH) >> 2, (flat % CH) & 3);
+                if (TYPE == MI355X_TYPE_Q8_0) c.v = q8_lds_chunk<false>(v_rawst, (flat / CH) * RS, (flat % CH) >> 2, (flat % CH) & 3);
+                else c = narrow_lds_chunk<RAW ? TYPE : MI355X_TYPE_Q4_0>(v_rawst, (flat / CH) * RS, (flat % CH) >> 2, (flat % CH) & 3);
             } else {
                 c = vraw[s][i];
             }
@@ -570,7 +610,7 @@ int launch_one(const FattnArgs & a, hipStream_t stream) {
     const int64_t wgs = (int64_t)a.n_splits * a.q_chunks * a.Hkv * a.B;
     if (wgs > 0x7fffffff || a.q_chunks != (a.Nq * a.gqa + 15) / 16) return (int)hipErrorInvalidValue;
     const dim3 grid((unsigned)wgs);
-    constexpr int lds = decode_lds_bytes<D, RAW, V8>();
+    constexpr int lds = decode_lds_bytes<D, TYPE, RAW, V8>();
     static std::atomic<uint64_t> lds_allowed{0};
     const hipError_t e = fattn_allow_lds((const void *)fattn_decode_kernel<D, TYPE, MASK, RAW, V8>, lds, lds_allowed);
     if (e != hipSuccess) return (int)e;
@@ -580,18 +620,20 @@ int launch_one(const FattnArgs & a, hipStream_t stream) {
 
 template <int D, int TYPE>
 int launch(const FattnArgs & a, hipStream_t stream) {
-    if (TYPE == MI355X_TYPE_Q8_0) {
+    if constexpr (FATTN_IS_BLOCK_TYPE(TYPE)) {
         // contiguous rows, and every step of every (head, batch, split) starts on a unit boundary
-        constexpr int RS   = D / 32 * FATTN_Q8_0_BYTES;
+        constexpr int RS   = D / 32 * raw_block_bytes<TYPE>();
         constexpr int UNIT = RS % 8 == 0 ? 8 : 4;
         const bool raw = a.nbk1 == RS && a.nbv1 == RS &&
                          !((uintptr_t)a.k % UNIT) && !((uintptr_t)a.v % UNIT) &&
                          !(a.nbk2 % UNIT) && !(a.nbk3 % UNIT) && !(a.nbv2 % UNIT) && !(a.nbv3 % UNIT);
-        if (raw) {
-            constexpr int T = MI355X_TYPE_Q8_0;     // (TYPE itself, spelled so that the f16 instantiation never names a RAW kernel)
-            static const bool f16_stage = getenv("MI355X_FATTN_DECODE_F16_STAGE") != nullptr;     // the earlier V path, for comparison runs
-            if (f16_stage) return a.mask ? launch_one<D, T, true, true>(a, stream) : launch_one<D, T, false, true>(a, stream);
-            return a.mask ? launch_one<D, T, true, true, true>(a, stream) : launch_one<D, T, false, true, true>(a, stream);
+        static const bool no_raw = getenv("MI355X_FATTN_DECODE_NO_STREAM") != nullptr;      // the per-lane path, for comparison runs
+        if (raw && !no_raw) {
+            if constexpr (TYPE == MI355X_TYPE_Q8_0) {
+                static const bool f16_stage = getenv("MI355X_FATTN_DECODE_F16_STAGE") != nullptr;     // the earlier V path, for comparison runs
+                if (!f16_stage) return a.mask ? launch_one<D, TYPE, true, true, true>(a, stream) : launch_one<D, TYPE, false, true, true>(a, stream);
+            }
+            return a.mask ? launch_one<D, TYPE, true, true>(a, stream) : launch_one<D, TYPE, false, true>(a, stream);
         }
     }
     return a.mask ? launch_one<D, TYPE, true, false>(a, stream) : launch_one<D, TYPE, false, false>(a, stream);
