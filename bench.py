@@ -225,12 +225,13 @@ def bench_decode(args, ca, ora, torch):
     def f16_buf(n):
         return torch.randn(n, device="cuda").half().view(torch.uint8)
 
-    def q8_buf(seed, n):
-        # N(0,1) values quantised by the library's own CPY F32 -> Q8_0 (bit-exact against the oracle in the tests)
+    def q8_buf(seed, n, dtype=None):
+        # N(0,1) values quantised by the library's own CPY F32 -> Q8_0 (or another block type; bit-exact against the
+        # oracle in the tests)
         gen = torch.Generator(device="cuda")
         gen.manual_seed(seed)
         src = ca.Tensor(torch.randn(n, device="cuda", generator=gen).view(torch.uint8), ca.F32, (n,))
-        dst = ca.Tensor.empty(ca.Q8_0, (n,))
+        dst = ca.Tensor.empty(ca.Q8_0 if dtype is None else dtype, (n,))
         ca.cpy(src, dst)
         torch.cuda.synchronize()
         return dst.buf
@@ -336,6 +337,20 @@ def bench_decode(args, ca, ora, torch):
                        "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 128))})
     run("llm_decode_q8_0_gqa4_4096x128seq", layers, 128 ** -0.5, 128 * (2 * Lk * Hkv * rs + 2 * Hq * D * 4), 10,
         "128 sequences x 4096-entry Q8_0 cache per call")
+    del layers
+    # the narrower cache types of src/core/attention.h:79-105 on the same shape (blocks of 18 and 22 bytes)
+    for kt, nm, bb in ((ca.Q4_0, "q4_0", 18), (ca.Q5_0, "q5_0", 22)):
+        rs = 4 * bb
+        nbk = (bb, rs, rs * Lk, rs * Lk * Hkv)
+        layers = []
+        for l in range(2):
+            layers.append({"q": ca.Tensor(torch.randn(64 * Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, 64)),
+                           "k": ca.Tensor(q8_buf(1300 + 2 * l, 64 * Hkv * Lk * D, kt), kt, (D, Lk, Hkv, 64), nbk),
+                           "v": ca.Tensor(q8_buf(1301 + 2 * l, 64 * Hkv * Lk * D, kt), kt, (D, Lk, Hkv, 64), nbk),
+                           "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 64))})
+        run(f"llm_decode_{nm}_gqa4_4096x64seq", layers, 128 ** -0.5, 64 * (2 * Lk * Hkv * rs + 2 * Hq * D * 4), 10,
+            f"64 sequences x 4096-entry {nm.upper()} cache per call (bound by dequantisation, not by bytes)")
+        del layers
     return out
 
 
