@@ -173,6 +173,26 @@ def test_attention_over_a_narrow_cache_matches_the_exact_oracle(spec, want_kerne
             ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA, **kw)
 
 
+@pytest.mark.parametrize("ktype", NARROW + [ora.Q8_0], ids=lambda t: NAMES[t])
+@pytest.mark.parametrize("D,mask", [(128, None), (64, "random_inf")])
+def test_decode_kernel_streamed_and_strided_rows_give_the_same_bits(ktype, D, mask):
+    # contiguous rows are streamed through the raw LDS stage, rows of a larger pitch are fetched chunk by chunk per lane:
+    # both dequantise to the same f16 values and feed the same MFMAs in the same order
+    spec = dict(seed=4430, D=D, Nq=2, Nkv=1237, Hq=8, Hkv=2, B=2, mask=mask)
+    outs = []
+    for layout in ("contig", "gap"):
+        case = make_case(ktype=ktype, kv_layout=layout, **spec)
+        q, k, v = upload(case["q"]), upload(case["k"]), upload(case["v"])
+        m = upload(case["mask"]) if case["mask"] is not None else None
+        print("streamed vs strided", NAMES[ktype], D, mask, layout, plan_details(case), flush=True)
+        outs.append(ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA).numpy_f32())
+        assert_parity(outs[-1], run_oracle(case), f"{NAMES[ktype]} {layout} {spec}")
+    if ktype == ora.Q8_0:       # its streamed path hands V to the MFMA in another key order: same values, another summation order
+        assert np.abs(outs[0] - outs[1]).max() <= 2e-6
+    else:
+        assert np.array_equal(outs[0], outs[1])
+
+
 def test_mixed_cache_types_are_left_to_the_cpu_backend():
     case = make_case(seed=4420, D=64, Nq=2, Nkv=40, Hq=2, ktype=ora.Q4_0, vtype=ora.Q5_1)
     assert ggml.flash_attn_supports(upload(case["q"]), upload(case["k"]), upload(case["v"]), None) == ggml.ERR_UNSUPPORTED
