@@ -82,3 +82,8 @@ def test_random_shape_matches_oracle_on_every_kernel(seed):
                 pass
         if kern == ggml.KERNEL_MMA and spec["Nkv"] > 64:       # key ranges of whole tiles + merge pass
             assert_parity(run_gpu(case, kernel=kern, n_splits=2 + seed % 3), ref, "tile kernel, split keys %s" % spec, **tol)
+            try:                                               # ... and in the instantiation named above
+                assert_parity(run_gpu(case, kernel=kern, n_splits=2 + seed % 3, tile_variant=variant), ref,
+                              "tile kernel variant %d, split keys %s" % (variant, spec), **tol)
+            except (ggml.UnsupportedError, ggml.InvalidError):
+                pass
