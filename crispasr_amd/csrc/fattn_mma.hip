@@ -142,6 +142,11 @@ template <int D> __device__ __forceinline__ int swz_v(int r) { return D == 64 ? 
 
 template <int D> __device__ __forceinline__ int swz_m(int r) { return (r >> 2) & 3; }     // mask half tile: 4 chunks per row
 
+// keys per tile of an instantiation (the launcher sizes the LDS from the same rule)
+template <int D, int KSP, bool MASK, bool DIRECT> struct FATTN_MMA_TILE_KEYS {
+    static constexpr int value = (KSP == 2 && D == 64 && !MASK && DIRECT) ? 2 * BC : BC;
+};
+
 template <int D, int NQB, int KSP, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA>
 __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnArgs a, const int n_qtiles) {
     static_assert(!DIRECT || TYPE == MI355X_TYPE_F16, "only f16 rows can go to LDS unconverted");
@@ -150,7 +155,10 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     constexpr int NMH   = NQB * 2;                 // MDMA: loads per wave and half tile (16 rows x 64 bytes each)
     constexpr int MHALF = NQB * 32 * 64;           //       bytes of a wave's half-tile block; a wave owns 2 of them
     constexpr int ROWB  = D * 2;                   // DIRECT: bytes per (unpadded) row
-    constexpr int TILEB = BC * ROWB;               //         bytes per K or V tile; LDS = K0 K1 V0 V1
+    // keys per tile: the key-split form of 64-wide heads without a mask walks tiles of 128 (each wave two 32-key blocks of its
+    // half): half the barriers per key, and the second block's operands are on their way while the first is in the softmax
+    constexpr int BCT   = FATTN_MMA_TILE_KEYS<D, KSP, MASK, DIRECT>::value;
+    constexpr int TILEB = BCT * ROWB;              //         bytes per K or V tile; LDS = K0 K1 V0 V1
     constexpr int NLD   = TILEB / 1024 / MMA_WAVES;   //      global->LDS loads per wave, tile and tensor
 
     constexpr int KS   = D / 16;                   // reduction steps of Q.K^T
@@ -162,7 +170,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     constexpr int PV   = Pitch<D>::V;
     constexpr int BMW  = 32 * NQB;                 // queries per wave
     constexpr int BMG  = BMW * MMA_WAVES / KSP;    // queries per workgroup
-    constexpr int NKB  = 2 / KSP;                  // 32-key blocks of a tile that one wave walks
+    constexpr int NKB  = BCT / 32 / KSP;           // 32-key blocks of a tile that one wave walks
     // Skipping excluded blocks adds a branch round the block's body.  The instantiations that already fill the register
     // file (two query blocks per wave, 128-wide heads without key split) answer it with spills inside the tile loop, so
     // it is left to the others: the key-split form and one query block of 64-wide heads.
@@ -430,7 +438,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                 for (int kbi = 0; kbi < NKB; kbi++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        const int key = j0 + (KSP == 2 ? khalf : kbi) * 32 + g * 8 + hh * 4;
+                        const int key = j0 + (KSP == 2 ? khalf * NKB + kbi : kbi) * 32 + g * 8 + hh * 4;
                         // Past Nkv the loads are clamped to the row's last valid pair (or element): branch-free and in
                         // bounds; what they return belongs to keys that the tail tile excludes anyway.
                         if (!TAIL) {
@@ -482,12 +490,12 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         // with few reduction steps the next block's K operands are requested a block ahead
         constexpr bool K_AHEAD = KS <= 4 && NKB == 2;
         half8 ka[K_AHEAD ? 2 : 1][KS];
-        load_k(KSP == 2 ? khalf : 0, ka[0]);
+        load_k(KSP == 2 ? khalf * NKB : 0, ka[0]);
 
         // the tile is consumed in blocks of 32 keys to keep the score registers few
 #pragma unroll
         for (int kbi = 0; kbi < NKB; kbi++) {
-            const int kb = KSP == 2 ? khalf : kbi;         // which 32 keys of the tile
+            const int kb = KSP == 2 ? khalf * NKB + kbi : kbi;      // which 32 keys of the tile
             if (MLDS && kbi == 1 && !TAIL) {
                 // the second half was requested when the tile began; the only requests that can be younger than
                 // it are the next tile's first mask half (they follow block 0)
@@ -510,7 +518,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                 excluded = __builtin_amdgcn_ballot_w64(mdiff != 0) == 0;
             }
             if (excluded) {
-                if (NKB == 2 && kbi == 0) load_k(1, ka[K_AHEAD ? 1 : 0]);
+                if (NKB == 2 && kbi == 0) load_k(kb + 1, ka[K_AHEAD ? 1 : 0]);
                 if (MLDS && kbi == 0 && !TAIL && mn) load_mask_half(j0 + BC, 0, mb, __uint_as_float(mdiff));
                 continue;
             }
@@ -533,7 +541,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             // operands needed next are requested now, so their LDS latency hides behind the softmax
             half8 va[2][DB];
             load_v(kb, va);
-            if (NKB == 2 && kbi == 0) load_k(1, ka[K_AHEAD ? 1 : 0]);
+            if (NKB == 2 && kbi == 0) load_k(kb + 1, ka[K_AHEAD ? 1 : 0]);
 
             // ---- soft cap (this path subtracts m explicitly), mask, key tail -----------------------------
             if (SOFTCAP) {
@@ -660,8 +668,8 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         }
     };
 
-    const int n_tiles = (k_end - k_begin + BC - 1) / BC;
-    const int n_full  = (k_end - k_begin) / BC;
+    const int n_tiles = (k_end - k_begin + BCT - 1) / BCT;
+    const int n_full  = (k_end - k_begin) / BCT;
     if (DIRECT) {
         char * const lb = (char *)lds_raw;               // K0 K1 V0 V1 [mask: per wave 2 half-tile blocks]
         char * const mb = lb + 4 * TILEB;
@@ -683,9 +691,9 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                 else                                            __builtin_amdgcn_s_setprio(0);
             }
             const int  cur = (t & 1) * TILEB, nxt = TILEB - cur;
-            const int  jn  = t + 1 < n_tiles ? k_begin + (t + 1) * BC : -1;
+            const int  jn  = t + 1 < n_tiles ? k_begin + (t + 1) * BCT : -1;
             const bool mn  = (MDMA || MPRE) && t + 1 < n_full;     // the next tile's mask is requested during this one
-            tile(k_begin + t * BC, 0, std::false_type{}, lb + cur, lb + 2 * TILEB + cur, lb + nxt, lb + 2 * TILEB + nxt, jn, t + 1 >= n_full, mb, mn);
+            tile(k_begin + t * BCT, 0, std::false_type{}, lb + cur, lb + 2 * TILEB + cur, lb + nxt, lb + 2 * TILEB + nxt, jn, t + 1 >= n_full, mb, mn);
             // everything requested during the tile has had at least half a tile to land
             __builtin_amdgcn_s_waitcnt(0x0F70);
             __syncthreads();
@@ -693,8 +701,8 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         __builtin_amdgcn_s_setprio(0);
         if (n_full < n_tiles) {
             const int cur = (n_full & 1) * TILEB;
-            if (MDMA) stage_mask_tail(k_begin + n_full * BC, mb);
-            tile(k_begin + n_full * BC, 0, std::true_type{}, lb + cur, lb + 2 * TILEB + cur, nullptr, nullptr, -1, false, mb, false);
+            if (MDMA) stage_mask_tail(k_begin + n_full * BCT, mb);
+            tile(k_begin + n_full * BCT, 0, std::true_type{}, lb + cur, lb + 2 * TILEB + cur, nullptr, nullptr, -1, false, mb, false);
         }
     } else {
     load_tile(k_begin);
@@ -831,7 +839,7 @@ int launch(const FattnArgs & a, hipStream_t stream) {
     const int n_qtiles = (a.Nq + bmg - 1) / bmg;
     if ((int64_t)n_qtiles * a.Hq * a.B * a.n_splits > 0x7fffffff) return (int)hipErrorInvalidValue;
     const dim3 grid((unsigned)((int64_t)n_qtiles * a.Hq * a.B * a.n_splits));
-    const size_t lds = DIRECT ? (size_t)4 * BC * D * sizeof(_Float16) + (MDMA ? (size_t)MMA_WAVES * NQB * 4096 : 0)
+    const size_t lds = DIRECT ? (size_t)4 * FATTN_MMA_TILE_KEYS<D, KSP, MASK, DIRECT>::value * D * sizeof(_Float16) + (MDMA ? (size_t)MMA_WAVES * NQB * 4096 : 0)
                               : (size_t)2 * BC * (Pitch<D>::K + Pitch<D>::V) * sizeof(_Float16);
     static std::atomic<uint64_t> lds_allowed{0};     // per instantiation
     const hipError_t ea = fattn_allow_lds((const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA>, (int)lds, lds_allowed);
