@@ -958,22 +958,22 @@ static int relpos_fused_run(const mi355x_tensor * q_u, const mi355x_tensor * q_v
     g.Hr = (int)r->ne[2]; g.Br = (int)r->ne[3];
     if (f.table_bytes) {
         char * r16 = (char *)ws + f.kv_bytes;
-        CpyArgs c;
         if (!table_done) {
-        memset(&c, 0, sizeof(c));
-        c.src = (const char *)r->data;
-        c.dst = r16;
-        int64_t nb = 2;
-        c.n = 1;
-        for (int i = 0; i < 4; i++) {
-            c.sne[i] = c.dne[i] = r->ne[i];
-            c.snb[i] = (int64_t)r->nb[i];
-            c.dnb[i] = nb;
-            nb *= r->ne[i];
-            c.n *= r->ne[i];
-        }
-        const int e = cpy_launch(c, r->type, MI355X_TYPE_F16, st);
-        if (e) return hip_fail((hipError_t)e, "table conversion launch");
+            CpyArgs c;
+            memset(&c, 0, sizeof(c));
+            c.src = (const char *)r->data;
+            c.dst = r16;
+            int64_t nb = 2;
+            c.n = 1;
+            for (int i = 0; i < 4; i++) {
+                c.sne[i] = c.dne[i] = r->ne[i];
+                c.snb[i] = (int64_t)r->nb[i];
+                c.dnb[i] = nb;
+                nb *= r->ne[i];
+                c.n *= r->ne[i];
+            }
+            const int e = cpy_launch(c, r->type, MI355X_TYPE_F16, st);
+            if (e) return hip_fail((hipError_t)e, "table conversion launch");
         }
         g.r = r16;
         g.nbr1 = (int64_t)a.D * 2; g.nbr2 = g.nbr1 * r->ne[1]; g.nbr3 = g.nbr2 * r->ne[2];
