@@ -188,6 +188,26 @@ def test_planning_sees_the_alignment_a_view_will_have():
     assert cpy_supports(ca.Tensor(None, ca.F32, (D, 4, H, 1), offset=2), _t(ca.F16, (D, 4, H, 1))) == ggml.ERR_UNSUPPORTED
 
 
+def test_planning_of_the_narrow_cache_types():
+    """Q4_0 .. Q5_1 K/V: up to 16 query rows per KV head go to the decode kernel (head sizes 64 / 128, no soft cap), more
+    rows to the tile kernel through f16 copies in the workspace, everything else to the vector kernel."""
+    for t, bb in ((ca.Q4_0, 18), (ca.Q4_1, 20), (ca.Q5_0, 22), (ca.Q5_1, 24)):
+        for D in (64, 128):
+            rs = D // 32 * bb
+            k = _t(t, (D, 700, 2, 1), (bb, rs, rs * 700, rs * 1400))
+            one = ggml.flash_attn_plan_details(_t(ca.F32, (D, 1, 8, 1)), k, k, None)              # 4 rows per KV head
+            assert one["kernel"] == ggml.KERNEL_DECODE_MMA and one["kv_to_f16"] == 0, (t, D, one)
+            many = ggml.flash_attn_plan_details(_t(ca.F32, (D, 40, 8, 1)), k, k, None)
+            assert many["kernel"] == ggml.KERNEL_MMA and many["kv_to_f16"] == 1, (t, D, many)
+            assert many["workspace"] >= 2 * D * 700 * 2 * 2
+            capped = ggml.flash_attn_plan_details(_t(ca.F32, (D, 1, 8, 1)), k, k, None, logit_softcap=30.0)
+            assert capped["kernel"] == ggml.KERNEL_VEC, (t, D, capped)
+        k96 = _t(t, (96, 700, 2, 1), (bb, 3 * bb, 3 * bb * 700, 3 * bb * 1400))
+        assert ggml.flash_attn_plan_details(_t(ca.F32, (96, 1, 8, 1)), k96, k96, None)["kernel"] == ggml.KERNEL_VEC
+        few = _t(t, (128, 9, 2, 1), (bb, 4 * bb, 4 * bb * 9, 4 * bb * 18))                        # a handful of keys: exact values
+        assert ggml.flash_attn_plan_details(_t(ca.F32, (128, 1, 8, 1)), few, few, None)["kernel"] == ggml.KERNEL_VEC
+
+
 def test_set_rows_supports_checks_shapes_types_and_alignment():
     D, rows = 128, 64
     dst = _t(ca.Q8_0, (D, rows, 8, 1))
