@@ -142,14 +142,13 @@ template <int D> __device__ __forceinline__ int swz_v(int r) { return D == 64 ? 
 
 template <int D> __device__ __forceinline__ int swz_m(int r) { return (r >> 2) & 3; }     // mask half tile: 4 chunks per row
 
-// keys per tile of an instantiation (the launcher sizes the LDS from the same rule)
-// (two query blocks per wave with such tiles: 240 bytes of scratch per lane in the loop, 110 us instead of 60 on the
+// TK: keys per tile.  64, except in the key-split form of 64-wide heads without a mask - the grids where a wave is alone on
+// its SIMD: tiles of 128 (each wave two 32-key blocks of its half: half the barriers per key, and the second block's
+// operands are on their way while the first is in the softmax), or of 256 when the workgroups number no more than the
+// CUs, since four such tiles are 128 KB of LDS and leave room for one workgroup per CU only.
+// (two query blocks per wave with 128-key tiles: 240 bytes of scratch per lane in the loop, 110 us instead of 60 on the
 //  large-v3 encoder layer)
-template <int D, int NQB, int KSP, bool MASK, bool DIRECT> struct FATTN_MMA_TILE_KEYS {
-    static constexpr int value = (KSP == 2 && D == 64 && !MASK && DIRECT) ? 2 * BC : BC;
-};
-
-template <int D, int NQB, int KSP, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA>
+template <int D, int NQB, int KSP, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA, int TK = BC>
 __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnArgs a, const int n_qtiles) {
     static_assert(!DIRECT || TYPE == MI355X_TYPE_F16, "only f16 rows can go to LDS unconverted");
     static_assert(!MDMA || (DIRECT && MASK), "the mask goes through LDS only beside directly loaded K/V");
@@ -157,9 +156,8 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     constexpr int NMH   = NQB * 2;                 // MDMA: loads per wave and half tile (16 rows x 64 bytes each)
     constexpr int MHALF = NQB * 32 * 64;           //       bytes of a wave's half-tile block; a wave owns 2 of them
     constexpr int ROWB  = D * 2;                   // DIRECT: bytes per (unpadded) row
-    // keys per tile: the key-split form of 64-wide heads without a mask walks tiles of 128 (each wave two 32-key blocks of its
-    // half): half the barriers per key, and the second block's operands are on their way while the first is in the softmax
-    constexpr int BCT   = FATTN_MMA_TILE_KEYS<D, NQB, KSP, MASK, DIRECT>::value;
+    constexpr int BCT   = TK;                      // keys per tile
+    static_assert(TK == BC || (KSP == 2 && D == 64 && !MASK && DIRECT), "larger tiles exist for the unmasked key-split form of 64-wide heads");
     constexpr int TILEB = BCT * ROWB;              //         bytes per K or V tile; LDS = K0 K1 V0 V1
     constexpr int NLD   = TILEB / 1024 / MMA_WAVES;   //      global->LDS loads per wave, tile and tensor
 
@@ -835,25 +833,25 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     }
 }
 
-template <int D, int NQB, int KSP, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA>
+template <int D, int NQB, int KSP, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA, int TK = BC>
 int launch(const FattnArgs & a, hipStream_t stream) {
     const int bmg = 32 * NQB * MMA_WAVES / KSP;
     const int n_qtiles = (a.Nq + bmg - 1) / bmg;
     if ((int64_t)n_qtiles * a.Hq * a.B * a.n_splits > 0x7fffffff) return (int)hipErrorInvalidValue;
     const dim3 grid((unsigned)((int64_t)n_qtiles * a.Hq * a.B * a.n_splits));
-    const size_t lds = DIRECT ? (size_t)4 * FATTN_MMA_TILE_KEYS<D, NQB, KSP, MASK, DIRECT>::value * D * sizeof(_Float16) + (MDMA ? (size_t)MMA_WAVES * NQB * 4096 : 0)
+    const size_t lds = DIRECT ? (size_t)4 * TK * D * sizeof(_Float16) + (MDMA ? (size_t)MMA_WAVES * NQB * 4096 : 0)
                               : (size_t)2 * BC * (Pitch<D>::K + Pitch<D>::V) * sizeof(_Float16);
     static std::atomic<uint64_t> lds_allowed{0};     // per instantiation
-    const hipError_t ea = fattn_allow_lds((const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA>, (int)lds, lds_allowed);
+    const hipError_t ea = fattn_allow_lds((const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA, TK>, (int)lds, lds_allowed);
     if (ea != hipSuccess) return (int)ea;
     static const bool debug = getenv("MI355X_FATTN_DEBUG") != nullptr;
     if (debug) {
         int nb = -1;
-        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA>, MMA_THREADS, lds);
+        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA, TK>, MMA_THREADS, lds);
         fprintf(stderr, "[mi355x] fattn_mma<%d,%d,%d,%d,%d,%d,%d,%d> grid %u lds %zu B, resident workgroups per CU: %d\n",
                 D, NQB, KSP, TYPE, (int)MASK, (int)SOFTCAP, (int)DIRECT, (int)MDMA, grid.x, lds, nb);
     }
-    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
+    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA, TK>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
     return (int)hipGetLastError();
 }
 
@@ -862,7 +860,15 @@ int launch_mask(const FattnArgs & a, const FattnMmaVariant & v, hipStream_t stre
     const bool mask = a.mask != nullptr;
     if (KSP == 1 && a.softcap != 0.0f)
         return mask ? launch<D, NQB, 1, TYPE, true, true, DIRECT, false>(a, stream) : launch<D, NQB, 1, TYPE, false, true, DIRECT, false>(a, stream);
-    if (!mask) return launch<D, NQB, KSP, TYPE, false, false, DIRECT, false>(a, stream);
+    if (!mask) {
+        if constexpr (KSP == 2 && D == 64 && DIRECT) {
+            const int64_t wgs = (int64_t)((a.Nq + 63) / 64) * a.Hq * a.B * a.n_splits;
+            if (a.n_cus > 0 && wgs <= a.n_cus) return launch<D, NQB, KSP, TYPE, false, false, DIRECT, false, 4 * BC>(a, stream);
+            return launch<D, NQB, KSP, TYPE, false, false, DIRECT, false, 2 * BC>(a, stream);
+        } else {
+            return launch<D, NQB, KSP, TYPE, false, false, DIRECT, false>(a, stream);
+        }
+    }
     if (KSP == 1 && DIRECT && v.mask_dma) return launch<D, NQB, 1, TYPE, true, false, DIRECT, DIRECT>(a, stream);
     return launch<D, NQB, KSP, TYPE, true, false, DIRECT, false>(a, stream);
 }
