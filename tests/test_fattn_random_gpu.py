@@ -8,9 +8,9 @@ import numpy as np
 import pytest
 
 import oracle as ora
-from cases import make_case
+from cases import make_case, to_f32
 from crispasr_amd import ggml
-from gpu_util import assert_parity, run_gpu, run_oracle
+from gpu_util import assert_parity, plan_details, run_gpu, run_oracle
 
 pytestmark = pytest.mark.gpu
 
@@ -51,6 +51,30 @@ def draw(seed: int) -> dict:
 N_CASES = int(os.environ.get("FATTN_RANDOM_CASES", "150"))        # more for a longer hunt
 
 
+def rows_seeing_few_keys(case: dict, limit: int = 16) -> np.ndarray:
+    """[B, Nq, Hq] bool: the query rows that the mask (or Nkv itself) leaves at most `limit` keys."""
+    _, Nq, Hq, B = case["q"].ne
+    Nkv = case["k"].ne[1]
+    if case["mask"] is None:
+        return np.full((B, Nq, Hq), Nkv <= limit)
+    vis = (to_f32(case["mask"])[:, :, :Nq, :Nkv] > -np.inf).sum(-1)          # [Bm, Hm, Nq]
+    Bm, Hm = vis.shape[:2]
+    return np.stack([np.stack([vis[b % Bm, h % Hm] for h in range(Hq)], axis=-1) for b in range(B)]) <= limit
+
+
+def assert_parity_by_rows(got, ref, case, what, exact_values, **tol):
+    """The MFMA kernels round F32 and quantised K/V to f16 (2^-11 relative).  Over many keys that averages out; a row that
+    sees a handful of keys keeps it - one key with |v| = 4.1 is already 2e-3 off (seeds 1932 and 12316 of the longer
+    sweeps: 2.01e-3 and 2.02e-3) - so such rows are held to 3e-3 unless the kernel works on the exact values."""
+    if exact_values:
+        return assert_parity(got, ref, what, **tol)
+    few = rows_seeing_few_keys(case)
+    if few.any():
+        assert_parity(got[few], ref[few], what + " (rows that see <= 16 keys)", **{**tol, "max_abs_tol": 3e-3})
+    if not few.all():
+        assert_parity(got[~few], ref[~few], what, **tol)
+
+
 @pytest.mark.parametrize("seed", range(N_CASES))
 def test_random_shape_matches_oracle_on_every_kernel(seed):
     spec = draw(seed)
@@ -64,26 +88,28 @@ def test_random_shape_matches_oracle_on_every_kernel(seed):
     # draws are held to 3e-3.
     hot = spec.get("scale", 0.0) * spec["D"] ** 0.5 > 1.2
     tol = dict(max_abs_tol=3e-3) if hot else {}
-    assert_parity(run_gpu(case), ref, "auto %s" % spec, **tol)
+    f16_kv = spec["ktype"] == ora.F16
+    auto_kernel = plan_details(case)["kernel"]
+    assert_parity_by_rows(run_gpu(case), ref, case, "auto %s" % spec, f16_kv or auto_kernel == ggml.KERNEL_VEC, **tol)
     for kern in (ggml.KERNEL_VEC, ggml.KERNEL_MMA, ggml.KERNEL_DECODE_MMA):
         try:
             got = run_gpu(case, kernel=kern)
         except ggml.UnsupportedError:
             continue
-        # a handful of keys in F32 or Q8_0: the automatic choice is the vector kernel (exact values); an MFMA kernel forced
-        # onto such a call rounds K/V to f16 with nothing to average the rounding over (2.01e-3 at 7 keys, seed 1932)
-        few = spec["Nkv"] <= 16 and spec["ktype"] != ora.F16 and kern != ggml.KERNEL_VEC
-        assert_parity(got, ref, "kernel %d %s" % (kern, spec), **(dict(max_abs_tol=3e-3) if few else tol))
+        # (the vector kernel works on the exact F32 / dequantised values; f16 K/V are exact in every kernel)
+        exact = f16_kv or kern == ggml.KERNEL_VEC
+        assert_parity_by_rows(got, ref, case, "kernel %d %s" % (kern, spec), exact, **tol)
         if kern == ggml.KERNEL_MMA:                             # one of the instantiations by name (refused where it does not exist)
             try:
-                assert_parity(run_gpu(case, kernel=kern, tile_variant=variant), ref, "tile kernel variant %d %s" % (variant, spec),
-                              **(dict(max_abs_tol=3e-3) if few else tol))
+                assert_parity_by_rows(run_gpu(case, kernel=kern, tile_variant=variant), ref, case,
+                                      "tile kernel variant %d %s" % (variant, spec), exact, **tol)
             except (ggml.UnsupportedError, ggml.InvalidError):
                 pass
         if kern == ggml.KERNEL_MMA and spec["Nkv"] > 64:       # key ranges of whole tiles + merge pass
-            assert_parity(run_gpu(case, kernel=kern, n_splits=2 + seed % 3), ref, "tile kernel, split keys %s" % spec, **tol)
+            assert_parity_by_rows(run_gpu(case, kernel=kern, n_splits=2 + seed % 3), ref, case, "tile kernel, split keys %s" % spec,
+                                  exact, **tol)
             try:                                               # ... and in the instantiation named above
-                assert_parity(run_gpu(case, kernel=kern, n_splits=2 + seed % 3, tile_variant=variant), ref,
-                              "tile kernel variant %d, split keys %s" % (variant, spec), **tol)
+                assert_parity_by_rows(run_gpu(case, kernel=kern, n_splits=2 + seed % 3, tile_variant=variant), ref, case,
+                                      "tile kernel variant %d, split keys %s" % (variant, spec), exact, **tol)
             except (ggml.UnsupportedError, ggml.InvalidError):
                 pass
