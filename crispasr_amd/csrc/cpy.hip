@@ -8,6 +8,11 @@
 
 #include <string.h>
 
+// The quantisers must round every product and every sum on its own, as the reference's scalar code does: hipcc's default
+// contraction turns x * id + c into one fused multiply-add (so do __fmul_rn / __fadd_rn, which inline as contractible), and
+// an element whose sum lands within half an ulp of an integer then truncates to the neighbouring level.
+#pragma clang fp contract(off)
+
 namespace {
 
 // byte offset of unit i, where a unit is `unit0` elements along dimension 0 and one step of
@@ -78,13 +83,15 @@ __device__ __forceinline__ void quantize_block_store(float x, char * blk, int e,
         if (!(amax > 0.0f)) ext = 0.0f;
         d = ext / (float)(-(F::LEVELS / 2));
         const float id = d != 0.0f ? 1.0f / d : 0.0f;
-        qi = (int)(int8_t)(int)__fadd_rn(__fmul_rn(x, id), (float)(F::LEVELS / 2) + 0.5f);
+        const float x0 = x * id;
+        qi = (int)(int8_t)(int)(x0 + ((float)(F::LEVELS / 2) + 0.5f));
     } else {
         m = group_min<32>(x);
         const float mx = group_max<32>(x);
-        d = __fsub_rn(mx, m) / (float)(F::LEVELS - 1);
+        d = (mx - m) / (float)(F::LEVELS - 1);
         const float id = d != 0.0f ? 1.0f / d : 0.0f;
-        qi = (int)(uint8_t)(int)__fadd_rn(__fmul_rn(__fsub_rn(x, m), id), 0.5f);
+        const float x0 = (x - m) * id;
+        qi = (int)(uint8_t)(int)(x0 + 0.5f);
     }
     qi = qi < F::LEVELS - 1 ? qi : F::LEVELS - 1;
     const int      hi = __shfl(qi, half + (e & 15) + 16, 64);       // the element that shares this lane's byte

@@ -72,6 +72,15 @@ static __device__ __forceinline__ float fattn_slope(const FattnArgs & a, int h) 
     return h < a.n_head_log2 ? powf(a.m0, (float)(h + 1)) : powf(a.m1, (float)(2 * (h - a.n_head_log2) + 1));
 }
 
+// a * b + c with the product and the sum each rounded to f32, as two graph nodes (or two scalar statements) round them.
+// hipcc contracts a * b + c into one fused multiply-add by default, also when it is spelled __fadd_rn(__fmul_rn(a, b), c):
+// those inline as contractible operations.  Only operations compiled under "contract(off)" stay apart.
+static __device__ __forceinline__ float mul_then_add(float a, float b, float c) {
+#pragma clang fp contract(off)
+    const float p = a * b;
+    return p + c;
+}
+
 static __device__ __forceinline__ float h2f_bits(uint16_t h) {
     return (float)__builtin_bit_cast(_Float16, h);
 }
@@ -163,8 +172,8 @@ static __device__ __forceinline__ void dequant8(const char * blk, int j0, float 
         const int      q0 = (int)(((w >> sh) & 15u) | (((hb >> (2 * i)) & 1u) << 4));
         const int      q1 = (int)(((w >> (8 + sh)) & 15u) | (((hb >> (2 * i + 1)) & 1u) << 4));
         if (F::HAS_M) {
-            out[2 * i]     = __fadd_rn(__fmul_rn((float)q0, d), m);
-            out[2 * i + 1] = __fadd_rn(__fmul_rn((float)q1, d), m);
+            out[2 * i]     = mul_then_add((float)q0, d, m);
+            out[2 * i + 1] = mul_then_add((float)q1, d, m);
         } else {
             out[2 * i]     = (float)(q0 - F::LEVELS / 2) * d;
             out[2 * i + 1] = (float)(q1 - F::LEVELS / 2) * d;

@@ -309,8 +309,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
             const float4v bd = *(const float4v *)&sq[il * FR_SQP + 8 * g + 4 * hh];
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                float mk = __fmul_rn(bd[c], a.scale);                                        // as the graph: scale, then add
-                if (ADD) mk = __fadd_rn(mk, av[4 * g + c]);
+                const float mk = ADD ? mul_then_add(bd[c], a.scale, av[4 * g + c]) : bd[c] * a.scale;   // as the graph: scale, then add
                 const _Float16 mh = (_Float16)mk;
                 s2[4 * g + c] = fmaf((float)mh, FR_LOG2E, s[4 * g + c]);
             }

@@ -253,7 +253,7 @@ __global__ void __launch_bounds__(RP_WAVES * 64, 2) relpos_bias_kernel(const Rel
         }
     };
     // scale, add and the rounding to f16 as the graph's nodes do them: an f32 multiply, an f32 add (not fused), RNE
-    auto finish = [&](float g, float add) { return (_Float16)__fadd_rn(__fmul_rn(g, a.scale), add); };
+    auto finish = [&](float g, float add) { return (_Float16)mul_then_add(g, a.scale, add); };
     auto flush = [&](int t) __attribute__((always_inline)) {         // t even: tiles t and t + 1
         __builtin_amdgcn_wave_barrier();
         const int nk = keys_left(t);

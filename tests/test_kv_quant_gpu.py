@@ -127,6 +127,59 @@ def test_reference_kv_quant_roundtrip_with_an_appended_row(dtype):
     assert np.array_equal(got, to_f32(ora.from_f32(wrote, dtype)))
 
 
+def _blocks_that_a_fused_multiply_add_would_change(dtype, n_blocks=4096):
+    """Blocks of 32 holding an element for which trunc(x * id + c) differs between a separately rounded product and sum
+    (the reference's scalar code) and one fused operation: the sum lies within half an ulp of an integer.  One element in
+    four million does that by chance, so the middle element of each random block is moved to such a value where the
+    129 floats around a level boundary hold one."""
+    f32, f64 = np.float32, np.float64
+    r = np.random.default_rng(4420 + dtype)
+    x = (ora.randn(4420 + dtype, (n_blocks, 32)) * f32(1e-3)).astype(f32)
+    levels = 16 if dtype in (ora.Q4_0, ora.Q4_1) else 32
+    rows = np.arange(n_blocks)
+    if dtype in (ora.Q4_0, ora.Q5_0):
+        first = np.argmax(np.abs(x) == np.abs(x).max(axis=1, keepdims=True), axis=1)
+        d = (x[rows, first] / f32(-(levels // 2))).astype(f32)
+        base, c = np.zeros(n_blocks, f32), f32(levels // 2 + 0.5)
+    else:
+        base = x.min(axis=1)
+        d = ((x.max(axis=1) - base).astype(f32) / f32(levels - 1)).astype(f32)
+        c = f32(0.5)
+    inv = (f32(1.0) / d).astype(f32)
+    # the level boundary to sit on.  With c = 0.5 the sum only rounds a second time where it leaves the product's binade
+    # for a coarser one, and among the boundaries that is the one between levels 0 and 1
+    k = r.integers(2, levels - 2, n_blocks) if c > 1 else np.ones(n_blocks, np.int64)
+    centre = (base.astype(f64) + (k - f64(c)) * d.astype(f64)).astype(f32)
+    cand = (centre.view(np.int32)[:, None] + np.arange(-64, 65, dtype=np.int32)[None, :]).view(f32)
+    xs = (cand - base[:, None]).astype(f32)
+    apart = ((xs * inv[:, None]).astype(f32) + c).astype(f32)
+    fused = (xs.astype(f64) * inv[:, None].astype(f64) + f64(c)).astype(f32)         # the f64 product is exact
+    differ = np.trunc(apart) != np.trunc(fused)
+    found = differ.any(axis=1)
+    middle = np.argsort(x, axis=1)[:, 16]                                 # neither the minimum nor an extreme value
+    x[rows[found], middle[found]] = cand[rows[found], np.argmax(differ[found], axis=1)]
+    return x[found]
+
+
+@pytest.mark.parametrize("dtype", NARROW, ids=lambda t: NAMES[t])
+def test_quantisers_round_the_product_and_the_sum_separately(dtype):
+    # the compiler's default contraction of x * id + c into a fused multiply-add moves such an element to the
+    # neighbouring level; the device code must keep the two roundings of the scalar quantisers
+    x = _blocks_that_a_fused_multiply_add_would_change(dtype)
+    assert len(x) >= 16, "the search found too few blocks to make the point"
+    x = np.concatenate([x, (ora.randn(4430, (256, 32)) * np.float32(1e-3)).astype(np.float32)])
+    n = len(x)
+    want = ora.from_f32(x.reshape(1, 1, n, 32), dtype)
+    print("straddling blocks", NAMES[dtype], n, flush=True)
+    got = ca.cpy(upload(ora.from_f32(x.reshape(1, 1, n, 32), ora.F32)), ca.Tensor.empty(dtype, (32, n, 1, 1)))
+    torch.cuda.synchronize()
+    assert np.array_equal(got.to_host()[: want.buf.size], want.buf)
+    cache = ca.Tensor.empty(dtype, (32, n, 1, 1))
+    ca.set_rows(cache, upload(ora.from_f32(x.reshape(1, 1, n, 32), ora.F32)), torch.arange(n, dtype=torch.int64, device="cuda"))
+    torch.cuda.synchronize()
+    assert np.array_equal(cache.to_host()[: want.buf.size], want.buf)
+
+
 ATTN = [
     # single-token decode against a strided cache view, GQA 4 (the decoder of src/canary.cpp:953-972 with a narrow cache)
     (dict(seed=4411, D=128, Nq=1, Nkv=300, Hq=8, Hkv=2, kv_layout="gap"), ggml.KERNEL_DECODE_MMA),
