@@ -6,6 +6,7 @@ tests upload the same bytes and call the HIP path through the C-ABI.
 from __future__ import annotations
 
 import math
+import os
 from typing import Optional
 
 import numpy as np
@@ -13,6 +14,13 @@ import numpy as np
 import oracle as ora
 
 NEG_INF_H = np.uint16(0xFC00)
+
+
+def sweep_seeds(count_variable: str, default: int) -> range:
+    """Seeds of a randomised test: `default` of them, or as many as the environment variable says (a longer hunt), from
+    RANDOM_FIRST_SEED on (0 by default: the cases every run repeats)."""
+    first = int(os.environ.get("RANDOM_FIRST_SEED", "0"))
+    return range(first, first + int(os.environ.get(count_variable, str(default))))
 
 
 def _store(x_f32: np.ndarray, type_: int, layout: str, pad_rows: int = 0) -> ora.Tensor:

@@ -1,15 +1,13 @@
 """Randomised cache writes: GGML_OP_CPY and SET_ROWS of F32 rows into views of a cache of every type (the writes of
 src/core/attention.h:342-378), over random row lengths, head counts, view offsets and permuted sources, every byte of the
 cache compared with the oracle's - the bytes outside the view included - and read back through the dequantising copy."""
-import os
-
 import numpy as np
 import pytest
 import torch
 
 import crispasr_amd as ca
 import oracle as ora
-from cases import to_f32
+from cases import sweep_seeds, to_f32
 from gpu_util import upload
 
 pytestmark = pytest.mark.gpu
@@ -42,7 +40,7 @@ def source(spec: dict):
     return x, ora.Tensor(xt.view(np.uint8).reshape(-1).copy(), ora.F32, (D, T, H, B), (4, 4 * D * H, 4 * D, 4 * D * H * T))
 
 
-@pytest.mark.parametrize("seed", range(int(os.environ.get("CPY_RANDOM_CASES", "40"))))
+@pytest.mark.parametrize("seed", sweep_seeds("CPY_RANDOM_CASES", 40))
 def test_random_cache_write_is_bit_exact(seed):
     spec = draw(seed)
     print("cpy case", spec, flush=True)

@@ -1,12 +1,10 @@
 """Randomised decode shapes: few query rows per KV head against long caches of every type, so that the decode kernel's
 key ranges, partial last steps, streamed and strided row paths and the merge pass meet in every combination."""
-import os
-
 import numpy as np
 import pytest
 
 import oracle as ora
-from cases import make_case
+from cases import make_case, sweep_seeds
 from crispasr_amd import ggml
 from gpu_util import assert_parity, plan_details, run_gpu, run_oracle
 
@@ -27,7 +25,7 @@ def draw(seed: int) -> dict:
                 kv_layout=str(r.choice(["contig", "contig", "gap", "thd"])))
 
 
-@pytest.mark.parametrize("seed", range(int(os.environ.get("DECODE_RANDOM_CASES", "40"))))
+@pytest.mark.parametrize("seed", sweep_seeds("DECODE_RANDOM_CASES", 40))
 def test_random_decode_shape_matches_oracle(seed):
     spec = draw(seed)
     print("decode case", spec, flush=True)

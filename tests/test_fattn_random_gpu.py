@@ -2,13 +2,11 @@
 accepts the shape.  The draws are made to hit the tile kernel's paths in every combination: K/V moved global->LDS
 directly or through registers, masks with dword-aligned and unaligned rows, even and odd Nkv, full and partial
 last tiles, few and many queries (the F32 -> f16 pre-conversion starts at 128)."""
-import os
-
 import numpy as np
 import pytest
 
 import oracle as ora
-from cases import make_case, to_f32
+from cases import make_case, sweep_seeds, to_f32
 from crispasr_amd import ggml
 from gpu_util import assert_parity, plan_details, run_gpu, run_oracle
 
@@ -48,7 +46,7 @@ def draw(seed: int) -> dict:
     return spec
 
 
-N_CASES = int(os.environ.get("FATTN_RANDOM_CASES", "150"))        # more for a longer hunt
+SEEDS = sweep_seeds("FATTN_RANDOM_CASES", 150)
 
 
 def rows_seeing_few_keys(case: dict, limit: int = 16) -> np.ndarray:
@@ -75,7 +73,7 @@ def assert_parity_by_rows(got, ref, case, what, exact_values, **tol):
         assert_parity(got[~few], ref[~few], what, **tol)
 
 
-@pytest.mark.parametrize("seed", range(N_CASES))
+@pytest.mark.parametrize("seed", SEEDS)
 def test_random_shape_matches_oracle_on_every_kernel(seed):
     spec = draw(seed)
     variant = spec.pop("variant")

@@ -1,12 +1,12 @@
 """GPU parity of FastConformer's relative-position mask kernel and of the fused rel-pos attention call against the
 CPU oracle's node-by-node restatement of the graph (src/core/fastconformer.h:98-102, 876-934)."""
 import math
-import os
 
 import numpy as np
 import pytest
 
 import oracle as ora
+from cases import sweep_seeds
 from crispasr_amd import ggml
 from gpu_util import assert_parity, upload
 
@@ -53,6 +53,8 @@ def check_mask(got_bits: np.ndarray, ref_bits: np.ndarray, what: str):
     assert np.array_equal(got_bits == NEG_INF_BITS, inf_ref), f"{what}: -inf positions differ"
     g, r = ora.fp16_to_fp32(got_bits), ora.fp16_to_fp32(ref_bits)
     fin = ~inf_ref
+    if not fin.any():           # e.g. a single key that the pad mask removes
+        return
     assert np.isfinite(g[fin]).all(), f"{what}: non-finite value at a finite position"
     err = np.abs(g[fin] - r[fin])
     # inputs of the products are rounded to f16 (relative 2^-11 each) before an f32 accumulation, and the result
@@ -180,7 +182,7 @@ def _draw(seed: int) -> dict:
                 add_type=(ora.F32, ora.F16)[r(9, 0, 1)])
 
 
-@pytest.mark.parametrize("seed", range(int(os.environ.get("RELPOS_RANDOM_CASES", "24"))))
+@pytest.mark.parametrize("seed", sweep_seeds("RELPOS_RANDOM_CASES", 24))
 def test_relpos_mask_random_shapes(seed):
     spec = _draw(seed)
     c = make(**spec)
@@ -191,7 +193,7 @@ def test_relpos_mask_random_shapes(seed):
     check_mask(got.to_host()[: 2 * n].view(np.uint16), ref.buf.view(np.uint16), str(spec))
 
 
-@pytest.mark.parametrize("seed", range(int(os.environ.get("RELPOS_ATTN_RANDOM_CASES", "20"))))
+@pytest.mark.parametrize("seed", sweep_seeds("RELPOS_ATTN_RANDOM_CASES", 20))
 def test_relpos_attention_random_shapes(seed):
     """the one-kernel form on seeded random shapes off the tile grid: broadcast tables, every K/V type, both mask types"""
     spec = _draw(100 + seed)
