@@ -124,35 +124,49 @@ struct Chunk {
 
 // Q4_0 / Q4_1 / Q5_0 / Q5_1: x, y = the 8 bytes that hold the chunk's nibbles, shifted so that they sit in the low halves;
 // z = d (low) and m (high halfword); w = the chunk's 8 fifth bits.  q0, q1: the 8 bytes at QS + 8 (c % 2) of the block,
-// h0, h1: the block's first 8 bytes, c: which 8 of the block's 32 elements.
-template <int TYPE>
-__device__ __forceinline__ Chunk narrow_chunk(uint32_t q0, uint32_t q1, uint32_t h0, uint32_t h1, int c) {
-    typedef BlockFormat<TYPE> F;
+// dm: d in the low halfword (and m in the high one), qh: the block's 32 fifth bits, c: which 8 of the block's 32 elements.
+__device__ __forceinline__ Chunk narrow_fields(uint32_t q0, uint32_t q1, uint32_t dm, uint32_t qh, int c) {
     Chunk r;
     const int sh = (c & 2) ? 4 : 0;
     r.v.x = (q0 >> sh) & 0x0F0F0F0Fu;
     r.v.y = (q1 >> sh) & 0x0F0F0F0Fu;
-    r.v.z = F::HAS_M ? h0 : h0 & 0xFFFFu;
-    const uint32_t qh = !F::QH ? 0u : F::QH == 4 ? h1 : __builtin_amdgcn_alignbyte(h1, h0, 2);
+    r.v.z = dm;
     r.v.w = (qh >> (c * 8)) & 0xFFu;
     return r;
 }
 
+// the same from the block's first 8 bytes h0, h1
+template <int TYPE>
+__device__ __forceinline__ Chunk narrow_chunk(uint32_t q0, uint32_t q1, uint32_t h0, uint32_t h1, int c) {
+    typedef BlockFormat<TYPE> F;
+    const uint32_t qh = !F::QH ? 0u : F::QH == 4 ? h1 : __builtin_amdgcn_alignbyte(h1, h0, 2);
+    return narrow_fields(q0, q1, F::HAS_M ? h0 : h0 & 0xFFFFu, qh, c);
+}
+
 // the same chunk cut out of a raw copy of the rows in LDS (row_off: byte offset of the row inside the stage, a multiple
-// of 4; blocks and their quants start on even bytes): aligned dword reads, shifted by two bytes where needed.  The
-// stage is padded, so the third dword of a pair is always inside it.
+// of 4; blocks and their quants start on even bytes) with aligned dword reads.  Whether a block starts on a dword or two
+// bytes past one depends on the block's index alone - 18- and 22-byte blocks alternate, 20- and 24-byte ones always start
+// on one - so with blk a constant after unrolling, every shift here is decided at compile time.  The stage is padded:
+// the dword after a pair is always inside it.
 template <int TYPE>
 __device__ __forceinline__ Chunk narrow_lds_chunk(const char * stage, int row_off, int blk, int c) {
     typedef BlockFormat<TYPE> F;
-    const int oh = row_off + blk * F::BYTES;
-    const int oq = oh + F::QS + (c & 1) * 8;
-    const uint32_t * ph = (const uint32_t *)(stage + (oh & ~3));
-    const uint32_t * pq = (const uint32_t *)(stage + (oq & ~3));
-    const uint32_t a0 = ph[0], a1 = ph[1], a2 = ph[2];
-    const uint32_t b0 = pq[0], b1 = pq[1], b2 = pq[2];
-    const uint32_t sa = oh & 2, sb = oq & 2;
-    return narrow_chunk<TYPE>(__builtin_amdgcn_alignbyte(b1, b0, sb), __builtin_amdgcn_alignbyte(b2, b1, sb),
-                              __builtin_amdgcn_alignbyte(a1, a0, sa), __builtin_amdgcn_alignbyte(a2, a1, sa), c);
+    const int mis  = (blk * F::BYTES) & 2;                   // bytes from the dword below to the block
+    const int misq = (mis + F::QS) & 2;                      // ... to its quants
+    const uint32_t * ph = (const uint32_t *)(stage + row_off + blk * F::BYTES - mis);
+    const uint32_t * pq = (const uint32_t *)(stage + row_off + blk * F::BYTES + F::QS + (c & 1) * 8 - misq);
+    const uint32_t a0 = ph[0];
+    uint32_t q0 = pq[0], q1 = pq[1];
+    if (misq) {
+        const uint32_t q2 = pq[2];
+        q0 = __builtin_amdgcn_alignbyte(q1, q0, 2);
+        q1 = __builtin_amdgcn_alignbyte(q2, q1, 2);
+    }
+    const uint32_t dm = F::HAS_M ? a0 : mis ? a0 >> 16 : a0 & 0xFFFFu;
+    uint32_t qh = 0;
+    if (F::QH == 4) qh = ph[1];                                                    // fifth bits at byte 4
+    if (F::QH == 2) qh = mis ? ph[1] : __builtin_amdgcn_alignbyte(ph[1], a0, 2);   // at byte 2
+    return narrow_fields(q0, q1, dm, qh, c);
 }
 
 // bytes per block of the types the raw stream carries (Q8_0 for the others: they never instantiate it)
@@ -443,12 +457,16 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
         for (int i = 0; i < (V8 ? 0 : NV); i++) {
             const int flat = i * 64 + lane;
             Chunk c;
-            if (RAW) {
-                if (TYPE == MI355X_TYPE_Q8_0) c.v = q8_lds_chunk<false>(v_rawst, (flat / CH) * RS, (flat % CH) >> 2, (flat % CH) & 3);
-                else c = narrow_lds_chunk<RAW ? TYPE : MI355X_TYPE_Q4_0>(v_rawst, (flat / CH) * RS, (flat % CH) >> 2, (flat % CH) & 3);
-            } else {
-                c = vraw[s][i];
+            if (RAW && TYPE != MI355X_TYPE_Q8_0) {
+                // one block of 16 rows per pass (4 lanes per row), so that the block index is a constant: pass i takes
+                // block i % KS of rows 16 (i / KS) ... + 15
+                const int row = (i / KS) * 16 + (lane >> 2), ch = (i % KS) * 4 + (lane & 3);
+                c = narrow_lds_chunk<RAW ? TYPE : MI355X_TYPE_Q4_0>(v_rawst, row * RS, i % KS, lane & 3);
+                *(half8 *)&v_stage[row * PV + ch * 8] = chunk_to_half8<TYPE>(c);
+                continue;
             }
+            if (RAW) c.v = q8_lds_chunk<false>(v_rawst, (flat / CH) * RS, (flat % CH) >> 2, (flat % CH) & 3);
+            else     c = vraw[s][i];
             *(half8 *)&v_stage[(flat / CH) * PV + (flat % CH) * 8] = chunk_to_half8<TYPE>(c);
         }
         __builtin_amdgcn_wave_barrier();      // LDS runs a wave's instructions in order; keep the compiler from reordering
