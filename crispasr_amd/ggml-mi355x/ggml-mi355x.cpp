@@ -300,7 +300,17 @@ static ggml_backend_device_i make_device_iface() {
 static const ggml_backend_device_i mi355x_device_iface = make_device_iface();
 
 static const char * reg_name(ggml_backend_reg_t) { return "MI355X"; }
-static size_t reg_count(ggml_backend_reg_t) { int n = 0; mi355x_device_count(&n); return n > 0 ? 1 : 0; }
+static size_t reg_count(ggml_backend_reg_t) {
+    // a library built from another revision of the header than this file offers no device: its structs may differ
+    if (mi355x_api_version() != MI355X_FATTN_API_VERSION) {
+        GGML_LOG_ERROR("ggml-mi355x: libmi355x_fattn has API version %d, this backend was built against %d\n",
+                       mi355x_api_version(), MI355X_FATTN_API_VERSION);
+        return 0;
+    }
+    int n = 0;
+    mi355x_device_count(&n);
+    return n > 0 ? 1 : 0;
+}
 static ggml_backend_dev_t reg_dev(ggml_backend_reg_t, size_t) { return g_dev(); }
 static void * reg_proc(ggml_backend_reg_t, const char *) { return nullptr; }
 
