@@ -45,16 +45,13 @@ constexpr int   STEP        = 32;                  // keys per wave step
 constexpr float LOG2E       = 1.4426950408889634f;
 constexpr float SUM_LIMIT   = 4096.0f;             // 8 probabilities per lane and step
 
-// K and V are read once per launch: loads marked non-temporal leave the rest of L2 alone and stream faster (a read-only
-// sweep of 2 GiB reaches 7.0-7.1 TB/s with them against 5.7-6.2 TB/s with plain loads on the same device; 64 sequences
-// x 4096 f16 entries: 169 against 188 us).  Only for loads whose wave instruction takes whole lines once - the coalesced
-// row streams and f16 rows.  Per-lane pieces of block rows come back to a line several times: the 8-byte pieces and
-// halfword scales of the int8 V stage lose 3-5% when marked, and the strided-row forms stay plain with them.
+// K and V are read once per launch and loaded with stream_load where a wave instruction takes whole lines once - the
+// coalesced row streams and f16 rows (64 sequences x 4096 f16 entries: 169 against 188 us).  Per-lane pieces of block
+// rows come back to a line several times: the 8-byte pieces and halfword scales of the int8 V stage lose 3-5% when
+// marked, and the strided-row forms stay plain with them.
 typedef uint32_t u32x2    __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4    __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_a2 __attribute__((ext_vector_type(2), aligned(2)));
-template <typename T>
-__device__ __forceinline__ T stream_load(const void * p) { return __builtin_nontemporal_load((const T *)p); }
 
 // ---- Q8_0 in registers ------------------------------------------------------------------
 
