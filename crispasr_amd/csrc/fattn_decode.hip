@@ -266,11 +266,13 @@ constexpr int decode_lds_bytes() {
 }
 
 // V8 (with RAW): V's quants go to LDS as bytes and come back through ds_read_b64_tr_b8 already in operand layout
-// (8 consecutive keys of one column per lane); the transposing read ignores the low three address bits, and the quants
-// of block b start at byte 34 b + 2 of a row, so V is not taken from the coalesced stream: each lane fetches the 8
-// quants of one chunk with one 8-byte load from its 2-byte aligned address, and the scales with halfword loads.
+// (8 consecutive keys of one column per lane).  The transposing read ignores the low three address bits and the quants
+// of block b start at byte 34 b + 2 of a row, so the rows cannot stay as they are in memory: V arrives as the same
+// coalesced stream as K, and each 2-byte piece of a unit is written to its place - a pair of quants to [key][column],
+// a scale to [block][key] - by one ds_write_b16 whose address depends on the lane alone (computed once, before the
+// key loop).
 template <int D, int TYPE, bool MASK, bool RAW, bool V8>
-__global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode_kernel(const FattnArgs a) {
+__global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const FattnArgs a) {
     static_assert(!V8 || RAW, "the int8 V stage belongs to the streamed Q8_0 path");
     constexpr int KS  = D / 32;                    // reduction steps of Q.K^T (one Q8_0 block each)
     constexpr int DBK = D / 16;                    // 16-wide blocks of the output's d
@@ -291,8 +293,9 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
     // the per-wave stages; after the key loop the same memory carries the cross-wave reduction
     extern __shared__ __attribute__((aligned(16))) char smem[];
     constexpr int VP8 = v8_pitch<D>();
-    constexpr int NV8 = STEP * (D / 8) / 64;       // 8-quant chunks of V per lane and step
-    constexpr int NSC = STEP * KS / 64;            // V scales per lane and step
+    constexpr int PCS = UNIT / 2;                  // (V8) 2-byte pieces per unit
+    constexpr bool ONE = V8;                       // one register stage: the next step is requested once this one is in LDS
+                                                   // (two stages, as the other forms have: 102-104 against 99 us at 64 x 4096)
     constexpr int WAVE_BYTES = V8 ? RAWSZ + STEP * VP8 + KS * STEP * 2 : STEP * PV * 2 + (RAW ? 2 * RAWSZ : 0);
     char * const wave_mem = smem + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * WAVE_BYTES;
     _Float16 * v_stage = (_Float16 *)wave_mem;                          // (!V8)
@@ -346,9 +349,22 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
     Chunk vraw[2][RAW ? 1 : NV];
     typedef typename std::conditional<UNIT == 8, u32x2, uint32_t>::type unit_t;
     // (V8 keeps one register stage: index 0 whatever the step's stage number)
-    unit_t kun[2][RAW ? NU : 1], vun[2][RAW && !V8 ? NU : 1];
-    u32x2_a2 v8q[1][V8 ? NV8 : 1];
-    uint16_t v8d[1][V8 ? NSC : 1];
+    unit_t kun[2][RAW ? NU : 1], vun[2][RAW ? NU : 1];
+    // (V8) LDS offsets from wave_mem of the pieces of this lane's V units, two to a register: byte o of a step's rows is
+    // byte o % RS of row o / RS; byte 0 of a block is its scale's, bytes 2.. its quants'
+    uint32_t vdst[V8 ? NU : 1][V8 ? PCS / 2 : 1];
+    if (V8) {
+#pragma unroll
+        for (int i = 0; i < NU; i++)
+#pragma unroll
+            for (int k = 0; k < PCS; k++) {
+                const int o   = (i * 64 + lane) * UNIT + 2 * k;
+                const int row = o / RS, rem = o % RS, blk = rem / BB, ib = rem % BB;
+                const uint32_t dst = ib == 0 ? RAWSZ + STEP * VP8 + (blk * STEP + row) * 2
+                                             : RAWSZ + row * VP8 + blk * 32 + ib - 2;
+                vdst[i][k / 2] = k % 2 ? vdst[i][k / 2] | dst << 16 : dst;
+            }
+    }
     // a partial last step: its loads are clamped to the last valid row or unit (branch-free, in bounds) and the
     // keys they stand for are excluded in the step
     auto issue = [&](int it, auto stage) __attribute__((always_inline)) {
@@ -362,23 +378,8 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
 #pragma unroll
             for (int i = 0; i < NU; i++) {
                 const uint32_t off = (uint32_t)min(i * 64 + lane, last) * UNIT;
-                kun[V8 ? 0 : s][i] = stream_load<unit_t>(kp + off);
-                if (!V8) vun[s][i] = stream_load<unit_t>(vp + off);
-            }
-            if (V8) {
-                const int last_row = min(STEP, k_end - j0) - 1;
-#pragma unroll
-                for (int i = 0; i < NV8; i++) {
-                    const int flat = i * 64 + lane;
-                    const int row  = min(flat / CH, last_row), c = flat % CH;
-                    v8q[0][i] = *(const u32x2_a2 *)(vp + row * RS + (c >> 2) * FATTN_Q8_0_BYTES + 2 + (c & 3) * 8);
-                }
-#pragma unroll
-                for (int i = 0; i < NSC; i++) {
-                    const int flat = i * 64 + lane;
-                    const int row  = min(flat / KS, last_row);
-                    v8d[0][i] = *(const uint16_t *)(vp + row * RS + (flat % KS) * FATTN_Q8_0_BYTES);
-                }
+                kun[ONE ? 0 : s][i] = stream_load<unit_t>(kp + off);
+                vun[ONE ? 0 : s][i] = stream_load<unit_t>(vp + off);
             }
             return;
         }
@@ -406,29 +407,38 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
         const int  j0   = k_begin + it * STEP;
         const bool tail = j0 + STEP > k_end;                  // wave-uniform
         // the following step's loads: into the other register stage, or (V8) into this one as soon as it is in LDS
-        if (!V8 && it + DEC_WAVES < n_steps) issue(it + DEC_WAVES, std::integral_constant<int, 1 - s>{});
+        if (!ONE && it + DEC_WAVES < n_steps) issue(it + DEC_WAVES, std::integral_constant<int, 1 - s>{});
 
         if (RAW) {
 #pragma unroll
             for (int i = 0; i < NU; i++) {
-                *(unit_t *)(k_rawst + (i * 64 + lane) * UNIT) = kun[V8 ? 0 : s][i];
+                *(unit_t *)(k_rawst + (i * 64 + lane) * UNIT) = kun[ONE ? 0 : s][i];
                 if (!V8) *(unit_t *)(v_rawst + (i * 64 + lane) * UNIT) = vun[s][i];
             }
             if (V8) {
 #pragma unroll
-                for (int i = 0; i < NV8; i++) {
-                    const int flat = i * 64 + lane;
-                    *(uint2 *)(v8_stage + (flat / CH) * VP8 + (flat % CH) * 8) = make_uint2(v8q[0][i][0], v8q[0][i][1]);
-                }
-                // rows past k_end repeat the last row's bytes: a zero scale makes exact zeros of them
+                for (int i = 0; i < NU; i++) {
+                    if ((i + 1) * 64 > UPS && i * 64 + lane >= UPS) continue;      // past the step's 32 rows
+                    uint32_t w[2];
+                    if constexpr (UNIT == 8) { w[0] = vun[ONE ? 0 : s][i][0]; w[1] = vun[ONE ? 0 : s][i][1]; }
+                    else                     { w[0] = vun[ONE ? 0 : s][i]; w[1] = 0; }
 #pragma unroll
-                for (int i = 0; i < NSC; i++) {
-                    const int flat = i * 64 + lane;
-                    const int row  = flat / KS;
-                    *(uint16_t *)(vsc_stage + ((flat % KS) * STEP + row) * 2) = (tail && j0 + row >= k_end) ? (uint16_t)0 : v8d[0][i];
+                    for (int k = 0; k < PCS; k++) {
+                        const uint32_t dst = k % 2 ? vdst[i][k / 2] >> 16 : vdst[i][k / 2] & 0xFFFFu;
+                        *(uint16_t *)(wave_mem + dst) = (uint16_t)(k % 2 ? w[k / 2] >> 16 : w[k / 2]);
+                    }
+                }
+                // rows past k_end hold bytes of other rows: a zero scale makes exact zeros of them (the LDS runs a wave's
+                // writes in order)
+                if (tail) {
+#pragma unroll
+                    for (int t = 0; t < STEP * KS / 64; t++) {
+                        const int idx = t * 64 + lane, row = idx / KS;
+                        if (j0 + row >= k_end) *(uint16_t *)(vsc_stage + ((idx % KS) * STEP + row) * 2) = 0;
+                    }
                 }
             }
-            if (V8 && it + DEC_WAVES < n_steps) issue(it + DEC_WAVES, stage);
+            if (ONE && it + DEC_WAVES < n_steps) issue(it + DEC_WAVES, stage);
             if (!V8 && tail) {
                 // rows past k_end hold bytes of no row: a zero scale keeps what is made of them finite
 #pragma unroll
@@ -575,7 +585,7 @@ __global__ void __launch_bounds__(DEC_THREADS, V8 && !MASK ? 3 : 2) fattn_decode
     }
     for (int it = wave; it < n_steps; it += 2 * DEC_WAVES) {
         step(it, S0{});
-        if (it + DEC_WAVES < n_steps) step(it + DEC_WAVES, std::integral_constant<int, V8 ? 0 : 1>{});
+        if (it + DEC_WAVES < n_steps) step(it + DEC_WAVES, std::integral_constant<int, ONE ? 0 : 1>{});
     }
 
     // ---- column totals, then the four waves through LDS ----------------------------------------------
