@@ -265,12 +265,35 @@ constexpr int decode_lds_bytes() {
     return stage > red ? stage : red;
 }
 
+// Where the 2-byte pieces of a step's 32 Q8_0 rows go in the int8 V stage, as offsets from the wave's LDS block: byte o
+// of the step is byte o % RS of row o / RS; byte 0 of a 34-byte block is its scale's (-> f16 [block][key] behind the
+// stage), bytes 2.. are its quants' (-> [key][column]).  Indexed by piece o / 2, padded to whole 64-lane loads of units.
+template <int D>
+struct V8Places {
+    static constexpr int RS = D / 32 * FATTN_Q8_0_BYTES, UNIT = RS % 8 == 0 ? 8 : 4;
+    static constexpr int UNITS = (STEP * RS / UNIT + 63) / 64 * 64;
+    static constexpr int RAWSZ = (STEP * RS + 511) / 512 * 512 + 64;
+    uint16_t at[UNITS * UNIT / 2];
+};
+template <int D>
+constexpr V8Places<D> v8_places() {
+    typedef V8Places<D> P;
+    P t{};
+    for (int o = 0; o < STEP * P::RS; o += 2) {
+        const int row = o / P::RS, rem = o % P::RS, blk = rem / FATTN_Q8_0_BYTES, ib = rem % FATTN_Q8_0_BYTES;
+        t.at[o / 2] = (uint16_t)(ib == 0 ? P::RAWSZ + STEP * v8_pitch<D>() + (blk * STEP + row) * 2
+                                         : P::RAWSZ + row * v8_pitch<D>() + blk * 32 + ib - 2);
+    }
+    return t;
+}
+template <int D> __device__ const V8Places<D> v8_places_table = v8_places<D>();
+
 // V8 (with RAW): V's quants go to LDS as bytes and come back through ds_read_b64_tr_b8 already in operand layout
 // (8 consecutive keys of one column per lane).  The transposing read ignores the low three address bits and the quants
 // of block b start at byte 34 b + 2 of a row, so the rows cannot stay as they are in memory: V arrives as the same
 // coalesced stream as K, and each 2-byte piece of a unit is written to its place - a pair of quants to [key][column],
-// a scale to [block][key] - by one ds_write_b16 whose address depends on the lane alone (computed once, before the
-// key loop).
+// a scale to [block][key] - by one ds_write_b16 whose address depends on the lane alone (read from a table behind the
+// first K/V request: computing the 36 of them costs more instructions than a 32-key step).
 template <int D, int TYPE, bool MASK, bool RAW, bool V8>
 __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const FattnArgs a) {
     static_assert(!V8 || RAW, "the int8 V stage belongs to the streamed Q8_0 path");
@@ -350,21 +373,8 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     typedef typename std::conditional<UNIT == 8, u32x2, uint32_t>::type unit_t;
     // (V8 keeps one register stage: index 0 whatever the step's stage number)
     unit_t kun[2][RAW ? NU : 1], vun[2][RAW ? NU : 1];
-    // (V8) LDS offsets from wave_mem of the pieces of this lane's V units, two to a register: byte o of a step's rows is
-    // byte o % RS of row o / RS; byte 0 of a block is its scale's, bytes 2.. its quants'
+    // (V8) LDS offsets from wave_mem of the pieces of this lane's V units, two to a register
     uint32_t vdst[V8 ? NU : 1][V8 ? PCS / 2 : 1];
-    if (V8) {
-#pragma unroll
-        for (int i = 0; i < NU; i++)
-#pragma unroll
-            for (int k = 0; k < PCS; k++) {
-                const int o   = (i * 64 + lane) * UNIT + 2 * k;
-                const int row = o / RS, rem = o % RS, blk = rem / BB, ib = rem % BB;
-                const uint32_t dst = ib == 0 ? RAWSZ + STEP * VP8 + (blk * STEP + row) * 2
-                                             : RAWSZ + row * VP8 + blk * 32 + ib - 2;
-                vdst[i][k / 2] = k % 2 ? vdst[i][k / 2] | dst << 16 : dst;
-            }
-    }
     // a partial last step: its loads are clamped to the last valid row or unit (branch-free, in bounds) and the
     // keys they stand for are excluded in the step
     auto issue = [&](int it, auto stage) __attribute__((always_inline)) {
@@ -571,6 +581,15 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     };
     if (wave < n_steps) issue(wave, S0{});
 
+    // (V8) where the pieces of this lane's V units go: read behind the first K/V request, needed when that has arrived
+    if (V8) {
+        static_assert(!V8 || (V8Places<D>::RAWSZ == RAWSZ && V8Places<D>::UNITS == NU * 64 && V8Places<D>::UNIT == UNIT), "table layout");
+        const uint32_t * places = (const uint32_t *)v8_places_table<D>.at;
+#pragma unroll
+        for (int i = 0; i < NU; i++)
+#pragma unroll
+            for (int k = 0; k < PCS / 2; k++) vdst[i][k] = places[(i * 64 + lane) * (PCS / 2) + k];
+    }
     // ---- Q -> f16 B operands in log2 units (after the first K/V request: the two cold misses overlap) ----
     {
         const float * qrow = (const float *)(a.q + (int64_t)iq1 * a.nbq1 + (int64_t)h * a.nbq2 + (int64_t)b * a.nbq3);
