@@ -791,7 +791,10 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             for (int k = 0; k < 32 / RPI; k++) {
                 const int row = k * RPI + lane / CPR, c = lane % CPR;
                 const float4 o = *(const float4 *)(stg + row * D + ((c ^ (row & (CPR - 1))) * 4));
-                if (q_first + row < a.Nq) *(float4 *)(out0 + row * row_stride + c * 4) = o;
+                // whole rows, written once: marked non-temporal (encoder launch 2% shorter; the scattered quarter-lines of
+                // the direct form were 12 us slower with the mark)
+                typedef float f32x4 __attribute__((ext_vector_type(4)));
+                if (q_first + row < a.Nq) __builtin_nontemporal_store(f32x4{o.x, o.y, o.z, o.w}, (f32x4 *)(out0 + row * row_stride + c * 4));
             }
             __builtin_amdgcn_wave_barrier();               // the next query block reuses the staging rows
             if (a.n_splits > 1 && hh == 0 && qi < a.Nq) {
