@@ -20,11 +20,12 @@
 // with one packed multiply (one rounding, = f16(q*d)).  When the rows of a Q8_0 cache are contiguous the
 // K bytes of a step are fetched as one coalesced stream of 8- (or 4-)byte units into a wave-private raw
 // stage in LDS and the chunks are cut out of LDS instead - three times fewer global load instructions.
-// V then skips the f16 stage: its quants are stored to LDS as bytes (one 8-byte load per chunk, from its
-// 2-byte aligned address, and one aligned 8-byte LDS store) and read back through ds_read_b64_tr_b8,
-// which hands every lane eight consecutive keys of one column - the A operand of the second product -
-// to be widened and multiplied by those keys' scales in registers: same values, a third of the LDS
-// instructions, half the LDS bytes, one register stage instead of two.
+// V then skips the f16 stage: it arrives as the same kind of stream, its quants are stored to LDS as bytes - every
+// 2-byte piece of a unit written to its place, [key][column] for quants and [block][key] for scales - and read back
+// through ds_read_b64_tr_b8, which hands every lane eight consecutive keys of one column - the A operand of the second
+// product - to be widened and multiplied by those keys' scales in registers: same values, half the LDS bytes, one
+// register stage instead of two.  Q4_0 / Q4_1 / Q5_0 / Q5_1 rows are streamed the same way into raw K and V stages and
+// dequantised out of LDS (V into the f16 stage).  Streams and f16 rows are loaded non-temporal: they are read once.
 // Loads of the next step are in flight while the current one is consumed.  Waves are merged through LDS, splits by fattn_merge_kernel.
 #include "fattn_common.h"
 
