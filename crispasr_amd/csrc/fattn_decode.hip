@@ -27,7 +27,7 @@
 // register stage instead of two.  Q4_0 / Q4_1 / Q5_0 / Q5_1 rows are streamed the same way into raw K and V stages and
 // dequantised out of LDS (V into the f16 stage).  Streams and f16 rows are loaded non-temporal: they are read once.
 // Loads of the next step are in flight while the current one is consumed.  Waves are merged through LDS, splits by fattn_merge_kernel.
-#include "fattn_common.h"
+#include "fattn_row.h"
 
 #include <stdlib.h>
 #include <type_traits>
@@ -625,6 +625,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
 
     // thread t: column t / 16, a strided set of d
     const int col = tid >> 4;
+    bool bad = false;                           // this column's result is not finite
     if (row0 + col < R) {
         float M = -INFINITY;
 #pragma unroll
@@ -637,6 +638,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
             f[w] = mw == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mw - M);
             L += red_ml[w][col][1] * f[w];
         }
+        bad = not_finite(L);
         const int     ciq1 = (row0 + col) / a.gqa;
         const int     ch   = hk * a.gqa + (row0 + col) % a.gqa;
         const int64_t row  = ((int64_t)b * a.Nq + ciq1) * a.Hq + ch;
@@ -644,6 +646,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
             float acc = 0.0f;
 #pragma unroll
             for (int w = 0; w < DEC_WAVES; w++) acc += red_o[w][col][d] * f[w];
+            bad = bad || not_finite(acc);
             if (a.n_splits == 1) {
                 a.dst[row * D + d] = L > 0.0f ? acc / L : 0.0f;
             } else {
@@ -655,6 +658,23 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
             float * pm = a.part_ml + (row * a.n_splits + split) * 2;
             pm[0] = M == -INFINITY ? -INFINITY : M * 0.6931471805599453f;
             pm[1] = L;
+        }
+    }
+    // An excluded key was multiplied by a probability of zero above, not skipped.  For finite K/V that is the same thing; a
+    // cache slot that holds NaN or inf bits (never written, and masked out for that reason) turns the products into NaN.
+    // Such a row shows in its result, and is computed again the way the CPU op does it - excluded keys not read at all.
+    // Without a mask every key is visible and a non-finite result is the answer.  (Columns 4w .. 4w + 3 belong to wave w
+    // in both passes: the second store follows the first in the same wave.)
+    if constexpr (MASK) {
+        const uint64_t badmask = __builtin_amdgcn_ballot_w64(bad);
+        if (badmask != 0) {
+            __threadfence();
+#pragma unroll 1
+            for (int c = 0; c < 4; c++) {
+                const int r = row0 + wave * 4 + c;
+                if (((badmask >> (16 * c)) & 0xFFFFu) != 0 && r < R)
+                    attn_row_redo<TYPE, D>(a, r / a.gqa, hk * a.gqa + r % a.gqa, b, split, k_begin, k_end);
+            }
         }
     }
 }

@@ -39,7 +39,7 @@
 //
 // A 32-key block whose mask excludes every key for all of the wave's queries is skipped outright (its probabilities
 // would all be exact zeros): the upper triangle of a causal prompt, the keys beyond a padded sequence's length.
-#include "fattn_common.h"
+#include "fattn_row.h"
 
 #include <stdio.h>
 #include <stdlib.h>
@@ -757,6 +757,21 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     // LDS; the other forms, whose launches are short, store from the accumulator layout (the detour costs them a
     // barrier and a round trip: the Whisper-base encoder layer 17.5 -> 18.4 us, against 61.4 -> 60.3 us on large-v3's).
     constexpr bool OUT_LDS = NQB == 2;
+    // Excluded keys were multiplied by probabilities of exactly zero, not skipped: the same for finite K/V, NaN for a cache
+    // slot that holds NaN or inf bits (never written, and masked out for that reason).  A query whose sum or accumulators
+    // are not finite is noted here and computed again below the way the CPU op does it.  (x * 0 is 0 for every finite x.)
+    uint64_t badbits[NQB];
+    if constexpr (MASK) {
+#pragma unroll
+        for (int qb = 0; qb < NQB; qb++) {
+            float chk = st[qb].l * 0.0f;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) chk = fmaf(oacc[qb][db][r], 0.0f, chk);
+            badbits[qb] = __builtin_amdgcn_ballot_w64(chk != 0.0f);         // NaN != 0
+        }
+    }
     if constexpr (OUT_LDS) {
         // A lane holds 16-byte pieces of its query's row, 32 bytes apart: stored from there, one instruction scatters 64
         // quarter-lines over 32 rows.  The rows go through LDS instead (free now: 32 x D floats per wave, chunks XOR-swizzled
@@ -830,6 +845,25 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                     float * pm = a.part_ml + (row * a.n_splits + split) * 2;
                     pm[0] = st[qb].have ? st[qb].m * 0.6931471805599453f : -INFINITY;
                     pm[1] = ltot;
+                }
+            }
+        }
+    }
+    // the queries noted above, one row at a time by the whole wave (lanes l and l + 32 hold the same query); the wave
+    // that stored a row is the one that stores it again
+    if constexpr (MASK) {
+        uint64_t any = 0;
+#pragma unroll
+        for (int qb = 0; qb < NQB; qb++) any |= badbits[qb];
+        if (any != 0) {
+            __threadfence();
+#pragma unroll 1
+            for (int qb = 0; qb < NQB; qb++) {
+                uint32_t bits = (uint32_t)badbits[qb] | (uint32_t)(badbits[qb] >> 32);
+                while (bits != 0) {
+                    const int qi = q0 + qb * 32 + __builtin_ctz(bits);
+                    bits &= bits - 1;
+                    if (qi < a.Nq) attn_row_redo<TYPE, D>(a, qi, h, b, split, k_begin, k_end);
                 }
             }
         }

@@ -27,7 +27,7 @@
 // 16-byte chunks of a row XOR-swizzled so that the operand reads are conflict-free), requested behind the first barrier
 // of a step and waited for before the second; V is fetched one step ahead into registers and written behind the second.  K, V and the table are f16 with 16-byte aligned rows (the caller rounds F32 ones first, as
 // the reference's own graph does for the mask product's operands).
-#include "fattn_common.h"
+#include "fattn_row.h"
 
 #include <stdlib.h>
 #include <type_traits>
@@ -369,6 +369,17 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 
     // ---- normalise and store: lane (il, hh) holds d = 32 db + 8 g + 4 hh + c of its query -------------------------------
     l += __shfl_xor(l, 32, 64);
+    // Excluded keys (add = -inf) were multiplied by probabilities of exactly zero, not skipped: the same for finite K/V, NaN
+    // otherwise.  Queries whose result is not finite are computed again below, excluded keys unread, as the CPU op does it.
+    uint64_t badbits = 0;
+    if constexpr (ADD) {
+        float chk = l * 0.0f;
+#pragma unroll
+        for (int db = 0; db < DBO; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) chk = fmaf(oacc[db][r], 0.0f, chk);
+        badbits = __builtin_amdgcn_ballot_w64(chk != 0.0f);
+    }
     if (i0w + il < a.Nq) {
         const float inv = l > 0.0f ? 1.0f / l : 0.0f;
         float * orow = a.dst + (((int64_t)b * a.Nq + (i0w + il)) * a.H + h) * D;
@@ -381,6 +392,17 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
                 for (int c = 0; c < 4; c++) o[c] = oacc[db][4 * g + c] * inv;
                 *(float4v *)(orow + 32 * db + 8 * g + 4 * hh) = o;
             }
+    }
+    if constexpr (ADD) {
+        if (badbits != 0) {
+            __threadfence();
+            uint32_t bits = (uint32_t)badbits | (uint32_t)(badbits >> 32);      // lanes l and l + 32 hold the same query
+            while (bits != 0) {
+                const int qi = i0w + __builtin_ctz(bits);
+                bits &= bits - 1;
+                if (qi < a.Nq) attn_row_redo_relpos<D>(a, qi, h, b);
+            }
+        }
     }
 }
 

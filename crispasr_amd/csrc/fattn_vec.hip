@@ -12,76 +12,20 @@
 // (src/crispasr.cpp:3208-3222, 3269-3282; src/core/attention.h:992; src/canary.cpp:966-972):
 // s = scale*<q,k> [soft-capped] + slope*mask, -inf mask entries exclude a key, GQA by
 // h / (Hq/Hkv), mask broadcast by h % Hm and b % Bm, output [D, Hq, Nq, B].
-#include "fattn_common.h"
+#include "fattn_row.h"
 
 namespace {
 
 constexpr int VEC_WAVES   = 4;
 constexpr int VEC_THREADS = VEC_WAVES * 64;
-constexpr int VEC_UNROLL  = 4;
-
-// 8 consecutive elements of a K/V row starting at element d0, as f32 (exact for all types)
-template <int TYPE>
-__device__ __forceinline__ void load8(const char * row, int d0, bool aligned16, float (&out)[8]) {
-    if constexpr (TYPE == MI355X_TYPE_F16) {
-        const char * p = row + (size_t)d0 * 2;
-        if (aligned16) {
-            const uint4 u = *(const uint4 *)p;
-            const uint32_t w[4] = {u.x, u.y, u.z, u.w};
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                out[2 * i]     = h2f_bits((uint16_t)(w[i] & 0xffffu));
-                out[2 * i + 1] = h2f_bits((uint16_t)(w[i] >> 16));
-            }
-        } else {
-            const uint16_t * h = (const uint16_t *)p;
-#pragma unroll
-            for (int i = 0; i < 8; i++) out[i] = h2f_bits(h[i]);
-        }
-    } else if constexpr (TYPE == MI355X_TYPE_F32) {
-        const char * p = row + (size_t)d0 * 4;
-        if (aligned16) {
-            const float4 a = *(const float4 *)p;
-            const float4 b = *(const float4 *)(p + 16);
-            out[0] = a.x; out[1] = a.y; out[2] = a.z; out[3] = a.w;
-            out[4] = b.x; out[5] = b.y; out[6] = b.z; out[7] = b.w;
-        } else {
-            const float * f = (const float *)p;
-#pragma unroll
-            for (int i = 0; i < 8; i++) out[i] = f[i];
-        }
-    } else {  // block-32 types: blocks are only 2-byte aligned
-        dequant8<TYPE>(row + (size_t)(d0 / FATTN_QK8_0) * fattn_block_bytes(TYPE), d0 % FATTN_QK8_0, out);
-    }
-}
-
-struct Partial {
-    float m, l;
-    float acc[8];
-};
-
-__device__ __forceinline__ void merge_partial(Partial & a, const Partial & b) {
-    const float mn = fmaxf(a.m, b.m);
-    // a state that has seen no key has m = -inf and l = 0: its factor must be 0, not NaN
-    const float fa = a.m == -INFINITY ? 0.0f : __expf(a.m - mn);
-    const float fb = b.m == -INFINITY ? 0.0f : __expf(b.m - mn);
-    a.l = a.l * fa + b.l * fb;
-#pragma unroll
-    for (int e = 0; e < 8; e++) a.acc[e] = a.acc[e] * fa + b.acc[e] * fb;
-    a.m = mn;
-}
 
 template <int TYPE, int LPR>
 __global__ void __launch_bounds__(VEC_THREADS) fattn_vec_kernel(const FattnArgs a) {
-    constexpr int G = 64 / LPR;                 // key rows per wave per load
     const int tid  = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
-    const int grp  = lane / LPR;
-    const int lig  = lane % LPR;                // lane in group
-    const int d0   = lig * 8;
+    const int d0   = (lane % LPR) * 8;          // the lane's 8 elements of d
     const bool dvalid = d0 < a.D;               // D is a multiple of 8
-    const int d0c  = dvalid ? d0 : 0;
 
     // blockIdx.x = row * n_splits + split, row = (b*Nq + iq1)*Hq + h  (the dst row order)
     const int split = blockIdx.x % a.n_splits;
@@ -103,81 +47,16 @@ __global__ void __launch_bounds__(VEC_THREADS) fattn_vec_kernel(const FattnArgs 
     }
     const char * kbase = a.k + hk * a.nbk2 + bk * a.nbk3;
     const char * vbase = a.v + hk * a.nbv2 + bk * a.nbv3;
-    const uint16_t * mrow = a.mask
-        ? (const uint16_t *)(a.mask + iq1 * a.nbm1 + (h % a.Hm) * a.nbm2 + (b % a.Bm) * a.nbm3)
-        : nullptr;
-    const float slope = fattn_slope(a, h);
-    const bool  al    = a.aligned16 != 0;
+    RowMaskTensor mask;
+    mask.row   = a.mask ? (const uint16_t *)(a.mask + iq1 * a.nbm1 + (h % a.Hm) * a.nbm2 + (b % a.Bm) * a.nbm3) : nullptr;
+    mask.slope = fattn_slope(a, h);
 
-    Partial st;
+    RowPartial st;
     st.m = -INFINITY;
     st.l = 0.0f;
 #pragma unroll
     for (int e = 0; e < 8; e++) st.acc[e] = 0.0f;
-
-    // every lane runs the same trip count so that the DPP reductions see full groups
-    const int stride = VEC_WAVES * G * VEC_UNROLL;
-    for (int j0 = k_begin; j0 < k_end; j0 += stride) {
-        float kf[VEC_UNROLL][8];
-        float vf[VEC_UNROLL][8];
-        float s[VEC_UNROLL];
-        int   jj[VEC_UNROLL];
-#pragma unroll
-        for (int u = 0; u < VEC_UNROLL; u++) {
-            jj[u] = j0 + (u * VEC_WAVES + wave) * G + grp;
-            const int jc = min(jj[u], k_end - 1);
-            load8<TYPE>(kbase + (size_t)jc * a.nbk1, d0c, al, kf[u]);
-        }
-#pragma unroll
-        for (int u = 0; u < VEC_UNROLL; u++) {
-            const int jc = min(jj[u], k_end - 1);
-            load8<TYPE>(vbase + (size_t)jc * a.nbv1, d0c, al, vf[u]);
-        }
-        float mloc = -INFINITY;
-#pragma unroll
-        for (int u = 0; u < VEC_UNROLL; u++) {
-            float dot = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 8; e++) dot = fmaf(q[e], kf[u][e], dot);
-            dot = group_sum<LPR>(dot);
-            float sc = dot * a.scale;
-            if (a.softcap != 0.0f) sc = a.softcap * tanhf(sc);
-            if (mrow) {
-                const int jc = min(jj[u], k_end - 1);
-                sc += slope * h2f_bits(mrow[jc]);
-            }
-            if (jj[u] >= k_end) sc = -INFINITY;
-            s[u] = sc;
-            mloc = fmaxf(mloc, sc);
-        }
-        if (mloc > st.m) {                       // uniform within a group
-            const float alpha = __expf(st.m - mloc);   // exp(-inf) = 0 on the first hit
-            st.l *= alpha;
-#pragma unroll
-            for (int e = 0; e < 8; e++) st.acc[e] *= alpha;
-            st.m = mloc;
-        }
-        if (st.m > -INFINITY) {
-#pragma unroll
-            for (int u = 0; u < VEC_UNROLL; u++) {
-                const float p = __expf(s[u] - st.m);   // 0 for excluded keys
-                st.l += p;
-#pragma unroll
-                for (int e = 0; e < 8; e++) st.acc[e] = fmaf(p, vf[u][e], st.acc[e]);
-            }
-        }
-    }
-
-    // merge the G groups of this wave (lanes with equal lig)
-#pragma unroll
-    for (int off = LPR; off < 64; off <<= 1) {
-        Partial o;
-        o.m = xor_shuffle(st.m, off);
-        o.l = xor_shuffle(st.l, off);
-#pragma unroll
-        for (int e = 0; e < 8; e++) o.acc[e] = xor_shuffle(st.acc[e], off);
-        merge_partial(st, o);
-    }
+    row_scan<TYPE, TYPE, LPR, VEC_WAVES>(row_scan_args(a), q, kbase, vbase, mask, k_begin, k_end, wave, lane, st);
 
     // merge the waves through LDS
     __shared__ float sh[VEC_WAVES][LPR][10];
@@ -191,30 +70,14 @@ __global__ void __launch_bounds__(VEC_THREADS) fattn_vec_kernel(const FattnArgs 
     if (wave == 0 && lane < LPR) {
 #pragma unroll
         for (int w = 1; w < VEC_WAVES; w++) {
-            Partial o;
+            RowPartial o;
             o.m = sh[w][lane][0];
             o.l = sh[w][lane][1];
 #pragma unroll
             for (int e = 0; e < 8; e++) o.acc[e] = sh[w][lane][2 + e];
-            merge_partial(st, o);
+            row_partial_merge(st, o);
         }
-        if (dvalid) {
-            if (a.n_splits == 1) {
-                const float inv = st.l > 0.0f ? 1.0f / st.l : 0.0f;
-                float * out = a.dst + (size_t)row * a.D + d0;
-#pragma unroll
-                for (int e = 0; e < 8; e++) out[e] = st.acc[e] * inv;
-            } else {
-                float * pa = a.part_acc + ((size_t)row * a.n_splits + split) * a.D + d0;
-#pragma unroll
-                for (int e = 0; e < 8; e++) pa[e] = st.acc[e];
-                if (lane == 0) {
-                    float * pm = a.part_ml + ((size_t)row * a.n_splits + split) * 2;
-                    pm[0] = st.m;
-                    pm[1] = st.l;
-                }
-            }
-        }
+        row_store<LPR>(a, st, row, split, lane);
     }
 }
 

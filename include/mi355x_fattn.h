@@ -140,7 +140,10 @@ int mi355x_stream_synchronize(void * stream);
  *        batch b reads b % Bm; -inf entries exclude the key
  *   Hq % Hkv == 0 (query head h reads KV head h / (Hq/Hkv)), B % Bk == 0.
  *   A row whose keys are all excluded (or Nkv == 0) yields zeros.
- *   Excluded keys still have to hold finite K/V values (they are multiplied by 0).
+ *   An excluded key contributes nothing whatever its K/V bytes are - NaN, inf, a Q8_0 block whose scale is NaN - as in
+ *   ggml-cpu, which skips it: cache slots that were never written may be masked out instead of cleared
+ *   (src/core/attention.h:680-683).  (The MFMA kernels multiply such a key by a probability of exactly zero, look at each
+ *   row's result before storing it, and compute a row that came out non-finite again with the excluded keys unread.)
  *
  * mi355x_fattn_supports is the predicate the backend's supports_op mirrors: it returns
  * MI355X_OK, MI355X_ERR_UNSUPPORTED or MI355X_ERR_INVALID without touching the device.
