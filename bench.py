@@ -9,7 +9,8 @@ resident in HBM before the timed region starts.  Prints ONE JSON line.
 Extra keys beside the contract's: `roofline` (dominant kernel against the f16 dense MFMA peak),
 `cpu_baseline` (the CPU oracle's ggml-like mode on a bounded sample, host cores of this box),
 `parity` (the timed configuration checked against the oracle on a sample of rows) and
-`decode` (the HBM-bound decode shapes, GB/s against 8 TB/s) and `host_resident` (the same calls on
+`roofline_decode` (the decode half of the metric: bytes of one decode step of the BASELINE shapes, and of the saturating
+ceiling shapes, over its time, against 8 TB/s), `decode` (more HBM-bound decode shapes, per call) and `host_resident` (the same calls on
 pinned host buffers: link-inclusive rates, never `value`).
 """
 from __future__ import annotations
@@ -354,6 +355,129 @@ def bench_decode(args, ca, ora, torch):
     return out
 
 
+def bench_roofline_decode(ca, ora, torch):
+    """The decode half of the metric as roofline entries: algorithmic bytes of one decode STEP (every layer's calls) over the
+    time of that step inside a HIP graph, against the 8 TB/s HBM peak.
+      C3_step: Whisper large-v3 decoder step with beam 5 - 32 layers x (self-attention, 1 query per beam against its own
+               224-entry f16 cache with a -inf mask beyond its position; cross-attention, 5 queries against one shared
+               1500-entry f16 K/V); 430 MB of distinct K/V per step.
+      C4_step: Voxtral-style LLM decode step - 30 layers x (1 token, 32 q / 8 kv heads x 128, Q8_0 cache of 663 entries, the
+               last of the 256 steps); 43 MB per step, so 8 steps' worth of distinct layers rotate through one replay.
+      ceilings: the same kernels with 64 independent sequences of 4096 entries per call (what the kernel's loop can do
+               when a launch has enough bytes to hide its fixed cost)."""
+    import numpy as np
+    res = {"bound": "hbm", "peak": PEAK_HBM_GBS, "unit": "GB/s"}
+
+    def f16_buf(n):
+        return torch.randn(n, device="cuda").half().view(torch.uint8)
+
+    def q8_buf(seed, n):
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(seed)
+        src = ca.Tensor(torch.randn(n, device="cuda", generator=gen).view(torch.uint8), ca.F32, (n,))
+        dst = ca.Tensor.empty(ca.Q8_0, (n,))
+        ca.cpy(src, dst)
+        torch.cuda.synchronize()
+        return dst.buf
+
+    def timed(name, label, calls, steps_in_graph, bytes_per_step, reps, note):
+        def replay_body():
+            for c in calls:
+                ca.flash_attn_ext(c["q"], c["k"], c["v"], c.get("mask"), c["scale"], out=c["out"])
+        for _ in range(2):
+            replay_body()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                replay_body()
+        torch.cuda.synchronize()
+        for _ in range(reps):                        # the clock settles
+            graph.replay()
+        torch.cuda.synchronize()
+        # five groups of `reps` replays that follow each other without the host in between; the median group
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
+        ev[0].record()
+        for i in range(5):
+            for _ in range(reps):
+                graph.replay()
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        ts = sorted(ev[i].elapsed_time(ev[i + 1]) / reps for i in range(5))
+        us_step = ts[len(ts) // 2] * 1e3 / steps_in_graph
+        gbs = bytes_per_step / (us_step * 1e-6) / 1e9
+        plans = sorted({ca.ggml.flash_attn_plan(c["q"], c["k"], c["v"], c.get("mask"), c["scale"]) for c in calls})
+        res[name] = {"label": label, "bytes": bytes_per_step, "us": us_step, "achieved": gbs, "frac": gbs / PEAK_HBM_GBS,
+                     "calls_per_step": len(calls) // steps_in_graph, "us_per_call": us_step * steps_in_graph / len(calls),
+                     "kernel_and_splits": [list(p) for p in plans], "note": note}
+        log(f"[bench] roofline_decode {name} ({label}): {bytes_per_step / 1e6:.1f} MB in {us_step:.1f} us per step = {gbs:.0f} GB/s "
+            f"= {gbs / PEAK_HBM_GBS:.3f} of HBM peak; {us_step * steps_in_graph / len(calls):.2f} us per call, plans {plans}")
+
+    # ---- C3: Whisper large-v3 decoder step, beam 5 ----
+    D, H, L = 64, 20, 32
+    n_state = D * H
+    Lk, Nenc = 224, 1500
+    mask = np.zeros((5, 1, 1, Lk), np.float32)
+    for b in range(5):
+        mask[b, 0, 0, ora.randint(31, b, 1, Lk):] = -np.inf
+    mask_d = ca.Tensor.from_host(ora.fp32_to_fp16(mask), ca.F16, (Lk, 1, 1, 5))
+    calls = []
+    for l in range(L):
+        nbs = (2, 2 * n_state, 2 * D, 2 * n_state * Lk)
+        calls.append({"q": ca.Tensor(torch.randn(5 * n_state, device="cuda").view(torch.uint8), ca.F32, (D, 1, H, 5),
+                                     (4, 4 * n_state, 4 * D, 4 * n_state)),
+                      "k": ca.Tensor(f16_buf(5 * Lk * n_state), ca.F16, (D, Lk, H, 5), nbs),
+                      "v": ca.Tensor(f16_buf(5 * Lk * n_state), ca.F16, (D, Lk, H, 5), nbs),
+                      "mask": mask_d, "scale": 1.0, "out": ca.Tensor.empty(ca.F32, (D, H, 1, 5))})
+        nbc = (2, 2 * n_state, 2 * D, 2 * n_state * Nenc)
+        calls.append({"q": ca.Tensor(torch.randn(5 * n_state, device="cuda").view(torch.uint8), ca.F32, (D, 5, H, 1),
+                                     (4, 4 * n_state, 4 * D, 4 * n_state * 5)),
+                      "k": ca.Tensor(f16_buf(Nenc * n_state), ca.F16, (D, Nenc, H, 1), nbc),
+                      "v": ca.Tensor(f16_buf(Nenc * n_state), ca.F16, (D, Nenc, H, 1), nbc),
+                      "scale": 64 ** -0.25, "out": ca.Tensor.empty(ca.F32, (D, H, 5, 1))})
+    b_self = 5 * (2 * Lk * n_state * 2 + 2 * n_state * 4 + Lk * 2)
+    b_cross = 2 * Nenc * n_state * 2 + 2 * 5 * n_state * 4
+    timed("C3_step", "BASELINE shape", calls, 1, L * (b_self + b_cross), 20,
+          "32 layers x (self: q [64,1,20,5] vs f16 K/V [64,224,20,5] + mask; cross: q [64,5,20,1] vs shared f16 K/V [64,1500,20,1])")
+    del calls
+
+    # ---- C4: Voxtral-style LLM decode step ----
+    D, Hq, Hkv, Lk, L, STEPS = 128, 32, 8, 663, 30, 8
+    rs = 136
+    nbk = (34, rs, rs * Lk, rs * Lk * Hkv)
+    calls = []
+    for l in range(L * STEPS):
+        calls.append({"q": ca.Tensor(torch.randn(Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, 1)),
+                      "k": ca.Tensor(q8_buf(900 + 2 * l, Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, 1), nbk),
+                      "v": ca.Tensor(q8_buf(901 + 2 * l, Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, 1), nbk),
+                      "scale": 128 ** -0.5, "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 1))})
+    per_call = 2 * Lk * Hkv * rs + 2 * Hq * D * 4
+    timed("C4_step", "BASELINE shape", calls, STEPS, L * per_call, 20,
+          "30 layers x (q [128,1,32,1] vs Q8_0 K/V [128,663,8,1], no mask); 8 steps' worth of distinct layers per replay (345 MB)")
+    del calls
+
+    # ---- ceilings: 64 sequences x 4096 entries per call ----
+    Lk = 4096
+    nbq = (34, rs, rs * Lk, rs * Lk * Hkv)
+    calls = [{"q": ca.Tensor(torch.randn(64 * Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, 64)),
+              "k": ca.Tensor(q8_buf(1100 + 2 * l, 64 * Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, 64), nbq),
+              "v": ca.Tensor(q8_buf(1101 + 2 * l, 64 * Hkv * Lk * D), ca.Q8_0, (D, Lk, Hkv, 64), nbq),
+              "scale": 128 ** -0.5, "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 64))} for l in range(2)]
+    timed("ceiling_q8_0_64seq_x4096", "ceiling", calls, 2, 64 * (2 * Lk * Hkv * rs + 2 * Hq * D * 4), 10,
+          "one call: 64 sequences x (32 q / 8 kv heads x 128) against 4096-entry Q8_0 caches; not a BASELINE configuration")
+    del calls
+    nbf = (2, 2 * D, 2 * D * Lk, 2 * D * Lk * Hkv)
+    calls = [{"q": ca.Tensor(torch.randn(64 * Hq * D, device="cuda").view(torch.uint8), ca.F32, (D, 1, Hq, 64)),
+              "k": ca.Tensor(f16_buf(64 * Hkv * Lk * D), ca.F16, (D, Lk, Hkv, 64), nbf),
+              "v": ca.Tensor(f16_buf(64 * Hkv * Lk * D), ca.F16, (D, Lk, Hkv, 64), nbf),
+              "scale": 128 ** -0.5, "out": ca.Tensor.empty(ca.F32, (D, Hq, 1, 64))} for l in range(2)]
+    timed("ceiling_f16_64seq_x4096", "ceiling", calls, 2, 64 * (2 * Lk * Hkv * D * 2 + 2 * Hq * D * 4), 10,
+          "one call: 64 sequences against 4096-entry f16 caches; not a BASELINE configuration")
+    del calls
+    return res
+
+
 def bench_host_resident(ca, ora, torch):
     """The same kernels with every tensor in pinned, GPU-mapped host memory (the is_host buffer type a backend
     that implements one op gives ggml, so that ggml-cpu keeps running the other ops on weights and caches):
@@ -569,7 +693,8 @@ def bench_relpos(ca, ora, torch, lengths):
     us_two = _time_calls(torch, lambda: ca.ggml.flash_attn_relpos(dqu, dqv, dk, dv, dr, da, scale, out=out,
                                                                    kernel=ca.ggml.KERNEL_MMA), 20)
     us_all = _time_calls(torch, lambda: ca.ggml.flash_attn_relpos(dqu, dqv, dk, dv, dr, da, scale, out=out), 20)
-    ws_one = ca.ggml.flash_attn_relpos_workspace_size(dqu, dqv, dk, dv, dr, da, scale)
+    # what the one-kernel form uses: f16 copies of K and V, then of the table (the size query itself answers for both forms)
+    ws_one = (2 * 2 * D * T * H * B + 255) // 256 * 256 + ca.ggml.relpos_bias_workspace_size(dr)
     got = out.numpy_f32()
     worst = [0.0, 0.0]
     for b in (0, B - 1):
@@ -731,6 +856,9 @@ def main():
     ap.add_argument("--no-decode", action="store_true")
     ap.add_argument("--no-scale-check", action="store_true", help="skip the half-size launches (keeps profiler means per kernel clean)")
     ap.add_argument("--no-configs", action="store_true", help="skip the other baseline configurations and the Whisper protocol")
+    ap.add_argument("--roofline-decode-only", action="store_true",
+                    help="run only the decode roofline entries (C3 step, C4 step, ceilings) and print them as the JSON line (profiling: "
+                         "every shape then has a (kernel, grid) pair of its own in the kernel trace)")
     ap.add_argument("--relpos-only", action="store_true",
                     help="run only the FastConformer rel-pos configuration and print its figures as the JSON line (profiling)")
     args = ap.parse_args()
@@ -750,6 +878,9 @@ def main():
     log(f"[bench] device {info['name']} {info['arch']} CUs={info['compute_units']} clock={info['clock_khz']} kHz; "
         f"roofline constants: f16 dense MFMA {PEAK_F16_TFLOPS} TFLOP/s, HBM {PEAK_HBM_GBS} GB/s")
 
+    if args.roofline_decode_only:
+        print(json.dumps({"roofline_decode": bench_roofline_decode(ca, ora, torch)}), flush=True)
+        return
     if args.relpos_only:
         lengths = [ora.randint(5, b, 400, 750) for b in range(8)]
         print(json.dumps({"config": "C5_fastconformer_relpos_f32", **bench_relpos(ca, ora, torch, lengths)}), flush=True)
@@ -770,6 +901,7 @@ def main():
     }
     line["copy_calibration"] = copy_calibration(ca, torch)
     if not args.no_decode:
+        line["roofline_decode"] = bench_roofline_decode(ca, ora, torch)
         line["decode"] = bench_decode(args, ca, ora, torch)
     if not args.no_configs:
         line["host_resident"] = bench_host_resident(ca, ora, torch)

@@ -154,7 +154,8 @@ struct Plan {
     int     keys_per_split;
     size_t  workspace;       // bytes in all: [f16 copies of K and V][split partials]
     size_t  ws_partials;     // offset of the split partials inside the workspace
-    bool    kv_to_f16;       // F32 K/V are converted to f16 in the workspace first (tile kernel only)
+    bool    kv_to_f16;       // K and V are rounded to f16 copies in the workspace first (F32 / quantised K/V before the tile kernel; a
+                             // K and a V of different types before any kernel)
 };
 
 int check(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
@@ -165,7 +166,7 @@ int check(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor 
         return fail(MI355X_ERR_INVALID, "negative or oversized extent");
     if (q->type != MI355X_TYPE_F32) return fail(MI355X_ERR_UNSUPPORTED, "q must be F32 (type %d)", q->type);
     if (!type_size(k->type)) return fail(MI355X_ERR_UNSUPPORTED, "K type %d not covered", k->type);
-    if (k->type != v->type) return fail(MI355X_ERR_UNSUPPORTED, "K and V types differ (%d, %d)", k->type, v->type);
+    if (!type_size(v->type)) return fail(MI355X_ERR_UNSUPPORTED, "V type %d not covered", v->type);
 
     const int64_t D = q->ne[0], Nq = q->ne[1], Hq = q->ne[2], B = q->ne[3];
     const int64_t Nkv = k->ne[1], Hkv = k->ne[2], Bk = k->ne[3];
@@ -174,16 +175,16 @@ int check(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor 
     if (Hkv <= 0 || Bk <= 0 || Hq % Hkv || B % Bk) return fail(MI355X_ERR_INVALID, "q heads/batch not a multiple of kv heads/batch");
     if (v->ne[0] != D) return fail(MI355X_ERR_UNSUPPORTED, "DV %lld != DK %lld", (long long)v->ne[0], (long long)D);
     if (D <= 0 || D % 8 || D > 256) return fail(MI355X_ERR_UNSUPPORTED, "head size %lld (need a multiple of 8, <= 256)", (long long)D);
-    if (FATTN_IS_BLOCK_TYPE(k->type) && D % FATTN_QK8_0) return fail(MI355X_ERR_INVALID, "quantised rows need D %% 32 == 0");
+    if ((FATTN_IS_BLOCK_TYPE(k->type) || FATTN_IS_BLOCK_TYPE(v->type)) && D % FATTN_QK8_0) return fail(MI355X_ERR_INVALID, "quantised rows need D %% 32 == 0");
     if (Nq < 0 || Nkv < 0 || Hq <= 0 || B <= 0) return fail(MI355X_ERR_INVALID, "negative or zero extent");
     if (q->nb[0] != 4) return fail(MI355X_ERR_UNSUPPORTED, "q rows must be contiguous (nb0 = %zu)", q->nb[0]);
     if (k->nb[0] != type_size(k->type) || v->nb[0] != type_size(v->type))
         return fail(MI355X_ERR_UNSUPPORTED, "k/v rows must be contiguous");
-    const size_t al = k->type == MI355X_TYPE_F32 ? 4 : 2;
+    const size_t alk = k->type == MI355X_TYPE_F32 ? 4 : 2, alv = v->type == MI355X_TYPE_F32 ? 4 : 2;
     for (int i = 1; i < 4; i++) {
-        if (q->nb[i] % 4 || k->nb[i] % al || v->nb[i] % al) return fail(MI355X_ERR_UNSUPPORTED, "misaligned strides");
+        if (q->nb[i] % 4 || k->nb[i] % alk || v->nb[i] % alv) return fail(MI355X_ERR_UNSUPPORTED, "misaligned strides");
     }
-    if (((uintptr_t)q->data % 4) || ((uintptr_t)k->data % al) || ((uintptr_t)v->data % al))
+    if (((uintptr_t)q->data % 4) || ((uintptr_t)k->data % alk) || ((uintptr_t)v->data % alv))
         return fail(MI355X_ERR_UNSUPPORTED, "misaligned data pointers");
     if (has_mask(mask)) {
         if (mask->type != MI355X_TYPE_F16) return fail(MI355X_ERR_UNSUPPORTED, "mask must be F16 (type %d)", mask->type);
@@ -275,7 +276,15 @@ void use_f16_copies(FattnArgs & a, void * ws) {
     a.aligned16 = a.q_aligned16;
 }
 
-void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Plan & plan) {
+// A K and a V of different storage types (CRISPASR_KV_QUANT_K / _V, src/core/attention.h:132-137) are both rounded to f16
+// copies first, whatever the kernel: the call is then planned and run as an F16 one.
+void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_params * p, Plan & plan) {
+    FattnArgs a = a0;
+    const bool mixed = ktype != vtype;
+    if (mixed) {
+        use_f16_copies(a, nullptr);
+        ktype = MI355X_TYPE_F16;
+    }
     int kernel = p->kernel;
     if (kernel == MI355X_FATTN_AUTO) {
         // The decode kernel takes the Nq * gqa rows that share a KV head 16 at a time, each chunk streaming the head's K/V
@@ -312,7 +321,7 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
     // touching registers) read the result: same values, same rounding.
     plan.ws_partials = 0;
     const bool convertible = (ktype == MI355X_TYPE_F32 && a.kv_aligned16) || (ktype == MI355X_TYPE_Q8_0 && a.kv_aligned2);
-    if (kernel == MI355X_FATTN_MMA && ((convertible && a.Nq >= 128) || narrow_quant(ktype))) {
+    if (mixed || (kernel == MI355X_FATTN_MMA && ((convertible && a.Nq >= 128) || narrow_quant(ktype)))) {
         plan.kv_to_f16 = true;
         plan.workspace = ((size_t)2 * a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t) + 255) / 256 * 256;
         plan.ws_partials = plan.workspace;
@@ -327,7 +336,7 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
         const int64_t rows    = (int64_t)a.Nq * a.Hq * a.B;
         FattnArgs b  = a;
         int       kt = ktype;
-        if (plan.kv_to_f16) {
+        if (plan.kv_to_f16 && !mixed) {
             use_f16_copies(b, nullptr);
             kt = MI355X_TYPE_F16;
         }
@@ -385,7 +394,7 @@ void make_plan(const FattnArgs & a, int ktype, const mi355x_fattn_params * p, Pl
         ns = a.Nkv > 0 ? (a.Nkv + kps - 1) / kps : 1;
         plan.n_splits = ns;
         plan.keys_per_split = a.Nkv > 0 ? kps : 0;
-        if (ns > 1) plan.workspace = (size_t)rows * ns * (a.D + 2) * sizeof(float);
+        if (ns > 1) plan.workspace += (size_t)rows * ns * (a.D + 2) * sizeof(float);
     }
 }
 
@@ -485,8 +494,12 @@ int mi355x_device_get_info(int device, mi355x_device_info * info) {
 
 int mi355x_set_device(int device) {
     HIP_TRY(hipSetDevice(device));
+    // Set-up of mi355x_flash_attn_ext_noalloc for this device happens here when the caller comes this way - as a courtesy:
+    // a failed lookup must not cost the caller the device (most never use that entry point, which reports the failure itself
+    // on its first call).
     void * ptr = nullptr;
-    return noalloc_scratch(&ptr);      // set-up of mi355x_flash_attn_ext_noalloc for this device happens here when the caller comes this way
+    if (noalloc_scratch(&ptr) != MI355X_OK) g_err[0] = 0;
+    return MI355X_OK;
 }
 
 int mi355x_stream_synchronize(void * stream) {
@@ -508,7 +521,7 @@ int mi355x_fattn_plan(const mi355x_tensor * q, const mi355x_tensor * k, const mi
     FattnArgs a;
     fill_args(a, q, k, v, mask, nullptr, params);
     Plan plan;
-    make_plan(a, k->type, params, plan);
+    make_plan(a, k->type, v->type, params, plan);
     if (kernel) *kernel = plan.kernel;
     if (n_splits) *n_splits = plan.n_splits;
     return MI355X_OK;
@@ -523,19 +536,21 @@ int mi355x_fattn_plan_details(const mi355x_tensor * q, const mi355x_tensor * k, 
     FattnArgs a;
     fill_args(a, q, k, v, mask, nullptr, params);
     Plan plan;
-    make_plan(a, k->type, params, plan);
+    make_plan(a, k->type, v->type, params, plan);
     memset(info, 0, sizeof(*info));
     info->kernel         = plan.kernel;
     info->n_splits       = plan.n_splits;
     info->keys_per_split = plan.keys_per_split;
     info->kv_to_f16      = plan.kv_to_f16 ? 1 : 0;
     info->workspace      = plan.workspace;
-    if (plan.kernel == MI355X_FATTN_MMA && fattn_mma_supported(a, k->type)) {
+    if (plan.kernel == MI355X_FATTN_MMA) {
+        // the order of the call itself: the f16 copies first, then the question whether the tile kernel takes the shape
         int ktype = k->type;
         if (plan.kv_to_f16) {
             use_f16_copies(a, nullptr);
             ktype = MI355X_TYPE_F16;
         }
+        if (!fattn_mma_supported(a, ktype)) return MI355X_OK;
         a.n_splits = plan.n_splits;
         a.keys_per_split = plan.keys_per_split;
         FattnMmaVariant var;
@@ -558,7 +573,7 @@ int mi355x_fattn_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k
     FattnArgs a;
     fill_args(a, q, k, v, mask, nullptr, params);
     Plan plan;
-    make_plan(a, k->type, params, plan);
+    make_plan(a, k->type, v->type, params, plan);
     *bytes = plan.workspace + (params->q_quant ? qq_q8_bytes(q) + qq_f32_bytes(q) : 0);
     return MI355X_OK;
 }
@@ -601,74 +616,52 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     if ((int64_t)a.Nq * a.Hq * a.B == 0) return MI355X_OK;
 
     Plan plan;
-    make_plan(a, k->type, params, plan);
+    make_plan(a, k->type, v->type, params, plan);
     hipStream_t st = (hipStream_t)stream;
 
+    int ktype = k->type;
     if (plan.kernel == MI355X_FATTN_MMA) {
-        {
-            FattnArgs b = a;
-            if (plan.kv_to_f16) use_f16_copies(b, nullptr);
-            if (!fattn_mma_supported(b, plan.kv_to_f16 ? MI355X_TYPE_F16 : k->type))
-                return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the MFMA kernel");
-        }
-        int ktype = k->type;
-        void * ws = nullptr;
-        if (plan.workspace) {
-            ws = params->workspace;
-            if (ws) {
-                if (params->workspace_size < plan.workspace)
-                    return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, plan.workspace);
-                if ((uintptr_t)ws % 16) return fail(MI355X_ERR_WORKSPACE, "workspace must be 16-byte aligned");
-            } else {
-                rc = get_scratch(plan.workspace, &ws, (hipStream_t)stream);
-                if (rc) return rc;
-            }
-        }
-        if (plan.kv_to_f16) {
-            const int e = kv_to_f16_launch(a, k->type, ws, st);
-            if (e) return hip_fail((hipError_t)e, "K/V conversion launch");
-            use_f16_copies(a, ws);
-            ktype = MI355X_TYPE_F16;
-        }
-        a.n_splits = plan.n_splits;
-        a.keys_per_split = plan.keys_per_split;
-        if (plan.n_splits > 1) {
-            const size_t rows = (size_t)a.Nq * a.Hq * a.B;
-            a.part_acc = (float *)((char *)ws + plan.ws_partials);
-            a.part_ml  = a.part_acc + rows * plan.n_splits * a.D;
-        }
-        int e = fattn_mma_launch(a, ktype, st);
-        if (e) return hip_fail((hipError_t)e, "fattn_mma launch");
-        if (plan.n_splits > 1) {
-            e = fattn_merge_launch(a, st);
-            if (e) return hip_fail((hipError_t)e, "fattn_merge launch");
-        }
-        return MI355X_OK;
-    }
-    if (plan.kernel == MI355X_FATTN_DECODE_MMA) {
-        if (!fattn_decode_supported(a, k->type)) return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the decode kernel");
+        FattnArgs b = a;
+        if (plan.kv_to_f16) use_f16_copies(b, nullptr);
+        if (!fattn_mma_supported(b, plan.kv_to_f16 ? MI355X_TYPE_F16 : ktype))
+            return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the MFMA kernel");
+    } else if (plan.kernel == MI355X_FATTN_DECODE_MMA) {
+        FattnArgs b = a;
+        if (plan.kv_to_f16) use_f16_copies(b, nullptr);
+        if (!fattn_decode_supported(b, plan.kv_to_f16 ? MI355X_TYPE_F16 : ktype))
+            return fail(MI355X_ERR_UNSUPPORTED, "shape not covered by the decode kernel");
     } else if (plan.kernel != MI355X_FATTN_VEC) {
         return fail(MI355X_ERR_UNSUPPORTED, "kernel %d not available", plan.kernel);
     }
-
-    a.n_splits = plan.n_splits;
-    a.keys_per_split = plan.keys_per_split;
-    if (plan.n_splits > 1) {
-        void * ws = params->workspace;
+    void * ws = nullptr;
+    if (plan.workspace) {
+        ws = params->workspace;
         if (ws) {
             if (params->workspace_size < plan.workspace)
                 return fail(MI355X_ERR_WORKSPACE, "workspace %zu < %zu bytes", params->workspace_size, plan.workspace);
             if ((uintptr_t)ws % 16) return fail(MI355X_ERR_WORKSPACE, "workspace must be 16-byte aligned");
         } else {
-            rc = get_scratch(plan.workspace, &ws, (hipStream_t)stream);
+            rc = get_scratch(plan.workspace, &ws, st);
             if (rc) return rc;
         }
+    }
+    if (plan.kv_to_f16) {
+        const int e = kv_to_f16_launch(a, k->type, v->type, ws, st);
+        if (e) return hip_fail((hipError_t)e, "K/V conversion launch");
+        use_f16_copies(a, ws);
+        ktype = MI355X_TYPE_F16;
+    }
+    a.n_splits = plan.n_splits;
+    a.keys_per_split = plan.keys_per_split;
+    if (plan.n_splits > 1) {
         const size_t rows = (size_t)a.Nq * a.Hq * a.B;
-        a.part_acc = (float *)ws;
+        a.part_acc = (float *)((char *)ws + plan.ws_partials);
         a.part_ml  = a.part_acc + rows * plan.n_splits * a.D;
     }
-    int e = plan.kernel == MI355X_FATTN_VEC ? fattn_vec_launch(a, k->type, st) : fattn_decode_launch(a, k->type, st);
-    if (e) return hip_fail((hipError_t)e, "split-KV kernel launch");
+    int e = plan.kernel == MI355X_FATTN_MMA   ? fattn_mma_launch(a, ktype, st)
+            : plan.kernel == MI355X_FATTN_VEC ? fattn_vec_launch(a, ktype, st)
+                                              : fattn_decode_launch(a, ktype, st);
+    if (e) return hip_fail((hipError_t)e, "attention kernel launch");
     if (plan.n_splits > 1) {
         e = fattn_merge_launch(a, st);
         if (e) return hip_fail((hipError_t)e, "fattn_merge launch");
@@ -880,7 +873,7 @@ static int relpos_fused_check(const mi355x_tensor * q_u, const mi355x_tensor * q
     FattnArgs a;
     fill_args(a, q_u, k, v, m, nullptr, params);
     Plan plan;
-    make_plan(a, k->type, params, plan);
+    make_plan(a, k->type, v->type, params, plan);
     *inner_bytes = plan.workspace;
     return MI355X_OK;
 }
@@ -907,9 +900,9 @@ static RelposFused relpos_fused_plan(const mi355x_tensor * q_u, const mi355x_ten
         const size_t es = type_size(add->type);
         if (add->nb[0] != es) return f;
     }
-    if (k->type == MI355X_TYPE_F16 && a.kv_aligned16) {
+    if (k->type == MI355X_TYPE_F16 && v->type == MI355X_TYPE_F16 && a.kv_aligned16) {
         f.kv_copy = false;
-    } else if ((k->type == MI355X_TYPE_F32 && a.kv_aligned16) || (FATTN_IS_BLOCK_TYPE(k->type) && a.kv_aligned2)) {
+    } else if (k->type != v->type || (k->type == MI355X_TYPE_F32 && a.kv_aligned16) || (FATTN_IS_BLOCK_TYPE(k->type) && a.kv_aligned2)) {
         f.kv_copy  = true;
         f.kv_bytes = ((size_t)2 * a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t) + 255) / 256 * 256;
     } else {
@@ -938,7 +931,7 @@ static int relpos_fused_run(const mi355x_tensor * q_u, const mi355x_tensor * q_v
     if (f.kv_copy) {
         F32Rider x;
         memset(&x, 0, sizeof(x));
-        if (f.table_bytes && r->type == MI355X_TYPE_F32 && aligned16_view(r)) {
+        if (f.table_bytes && r->type == MI355X_TYPE_F32 && aligned16_view(r) && k->type == v->type) {
             x.src = (const char *)r->data;
             x.dst = (char *)ws + f.kv_bytes;
             x.ne1 = r->ne[1]; x.ne2 = r->ne[2];
@@ -946,7 +939,7 @@ static int relpos_fused_run(const mi355x_tensor * q_u, const mi355x_tensor * q_v
             x.n   = (int64_t)(a.D / 8) * r->ne[1] * r->ne[2] * r->ne[3];
             table_done = true;
         }
-        const int e = kv_to_f16_launch(a, k->type, ws, st, table_done ? &x : nullptr);
+        const int e = kv_to_f16_launch(a, k->type, v->type, ws, st, table_done ? &x : nullptr);
         if (e) return hip_fail((hipError_t)e, "K/V conversion launch");
         use_f16_copies(a, ws);
     }
@@ -1005,8 +998,11 @@ int mi355x_fattn_relpos_workspace_size(const mi355x_tensor * q_u, const mi355x_t
     size_t mb = 0, ib = 0;
     const int rc = relpos_fused_check(q_u, q_v, k, v, r, add, nullptr, params, &m, &mb, &ib);
     if (rc) return rc;
+    // Which form a call takes depends on the alignment of its data pointers, and a size query may come before those exist
+    // (NULL looks aligned): the answer covers both forms, so that a workspace of this size never turns out too small.
     const RelposFused f = relpos_fused_plan(q_u, q_v, k, v, r, add, params);
-    *bytes = f.ok ? f.kv_bytes + f.table_bytes : mb + ib;
+    const size_t one = f.kv_bytes + f.table_bytes, two = mb + ib;
+    *bytes = f.ok && one > two ? one : two;
     return MI355X_OK;
 }
 

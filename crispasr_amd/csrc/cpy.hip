@@ -237,6 +237,47 @@ __global__ void __launch_bounds__(256) kv_to_f16_kernel(const FattnArgs a, char 
     *(h8 *)(dst + ((is_v ? half : 0) + i) * 16) = y;
 }
 
+// The same for a K and a V of different storage types (CRISPASR_KV_QUANT_K / _V, src/core/attention.h:132-137; the
+// Canary decoder hands both cache views to the op as they are, src/canary.cpp:953-972): the type is looked up per
+// tensor at run time.  Scalar loads: such rows are only as aligned as their type.
+__global__ void __launch_bounds__(256) kv_to_f16_mixed_kernel(const FattnArgs a, const int ktype, const int vtype, char * dst) {
+    const int     cpr  = a.D / 8;
+    const int64_t half = (int64_t)cpr * a.Nkv * a.Hkv * a.Bk;
+    int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= 2 * half) return;
+    const bool is_v = i >= half;
+    if (is_v) i -= half;
+    const int     c = (int)(i % cpr);
+    int64_t       r = i / cpr;
+    const int64_t j = r % a.Nkv;  r /= a.Nkv;
+    const int64_t h = r % a.Hkv;
+    const int64_t b = r / a.Hkv;
+    const char * row = is_v ? a.v + j * a.nbv1 + h * a.nbv2 + b * a.nbv3
+                            : a.k + j * a.nbk1 + h * a.nbk2 + b * a.nbk3;
+    float f[8];
+    const char * blk = row + (c >> 2) * fattn_block_bytes(is_v ? vtype : ktype);
+    switch (is_v ? vtype : ktype) {
+        case MI355X_TYPE_F32:
+#pragma unroll
+            for (int e = 0; e < 8; e++) f[e] = ((const float *)row)[c * 8 + e];
+            break;
+        case MI355X_TYPE_F16:
+#pragma unroll
+            for (int e = 0; e < 8; e++) f[e] = h2f_bits(((const uint16_t *)row)[c * 8 + e]);
+            break;
+        case MI355X_TYPE_Q8_0: dequant8<MI355X_TYPE_Q8_0>(blk, (c & 3) * 8, f); break;
+        case MI355X_TYPE_Q4_0: dequant8<MI355X_TYPE_Q4_0>(blk, (c & 3) * 8, f); break;
+        case MI355X_TYPE_Q4_1: dequant8<MI355X_TYPE_Q4_1>(blk, (c & 3) * 8, f); break;
+        case MI355X_TYPE_Q5_0: dequant8<MI355X_TYPE_Q5_0>(blk, (c & 3) * 8, f); break;
+        default:               dequant8<MI355X_TYPE_Q5_1>(blk, (c & 3) * 8, f); break;
+    }
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    h8 y;
+#pragma unroll
+    for (int e = 0; e < 8; e++) y[e] = (_Float16)f[e];
+    *(h8 *)(dst + ((is_v ? half : 0) + i) * 16) = y;
+}
+
 // memset as a kernel: a memset node recorded into a captured graph is what a fill kernel avoids.
 // 16-byte stores over the aligned middle, single bytes for the (< 16-byte) head and tail.
 __global__ void __launch_bounds__(256) fill_kernel(unsigned char * p, unsigned value, size_t head, size_t n16, size_t tail) {
@@ -263,7 +304,7 @@ int fill_launch(void * ptr, int value, size_t size, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
-int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t stream, const F32Rider * rider) {
+int kv_to_f16_launch(const FattnArgs & a, int ktype, int vtype, void * dst, hipStream_t stream, const F32Rider * rider) {
     F32Rider x;
     memset(&x, 0, sizeof(x));
     if (rider) x = *rider;
@@ -271,6 +312,11 @@ int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t str
     if (n == 0) return 0;
     if ((n + 255) / 256 > 0x7fffffff) return (int)hipErrorInvalidValue;
     const unsigned g = (unsigned)((n + 255) / 256);
+    if (ktype != vtype) {
+        if (rider) return (int)hipErrorInvalidValue;
+        hipLaunchKernelGGL(kv_to_f16_mixed_kernel, dim3(g), dim3(256), 0, stream, a, ktype, vtype, (char *)dst);
+        return (int)hipGetLastError();
+    }
     switch (ktype) {
 #define KV16(T) case T: hipLaunchKernelGGL((kv_to_f16_kernel<T>), dim3(g), dim3(256), 0, stream, a, (char *)dst, x); break
         KV16(MI355X_TYPE_F32);

@@ -250,15 +250,16 @@ bool fattn_decode_supported(const FattnArgs & a, int ktype);
 int cpy_launch(const CpyArgs & a, int stype, int dtype, hipStream_t stream);
 int set_rows_launch(const CpyArgs & a, int dtype, hipStream_t stream);
 int fill_launch(void * ptr, int value, size_t size, hipStream_t stream);      // memset by a kernel
-// K and V (F32 or Q8_0, any strides) -> contiguous f16 [D, Nkv, Hkv, Bk] at dst and right behind it
 int relpos_bias_launch(RelposArgs a, int rtype, hipStream_t stream);
 int fattn_relpos_launch(const FattnRelposArgs & a, hipStream_t stream);
 bool fattn_relpos_supported(const FattnRelposArgs & a);
 // an F32 tensor [D, ne1, ne2, ne3] (D = the attention call's head size, rows 16-byte aligned) converted to a contiguous f16
 // copy by the same launch; n = its 8-element chunks
+// (kv_to_f16_launch: K and V, of any storage type each and any strides, -> contiguous f16 [D, Nkv, Hkv, Bk] at dst and right
+//  behind it; the rider only beside a K and V of one type)
 struct F32Rider {
     const char * src;
     char *       dst;
     int64_t ne1, ne2, nb1, nb2, nb3, n;
 };
-int kv_to_f16_launch(const FattnArgs & a, int ktype, void * dst, hipStream_t stream, const F32Rider * rider = nullptr);
+int kv_to_f16_launch(const FattnArgs & a, int ktype, int vtype, void * dst, hipStream_t stream, const F32Rider * rider = nullptr);

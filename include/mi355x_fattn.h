@@ -132,7 +132,8 @@ int mi355x_stream_synchronize(void * stream);
  *
  *   q    F32  [D,  Nq,  Hq,  B ]   any strides with nb[0] == 4
  *   k    F16 | F32 | Q8_0 | Q4_0 | Q4_1 | Q5_0 | Q5_1 [D,  Nkv, Hkv, Bk]   rows contiguous (nb[0] == type size)
- *   v    same type as k   [DV, Nkv, Hkv, Bk]   DV == D
+ *   v    any of k's types [DV, Nkv, Hkv, Bk]   DV == D.  A V of another type than K's (CRISPASR_KV_QUANT_K / _V,
+ *        src/core/attention.h:132-137) costs one conversion of both to f16 copies in the workspace before the kernel.
  *        (Q4_0 .. Q5_1: up to 16 query rows per KV head read the blocks in the decode kernel (head sizes 64 and 128, no
  *         soft cap; other shapes in the vector kernel); more rows go through one conversion of K and V to f16 in the
  *         workspace and the tile kernel)
@@ -254,7 +255,8 @@ int mi355x_relpos_bias(const mi355x_tensor * q_v, const mi355x_tensor * r, const
 int mi355x_flash_attn_relpos(const mi355x_tensor * q_u, const mi355x_tensor * q_v, const mi355x_tensor * k,
                              const mi355x_tensor * v, const mi355x_tensor * r, const mi355x_tensor * add,
                              const mi355x_tensor * dst, const mi355x_fattn_params * params, void * stream);
-/* bytes of workspace the call above uses (the mask plus what the attention call itself needs) */
+/* bytes of workspace that are enough for the call above in either form (the larger of the two needs: which form a call takes
+ * depends on the alignment of its data pointers, which a size query made before allocation cannot know) */
 int mi355x_fattn_relpos_workspace_size(const mi355x_tensor * q_u, const mi355x_tensor * q_v, const mi355x_tensor * k,
                                        const mi355x_tensor * v, const mi355x_tensor * r, const mi355x_tensor * add,
                                        const mi355x_fattn_params * params, size_t * bytes);

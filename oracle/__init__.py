@@ -21,7 +21,7 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 
 F32, F16, Q4_0, Q4_1, Q5_0, Q5_1, Q8_0 = 0, 1, 2, 3, 6, 7, 8
 BLOCK_TYPES = (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0)
-MODE_EXACT, MODE_GGML_LIKE, MODE_GGML_LIKE_F16_ACC = 0, 1, 2
+MODE_EXACT, MODE_GGML_LIKE = 0, 1
 ROUND_NEAREST_EVEN, ROUND_HALF_AWAY = 0, 1
 QK8_0 = 32
 BLOCK_Q8_0_BYTES = 34

@@ -409,11 +409,10 @@ static void fa_row_exact(const fa_args * a, int64_t iq1, int64_t iq2, int64_t iq
  * F32 for F32/F16 K in the fork (tools/upstream-prs/01-cpu-f16-saturation.md:17-23), Q8_0 for Q8_0 K,
  * the row quantiser and the block dot product being the ones the reference's note
  * tools/upstream-prs/09-metal-q8_0-bit-match.md:24-36 writes down; that FLASH_ATTN_EXT routes a Q8_0 K
- * through them is recalled.  f16_acc (ORA_MODE_GGML_LIKE_F16_ACC only): the P.V accumulator is kept in
- * fp16 when V is F16 - recalled, held by nothing in the reference's tree: a diagnostic, PARITY UNPINNED,
- * no test asserts against it. */
+ * through them is recalled.  K of the narrower block types is not taken in this mode (ggml-cpu's integer block dot
+ * products for them are written down nowhere in the reference's tree): the entry point refuses it. */
 static void fa_row_ggml_like(const fa_args * a, int64_t iq1, int64_t iq2, int64_t iq3,
-                             float * tmp, float * acc32, uint16_t * acc16, ora_block_q8_0 * qq, int f16_acc) {
+                             float * tmp, float * acc32, ora_block_q8_0 * qq) {
     const int64_t ik2 = iq2 / (a->Hq / a->Hkv);
     const int64_t ik3 = iq3 / (a->B / a->Bk);
     const float * qrow = (const float *)row_ptr(a->q, iq1, iq2, iq3);
@@ -429,17 +428,12 @@ static void fa_row_ggml_like(const fa_args * a, int64_t iq1, int64_t iq2, int64_
     const int     vtype  = a->v->type;
     const int64_t D      = a->D;
     const int64_t DV     = a->DV;
-    const int     v_f16  = f16_acc && vtype == ORA_TYPE_F16;
 
-    float qdq[512];
-    if (ktype == ORA_TYPE_Q8_0 || ora_block_bytes(ktype)) {
-        ora_quantize_row_q8_0(qrow, qq, D, ORA_ROUND_NEAREST_EVEN);
-        ora_dequantize_row_q8_0(qq, qdq, D);
-    }
+    if (ktype == ORA_TYPE_Q8_0) ora_quantize_row_q8_0(qrow, qq, D, ORA_ROUND_NEAREST_EVEN);
 
     float S = 0.0f;
     float M = -INFINITY;
-    if (v_f16) memset(acc16, 0, (size_t)DV * 2); else memset(acc32, 0, (size_t)DV * 4);
+    memset(acc32, 0, (size_t)DV * 4);
 
     for (int64_t j = 0; j < a->Nkv; j++) {
         const float mv = mrow ? slope * h2f(mrow[j]) : 0.0f;
@@ -468,15 +462,8 @@ static void fa_row_ggml_like(const fa_args * a, int64_t iq1, int64_t iq2, int64_
 #else
             for (int64_t d = 0; d < D; d++) s += h2f(kh[d]) * qrow[d];
 #endif
-        } else if (ktype == ORA_TYPE_Q8_0) {
-            s = vec_dot_q8_0_q8_0((const ora_block_q8_0 *)kp, qq, D);
         } else {
-            /* Q4_0 .. Q5_1: the rounded query row against the dequantised key row, summed in f32 in element order.
-             * ggml-cpu's integer block dot products for these types are not written down anywhere in the reference's
-             * tree: this stands in for them as a diagnostic, PARITY UNPINNED. */
-            float kf[512];
-            ora_dequantize_row(ktype, kp, kf, D);
-            for (int64_t d = 0; d < D; d++) s += kf[d] * qdq[d];
+            s = vec_dot_q8_0_q8_0((const ora_block_q8_0 *)kp, qq, D);
         }
         s *= scale;
         if (a->softcap != 0.0f) s = a->softcap * tanhf(s);
@@ -485,37 +472,22 @@ static void fa_row_ggml_like(const fa_args * a, int64_t iq1, int64_t iq2, int64_
         const float Mold = M;
         float ms = 1.0f, vs = 1.0f;
         const char * vp = row_ptr(a->v, j, ik2, ik3);
-        if (v_f16) {
-            const uint16_t * vh = (const uint16_t *)vp;
-            if (s > M) {
-                M  = s;
-                ms = expf(Mold - M);
-                for (int64_t d = 0; d < DV; d++) acc16[d] = f2h(h2f(acc16[d]) * ms);
-            } else {
-                vs = expf(s - M);
-            }
-            for (int64_t d = 0; d < DV; d++) acc16[d] = f2h(h2f(acc16[d]) + h2f(vh[d]) * vs);
+        if (s > M) {
+            M  = s;
+            ms = expf(Mold - M);
+            for (int64_t d = 0; d < DV; d++) acc32[d] *= ms;
         } else {
-            if (s > M) {
-                M  = s;
-                ms = expf(Mold - M);
-                for (int64_t d = 0; d < DV; d++) acc32[d] *= ms;
-            } else {
-                vs = expf(s - M);
-            }
-            const float * vf;
-            if (vtype == ORA_TYPE_F32) {
-                vf = (const float *)vp;
-            } else {
-                row_to_f32(vp, vtype, DV, tmp);
-                vf = tmp;
-            }
-            for (int64_t d = 0; d < DV; d++) acc32[d] += vf[d] * vs;
+            vs = expf(s - M);
         }
+        const float * vf;
+        if (vtype == ORA_TYPE_F32) {
+            vf = (const float *)vp;
+        } else {
+            row_to_f32(vp, vtype, DV, tmp);
+            vf = tmp;
+        }
+        for (int64_t d = 0; d < DV; d++) acc32[d] += vf[d] * vs;
         S = S * ms + vs;
-    }
-    if (v_f16) {
-        for (int64_t d = 0; d < DV; d++) acc32[d] = h2f(acc16[d]);
     }
     const float S_inv = S == 0.0f ? 0.0f : 1.0f / S;
     float * out = a->dst + ((iq3 * a->Nq + iq1) * a->Hq + iq2) * a->DV;
@@ -549,6 +521,10 @@ int ora_flash_attn_ext(const ora_tensor * q, const ora_tensor * k, const ora_ten
     }
     if (max_bias > 0.0f && !mask) return -5;
     if (q->nb[0] != 4) return -6;
+    if (mode != ORA_MODE_EXACT && mode != ORA_MODE_GGML_LIKE) return -7;
+    /* ggml-like mode takes K as F32, F16 or Q8_0: nothing in the reference's tree says how ggml-cpu multiplies a query row
+     * with Q4_0 .. Q5_1 blocks */
+    if (mode == ORA_MODE_GGML_LIKE && ora_block_bytes(k->type) && k->type != ORA_TYPE_Q8_0) return -7;
 
     const int64_t n_rows = a.Nq * a.Hq * a.B;
     int nt = n_threads > 0 ? n_threads : 1;
@@ -563,7 +539,6 @@ int ora_flash_attn_ext(const ora_tensor * q, const ora_tensor * k, const ora_ten
         double *        acc   = (double *)malloc((size_t)Dm * 8);
         float *         tmp   = (float *)malloc((size_t)Dm * 4);
         float *         acc32 = (float *)malloc((size_t)Dm * 4);
-        uint16_t *      acc16 = (uint16_t *)malloc((size_t)Dm * 2);
         ora_block_q8_0 * qq   = (ora_block_q8_0 *)malloc(sizeof(ora_block_q8_0) * (size_t)(a.D / ORA_QK8_0 + 1));
 #pragma omp for schedule(dynamic, 16)
         for (int64_t ir = 0; ir < n_rows; ir++) {
@@ -573,10 +548,10 @@ int ora_flash_attn_ext(const ora_tensor * q, const ora_tensor * k, const ora_ten
             if (mode == ORA_MODE_EXACT) {
                 fa_row_exact(&a, iq1, iq2, iq3, s, tmp, acc);
             } else {
-                fa_row_ggml_like(&a, iq1, iq2, iq3, tmp, acc32, acc16, qq, mode == ORA_MODE_GGML_LIKE_F16_ACC);
+                fa_row_ggml_like(&a, iq1, iq2, iq3, tmp, acc32, qq);
             }
         }
-        free(s); free(acc); free(tmp); free(acc32); free(acc16); free(qq);
+        free(s); free(acc); free(tmp); free(acc32); free(qq);
     }
     return 0;
 }

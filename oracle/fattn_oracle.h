@@ -31,9 +31,6 @@
  *       Q8_0 K, f32 accumulator) : the recurrence is the reference's own (src/core/cpu_attention.h:53-83, compiled
  *       into oracle/_ref/ and compared where its tree is present); that the op quantises Q for a Q8_0 K is
  *       recalled.  logit_softcap is pinned by its closed form only.
- *   ora_flash_attn_ext, mode ORA_MODE_GGML_LIKE_F16_ACC (the same with the P.V accumulator rounded to fp16 at
- *       every key when V is F16) : PARITY UNPINNED - recalled behaviour of ggml-cpu that no file, test or
- *       fixture of the reference holds.  A diagnostic: reported by the benchmark, asserted by no test.
  *   ora_relpos_bias : pinned by the reference's own graph (src/core/fastconformer.h:98-102,
  *       876-918, every node of which is restated literally, the rel_shift view as byte strides)
  *       and by the mathematics: numpy matmul + numpy.lib.stride_tricks.as_strided with the
@@ -52,7 +49,7 @@ extern "C" {
 /* ggml type ids of the types this path meets */
 enum { ORA_TYPE_F32 = 0, ORA_TYPE_F16 = 1, ORA_TYPE_Q4_0 = 2, ORA_TYPE_Q4_1 = 3, ORA_TYPE_Q5_0 = 6, ORA_TYPE_Q5_1 = 7, ORA_TYPE_Q8_0 = 8 };
 
-enum { ORA_MODE_EXACT = 0, ORA_MODE_GGML_LIKE = 1, ORA_MODE_GGML_LIKE_F16_ACC = 2 };
+enum { ORA_MODE_EXACT = 0, ORA_MODE_GGML_LIKE = 1 };
 
 /* rounding of x/d in the Q8_0 quantiser */
 enum { ORA_ROUND_NEAREST_EVEN = 0, ORA_ROUND_HALF_AWAY = 1 };

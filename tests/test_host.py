@@ -71,11 +71,12 @@ def test_supports_rejects_contract_violations_and_uncovered_ops():
     assert ggml.flash_attn_supports(q, k, k, _t(ca.F16, (8, 4, 1, 1))) == ggml.ERR_INVALID               # mask too narrow
     assert ggml.flash_attn_supports(q, k, k, _t(ca.F16, (16, 4, 3, 1))) == ggml.ERR_INVALID              # 8 % 3
     # valid for ggml, outside these kernels: goes to the CPU backend
-    assert ggml.flash_attn_supports(q, k, _t(ca.F32, (64, 16, 8, 1)), None) == ggml.ERR_UNSUPPORTED      # mixed K/V types
+    assert ggml.flash_attn_supports(q, k, _t(ca.F32, (64, 16, 8, 1)), None) == ggml.OK                   # a K and a V of different types: both rounded to f16 first
+    assert ggml.flash_attn_supports(q, k, _t(30, (64, 16, 8, 1), (2, 128, 2048, 16384)), None) == ggml.ERR_UNSUPPORTED    # a V type outside the cache types
     assert ggml.flash_attn_supports(_t(ca.F16, (64, 4, 8, 1)), k, k, None) == ggml.ERR_UNSUPPORTED       # q not F32
     k4 = _t(ca.Q4_0, (64, 16, 8, 1), (18, 36, 576, 4608))
     assert ggml.flash_attn_supports(q, k4, k4, None) == ggml.OK                                          # Q4_0 cache view
-    assert ggml.flash_attn_supports(q, k4, _t(ca.Q5_1, (64, 16, 8, 1)), None) == ggml.ERR_UNSUPPORTED    # mixed K/V types
+    assert ggml.flash_attn_supports(q, k4, _t(ca.Q5_1, (64, 16, 8, 1)), None) == ggml.OK                 # -ctk q4_0 -ctv q5_1
     assert ggml.flash_attn_supports(_t(ca.F32, (48, 4, 8, 1)), _t(ca.Q4_0, (32, 16, 8, 1), (18, 18, 288, 2304)),
                                     _t(ca.Q4_0, (32, 16, 8, 1), (18, 18, 288, 2304)), None) == ggml.ERR_INVALID
     k12 = ca.Tensor.__new__(ca.Tensor); k12.__dict__.update(_t(ca.F16, (64, 16, 8, 1)).__dict__); k12.type = 12   # a k-quant

@@ -246,6 +246,31 @@ def test_decode_kernel_streamed_and_strided_rows_give_the_same_bits(ktype, D, ma
         assert np.array_equal(outs[0], outs[1])
 
 
-def test_mixed_cache_types_are_left_to_the_cpu_backend():
-    case = make_case(seed=4420, D=64, Nq=2, Nkv=40, Hq=2, ktype=ora.Q4_0, vtype=ora.Q5_1)
-    assert ggml.flash_attn_supports(upload(case["q"]), upload(case["k"]), upload(case["v"]), None) == ggml.ERR_UNSUPPORTED
+MIXED = [
+    # CRISPASR_KV_QUANT_K / CRISPASR_KV_QUANT_V (src/core/attention.h:132-137): the two halves of the cache in different types,
+    # both views handed to the op as they are (src/canary.cpp:953-972)
+    (ora.Q8_0, ora.Q4_0, dict(seed=4440, D=128, Nq=1, Nkv=300, Hq=8, kv_layout="gap")),                 # -ctk q8_0 -ctv q4_0, a decode step
+    (ora.Q8_0, ora.Q4_0, dict(seed=4441, D=128, Nq=24, Nkv=24, Hq=8, mask="causal")),                    # its prompt step
+    (ora.F16, ora.Q5_1, dict(seed=4442, D=64, Nq=2, Nkv=1237, Hq=8, Hkv=2, B=2, mask="random_inf")),
+    (ora.Q5_0, ora.F16, dict(seed=4443, D=128, Nq=200, Nkv=260, Hq=4, mask="causal")),                   # tile kernel
+    (ora.Q4_1, ora.Q8_0, dict(seed=4444, D=96, Nq=3, Nkv=70, Hq=2)),                                     # vector kernel
+    (ora.F32, ora.Q8_0, dict(seed=4445, D=64, Nq=5, Nkv=333, Hq=4, q_layout="thd")),
+]
+
+
+@pytest.mark.parametrize("ktype,vtype,spec", MIXED, ids=lambda x: "seed%d" % x["seed"] if isinstance(x, dict) else NAMES.get(x, str(x)))
+def test_k_and_v_of_different_cache_types(ktype, vtype, spec):
+    case = make_case(ktype=ktype, vtype=vtype, **spec)
+    q, k, v = upload(case["q"]), upload(case["k"]), upload(case["v"])
+    m = upload(case["mask"]) if case["mask"] is not None else None
+    assert ggml.flash_attn_supports(q, k, v, m, case["scale"]) == ggml.OK
+    plan = plan_details(case)
+    print("mixed cache types", ktype, vtype, spec, plan, flush=True)
+    assert plan["kv_to_f16"] == 1 and plan["workspace"] >= 2 * 2 * spec["D"] * spec["Nkv"] * spec.get("Hkv", spec["Hq"]) * spec.get("B", 1)
+    ref = run_oracle(case)
+    got = ggml.flash_attn_ext(q, k, v, m, case["scale"]).numpy_f32()
+    assert_parity(got, ref, "mixed %s" % spec)
+    ws = torch.empty(ggml.flash_attn_workspace_size(q, k, v, m, case["scale"]), dtype=torch.uint8, device="cuda")
+    assert np.array_equal(ggml.flash_attn_ext(q, k, v, m, case["scale"], workspace=ws).numpy_f32(), got)
+    for kern in (ggml.KERNEL_VEC, ggml.KERNEL_DECODE_MMA if spec["D"] in (64, 128) else ggml.KERNEL_VEC):
+        assert_parity(ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=kern, n_splits=2).numpy_f32(), ref, "mixed, kernel %d" % kern)

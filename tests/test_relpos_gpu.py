@@ -135,13 +135,17 @@ def test_relpos_attention_in_one_kernel_and_as_two_launches_matches_oracle(spec)
     pitch = (Nkv * 2 + 127) // 128 * 128
     need = ggml.flash_attn_relpos_workspace_size(dq, dqv, dk, dv, dr, da, c["scale"])
     kv16 = 0 if ktype == ora.F16 else (2 * D * Nkv * H * B * 2 + 255) // 256 * 256
-    assert need == kv16 + ggml.relpos_bias_workspace_size(dr)
+    # the size query answers for both forms of the call (which one a call takes depends on its pointers' alignment, unknown
+    # when a graph is planned): at least what the one-kernel form uses, and that form runs in exactly its own share
+    one = kv16 + ggml.relpos_bias_workspace_size(dr)
+    assert need >= one
     ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
     got_ws = ggml.flash_attn_relpos(dq, dqv, dk, dv, dr, da, c["scale"], workspace=ws).numpy_f32()
     assert np.array_equal(got_ws, got)
-    if need:
+    if one:
+        assert np.array_equal(ggml.flash_attn_relpos(dq, dqv, dk, dv, dr, da, c["scale"], workspace=ws[:one]).numpy_f32(), got)
         with pytest.raises(ggml.Mi355xError):
-            ggml.flash_attn_relpos(dq, dqv, dk, dv, dr, da, c["scale"], workspace=ws[: need - 256])
+            ggml.flash_attn_relpos(dq, dqv, dk, dv, dr, da, c["scale"], workspace=ws[: one - 256])
     # a kernel asked for by name: the mask is written out and the attention call reads it - the same bits as the two
     # calls made separately
     kern = ggml.KERNEL_MMA if Nq >= 16 else ggml.KERNEL_VEC
