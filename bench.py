@@ -520,6 +520,26 @@ def bench_host_resident(ca, ora, torch):
     ref = ca.flash_attn_ext(qd, kd, vd, None, 64 ** -0.25).numpy_f32()
     torch.cuda.synchronize()
     out["whisper_cross_beam5_f16"]["equals_device_resident"] = bool(np.array_equal(o.numpy_f32(), ref))
+    out["whisper_cross_beam5_f16"]["note"] += ("; K/V stored into the host buffer by the CPU, so the buffer has no mirror in HBM: "
+                                               "every call pulls them over the link")
+
+    # the same call on a cache that the graph's own KV write has filled (ggml_cpy F32 -> F16 into the cache view,
+    # src/crispasr.cpp:2956-2973): the write creates the buffer's mirror in HBM and attention reads that
+    kv2 = [host(Nkv * n_state * 2) for _ in range(2)]
+    for b, hb in zip(kv2, kv):
+        f32 = torch.from_numpy(hb.array.view(np.float16).astype(np.float32)).cuda()
+        ca.cpy(ca.Tensor(f32.view(torch.uint8), ca.F32, (Nkv * n_state,)), ca.Tensor(b, ca.F16, (Nkv * n_state,)))
+    torch.cuda.synchronize()
+    k2, v2 = ca.Tensor(kv2[0], ca.F16, (D, Nkv, H, 1), nbk), ca.Tensor(kv2[1], ca.F16, (D, Nkv, H, 1), nbk)
+    timed("whisper_cross_beam5_f16_cache_written_by_cpy", lambda: ca.flash_attn_ext(q, k2, v2, None, 64 ** -0.25, out=o),
+          2 * Nkv * n_state * 2 + 2 * 5 * n_state * 4, 20,
+          "the cache in a host buffer, filled by the library's copy kernel as the graph's KV write does: mirrored in HBM, only "
+          "Q and the result (51 KB) cross the link")
+    torch.cuda.synchronize()
+    e = out["whisper_cross_beam5_f16_cache_written_by_cpy"]
+    e["equals_device_resident"] = bool(np.array_equal(o.numpy_f32(), ref))
+    e["host_bytes_equal"] = bool(np.array_equal(kv2[0].array, kv[0].array) and np.array_equal(kv2[1].array, kv[1].array))
+    e["mirror"] = kv2[0].mirror_stats()
 
     # one encoder layer of the headline workload, one window, everything in host memory
     N = 1500
@@ -808,19 +828,21 @@ def bench_whisper_protocol(args, ca, ora, torch):
     return res
 
 
-def bench_whisper_protocol_native():
+def bench_whisper_protocol_native(*mode):
     """The same protocol driven by the native host driver (C++ above the C ABI, no Python between the calls): what a
-    ggml backend's graph_compute would pay per node.  Runs as a child process."""
+    ggml backend's graph_compute would pay per node.  Runs as a child process.  mode: () = everything in HBM, attention
+    calls only; ("host", "write") = caches, Q and results in host-visible buffers (the caches mirrored in HBM) and every
+    decode writing its new K/V rows first - the calls an unmodified runtime would make."""
     import subprocess
     exe = os.path.join(ROOT, "crispasr_amd", "host", "mi355x_attn_protocol")
     if not os.path.exists(exe):
         return {"error": "host driver not built"}
-    res = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    res = subprocess.run([exe, "32", *mode], capture_output=True, text=True, timeout=300)
     if res.returncode != 0:
         return {"error": "exit code %d: %s" % (res.returncode, res.stderr[-300:])}
     out = json.loads(res.stdout.strip().splitlines()[-1])
     for k in ("single_token_x256", "batch5_x64", "prompt256_x16"):
-        log(f"[bench] whisper protocol, native host driver, {k}: {out[k]['ms_per_decode']:.3f} ms per decode, "
+        log(f"[bench] whisper protocol, native host driver{' ' + '+'.join(mode) if mode else ''}, {k}: {out[k]['ms_per_decode']:.3f} ms per decode, "
             f"{out[k]['us_per_attention_call']:.1f} us per call incl. host launch")
     return out
 
@@ -908,6 +930,7 @@ def main():
         line["configs"] = bench_configs(args, ca, ora, torch)
         line["whisper_bench_protocol"] = bench_whisper_protocol(args, ca, ora, torch)
         line["whisper_bench_protocol_native"] = bench_whisper_protocol_native()
+        line["whisper_bench_protocol_native_host_buffers"] = bench_whisper_protocol_native("host", "write")
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(args, ora, host0)
     if not enc["parity"]["ok"]:

@@ -145,6 +145,131 @@ int noalloc_scratch(void ** out) {
     return MI355X_OK;
 }
 
+// ---- host-visible buffers and their mirrors in HBM ---------------------------------------------------------------
+// A buffer from mi355x_host_buffer_alloc is pinned host memory that the CPU backend works on in place.  What the GPU
+// reads from it again and again - a KV cache - would cross the host link on every call, so such a buffer grows a mirror:
+// an HBM allocation of the same size, created by the first KV write into the buffer.  The host copy stays complete and
+// authoritative; a page of the mirror is VALID when it holds the same bytes.  Every write that goes through this library
+// (copy / set_rows kernels, memset, set, copy) stores to both copies, after bringing the pages it touches up to date, so
+// pages that are VALID stay so; attention reads K and V from the mirror, bringing stale pages up to date first.  In the
+// steady state of a decoder loop nothing but the new rows (to the host copy), Q and the result cross the link.
+constexpr size_t MIRROR_PAGE = 64 * 1024;
+struct HostBuf {
+    char * base   = nullptr;
+    size_t size   = 0;
+    char * mirror = nullptr;
+    std::vector<uint8_t> valid;        // per page
+    size_t uploaded = 0;               // bytes brought up to date so far (statistics)
+};
+std::vector<HostBuf *> g_hostbufs;     // guarded by g_mu
+const bool g_no_mirror = getenv("MI355X_NO_MIRROR") != nullptr;      // comparison runs: every read and write goes to the host copy
+
+// the registered buffer that holds [p, p + n), or nullptr (g_mu held)
+HostBuf * hostbuf_of(const void * p, size_t n) {
+    for (HostBuf * b : g_hostbufs)
+        if ((const char *)p >= b->base && (const char *)p + n <= b->base + b->size) return b;
+    return nullptr;
+}
+
+// first and one-past-last byte that a view touches, relative to its data pointer
+void view_span(const mi355x_tensor * t, size_t * bytes) {
+    size_t hi = 0;
+    bool   empty = false;
+    for (int i = 0; i < 4; i++) empty = empty || t->ne[i] <= 0;
+    if (!empty) {
+        hi = (size_t)(t->ne[0] / block_size(t->type)) * t->nb[0];
+        for (int i = 1; i < 4; i++) hi += (size_t)(t->ne[i] - 1) * t->nb[i];
+    }
+    *bytes = hi;
+}
+
+// bring the mirror's pages that overlap [off, off + n) up to date (g_mu held)
+int mirror_make_valid(HostBuf * b, size_t off, size_t n, hipStream_t st) {
+    if (!b->mirror || n == 0) return MI355X_OK;
+    const size_t p0 = off / MIRROR_PAGE, p1 = (off + n + MIRROR_PAGE - 1) / MIRROR_PAGE;
+    size_t run = (size_t)-1;
+    for (size_t p = p0; p <= p1; p++) {
+        const bool stale = p < p1 && !b->valid[p];
+        if (stale && run == (size_t)-1) run = p;
+        if (!stale && run != (size_t)-1) {
+            const size_t lo = run * MIRROR_PAGE, hi = p * MIRROR_PAGE < b->size ? p * MIRROR_PAGE : b->size;
+            HIP_TRY(hipMemcpyAsync(b->mirror + lo, b->base + lo, hi - lo, hipMemcpyHostToDevice, st));
+            b->uploaded += hi - lo;
+            for (size_t k = run; k < p; k++) b->valid[k] = 1;
+            run = (size_t)-1;
+        }
+    }
+    return MI355X_OK;
+}
+
+// pages that lie inside [off, off + n) altogether have just been written in both copies
+void mirror_mark_written(HostBuf * b, size_t off, size_t n) {
+    if (!b->mirror) return;
+    const size_t p0 = (off + MIRROR_PAGE - 1) / MIRROR_PAGE;
+    const size_t end = off + n == b->size ? (b->size + MIRROR_PAGE - 1) / MIRROR_PAGE : (off + n) / MIRROR_PAGE;
+    for (size_t p = p0; p < end; p++) b->valid[p] = 1;
+}
+
+// A kernel is about to write the view `dst`.  If it lies in a host buffer: create that buffer's mirror if need be (never
+// while the stream is being captured: the write then goes to the host copy alone and the pages turn stale), bring the
+// pages of the view's span up to date, and return the distance from the host copy to the mirror (0: write the view only).
+int mirror_for_write(const mi355x_tensor * dst, hipStream_t st, int64_t * delta) {
+    *delta = 0;
+    if (g_no_mirror || !dst->data) return MI355X_OK;
+    size_t n = 0;
+    view_span(dst, &n);
+    std::lock_guard<std::mutex> lk(g_mu);
+    HostBuf * b = hostbuf_of(dst->data, n);
+    if (!b) return MI355X_OK;
+    const size_t off = (size_t)((const char *)dst->data - b->base);
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess) (void)hipGetLastError();
+    if (!b->mirror) {
+        void * m = nullptr;
+        if (cs != hipStreamCaptureStatusNone || hipMalloc(&m, b->size) != hipSuccess) {
+            (void)hipGetLastError();
+            return MI355X_OK;                        // no mirror: the buffer stays a plain host buffer
+        }
+        b->mirror = (char *)m;
+        b->valid.assign((b->size + MIRROR_PAGE - 1) / MIRROR_PAGE, 0);
+    }
+    if (cs != hipStreamCaptureStatusNone) {
+        // a captured write would be replayed without this bookkeeping: keep it to the host copy, pages become stale
+        const size_t p0 = off / MIRROR_PAGE, p1 = (off + n + MIRROR_PAGE - 1) / MIRROR_PAGE;
+        for (size_t p = p0; p < p1; p++) b->valid[p] = 0;
+        return MI355X_OK;
+    }
+    const int rc = mirror_make_valid(b, off, n, st);
+    if (rc) return rc;
+    *delta = b->mirror - b->base;
+    return MI355X_OK;
+}
+
+// A kernel is about to read the view `t` many times over (K or V).  If it lies in a host buffer that has a mirror, bring
+// the span's pages up to date and return the view's address in the mirror; otherwise the address it has.
+int mirror_for_read(const mi355x_tensor * t, hipStream_t st, void ** data) {
+    *data = t->data;
+    if (g_no_mirror || !t->data) return MI355X_OK;
+    size_t n = 0;
+    view_span(t, &n);
+    std::lock_guard<std::mutex> lk(g_mu);
+    HostBuf * b = hostbuf_of(t->data, n);
+    if (!b || !b->mirror) return MI355X_OK;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess) (void)hipGetLastError();
+    const size_t off = (size_t)((const char *)t->data - b->base);
+    if (cs != hipStreamCaptureStatusNone) {
+        // under capture only pages that are up to date already may be read from the mirror
+        for (size_t p = off / MIRROR_PAGE; p < (off + n + MIRROR_PAGE - 1) / MIRROR_PAGE; p++)
+            if (!b->valid[p]) return MI355X_OK;
+    } else {
+        const int rc = mirror_make_valid(b, off, n, st);
+        if (rc) return rc;
+    }
+    *data = b->mirror + off;
+    return MI355X_OK;
+}
+
 // a mask argument with no extent is the same as no mask
 bool has_mask(const mi355x_tensor * mask) { return mask && mask->ne[0] > 0; }
 
@@ -611,6 +736,16 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
         inner.workspace_size = need;
         return mi355x_flash_attn_ext(&qd, k, v, mask, dst, &inner, stream);
     }
+    // K and V of a cache that lives in a host buffer are read from that buffer's mirror in HBM
+    mi355x_tensor km = *k, vm = *v;
+    if ((int64_t)q->ne[1] * q->ne[2] * q->ne[3] > 0 && k->ne[1] > 0) {
+        rc = mirror_for_read(k, (hipStream_t)stream, &km.data);
+        if (rc) return rc;
+        rc = mirror_for_read(v, (hipStream_t)stream, &vm.data);
+        if (rc) return rc;
+    }
+    k = &km;
+    v = &vm;
     FattnArgs a;
     fill_args(a, q, k, v, mask, (float *)dst->data, params);
     if ((int64_t)a.Nq * a.Hq * a.B == 0) return MI355X_OK;
@@ -1069,6 +1204,14 @@ int mi355x_cpy(const mi355x_tensor * src, const mi355x_tensor * dst, void * stre
     if (a.n == 0) return MI355X_OK;
     if (!a.src || !a.dst) return fail(MI355X_ERR_INVALID, "null data pointer");
     if (a.n > ((int64_t)1 << 38)) return fail(MI355X_ERR_UNSUPPORTED, "copy too large");
+    const int rm = mirror_for_write(dst, (hipStream_t)stream, &a.mirror);
+    if (rm) return rm;
+    {   // a source inside a mirrored buffer (ggml_cont of a cache slice, src/core/attention.h:919-920) is read from HBM
+        void * sdata = nullptr;
+        const int rs = mirror_for_read(src, (hipStream_t)stream, &sdata);
+        if (rs) return rs;
+        a.src = (const char *)sdata;
+    }
     const int e = cpy_launch(a, src->type, dst->type, (hipStream_t)stream);
     if (e) return hip_fail((hipError_t)e, "cpy launch");
     return MI355X_OK;
@@ -1116,6 +1259,8 @@ int mi355x_set_rows(const mi355x_tensor * src, const void * idx, int32_t idx_typ
     a.n = FATTN_IS_BLOCK_TYPE(dst->type) ? n / FATTN_QK8_0 : n;
     if (a.n == 0) return MI355X_OK;
     if (!a.src || !a.dst || !a.idx) return fail(MI355X_ERR_INVALID, "null data pointer");
+    const int rm = mirror_for_write(dst, (hipStream_t)stream, &a.mirror);
+    if (rm) return rm;
     const int e = set_rows_launch(a, dst->type, (hipStream_t)stream);
     if (e) return hip_fail((hipError_t)e, "set_rows launch");
     return MI355X_OK;
@@ -1139,11 +1284,76 @@ int mi355x_host_buffer_alloc(size_t size, void ** ptr) {
     if (!ptr) return fail(MI355X_ERR_INVALID, "null argument");
     *ptr = nullptr;
     HIP_TRY(hipHostMalloc(ptr, size ? size : 1, hipHostMallocMapped | hipHostMallocCoherent));
+    HostBuf * b = new HostBuf();
+    b->base = (char *)*ptr;
+    b->size = size ? size : 1;
+    std::lock_guard<std::mutex> lk(g_mu);
+    g_hostbufs.push_back(b);
     return MI355X_OK;
 }
 
 int mi355x_host_buffer_free(void * ptr) {
-    if (ptr) HIP_TRY(hipHostFree(ptr));
+    if (!ptr) return MI355X_OK;
+    HostBuf * b = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        for (size_t i = 0; i < g_hostbufs.size(); i++)
+            if (g_hostbufs[i]->base == (char *)ptr) {
+                b = g_hostbufs[i];
+                g_hostbufs.erase(g_hostbufs.begin() + i);
+                break;
+            }
+    }
+    if (b) {
+        if (b->mirror) HIP_TRY(hipFree(b->mirror));
+        delete b;
+    }
+    HIP_TRY(hipHostFree(ptr));
+    return MI355X_OK;
+}
+
+int mi355x_host_buffer_mirror_stats(const void * ptr, size_t * mirror_bytes, size_t * valid_bytes, size_t * uploaded_bytes) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    HostBuf * b = hostbuf_of(ptr, 1);
+    if (!b) return fail(MI355X_ERR_INVALID, "not inside a buffer of mi355x_host_buffer_alloc");
+    size_t valid = 0;
+    for (size_t p = 0; p < b->valid.size(); p++)
+        if (b->valid[p]) valid += (p + 1) * MIRROR_PAGE <= b->size ? MIRROR_PAGE : b->size - p * MIRROR_PAGE;
+    if (mirror_bytes)   *mirror_bytes   = b->mirror ? b->size : 0;
+    if (valid_bytes)    *valid_bytes    = valid;
+    if (uploaded_bytes) *uploaded_bytes = b->uploaded;
+    return MI355X_OK;
+}
+
+int mi355x_host_buffer_invalidate(void * ptr, size_t size) {
+    if (size == 0) return MI355X_OK;
+    std::lock_guard<std::mutex> lk(g_mu);
+    HostBuf * b = hostbuf_of(ptr, size);
+    if (!b) return fail(MI355X_ERR_INVALID, "not inside a buffer of mi355x_host_buffer_alloc");
+    if (!b->mirror) return MI355X_OK;
+    const size_t off = (size_t)((char *)ptr - b->base);
+    for (size_t p = off / MIRROR_PAGE; p < (off + size + MIRROR_PAGE - 1) / MIRROR_PAGE; p++) b->valid[p] = 0;
+    return MI355X_OK;
+}
+
+// The place of [ptr, ptr + size) in the mirror of the host buffer that holds it, if that buffer has one (g_mu held).  The
+// callers below write the same bytes to both copies: a page they cover only in part keeps its state - up to date stays up
+// to date, stale stays stale and is fetched whole from the host copy when it is next needed.
+static int mirror_of_range(void * ptr, size_t size, hipStream_t st, HostBuf ** buf, char ** mirror) {
+    *buf = nullptr;
+    *mirror = nullptr;
+    if (g_no_mirror) return MI355X_OK;
+    HostBuf * b = hostbuf_of(ptr, size);
+    if (!b || !b->mirror) return MI355X_OK;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess) (void)hipGetLastError();
+    const size_t off = (size_t)((char *)ptr - b->base);
+    if (cs != hipStreamCaptureStatusNone) {           // replays would bypass the bookkeeping: host copy only, pages stale
+        for (size_t p = off / MIRROR_PAGE; p < (off + size + MIRROR_PAGE - 1) / MIRROR_PAGE; p++) b->valid[p] = 0;
+        return MI355X_OK;
+    }
+    *buf = b;
+    *mirror = b->mirror + off;
     return MI355X_OK;
 }
 
@@ -1151,8 +1361,15 @@ int mi355x_buffer_memset(void * ptr, int value, size_t size, void * stream) {
     if (size == 0) return MI355X_OK;
     if (!ptr) return fail(MI355X_ERR_INVALID, "null argument");
     // a fill kernel, not hipMemsetAsync: safe to record into a graph the caller captures
-    const int e = fill_launch(ptr, value, size, (hipStream_t)stream);
+    int e = fill_launch(ptr, value, size, (hipStream_t)stream);
     if (e) return hip_fail((hipError_t)e, "fill launch");
+    std::lock_guard<std::mutex> lk(g_mu);
+    HostBuf * b; char * m;
+    const int rc = mirror_of_range(ptr, size, (hipStream_t)stream, &b, &m);
+    if (rc || !m) return rc;
+    e = fill_launch(m, value, size, (hipStream_t)stream);
+    if (e) return hip_fail((hipError_t)e, "fill launch");
+    mirror_mark_written(b, (size_t)((char *)ptr - b->base), size);      // (pages covered in part keep their state: both copies got the same bytes)
     return MI355X_OK;
 }
 
@@ -1161,6 +1378,16 @@ int mi355x_buffer_set(void * dst, const void * host_src, size_t size, void * str
     if (size == 0) return MI355X_OK;
     if (!dst || !host_src) return fail(MI355X_ERR_INVALID, "null argument");
     HIP_TRY(hipMemcpyAsync(dst, host_src, size, hipMemcpyDefault, (hipStream_t)stream));
+    {
+        std::lock_guard<std::mutex> lk(g_mu);
+        HostBuf * b; char * m;
+        const int rc = mirror_of_range(dst, size, (hipStream_t)stream, &b, &m);
+        if (rc) return rc;
+        if (m) {
+            HIP_TRY(hipMemcpyAsync(m, host_src, size, hipMemcpyDefault, (hipStream_t)stream));
+            mirror_mark_written(b, (size_t)((char *)dst - b->base), size);
+        }
+    }
     HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
     return MI355X_OK;
 }
@@ -1177,6 +1404,21 @@ int mi355x_buffer_copy(void * dst, const void * src, size_t size, void * stream)
     if (size == 0) return MI355X_OK;
     if (!dst || !src) return fail(MI355X_ERR_INVALID, "null argument");
     HIP_TRY(hipMemcpyAsync(dst, src, size, hipMemcpyDefault, (hipStream_t)stream));
+    std::lock_guard<std::mutex> lk(g_mu);
+    HostBuf * b; char * m;
+    const int rc = mirror_of_range(dst, size, (hipStream_t)stream, &b, &m);
+    if (rc || !m) return rc;
+    // from the source's own mirror where that is up to date (a cache snapshot then never leaves HBM), else from the source
+    const void * from = src;
+    HostBuf * sb = hostbuf_of(src, size);
+    if (sb && sb->mirror) {
+        const size_t so = (size_t)((const char *)src - sb->base);
+        bool ok = true;
+        for (size_t p = so / MIRROR_PAGE; p < (so + size + MIRROR_PAGE - 1) / MIRROR_PAGE; p++) ok = ok && sb->valid[p];
+        if (ok) from = sb->mirror + so;
+    }
+    HIP_TRY(hipMemcpyAsync(m, from, size, hipMemcpyDefault, (hipStream_t)stream));
+    mirror_mark_written(b, (size_t)((char *)dst - b->base), size);
     return MI355X_OK;
 }
 

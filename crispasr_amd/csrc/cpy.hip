@@ -32,7 +32,9 @@ __global__ void __launch_bounds__(256) cpy_scalar_kernel(const CpyArgs a) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i >= a.n) return;
     const TS x = *(const TS *)(a.src + offset_of(i, a.sne, a.snb, 1));
-    *(TD *)(a.dst + offset_of(i, a.dne, a.dnb, 1)) = (TD)x;     // f32 -> f16 is round-to-nearest-even
+    char * dp = a.dst + offset_of(i, a.dne, a.dnb, 1);
+    *(TD *)dp = (TD)x;                                          // f32 -> f16 is round-to-nearest-even
+    if (a.mirror) *(TD *)(dp + a.mirror) = (TD)x;
 }
 
 // 8 consecutive elements of dimension 0 per lane: 128-bit loads and stores for f16 <-> f32 and same-type copies.
@@ -50,6 +52,7 @@ __global__ void __launch_bounds__(256) cpy_vec8_kernel(const CpyArgs a) {
 #pragma unroll
     for (int e = 0; e < 8; e++) y[e] = (TD)x[e];
     *(vd8 *)dp = y;
+    if (a.mirror) *(vd8 *)((char *)dp + a.mirror) = y;
 }
 
 // quantise one block of 32 held one element per lane (32 consecutive lanes) and store it
@@ -58,17 +61,21 @@ __global__ void __launch_bounds__(256) cpy_vec8_kernel(const CpyArgs a) {
 //   Q4_0 / Q5_0: d = (signed value of largest magnitude, the first one) / -8 (-16), q = min(15 (31), trunc(x/d + 8.5 (16.5)))
 //   Q4_1 / Q5_1: d = (max - min) / 15 (31), m = min, q = min(15 (31), trunc((x - min)/d + 0.5))
 // every product and sum is a single f32 operation, none fused.
+// mirror: 0, or the distance to a second copy of the destination that gets the same bytes
 template <int TYPE>
-__device__ __forceinline__ void quantize_block_store(float x, char * blk, int e, bool ok) {
+__device__ __forceinline__ void quantize_block_store(float x, char * blk, int e, bool ok, int64_t mirror) {
     typedef BlockFormat<TYPE> F;
+    const int copies = mirror ? 2 : 1;
     if (TYPE == MI355X_TYPE_Q8_0) {
         const float amax = group_max<32>(fabsf(x));
         const float d    = amax / 127.0f;
         const float id   = d != 0.0f ? 1.0f / d : 0.0f;
         const int   qi   = (int)rintf(x * id);
         if (ok) {
-            ((int8_t *)(blk + 2))[e] = (int8_t)qi;
-            if (e == 0) *(_Float16 *)blk = (_Float16)d;
+            for (int c = 0; c < copies; c++, blk += mirror) {
+                ((int8_t *)(blk + 2))[e] = (int8_t)qi;
+                if (e == 0) *(_Float16 *)blk = (_Float16)d;
+            }
         }
         return;
     }
@@ -97,11 +104,13 @@ __device__ __forceinline__ void quantize_block_store(float x, char * blk, int e,
     const int      hi = __shfl(qi, half + (e & 15) + 16, 64);       // the element that shares this lane's byte
     const uint32_t qh = (uint32_t)(__ballot((qi & 0x10) != 0) >> half);
     if (ok) {
-        if (e < 16) ((uint8_t *)(blk + F::QS))[e] = (uint8_t)((qi & 15) | ((hi & 15) << 4));
-        if (e == 16) *(_Float16 *)blk = (_Float16)d;
-        if (F::HAS_M && e == 17) *(_Float16 *)(blk + 2) = (_Float16)m;
-        if (F::QH && e == 18) *(uint16_t *)(blk + F::QH) = (uint16_t)qh;
-        if (F::QH && e == 19) *(uint16_t *)(blk + F::QH + 2) = (uint16_t)(qh >> 16);
+        for (int c = 0; c < copies; c++, blk += mirror) {
+            if (e < 16) ((uint8_t *)(blk + F::QS))[e] = (uint8_t)((qi & 15) | ((hi & 15) << 4));
+            if (e == 16) *(_Float16 *)blk = (_Float16)d;
+            if (F::HAS_M && e == 17) *(_Float16 *)(blk + 2) = (_Float16)m;
+            if (F::QH && e == 18) *(uint16_t *)(blk + F::QH) = (uint16_t)qh;
+            if (F::QH && e == 19) *(uint16_t *)(blk + F::QH + 2) = (uint16_t)(qh >> 16);
+        }
     }
 }
 
@@ -115,7 +124,7 @@ __global__ void __launch_bounds__(256) cpy_f32_block_kernel(const CpyArgs a) {
     const char *  sp  = a.src + offset_of(bc, a.sne, a.snb, FATTN_QK8_0) + e * a.snb[0];
     const float   x   = ok ? *(const float *)sp : 0.0f;
     char * dp = a.dst + offset_of(bc, a.dne, a.dnb, FATTN_QK8_0, FATTN_QK8_0);
-    quantize_block_store<TYPE>(x, dp, e, ok);
+    quantize_block_store<TYPE>(x, dp, e, ok, a.mirror);
 }
 
 // block type -> F32; 8 elements per lane, four lanes per block
@@ -131,6 +140,10 @@ __global__ void __launch_bounds__(256) cpy_block_f32_kernel(const CpyArgs a) {
     char * dp = a.dst + offset_of(blk, a.dne, a.dnb, FATTN_QK8_0) + j0 * a.dnb[0];
 #pragma unroll
     for (int i = 0; i < 8; i++) *(float *)(dp + i * a.dnb[0]) = y[i];
+    if (a.mirror) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) *(float *)(dp + a.mirror + i * a.dnb[0]) = y[i];
+    }
 }
 
 // same block type on both sides: move the blocks as halfwords
@@ -144,6 +157,7 @@ __global__ void __launch_bounds__(256) cpy_block_block_kernel(const CpyArgs a) {
     const uint16_t * sp = (const uint16_t *)(a.src + offset_of(blk, a.sne, a.snb, FATTN_QK8_0, FATTN_QK8_0));
     uint16_t *       dp = (uint16_t *)(a.dst + offset_of(blk, a.dne, a.dnb, FATTN_QK8_0, FATTN_QK8_0));
     dp[w] = sp[w];
+    if (a.mirror) *(uint16_t *)((char *)(dp + w) + a.mirror) = sp[w];
 }
 
 // SET_ROWS: dst[:, idx[i1, i2 % ine1, i3 % ine2], i2, i3] = convert(src[:, i1, i2, i3]), src F32
@@ -176,10 +190,12 @@ __global__ void __launch_bounds__(256) set_rows_kernel(const CpyArgs a) {
     const float  x  = ok ? *(const float *)sp : 0.0f;
     char * dp = a.dst + i0 * a.dnb[0] + (inside ? drow : 0) * a.dnb[1] + i2 * a.dnb[2] + i3 * a.dnb[3];
     if constexpr (BLOCKS) {
-        quantize_block_store<DTYPE>(x, dp, e, inside);
+        quantize_block_store<DTYPE>(x, dp, e, inside, a.mirror);
     } else if (inside) {
-        if (DTYPE == MI355X_TYPE_F16) *(_Float16 *)dp = (_Float16)x;
-        else                          *(float *)dp = x;
+        for (int c = 0; c < (a.mirror ? 2 : 1); c++, dp += a.mirror) {
+            if (DTYPE == MI355X_TYPE_F16) *(_Float16 *)dp = (_Float16)x;
+            else                          *(float *)dp = x;
+        }
     }
 }
 

@@ -196,6 +196,7 @@ struct CpyArgs {
     int64_t sne[4], dne[4];
     int64_t snb[4], dnb[4];
     int64_t n;                 // elements (or blocks of 32 when a side is a block type)
+    int64_t mirror;            // 0, or the distance in bytes from dst to a second copy that gets the same stores
     // SET_ROWS only
     const char * idx;
     int32_t idx_is_i64;

@@ -64,8 +64,12 @@ static mi355x_fattn_params fa_params(const ggml_tensor * node) {
 // The runtimes place weights and KV caches in the first GPU device's default buffer type
 // (src/crispasr.cpp:1940-1944, 3942-3971; src/core/gguf_loader.cpp:722-741).  For ggml-cpu to keep running
 // every other op on those tensors the buffer must be host memory (is_host = true); the GPU addresses the same
-// pages.  Tensors that only attention reads (the scheduler's copies at split boundaries) live in HBM buffers
-// of the second buffer type below.
+// pages.  A KV cache in such a buffer does not cross the host link on every attention call: the library gives the
+// buffer a mirror in HBM when the graph's first KV write (a CPY or SET_ROWS node whose destination lies in it - this
+// backend is the first one that supports both the buffer and the op, so the scheduler hands those nodes here) reaches
+// it, keeps both copies equal on every write that goes through its entry points - which is every call of the buffer
+// vtable below - and reads K and V from the mirror (mi355x_fattn.h, mi355x_host_buffer_alloc).  Nothing here has to
+// know: the vtable passes host pointers.  A second buffer type in plain HBM exists for callers that ask for it by name.
 
 struct mi355x_buffer_ctx { void * base; bool device; };
 

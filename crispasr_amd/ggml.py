@@ -84,7 +84,7 @@ EXPORTS = [
     "mi355x_fattn_supports", "mi355x_flash_attn_ext", "mi355x_flash_attn_ext_noalloc", "mi355x_fattn_workspace_size", "mi355x_fattn_plan", "mi355x_fattn_plan_details",
     "mi355x_relpos_bias_supports", "mi355x_relpos_bias", "mi355x_relpos_bias_workspace_size", "mi355x_flash_attn_relpos", "mi355x_fattn_relpos_workspace_size",
     "mi355x_cpy_supports", "mi355x_cpy", "mi355x_set_rows", "mi355x_set_rows_supports",
-    "mi355x_buffer_alloc", "mi355x_buffer_free", "mi355x_host_buffer_alloc", "mi355x_host_buffer_free", "mi355x_buffer_memset", "mi355x_buffer_set",
+    "mi355x_buffer_alloc", "mi355x_buffer_free", "mi355x_host_buffer_alloc", "mi355x_host_buffer_free", "mi355x_host_buffer_mirror_stats", "mi355x_host_buffer_invalidate", "mi355x_buffer_memset", "mi355x_buffer_set",
     "mi355x_buffer_get", "mi355x_buffer_copy",
 ]
 
@@ -129,6 +129,8 @@ def lib() -> ctypes.CDLL:
         L.mi355x_buffer_free.argtypes = [ctypes.c_void_p]
         L.mi355x_host_buffer_alloc.argtypes = [ctypes.c_size_t, ctypes.POINTER(ctypes.c_void_p)]
         L.mi355x_host_buffer_free.argtypes = [ctypes.c_void_p]
+        L.mi355x_host_buffer_mirror_stats.argtypes = [ctypes.c_void_p] + [ctypes.POINTER(ctypes.c_size_t)] * 3
+        L.mi355x_host_buffer_invalidate.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
         L.mi355x_buffer_memset.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t, ctypes.c_void_p]
         L.mi355x_buffer_set.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
         L.mi355x_buffer_get.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
@@ -181,6 +183,16 @@ class HostBuffer:
 
     def data_ptr(self) -> int:
         return self.ptr
+
+    def mirror_stats(self) -> dict:
+        """the buffer's mirror in HBM: its size (0: none yet), the bytes that are up to date, the bytes fetched so far"""
+        m, v, u = ctypes.c_size_t(0), ctypes.c_size_t(0), ctypes.c_size_t(0)
+        _check(lib().mi355x_host_buffer_mirror_stats(self.ptr, ctypes.byref(m), ctypes.byref(v), ctypes.byref(u)))
+        return {"mirror_bytes": m.value, "valid_bytes": v.value, "uploaded_bytes": u.value}
+
+    def invalidate(self, offset: int = 0, nbytes: Optional[int] = None) -> None:
+        """the CPU has written [offset, offset + nbytes) through `array`: the mirror's pages there are stale"""
+        _check(lib().mi355x_host_buffer_invalidate(self.ptr + offset, self.nbytes - offset if nbytes is None else nbytes))
 
     def __del__(self):
         if getattr(self, "ptr", None):

@@ -8,7 +8,13 @@
 // A small self-check (one masked GQA-free call against a double-precision loop) guards the timings; the parity
 // tests proper live in tests/.
 //
-// usage: mi355x_attn_protocol [n_layers]      -> one JSON line on stdout, exit code 0 when the self-check passes
+// usage: mi355x_attn_protocol [n_layers] [hbm|host] [write]
+//   host : the KV caches, Q and the result live in host-visible buffers (mi355x_host_buffer_alloc), which is where an
+//          unmodified runtime puts them when this library is its GPU backend (src/crispasr.cpp:3942-3971); the caches are
+//          filled the way the graphs fill them, by F32 -> F16 copies into cache views (src/crispasr.cpp:2956-2973,
+//          3185-3203), so they are mirrored in HBM and attention reads the mirror
+//   write: every decode also writes its new K and V rows into the self-attention cache first (two copies per layer)
+// -> one JSON line on stdout, exit code 0 when the self-check passes
 #include "mi355x_fattn.h"
 
 #include <chrono>
@@ -73,12 +79,43 @@ float rnd() {                                   // uniform in [-1, 1)
     return (float)((rng_state >> 40) / 8388608.0 - 1.0);
 }
 
+bool g_host = false;                            // caches, Q and the result in host-visible buffers
+
 void * dev_alloc(size_t n) {
     void * p = nullptr;
     CHECK(mi355x_buffer_alloc(n, &p));
     return p;
 }
+void * cache_alloc(size_t n) {
+    if (!g_host) return dev_alloc(n);
+    void * p = nullptr;
+    CHECK(mi355x_host_buffer_alloc(n, &p));
+    return p;
+}
+mi355x_tensor flat(void * data, int type, int64_t n) {
+    mi355x_tensor t;
+    t.data = data;
+    t.type = type;
+    t.ne[0] = n; t.ne[1] = t.ne[2] = t.ne[3] = 1;
+    t.nb[0] = type == MI355X_TYPE_F32 ? 4 : 2;
+    t.nb[1] = t.nb[2] = t.nb[3] = t.nb[0] * (size_t)n;
+    return t;
+}
+// a cache of n f16 values, zeros from zero_from on.  In host mode it is written as the graphs write it: an F32 tensor
+// copied (F32 -> F16) into the cache by the library's copy kernel, which is also what gives the buffer its mirror.
 void * dev_f16(size_t n, size_t zero_from = (size_t)-1) {
+    if (g_host) {
+        std::vector<float> f(n);
+        for (size_t i = 0; i < n; i++) f[i] = i >= zero_from ? 0.0f : rnd();
+        void * src = dev_alloc(n * 4);
+        CHECK(mi355x_buffer_set(src, f.data(), n * 4, nullptr));
+        void * p = cache_alloc(n * 2);
+        const mi355x_tensor s = flat(src, MI355X_TYPE_F32, (int64_t)n), d = flat(p, MI355X_TYPE_F16, (int64_t)n);
+        CHECK(mi355x_cpy(&s, &d, nullptr));
+        CHECK(mi355x_stream_synchronize(nullptr));
+        CHECK(mi355x_buffer_free(src));
+        return p;
+    }
     std::vector<uint16_t> h(n);
     for (size_t i = 0; i < n; i++) h[i] = i >= zero_from ? 0 : f2h(rnd());
     void * p = dev_alloc(n * 2);
@@ -147,6 +184,11 @@ double self_check(void * q_dev, const std::vector<float> & q_host, void * out_de
 
 int main(int argc, char ** argv) {
     const int L = argc > 1 ? atoi(argv[1]) : 32;
+    bool with_write = false;
+    for (int i = 2; i < argc; i++) {
+        if (!strcmp(argv[i], "host")) g_host = true;
+        if (!strcmp(argv[i], "write")) with_write = true;
+    }
     int n_dev = 0;
     CHECK(mi355x_device_count(&n_dev));
     if (n_dev < 1) { fprintf(stderr, "no device\n"); return 3; }
@@ -161,9 +203,12 @@ int main(int argc, char ** argv) {
     }
     std::vector<float> qh((size_t)256 * NSTATE);
     for (auto & x : qh) x = rnd();
-    void * q_dev = dev_alloc(qh.size() * 4);
+    void * q_dev = cache_alloc(qh.size() * 4);
     CHECK(mi355x_buffer_set(q_dev, qh.data(), qh.size() * 4, nullptr));
-    void * out_dev = dev_alloc(qh.size() * 4);
+    void * out_dev = cache_alloc(qh.size() * 4);
+    // the rows a decode writes into the cache: Kcur / Vcur of the graph, F32 [n_state, n_tok]
+    void * kv_new = cache_alloc(qh.size() * 4);
+    CHECK(mi355x_buffer_set(kv_new, qh.data(), qh.size() * 4, nullptr));
 
     const double err = self_check(q_dev, qh, out_dev);
 
@@ -173,7 +218,7 @@ int main(int argc, char ** argv) {
         std::vector<uint16_t> mh((size_t)n_tok * n_kv);
         for (int t = 0; t < n_tok; t++)
             for (int j = 0; j < n_kv; j++) mh[(size_t)t * n_kv + j] = j > n_past + t ? 0xfc00u : 0;
-        void * d = dev_alloc(mh.size() * 2);
+        void * d = cache_alloc(mh.size() * 2);          // a graph input: in the backend's compute buffer
         CHECK(mi355x_buffer_set(d, mh.data(), mh.size() * 2, nullptr));
         return d;
     };
@@ -193,6 +238,14 @@ int main(int argc, char ** argv) {
         const mi355x_tensor o = view(out_dev, MI355X_TYPE_F32, D, H, n_tok, 4, 4 * D, 4 * NSTATE);
         const mi355x_tensor m = view(mask, MI355X_TYPE_F16, n_kv, n_tok, 1, 2, 2 * (size_t)n_kv, 2 * (size_t)n_kv * n_tok);
         for (const auto & l : layers) {
+            if (with_write) {
+                // ggml_cpy(Kcur, ggml_view_1d(kv_self.k, n_tokens * n_state, offset of row n_past)), src/crispasr.cpp:3185-3203
+                const mi355x_tensor src = flat(kv_new, MI355X_TYPE_F32, (int64_t)n_tok * NSTATE);
+                const mi355x_tensor dk = flat((char *)l.ks + (size_t)n_past * NSTATE * 2, MI355X_TYPE_F16, (int64_t)n_tok * NSTATE);
+                const mi355x_tensor dv = flat((char *)l.vs + (size_t)n_past * NSTATE * 2, MI355X_TYPE_F16, (int64_t)n_tok * NSTATE);
+                CHECK(mi355x_cpy(&src, &dk, nullptr));
+                CHECK(mi355x_cpy(&src, &dv, nullptr));
+            }
             const mi355x_tensor ks = view(l.ks, MI355X_TYPE_F16, D, n_kv, H, 2, 2 * NSTATE, 2 * D);
             const mi355x_tensor vs = view(l.vs, MI355X_TYPE_F16, D, n_kv, H, 2, 2 * NSTATE, 2 * D);
             const mi355x_tensor kc = view(l.kc, MI355X_TYPE_F16, D, NENC, H, 2, 2 * NSTATE, 2 * D);
@@ -219,7 +272,11 @@ int main(int argc, char ** argv) {
         CHECK(mi355x_stream_synchronize(nullptr));
         phases[ph].ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     }
-    printf("{\"layers\": %d, \"self_check_max_abs\": %.3e", L, err);
+    size_t mirror = 0, valid = 0, uploaded = 0;
+    if (g_host) CHECK(mi355x_host_buffer_mirror_stats(layers[0].kc, &mirror, &valid, &uploaded));
+    printf("{\"layers\": %d, \"buffers\": \"%s\", \"kv_write_per_decode\": %s, \"self_check_max_abs\": %.3e", L, g_host ? "host-visible, caches mirrored in HBM" : "HBM",
+           with_write ? "true" : "false", err);
+    if (g_host) printf(", \"cross_cache_mirror\": {\"mirror_bytes\": %zu, \"valid_bytes\": %zu, \"uploaded_bytes\": %zu}", mirror, valid, uploaded);
     for (const auto & p : phases)
         printf(", \"%s\": {\"ms_total\": %.3f, \"ms_per_decode\": %.4f, \"us_per_attention_call\": %.2f}", p.name, p.ms, p.ms / p.n,
                p.ms * 1e3 / ((double)p.n * 2 * L));

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define MI355X_FATTN_API_VERSION 4
+#define MI355X_FATTN_API_VERSION 5
 
 /* ggml type ids of the storage types this path meets */
 enum mi355x_type {
@@ -297,9 +297,31 @@ int mi355x_set_rows(const mi355x_tensor * src, const void * idx, int32_t idx_typ
 int mi355x_buffer_alloc(size_t size, void ** ptr);                 /* alloc_buffer (256-byte aligned) */
 int mi355x_buffer_free(void * ptr);                                /* free_buffer */
 /* pinned host memory the GPU can address at the same pointer (hipHostMalloc, mapped + coherent): the
- * is_host buffer type a one-op backend needs so that ggml-cpu keeps running every other op on it */
+ * is_host buffer type a one-op backend needs so that ggml-cpu keeps running every other op on it.
+ *
+ * The runtimes put their KV caches into the first GPU device's default buffer type (src/crispasr.cpp:3942-3971,
+ * src/voxtral.cpp:1137-1145), i.e. into such a buffer, and attention reads them on every call.  So that those reads do not
+ * cross the host link each time, a buffer grows a MIRROR in HBM - an allocation of its own size - when mi355x_cpy or
+ * mi355x_set_rows first writes into it (the KV writes of the graphs).  From then on:
+ *   - the host copy stays complete and authoritative; the mirror is kept page by page (64 KiB), a page being up to date or
+ *     stale.  Every write through this library - mi355x_cpy, mi355x_set_rows, mi355x_buffer_memset / _set / _copy -
+ *     stores the same bytes to both copies (the kernels store twice; no second launch), having fetched the stale pages it
+ *     touches from the host copy first;
+ *   - mi355x_flash_attn_ext reads a K or V that lies in the buffer from the mirror (stale pages of the view's span are
+ *     fetched first, once), and mi355x_cpy a source that lies there; Q, the mask and the result stay where they are;
+ *   - nothing but this library may write into the buffer's memory once it has a mirror - a caller that lets the CPU store
+ *     into it directly (or another device) says so with mi355x_host_buffer_invalidate before the next call;
+ *   - all calls that touch one buffer belong on one stream at a time (the bookkeeping is done when a call is enqueued).
+ *     While a stream is being captured into a HIP graph, writes go to the host copy alone (their pages turn stale) and
+ *     reads take the mirror only where it is up to date already: replays bypass the bookkeeping.
+ * MI355X_NO_MIRROR=1 in the environment switches mirrors off (comparison runs). */
 int mi355x_host_buffer_alloc(size_t size, void ** ptr);
 int mi355x_host_buffer_free(void * ptr);
+/* ptr: any address inside a host buffer.  mirror_bytes: 0 while the buffer has no mirror, else its size; valid_bytes:
+ * bytes of pages that are up to date; uploaded_bytes: bytes fetched from the host copy so far.  Any of the three may be NULL. */
+int mi355x_host_buffer_mirror_stats(const void * ptr, size_t * mirror_bytes, size_t * valid_bytes, size_t * uploaded_bytes);
+/* [ptr, ptr + size) of a host buffer has been written behind the library's back: its pages are stale */
+int mi355x_host_buffer_invalidate(void * ptr, size_t size);
 /* memset_tensor / clear: asynchronous on the stream, done by a fill kernel (no memset node if the caller captures a graph) */
 int mi355x_buffer_memset(void * ptr, int value, size_t size, void * stream);
 int mi355x_buffer_set(void * dst, const void * host_src, size_t size, void * stream);   /* set_tensor  (sync) */
