@@ -270,6 +270,19 @@ int mirror_for_read(const mi355x_tensor * t, hipStream_t st, void ** data) {
     return MI355X_OK;
 }
 
+// A kernel is about to write the view `t` through its host address alone (an attention result, a mask): should the
+// buffer have a mirror, the pages of the view's span are stale from now on.
+void mirror_note_host_write(const mi355x_tensor * t) {
+    if (g_no_mirror || !t || !t->data) return;
+    size_t n = 0;
+    view_span(t, &n);
+    std::lock_guard<std::mutex> lk(g_mu);
+    HostBuf * b = hostbuf_of(t->data, n);
+    if (!b || !b->mirror || n == 0) return;
+    const size_t off = (size_t)((const char *)t->data - b->base);
+    for (size_t p = off / MIRROR_PAGE; p < (off + n + MIRROR_PAGE - 1) / MIRROR_PAGE; p++) b->valid[p] = 0;
+}
+
 // a mask argument with no extent is the same as no mask
 bool has_mask(const mi355x_tensor * mask) { return mask && mask->ne[0] > 0; }
 
@@ -746,6 +759,7 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     }
     k = &km;
     v = &vm;
+    mirror_note_host_write(dst);
     FattnArgs a;
     fill_args(a, q, k, v, mask, (float *)dst->data, params);
     if ((int64_t)a.Nq * a.Hq * a.B == 0) return MI355X_OK;
@@ -945,6 +959,7 @@ static int relpos_run(const mi355x_tensor * qv, const mi355x_tensor * r, const m
         a.Ha = (int)add->ne[2]; a.Ba = (int)add->ne[3];
         a.add_f16 = add->type == MI355X_TYPE_F16;
     }
+    mirror_note_host_write(dst);
     a.out = (char *)dst->data; a.nbo1 = dst->nb[1]; a.nbo2 = dst->nb[2]; a.nbo3 = dst->nb[3];
     a.out_al4 = !((uintptr_t)dst->data % 4) && !(dst->nb[1] % 4) && !(dst->nb[2] % 4) && !(dst->nb[3] % 4);
     a.scale = scale;
@@ -1115,6 +1130,7 @@ static int relpos_fused_run(const mi355x_tensor * q_u, const mi355x_tensor * q_v
         g.Ha = (int)add->ne[2]; g.Ba = (int)add->ne[3];
         g.add_f16 = add->type == MI355X_TYPE_F16;
     }
+    mirror_note_host_write(dst);
     g.dst = (float *)dst->data;
     g.D = a.D; g.Nq = a.Nq; g.Nkv = a.Nkv; g.H = a.Hq; g.B = a.B; g.gqa = a.gqa; g.bq = a.bq;
     g.scale = params->scale;

@@ -148,6 +148,16 @@ def test_writes_behind_the_librarys_back_need_invalidate_and_buffer_calls_keep_b
     up_before = vbuf.mirror_stats()["uploaded_bytes"]
     check("again")
     assert vbuf.mirror_stats()["uploaded_bytes"] == up_before                    # nothing more crossed the link
+    # 4. an attention result goes to its host address alone: where that lies in a mirrored buffer (a compute buffer whose
+    #    regions the graph allocator hands out again and again) a later read through the mirror must not see the old bytes
+    obuf = ca.HostBuffer(4 * D * H * 3)
+    o = ca.Tensor(obuf, ca.F32, (D, H, 3, 1))
+    K.cpy(ca.Tensor.from_host(np.zeros(D * H * 3, np.float32).view(np.uint8), ca.F32, (D, H, 3, 1)), o)     # mirrored, up to date: zeros
+    K.flash_attn_ext(dq, k, v, None, 0.125, out=o)
+    back = ca.Tensor.empty(ca.F32, (D, H, 3, 1))
+    K.cpy(o, back)                                                                # a source inside a mirrored buffer
+    torch.cuda.synchronize()
+    assert np.array_equal(back.numpy_f32(), o.numpy_f32()) and np.abs(o.numpy_f32()).max() > 0
 
 
 def test_a_graph_capture_never_reads_a_stale_mirror():
