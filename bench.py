@@ -355,7 +355,7 @@ def bench_decode(args, ca, ora, torch):
     return out
 
 
-def bench_roofline_decode(ca, ora, torch):
+def bench_roofline_decode(ca, ora, torch, quick=False):
     """The decode half of the metric as roofline entries: algorithmic bytes of one decode STEP (every layer's calls) over the
     time of that step inside a HIP graph, against the 8 TB/s HBM peak.
       C3_step: Whisper large-v3 decoder step with beam 5 - 32 layers x (self-attention, 1 query per beam against its own
@@ -381,6 +381,9 @@ def bench_roofline_decode(ca, ora, torch):
         return dst.buf
 
     def timed(name, label, calls, steps_in_graph, bytes_per_step, reps, note):
+        if quick:                                    # counter runs serialise every dispatch: a couple of replays are enough
+            reps = 1
+
         def replay_body():
             for c in calls:
                 ca.flash_attn_ext(c["q"], c["k"], c["v"], c.get("mask"), c["scale"], out=c["out"])
@@ -393,8 +396,16 @@ def bench_roofline_decode(ca, ora, torch):
             with torch.cuda.graph(graph, stream=side):
                 replay_body()
         torch.cuda.synchronize()
-        for _ in range(reps):                        # the clock settles
-            graph.replay()
+        # the clock controller takes some 15 ms of load to settle after an idle spell (kernel durations rise by a third a few
+        # milliseconds in and come back): replay for 40 ms before timing
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        if not quick:
+            for _ in range(min(400, max(reps, int(40.0 / max(e0.elapsed_time(e1), 1e-3))))):
+                graph.replay()
         torch.cuda.synchronize()
         # five groups of `reps` replays that follow each other without the host in between; the median group
         ev = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
@@ -881,6 +892,7 @@ def main():
     ap.add_argument("--roofline-decode-only", action="store_true",
                     help="run only the decode roofline entries (C3 step, C4 step, ceilings) and print them as the JSON line (profiling: "
                          "every shape then has a (kernel, grid) pair of its own in the kernel trace)")
+    ap.add_argument("--quick", action="store_true", help="with --roofline-decode-only: few replays (runs under rocprofv3 --pmc)")
     ap.add_argument("--relpos-only", action="store_true",
                     help="run only the FastConformer rel-pos configuration and print its figures as the JSON line (profiling)")
     args = ap.parse_args()
@@ -901,7 +913,7 @@ def main():
         f"roofline constants: f16 dense MFMA {PEAK_F16_TFLOPS} TFLOP/s, HBM {PEAK_HBM_GBS} GB/s")
 
     if args.roofline_decode_only:
-        print(json.dumps({"roofline_decode": bench_roofline_decode(ca, ora, torch)}), flush=True)
+        print(json.dumps({"roofline_decode": bench_roofline_decode(ca, ora, torch, args.quick)}), flush=True)
         return
     if args.relpos_only:
         lengths = [ora.randint(5, b, 400, 750) for b in range(8)]
