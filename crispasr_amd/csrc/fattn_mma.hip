@@ -497,10 +497,14 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         for (int kbi = 0; kbi < NKB; kbi++) {
             const int kb = KSP == 2 ? khalf * NKB + kbi : kbi;      // which 32 keys of the tile
             if (MLDS && kbi == 1 && !TAIL) {
-                // the second half was requested when the tile began; the only requests that can be younger than
-                // it are the next tile's first mask half (they follow block 0)
-                if (mn) __builtin_amdgcn_s_waitcnt(0x0F70 | NMH);
-                else    __builtin_amdgcn_s_waitcnt(0x0F70);
+                // the second half was requested when the tile began; younger than it are the next tile's K and V (requested
+                // right behind it) and the next tile's first mask half (behind block 0).  Loads return in order, so waiting
+                // until no more than those are outstanding is waiting for the half - and not for the K/V tile, which
+                // has until the end of this tile to land
+                static_assert(!MDMA || 2 * NLD + NMH <= 15, "wait count encoding");
+                if (mn)           __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * NLD + NMH));
+                else if (jn >= 0) __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * NLD));
+                else              __builtin_amdgcn_s_waitcnt(0x0F70);
             }
             // A block that the mask excludes altogether for this wave's queries - every entry -inf - contributes exact
             // zeros: it is skipped (wave-uniform), and the softmax state stays as it is.
