@@ -14,6 +14,13 @@
 // an address (here it is only a handle for the lookup below): each device holds its own copy at its own address.
 static __device__ __align__(256) unsigned char scratch[MI355X_NOALLOC_SCRATCH_BYTES];
 
+// Counters of launches that merge their split-KV partials in the kernel (FattnArgs::counters): zero when the library is
+// loaded, and left at zero by every launch.  Set 0 serves calls that run on the library's own scratch block, set 1 the
+// allocation-free entry point: each of the two is one-call-at-a-time per GPU by its contract, and a call of one may
+// overlap a call of the other.  A call on a caller's workspace may overlap anything and merges in a launch of its own.
+constexpr int MERGE_COUNTERS = 16384;
+static __device__ __align__(256) unsigned merge_counters[2 * MERGE_COUNTERS];
+
 namespace {
 
 thread_local char g_err[512] = "";
@@ -143,6 +150,30 @@ int noalloc_scratch(void ** out) {
     }
     *out = g_noalloc_scratch[dev];
     return MI355X_OK;
+}
+
+unsigned * g_merge_counters[64];   // per device: the address of merge_counters there
+bool       g_merge_counters_failed[64];
+const bool g_no_fused_merge = getenv("MI355X_NO_FUSED_MERGE") != nullptr;      // comparison runs: always the merge launch
+
+// the current device's counters of set `set`, or nullptr (then the caller merges in a launch of its own)
+unsigned * merge_counter_set(int set) {
+    if (set < 0 || g_no_fused_merge) return nullptr;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_merge_counters[dev] && !g_merge_counters_failed[dev]) {
+        void * ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(merge_counters)) != hipSuccess || !ptr) {
+            (void)hipGetLastError();
+            g_merge_counters_failed[dev] = true;
+        }
+        g_merge_counters[dev] = (unsigned *)ptr;
+    }
+    return g_merge_counters[dev] ? g_merge_counters[dev] + (size_t)set * MERGE_COUNTERS : nullptr;
 }
 
 // ---- host-visible buffers and their mirrors in HBM ---------------------------------------------------------------
@@ -292,6 +323,7 @@ struct Plan {
     int     keys_per_split;
     size_t  workspace;       // bytes in all: [f16 copies of K and V][split partials]
     size_t  ws_partials;     // offset of the split partials inside the workspace
+    int64_t merge_sets;      // > 0: the kernel can merge its splits itself, given this many counters
     bool    kv_to_f16;       // K and V are rounded to f16 copies in the workspace first (F32 / quantised K/V before the tile kernel; a
                              // K and a V of different types before any kernel)
 };
@@ -400,6 +432,8 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
     a.m1 = powf(2.0f, -(p->max_bias / 2.0f) / n2);
     a.n_splits = 1;
     a.keys_per_split = a.Nkv;
+    a.part_acc = a.part_ml = nullptr;
+    a.counters = nullptr;
 }
 
 // the same call on the f16 copies of K and V that kv_to_f16_launch leaves at ws: contiguous [D, Nkv, Hkv, Bk], V behind K
@@ -452,6 +486,7 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
     plan.workspace = 0;
     plan.kv_to_f16 = false;
     plan.ws_partials = 0;
+    plan.merge_sets = 0;
     // nothing to launch (no query rows) or nothing to read (no keys: the result is zeros): one range, no workspace
     if ((int64_t)a.Nq * a.Hq * a.B == 0 || a.Nkv == 0) return;
     // The tile kernel rounds F32 and Q8_0 K/V to f16 on their way into LDS anyway.  With enough queries to share the work it
@@ -533,6 +568,7 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         plan.n_splits = ns;
         plan.keys_per_split = a.Nkv > 0 ? kps : 0;
         if (ns > 1) plan.workspace += (size_t)rows * ns * (a.D + 2) * sizeof(float);
+        if (ns > 1 && kernel == MI355X_FATTN_DECODE_MMA && groups <= MERGE_COUNTERS) plan.merge_sets = groups;
     }
 }
 
@@ -681,6 +717,7 @@ int mi355x_fattn_plan_details(const mi355x_tensor * q, const mi355x_tensor * k, 
     info->keys_per_split = plan.keys_per_split;
     info->kv_to_f16      = plan.kv_to_f16 ? 1 : 0;
     info->workspace      = plan.workspace;
+    info->merge_in_kernel = plan.merge_sets > 0 && !params->workspace && !g_no_fused_merge ? 1 : 0;
     if (plan.kernel == MI355X_FATTN_MMA) {
         // the order of the call itself: the f16 copies first, then the question whether the tile kernel takes the shape
         int ktype = k->type;
@@ -716,9 +753,10 @@ int mi355x_fattn_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k
     return MI355X_OK;
 }
 
-int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+// counter_set: which of the library's counter sets a launch that merges its splits in the kernel may use (-1: none)
+static int flash_attn_run(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
                           const mi355x_tensor * mask, const mi355x_tensor * dst,
-                          const mi355x_fattn_params * params, void * stream) {
+                          const mi355x_fattn_params * params, void * stream, int counter_set) {
     if (!dst) return fail(MI355X_ERR_INVALID, "null dst");
     int rc = check(q, k, v, mask, dst, params);
     if (rc) return rc;
@@ -747,7 +785,7 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
         qq_view(q, (char *)ws + qq_q8_bytes(q), &qd);
         inner.workspace      = need ? (char *)ws + qb : nullptr;
         inner.workspace_size = need;
-        return mi355x_flash_attn_ext(&qd, k, v, mask, dst, &inner, stream);
+        return flash_attn_run(&qd, k, v, mask, dst, &inner, stream, counter_set);
     }
     // K and V of a cache that lives in a host buffer are read from that buffer's mirror in HBM
     mi355x_tensor km = *k, vm = *v;
@@ -806,16 +844,24 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
         const size_t rows = (size_t)a.Nq * a.Hq * a.B;
         a.part_acc = (float *)((char *)ws + plan.ws_partials);
         a.part_ml  = a.part_acc + rows * plan.n_splits * a.D;
+        if (plan.merge_sets > 0) a.counters = merge_counter_set(counter_set);
     }
     int e = plan.kernel == MI355X_FATTN_MMA   ? fattn_mma_launch(a, ktype, st)
             : plan.kernel == MI355X_FATTN_VEC ? fattn_vec_launch(a, ktype, st)
                                               : fattn_decode_launch(a, ktype, st);
     if (e) return hip_fail((hipError_t)e, "attention kernel launch");
-    if (plan.n_splits > 1) {
+    if (plan.n_splits > 1 && !a.counters) {
         e = fattn_merge_launch(a, st);
         if (e) return hip_fail((hipError_t)e, "fattn_merge launch");
     }
     return MI355X_OK;
+}
+
+int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                          const mi355x_tensor * mask, const mi355x_tensor * dst,
+                          const mi355x_fattn_params * params, void * stream) {
+    // on the library's scratch block (one call at a time per GPU by contract) the kernel may merge its splits itself
+    return flash_attn_run(q, k, v, mask, dst, params, stream, params && !params->workspace ? 0 : -1);
 }
 
 int mi355x_flash_attn_ext_noalloc(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
@@ -834,7 +880,7 @@ int mi355x_flash_attn_ext_noalloc(const mi355x_tensor * q, const mi355x_tensor *
     mi355x_fattn_params inner = *params;
     inner.workspace      = ptr;          // the kernels take the array's device address as they take any workspace
     inner.workspace_size = (size_t)MI355X_NOALLOC_SCRATCH_BYTES;
-    return mi355x_flash_attn_ext(q, k, v, mask, dst, &inner, stream);
+    return flash_attn_run(q, k, v, mask, dst, &inner, stream, 1);
 }
 
 // ---- copies ------------------------------------------------------------------------------

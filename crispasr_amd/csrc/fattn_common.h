@@ -50,6 +50,10 @@ struct FattnArgs {
     int32_t keys_per_split;
     float * part_acc;    // [rows, n_splits, D]  unnormalised accumulators
     float * part_ml;     // [rows, n_splits, 2]  running max, running sum
+    // nullptr: the partials are merged by fattn_merge_kernel, a launch of its own.  Else one counter per set of
+    // workgroups that share output rows (zero between launches): every workgroup adds one when its partials are out, and
+    // the one that finds the set complete merges the rows itself and leaves the counter at zero again.
+    unsigned * counters;
 };
 
 // Workgroups that use more than 64 KiB of dynamic LDS need hipFuncAttributeMaxDynamicSharedMemorySize raised, and that
@@ -125,6 +129,86 @@ static __device__ __forceinline__ float group_max(float x) {
     if (GROUP >= 32) x = fmaxf(x, xor_shuffle(x, 16));
     if (GROUP >= 64) x = fmaxf(x, xor_shuffle(x, 32));
     return x;
+}
+
+// ---- merging split-KV partials ---------------------------------------------------------
+// Loads and stores that are coherent across the whole device while the kernel runs (the L2 caches of the chip's eight
+// dies are not, for ordinary accesses): what workgroups of one launch hand to each other goes through these.
+static __device__ __forceinline__ void device_store(float * p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+static __device__ __forceinline__ float2 device_load2(const float2 * p) {
+    const uint64_t u = __hip_atomic_load((const uint64_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __builtin_bit_cast(float2, u);
+}
+static __device__ __forceinline__ float4 device_load4(const float4 * p) {
+    const float2 lo = device_load2((const float2 *)p), hi = device_load2((const float2 *)p + 1);
+    return make_float4(lo.x, lo.y, hi.x, hi.y);
+}
+
+// out[row] = sum_s acc_s * exp(m_s - M) / sum_s l_s * exp(m_s - M), for the four values d4*4 .. d4*4+3 of the row.
+// The (m, l) pairs and the accumulators of the first FATTN_MERGE_BATCH splits are requested together, so a row costs
+// one memory round trip, not one per split.  DEVICE: the partials come from other workgroups of this launch.
+constexpr int FATTN_MERGE_BATCH = 8;
+template <bool DEVICE>
+static __device__ __forceinline__ void fattn_merge_row(const FattnArgs & a, int64_t row, int d4) {
+    const int lpr = a.D / 4;
+    const float2 * pm = (const float2 *)(a.part_ml + (size_t)row * a.n_splits * 2);
+    const float4 * pa = (const float4 *)(a.part_acc + (size_t)row * a.n_splits * a.D) + d4;
+    float4 out = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    float  M = -INFINITY, L = 0.0f;
+    for (int s0 = 0; s0 < a.n_splits; s0 += FATTN_MERGE_BATCH) {
+        float2 ml[FATTN_MERGE_BATCH];
+        float4 v[FATTN_MERGE_BATCH];
+#pragma unroll
+        for (int i = 0; i < FATTN_MERGE_BATCH; i++) {
+            const int s = min(s0 + i, a.n_splits - 1);          // (past the end: a second look at the last one, not used)
+            ml[i] = DEVICE ? device_load2(pm + s) : pm[s];
+            v[i]  = DEVICE ? device_load4(pa + (size_t)s * lpr) : pa[(size_t)s * lpr];
+            if (s0 + i >= a.n_splits) ml[i] = make_float2(-INFINITY, 0.0f);
+        }
+        float Mb = M;
+#pragma unroll
+        for (int i = 0; i < FATTN_MERGE_BATCH; i++) Mb = fmaxf(Mb, ml[i].x);
+        if (Mb == -INFINITY) continue;              // nothing visible so far
+        const float f = __expf(M - Mb);             // M = -inf gives 0
+        L *= f; out.x *= f; out.y *= f; out.z *= f; out.w *= f;
+        M = Mb;
+#pragma unroll
+        for (int i = 0; i < FATTN_MERGE_BATCH; i++) {
+            // a split that saw no key carries m = -inf and an accumulator that must not be touched (select, not multiply)
+            const bool  seen = ml[i].x != -INFINITY;
+            const float w    = seen ? __expf(ml[i].x - M) : 0.0f;
+            L     += seen ? ml[i].y * w : 0.0f;
+            out.x += seen ? v[i].x * w : 0.0f;
+            out.y += seen ? v[i].y * w : 0.0f;
+            out.z += seen ? v[i].z * w : 0.0f;
+            out.w += seen ? v[i].w * w : 0.0f;
+        }
+    }
+    const float inv = L > 0.0f ? 1.0f / L : 0.0f;
+    out.x *= inv; out.y *= inv; out.z *= inv; out.w *= inv;
+    *((float4 *)(a.dst + (size_t)row * a.D) + d4) = out;
+}
+
+// The end of a workgroup that has stored its partials, when the launch merges in the kernel (a.counters): true for the
+// one workgroup of set `group` that finds the other n - 1 done.  The partials were stored by device_store (a thread that
+// used ordinary stores says so with `wrote_plain`, and pays for a write-back of its die's whole L2): every thread waits
+// for its stores to be acknowledged before the workgroup counts itself done, and the merging workgroup reads by
+// device_load.  All threads of the workgroup must call this; `flag` is a word of LDS that nothing else uses from here on.
+// The counter is zero again when the set is complete.
+static __device__ __forceinline__ bool fattn_last_of_set(const FattnArgs & a, int64_t group, int n, int * flag, bool wrote_plain) {
+    if (wrote_plain) __threadfence();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned old = __hip_atomic_fetch_add(a.counters + group, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool     all = old == (unsigned)(n - 1);
+        if (all) __hip_atomic_store(a.counters + group, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *flag = all;
+    }
+    __syncthreads();
+    return *flag != 0;
 }
 
 template <int GROUP>

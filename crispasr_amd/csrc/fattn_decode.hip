@@ -649,15 +649,23 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
             bad = bad || not_finite(acc);
             if (a.n_splits == 1) {
                 a.dst[row * D + d] = L > 0.0f ? acc / L : 0.0f;
+            } else if (a.counters) {
+                device_store(a.part_acc + (row * a.n_splits + split) * D + d, acc);
             } else {
                 a.part_acc[(row * a.n_splits + split) * D + d] = acc;
             }
         }
         if (a.n_splits > 1 && (tid & 15) == 0) {
-            // natural-log units, as the merge kernel expects them
+            // natural-log units, as the merge expects them
             float * pm = a.part_ml + (row * a.n_splits + split) * 2;
-            pm[0] = M == -INFINITY ? -INFINITY : M * 0.6931471805599453f;
-            pm[1] = L;
+            const float mn = M == -INFINITY ? -INFINITY : M * 0.6931471805599453f;
+            if (a.counters) {
+                device_store(pm, mn);
+                device_store(pm + 1, L);
+            } else {
+                pm[0] = mn;
+                pm[1] = L;
+            }
         }
     }
     // An excluded key was multiplied by a probability of zero above, not skipped.  For finite K/V that is the same thing; a
@@ -665,9 +673,11 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     // Such a row shows in its result, and is computed again the way the CPU op does it - excluded keys not read at all.
     // Without a mask every key is visible and a non-finite result is the answer.  (Columns 4w .. 4w + 3 belong to wave w
     // in both passes: the second store follows the first in the same wave.)
+    bool redone = false;
     if constexpr (MASK) {
         const uint64_t badmask = __builtin_amdgcn_ballot_w64(bad);
         if (badmask != 0) {
+            redone = true;
             __threadfence();
 #pragma unroll 1
             for (int c = 0; c < 4; c++) {
@@ -675,6 +685,15 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
                 if (((badmask >> (16 * c)) & 0xFFFFu) != 0 && r < R)
                     attn_row_redo<TYPE, D>(a, r / a.gqa, hk * a.gqa + r % a.gqa, b, split, k_begin, k_end);
             }
+        }
+    }
+    // the last of the n_splits workgroups of this (chunk, KV head, batch) merges its rows: no launch for the merge
+    if (a.n_splits > 1 && a.counters) {
+        if (!fattn_last_of_set(a, blockIdx.x / a.n_splits, a.n_splits, (int *)smem, redone)) return;
+        constexpr int LPR = D / 4;                  // lanes per row: 8 or 4 rows per pass
+        for (int c = tid / LPR; c < 16 && row0 + c < R; c += DEC_THREADS / LPR) {
+            const int r = row0 + c;
+            fattn_merge_row<true>(a, ((int64_t)b * a.Nq + r / a.gqa) * a.Hq + hk * a.gqa + r % a.gqa, tid % LPR);
         }
     }
 }

@@ -81,10 +81,7 @@ __global__ void __launch_bounds__(VEC_THREADS) fattn_vec_kernel(const FattnArgs 
     }
 }
 
-// out[row] = sum_s acc_s * exp(m_s - M) / sum_s l_s * exp(m_s - M)
-// D/4 lanes per row (one float4 of d each), 64 / (D/4) rows per wave.  The (m, l) pairs and the accumulators of the
-// first MERGE_BATCH splits are requested together, so a row costs one memory round trip, not one per split.
-constexpr int MERGE_BATCH = 8;
+// One row per D/4 lanes (a float4 of d each), 64 / (D/4) rows per wave.
 __global__ void __launch_bounds__(256) fattn_merge_kernel(const FattnArgs a, int rows) {
     const int lpr  = a.D / 4;                       // lanes per row
     const int rpw  = 64 / lpr;                      // rows per wave
@@ -92,42 +89,7 @@ __global__ void __launch_bounds__(256) fattn_merge_kernel(const FattnArgs a, int
     const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int row  = wave * rpw + lane / lpr;
     if (lane >= rpw * lpr || row >= rows) return;
-    const int d4 = lane % lpr;
-    const float2 * pm = (const float2 *)(a.part_ml + (size_t)row * a.n_splits * 2);
-    const float4 * pa = (const float4 *)(a.part_acc + (size_t)row * a.n_splits * a.D) + d4;
-    float4 out = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    float  M = -INFINITY, L = 0.0f;
-    for (int s0 = 0; s0 < a.n_splits; s0 += MERGE_BATCH) {
-        float2 ml[MERGE_BATCH];
-        float4 v[MERGE_BATCH];
-#pragma unroll
-        for (int i = 0; i < MERGE_BATCH; i++) {
-            const bool ok = s0 + i < a.n_splits;
-            ml[i] = ok ? pm[s0 + i] : make_float2(-INFINITY, 0.0f);
-            v[i]  = ok ? pa[(size_t)(s0 + i) * lpr] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-        }
-        float Mb = M;
-#pragma unroll
-        for (int i = 0; i < MERGE_BATCH; i++) Mb = fmaxf(Mb, ml[i].x);
-        if (Mb == -INFINITY) continue;              // nothing visible so far
-        const float f = __expf(M - Mb);             // M = -inf gives 0
-        L *= f; out.x *= f; out.y *= f; out.z *= f; out.w *= f;
-        M = Mb;
-#pragma unroll
-        for (int i = 0; i < MERGE_BATCH; i++) {
-            // a split that saw no key carries m = -inf and an accumulator that must not be touched (select, not multiply)
-            const bool  seen = ml[i].x != -INFINITY;
-            const float w    = seen ? __expf(ml[i].x - M) : 0.0f;
-            L     += seen ? ml[i].y * w : 0.0f;
-            out.x += seen ? v[i].x * w : 0.0f;
-            out.y += seen ? v[i].y * w : 0.0f;
-            out.z += seen ? v[i].z * w : 0.0f;
-            out.w += seen ? v[i].w * w : 0.0f;
-        }
-    }
-    const float inv = L > 0.0f ? 1.0f / L : 0.0f;
-    out.x *= inv; out.y *= inv; out.z *= inv; out.w *= inv;
-    *((float4 *)(a.dst + (size_t)row * a.D) + d4) = out;
+    fattn_merge_row<false>(a, row, lane % lpr);
 }
 
 template <int TYPE>

@@ -66,7 +66,7 @@ class CPlanInfo(ctypes.Structure):
     _fields_ = [("kernel", ctypes.c_int32), ("n_splits", ctypes.c_int32), ("keys_per_split", ctypes.c_int32),
                 ("kv_to_f16", ctypes.c_int32), ("workspace", ctypes.c_size_t),
                 ("queries_per_workgroup", ctypes.c_int32), ("query_blocks", ctypes.c_int32), ("key_split", ctypes.c_int32),
-                ("direct", ctypes.c_int32), ("mask_dma", ctypes.c_int32)]
+                ("direct", ctypes.c_int32), ("mask_dma", ctypes.c_int32), ("merge_in_kernel", ctypes.c_int32)]
 
 
 class CDeviceInfo(ctypes.Structure):
@@ -361,9 +361,9 @@ def flash_attn_plan(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor] = No
 
 def flash_attn_plan_details(q: Tensor, k: Tensor, v: Tensor, mask: Optional[Tensor] = None, scale: float = 1.0,
                             max_bias: float = 0.0, logit_softcap: float = 0.0, kernel: int = KERNEL_AUTO,
-                            n_splits: int = 0, tile_variant: int = 0) -> dict:
+                            n_splits: int = 0, tile_variant: int = 0, workspace: Optional[torch.Tensor] = None) -> dict:
     """Kernel, split count and - for the tile kernel - the instantiation the call takes."""
-    p = _params(scale, max_bias, logit_softcap, PREC_DEFAULT, kernel, n_splits, None, 0, tile_variant)
+    p = _params(scale, max_bias, logit_softcap, PREC_DEFAULT, kernel, n_splits, workspace, 0, tile_variant)
     info = CPlanInfo()
     _check(lib().mi355x_fattn_plan_details(q.ref(), k.ref(), v.ref(), mask.ref() if mask is not None else None,
                                            ctypes.byref(p), ctypes.byref(info)))

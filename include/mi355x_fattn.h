@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define MI355X_FATTN_API_VERSION 5
+#define MI355X_FATTN_API_VERSION 6
 
 /* ggml type ids of the storage types this path meets */
 enum mi355x_type {
@@ -87,7 +87,10 @@ typedef struct mi355x_fattn_params {
     void *  workspace;       /* NULL = library-owned scratch: one block per device, grown with hipMalloc when needed and
                               * shared by every call that passes NULL, so such calls (and replays of graphs that recorded
                               * them) belong on one stream at a time; while its stream is capturing, a call that would
-                              * have to grow the block is refused with MI355X_ERR_WORKSPACE instead.
+                              * have to grow the block is refused with MI355X_ERR_WORKSPACE instead.  (Such a call of the
+                              * split-KV decode kernel also merges its partial results inside the kernel - the last workgroup
+                              * to finish a set of key ranges does it - where a call on a caller's workspace, which may overlap
+                              * others, uses a second launch: same arithmetic, same bits.)
                               * Else 16-byte aligned.  With a caller's workspace of mi355x_fattn_workspace_size bytes the call allocates nothing
                               * and launches kernels only (no memset or copy nodes): it may be recorded into a HIP graph. */
     size_t  workspace_size;
@@ -204,6 +207,9 @@ typedef struct mi355x_fattn_plan_info {
     int32_t key_split;               /* 2: the waves of a workgroup pair up over the two halves of every 64-key tile */
     int32_t direct;                  /* K/V tiles move global -> LDS without passing registers */
     int32_t mask_dma;                /* the mask takes the same road */
+    int32_t merge_in_kernel;         /* 1: the split-KV partials are merged by the last workgroup to finish each set of ranges (no
+                                      * merge launch): calls on the library's scratch (params->workspace == NULL); the
+                                      * allocation-free entry point does the same for the same shapes */
 } mi355x_fattn_plan_info;
 int mi355x_fattn_plan_details(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
                               const mi355x_tensor * mask, const mi355x_fattn_params * params,

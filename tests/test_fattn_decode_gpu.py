@@ -130,3 +130,29 @@ def test_split_counts_and_caller_workspace():
     small = torch.empty(16, dtype=torch.float32, device="cuda")
     with pytest.raises(ggml.Mi355xError):
         ggml.flash_attn_ext(q, k, v, None, case["scale"], kernel=ggml.KERNEL_DECODE_MMA, n_splits=4, workspace=small)
+
+
+@pytest.mark.parametrize("spec", [
+    dict(seed=241, D=128, Nq=1, Nkv=663, Hq=32, Hkv=8, ktype=ora.Q8_0),                          # 7 ranges x 8 KV heads
+    dict(seed=242, D=64, Nq=5, Nkv=1500, Hq=20, q_layout="thd", kv_layout="thd", scale=64 ** -0.25),
+    dict(seed=243, D=64, Nq=1, Nkv=900, Hq=12, Hkv=4, B=3, ktype=ora.F16, mask="random_inf_batched"),
+    dict(seed=244, D=128, Nq=20, Nkv=700, Hq=4, Hkv=2, ktype=ora.F16, mask="causal"),            # 40 rows per KV head: three 16-row chunks
+], ids=lambda s: "seed%d" % s["seed"])
+def test_merge_in_the_kernel_equals_the_merge_launch(spec):
+    """On the library's scratch the last workgroup of every set of key ranges merges the set's rows itself; with a caller's
+    workspace the merge is a launch of its own.  Same arithmetic, same bits - call after call (the counters the first
+    form uses must be back at zero after every launch)."""
+    import torch
+    case = make_case(**spec)
+    q, k, v = upload(case["q"]), upload(case["k"]), upload(case["v"])
+    m = upload(case["mask"]) if case["mask"] is not None else None
+    info = ggml.flash_attn_plan_details(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA)
+    assert info["n_splits"] > 1 and info["merge_in_kernel"] == 1, info
+    ws = torch.empty(max(info["workspace"], 16), dtype=torch.uint8, device="cuda")
+    assert ggml.flash_attn_plan_details(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA, workspace=ws)["merge_in_kernel"] == 0
+    ref = run_oracle(case)
+    launch = ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA, workspace=ws).numpy_f32()
+    assert_parity(launch, ref, "merge launch")
+    for rep in range(3):
+        fused = ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA).numpy_f32()
+        assert np.array_equal(fused, launch), rep

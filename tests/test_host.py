@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(L, n), f"{n} declared in include/mi355x_fattn.h but not exported"
     assert sorted(ggml.EXPORTS) == names
-    assert L.mi355x_api_version() == 5
+    assert L.mi355x_api_version() == 6
     assert L.mi355x_status_string(0) == b"ok"
 
 

@@ -126,6 +126,25 @@ TILE = [
 ]
 
 
+def test_rows_computed_again_reach_the_merge_in_the_kernel():
+    """A row of a split launch that is computed a second time stores its partial with ordinary stores; the workgroup that
+    merges the set (possibly on another die) must still see it: the same bits as with the merge as a launch of its own."""
+    import torch
+    case = dead_key_case(list(TAIL(900, 600)) + [3, 64, 65], D=128, Nq=1, Nkv=900, Hq=16, Hkv=4, B=2, seed=951, ktype=ora.F16)
+    ref = run_oracle(case)
+    assert np.isfinite(ref).all()
+    q, k, v, m = (upload(case[n]) for n in ("q", "k", "v", "mask"))
+    info = ggml.flash_attn_plan_details(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA)
+    assert info["n_splits"] > 1 and info["merge_in_kernel"] == 1, info
+    ws = torch.empty(info["workspace"], dtype=torch.uint8, device="cuda")
+    launch = ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA, workspace=ws).numpy_f32()
+    assert_parity(launch, ref, "merge launch")
+    for rep in range(3):
+        fused = ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA).numpy_f32()
+        assert np.array_equal(fused, launch), rep
+
+
+
 @pytest.mark.parametrize("spec,variant,n_splits", TILE, ids=lambda s: "seed%d" % s["seed"] if isinstance(s, dict) else str(s))
 def test_tile_kernel_skips_excluded_keys(spec, variant, n_splits):
     n, nq = spec["Nkv"], spec["Nq"]
