@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import oracle as ora
-from cases import make_case, sweep_seeds, to_f32
+from cases import make_case, poison_rows, sweep_seeds, to_f32
 from crispasr_amd import ggml
 from gpu_util import assert_parity, plan_details, run_gpu, run_oracle
 
@@ -111,3 +111,58 @@ def test_random_shape_matches_oracle_on_every_kernel(seed):
                                       "tile kernel variant %d, split keys %s" % (variant, spec), exact, **tol)
             except (ggml.UnsupportedError, ggml.InvalidError):
                 pass
+
+
+def hidden_keys(case: dict):
+    """{(bk, hk): keys that no query row reading that K/V plane can see}: -inf for every query of every q head of the
+    GQA group and every batch entry that shares the plane."""
+    _, Nq, Hq, B = case["q"].ne
+    _, Nkv, Hkv, Bk = case["k"].ne
+    m = np.isneginf(to_f32(case["mask"])[:, :, :Nq, :Nkv])                  # [Bm, Hm, Nq, Nkv]
+    Bm, Hm = m.shape[:2]
+    out = {}
+    for bk in range(Bk):
+        for hk in range(Hkv):
+            dead = np.ones(Nkv, bool)
+            for b in range(bk * (B // Bk), (bk + 1) * (B // Bk)):
+                for h in range(hk * (Hq // Hkv), (hk + 1) * (Hq // Hkv)):
+                    dead &= m[b % Bm, h % Hm].all(axis=0)
+            if dead.any():
+                out[bk, hk] = np.nonzero(dead)[0]
+    return out
+
+
+@pytest.mark.parametrize("seed", [s for s in SEEDS if draw(s)["mask"] is not None][:40])
+def test_random_shape_with_non_finite_bits_in_hidden_cells(seed):
+    """The masked draws with a tenth of the keys hidden from every query on top of what the mask hides already, and NaN /
+    inf bit patterns written into every K/V row that no row reading it can see (the state of a cache that was never
+    cleared, src/voxtral.cpp:1137-1145): the result is the one over clean rows."""
+    spec = draw(seed)
+    spec.pop("variant")
+    case = make_case(**spec)
+    r = np.random.default_rng(77000 + seed)
+    m = ora.fp16_to_fp32(case["mask"].buf.view(np.uint16)).reshape(tuple(reversed(case["mask"].ne))).astype(np.float32)
+    Nkv = spec["Nkv"]
+    extra = np.nonzero(r.random(Nkv) < 0.1)[0]
+    extra = extra[extra > 0]                                   # key 0 stays as the draw has it
+    m[..., extra] = -np.inf
+    case["mask"] = ora.from_f32(m, ora.F16)
+    ref = run_oracle(case)
+    dead = hidden_keys(case)
+    for (bk, hk), keys in dead.items():
+        poison_rows(case["k"], keys, seed % 2, head=hk, batch=bk)
+        poison_rows(case["v"], keys, 1 - seed % 2, head=hk, batch=bk)
+    print("case", spec, "hidden keys per plane", {k: len(v) for k, v in dead.items()}, flush=True)
+    assert np.array_equal(run_oracle(case), ref)               # the oracle skips them
+    hot = spec.get("scale", 0.0) * spec["D"] ** 0.5 > 1.2
+    tol = dict(max_abs_tol=3e-3) if hot else {}
+    f16_kv = spec["ktype"] == ora.F16
+    auto_kernel = plan_details(case)["kernel"]
+    assert_parity_by_rows(run_gpu(case), ref, case, "auto %s" % spec, f16_kv or auto_kernel == ggml.KERNEL_VEC, **tol)
+    for kern in (ggml.KERNEL_VEC, ggml.KERNEL_MMA, ggml.KERNEL_DECODE_MMA):
+        for ns in (0, 3):
+            try:
+                got = run_gpu(case, kernel=kern, n_splits=ns)
+            except ggml.UnsupportedError:
+                continue
+            assert_parity_by_rows(got, ref, case, "kernel %d splits %d %s" % (kern, ns, spec), f16_kv or kern == ggml.KERNEL_VEC, **tol)

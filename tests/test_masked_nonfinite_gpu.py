@@ -11,38 +11,11 @@ import numpy as np
 import pytest
 
 import oracle as ora
-from cases import make_case
+from cases import poison_rows, make_case
 from crispasr_amd import ggml
 from gpu_util import assert_parity, plan_details, run_gpu, run_oracle, upload
 
 pytestmark = pytest.mark.gpu
-
-
-def poison_rows(t: ora.Tensor, keys, pattern: int):
-    """overwrite rows `keys` (dimension 1) of every head and batch of a K or V tensor with non-finite bit patterns"""
-    D, N, H, B = t.ne
-    rs = ora.row_size(t.type, D)
-    if t.type == ora.F16:
-        words = np.array([[0x7E00, 0xFFFF, 0x7C00, 0xFC00], [0x7C00, 0x7C00, 0xFC00, 0x7E01]][pattern], np.uint16)
-        row = np.resize(words, D).view(np.uint8)
-    elif t.type == ora.F32:
-        words = np.array([[0x7FC00000, 0xFFFFFFFF, 0x7F800000, 0xFF800000], [0x7F800000, 0x7F800000, 0xFF800000, 0x7FC00001]][pattern], np.uint32)
-        row = np.resize(words, D).view(np.uint8)
-    else:
-        bs = ora.TYPE_SIZE[t.type]
-        blk = np.full(bs, 0x5A, np.uint8)                       # arbitrary quants
-        blk[0:2] = np.array([[0x7E00], [0x7C00]][pattern], np.uint16).view(np.uint8)     # d = NaN / +inf
-        if t.type in (ora.Q4_1, ora.Q5_1):
-            blk[2:4] = np.array([[0xFC00], [0x7E00]][pattern], np.uint16).view(np.uint8)  # m = -inf / NaN
-        if t.type == ora.Q8_0 and pattern == 1:
-            blk[2:10] = 0                                       # inf * 0 quants as well
-        row = np.tile(blk, D // 32)
-    assert row.size == rs
-    for b in range(B):
-        for h in range(H):
-            for j in keys:
-                o = t.offset + j * t.nb[1] + h * t.nb[2] + b * t.nb[3]
-                t.buf[o:o + rs] = row
 
 
 def dead_key_case(dead, pattern=0, extra=None, **spec):
