@@ -394,7 +394,11 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     };
 
     float16v oacc[NQB][DB];
-    float16v negm[NQB];            // -m in all 16 slots: the C operand of the first Q.K^T MFMA
+    // -m in all 16 slots: the C operand of the first Q.K^T MFMA.  The masked form of 128-wide heads has no 16 registers for
+    // it (it answered with spills inside the tile loop, whose reloads wait for the tile's loads): it starts from zero and
+    // subtracts m with the mask.
+    constexpr bool SPLAT = !SOFTCAP && (KSP == 2 || (DIRECT && !MASK) || (NQB == 1 && D == 64));
+    float16v negm[SPLAT ? NQB : 1];
     RowState st[NQB];
 #pragma unroll
     for (int qb = 0; qb < NQB; qb++) {
@@ -402,7 +406,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         st[qb].l = 0.0f;
         st[qb].have = false;
 #pragma unroll
-        for (int r = 0; r < 16; r++) negm[qb][r] = 0.0f;
+        for (int r = 0; r < 16; r++) negm[SPLAT ? qb : 0][r] = 0.0f;
 #pragma unroll
         for (int db = 0; db < DB; db++)
 #pragma unroll
@@ -508,17 +512,27 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             }
             // A block that the mask excludes altogether for this wave's queries - every entry -inf - contributes exact
             // zeros: it is skipped (wave-uniform), and the softmax state stays as it is.
+            // The block's mask values leave LDS first, in one go and ahead of the operand reads below: LDS answers a wave in
+            // order, so a mask read issued behind those would make its consumer wait for all of them (and four reads issued
+            // one by one between the additions, as the compiler places them when left to itself, expose four round trips).
+            uint2 mval[NQB][4];
+            auto read_mask = [&]() __attribute__((always_inline)) {
+#pragma unroll
+                for (int qb = 0; qb < NQB; qb++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++)
+                        mval[qb][g] = MLDS ? *(const uint2 *)(mb + wave * (2 * MHALF) + kb * MHALF + qb * 2048 + maddr[g])
+                                           : mraw[MLDS ? 0 : qb][kbi][g];
+                if (MLDS) __builtin_amdgcn_sched_barrier(0);
+            };
+            if (SKIP) read_mask();          // (needed for the test below; the other forms read behind the score MFMAs)
             bool     excluded = false;
             uint32_t mdiff    = 0;
             if (SKIP) {
 #pragma unroll
                 for (int qb = 0; qb < NQB; qb++)
 #pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        const uint2 mv = MLDS ? *(const uint2 *)(mb + wave * (2 * MHALF) + kb * MHALF + qb * 2048 + maddr[g])
-                                              : mraw[MLDS ? 0 : qb][kbi][g];
-                        mdiff |= (mv.x ^ 0xFC00FC00u) | (mv.y ^ 0xFC00FC00u);
-                    }
+                    for (int g = 0; g < 4; g++) mdiff |= (mval[qb][g].x ^ 0xFC00FC00u) | (mval[qb][g].y ^ 0xFC00FC00u);
                 excluded = __builtin_amdgcn_ballot_w64(mdiff != 0) == 0;
             }
             if (excluded) {
@@ -530,7 +544,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             float16v s[NQB];
 #pragma unroll
             for (int qb = 0; qb < NQB; qb++) {
-                if (SOFTCAP) {          // the cap applies to the raw score: m is subtracted afterwards
+                if (!SPLAT) {           // (the cap applies to the raw score: m is subtracted afterwards)
 #pragma unroll
                     for (int r = 0; r < 16; r++) s[qb][r] = 0.0f;
                 } else {
@@ -542,6 +556,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
 #pragma unroll
                 for (int qb = 0; qb < NQB; qb++)
                     s[qb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka[K_AHEAD ? kbi & 1 : 0][ks], qreg[qb][ks], s[qb], 0, 0, 0);
+            if (MASK && !SKIP) read_mask();
             // operands needed next are requested now, so their LDS latency hides behind the softmax
             half8 va[2][DB];
             load_v(kb, va);
@@ -561,15 +576,14 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
                         // f16 halves enter the FMA directly (mixed-precision FMA, no separate conversion)
-                        const uint2 mv = MLDS ? *(const uint2 *)(mb + wave * (2 * MHALF) + kb * MHALF + qb * 2048 + maddr[g])
-                                              : mraw[MLDS ? 0 : qb][kbi][g];
+                        const uint2 mv = mval[qb][g];
                         const half2v w[2] = {__builtin_bit_cast(half2v, mv.x), __builtin_bit_cast(half2v, mv.y)};
 #pragma unroll
                         for (int e = 0; e < 4; e++)
                             s[qb][g * 4 + e] = fmaf(mslope, (float)w[e >> 1][e & 1], s[qb][g * 4 + e]);
                     }
             }
-            if (SOFTCAP) {
+            if (!SPLAT) {
 #pragma unroll
                 for (int qb = 0; qb < NQB; qb++)
 #pragma unroll
@@ -643,7 +657,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                     st[qb].m += delta;
                     st[qb].l *= f;
 #pragma unroll
-                    for (int r = 0; r < 16; r++) negm[qb][r] = -st[qb].m;
+                    for (int r = 0; r < 16; r++) negm[SPLAT ? qb : 0][r] = -st[qb].m;
 #pragma unroll
                     for (int db = 0; db < DB; db++)
 #pragma unroll
