@@ -256,27 +256,22 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
 #pragma unroll 1
     for (int t = 0; t < NTL; t++) {
         const bool tail = 32 * t + 32 > a.Nkv;             // uniform
-        // the additive mask of this tile: requested first, used after the products
-        float av[16];
+        // the additive mask of this tile: requested first, used after the products.  The values stay as loaded until
+        // then (a conversion inside the branch below would have to wait for its load right there, four round trips a step)
+        typedef typename std::conditional<ADD_F16, half4_a2, float4_a4>::type araw_t;
+        araw_t araw[4];
         if (ADD) {
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int key0 = 32 * t + 8 * g + 4 * hh;
                 if (!tail) {
-                    if (ADD_F16) {
-                        const half4_a2 x = *(const half4_a2 *)(addp + 8 * g * AES);
-#pragma unroll
-                        for (int c = 0; c < 4; c++) av[4 * g + c] = (float)x[c];
-                    } else {
-                        const float4_a4 x = *(const float4_a4 *)(addp + 8 * g * AES);
-#pragma unroll
-                        for (int c = 0; c < 4; c++) av[4 * g + c] = x[c];
-                    }
+                    araw[g] = *(const araw_t *)(addp + 8 * g * AES);
                 } else {
 #pragma unroll
                     for (int c = 0; c < 4; c++) {
                         const int key = min(key0 + c, a.Nkv - 1);
-                        av[4 * g + c] = ADD_F16 ? (float)*(const _Float16 *)(addrow + (int64_t)key * 2) : *(const float *)(addrow + (int64_t)key * 4);
+                        if constexpr (ADD_F16) araw[g][c] = *(const _Float16 *)(addrow + (int64_t)key * 2);
+                        else                   araw[g][c] = *(const float *)(addrow + (int64_t)key * 4);
                     }
                 }
             }
@@ -309,7 +304,7 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
             const float4v bd = *(const float4v *)&sq[il * FR_SQP + 8 * g + 4 * hh];
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                const float mk = ADD ? mul_then_add(bd[c], a.scale, av[4 * g + c]) : bd[c] * a.scale;   // as the graph: scale, then add
+                const float mk = ADD ? mul_then_add(bd[c], a.scale, (float)araw[g][c]) : bd[c] * a.scale;   // as the graph: scale, then add
                 const _Float16 mh = (_Float16)mk;
                 s2[4 * g + c] = fmaf((float)mh, FR_LOG2E, s[4 * g + c]);
             }
