@@ -621,8 +621,11 @@ def bench_configs(args, ca, ora, torch):
     Bytes = Q f32 + K,V in storage type once per KV head + mask f16 + out f32."""
     from cases import make_case, errors, MAX_ABS_TOL, REL_L2_TOL
     res = {}
+    only = getattr(args, "only_config", None)
 
     def run(name, spec, causal=False, note=""):
+        if only and only not in name:
+            return
         case = make_case(**spec)
         q, k, v = (ca.Tensor.from_host(t.buf, t.type, t.ne, t.nb, t.offset) for t in (case["q"], case["k"], case["v"]))
         mt = case["mask"]
@@ -675,7 +678,8 @@ def bench_configs(args, ca, ora, torch):
         run(f"C5_fastconformer_kv_{nm}", dict(seed=5, D=128, Nq=750, Nkv=750, Hq=8, B=8, ktype=kt, mask="bias_perhead_pad",
                                               lengths=lengths),
             note="8 heads x 128, T=750, batch 8, per-head f16 bias N(0, std 0.5) with -inf beyond each length (1 layer)")
-    res["C5_fastconformer_relpos_f32"] = bench_relpos(ca, ora, torch, lengths)
+    if not only:
+        res["C5_fastconformer_relpos_f32"] = bench_relpos(ca, ora, torch, lengths)
     # the reference's other call sites of the op, at their shapes
     run("voxtral_audio_encoder_f32", dict(seed=6, D=64, Nq=1500, Nkv=1500, Hq=20, ktype=ora.F32, q_layout="thd", kv_layout="thd"),
         note="core_attn::encoder_self_attn (src/core/attention.h:517-580, src/voxtral.cpp:676-687): 20 heads x 64, "
@@ -893,6 +897,9 @@ def main():
                     help="run only the decode roofline entries (C3 step, C4 step, ceilings) and print them as the JSON line (profiling: "
                          "every shape then has a (kernel, grid) pair of its own in the kernel trace)")
     ap.add_argument("--quick", action="store_true", help="with --roofline-decode-only: few replays (runs under rocprofv3 --pmc)")
+    ap.add_argument("--only-config", default=None, metavar="NAME",
+                    help="run only the baseline configurations whose name contains NAME (say C5_fastconformer_kv) and print "
+                         "their figures as the JSON line (profiling: the kernel trace then holds that configuration alone)")
     ap.add_argument("--relpos-only", action="store_true",
                     help="run only the FastConformer rel-pos configuration and print its figures as the JSON line (profiling)")
     args = ap.parse_args()
@@ -914,6 +921,9 @@ def main():
 
     if args.roofline_decode_only:
         print(json.dumps({"roofline_decode": bench_roofline_decode(ca, ora, torch, args.quick)}), flush=True)
+        return
+    if args.only_config:
+        print(json.dumps({"configs": bench_configs(args, ca, ora, torch)}), flush=True)
         return
     if args.relpos_only:
         lengths = [ora.randint(5, b, 400, 750) for b in range(8)]
