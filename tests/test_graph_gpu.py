@@ -85,6 +85,42 @@ def test_graph_replays_match_eager_calls():
     assert_parity(e_dec.numpy_f32(), run_oracle(host_case), "decode step after the replays")
 
 
+def test_graph_replays_of_a_call_that_merges_its_key_ranges_in_the_kernel():
+    """A split decode call on the library's scratch (sized by an eager call first) merges inside the kernel through counters
+    that every launch must leave at zero: recorded once and replayed with new contents, eager calls of the same kind in
+    between, it must keep giving what the call with a merge launch (a caller's workspace) gives."""
+    case = make_case(seed=961, D=128, Nq=1, Nkv=663, Hq=32, Hkv=8, ktype=ora.Q8_0)
+    q, k, v = upload(case["q"]), upload(case["k"]), upload(case["v"])
+    info = ggml.flash_attn_plan_details(q, k, v, None, case["scale"])
+    assert info["kernel"] == ggml.KERNEL_DECODE_MMA and info["n_splits"] > 1 and info["merge_in_kernel"] == 1, info
+    ws = torch.empty(info["workspace"], dtype=torch.uint8, device="cuda")
+    g_out, e_out, w_out = (ca.Tensor.empty(ca.F32, (128, 32, 1, 1)) for _ in range(3))
+    ggml.flash_attn_ext(q, k, v, None, case["scale"], out=e_out)       # sizes the scratch, loads the module
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(3):                                          # three launches share the counters back to back
+                ggml.flash_attn_ext(q, k, v, None, case["scale"], out=g_out, stream=side)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(6)
+    for replay in range(4):
+        q.buf.copy_(torch.from_numpy(rng.standard_normal(128 * 32, dtype=np.float32).view(np.uint8)).cuda())
+        g_out.buf.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ggml.flash_attn_ext(q, k, v, None, case["scale"], out=e_out)                   # eager, same counters
+        ggml.flash_attn_ext(q, k, v, None, case["scale"], out=w_out, workspace=ws)     # merge launch
+        torch.cuda.synchronize()
+        assert np.array_equal(g_out.numpy_f32(), w_out.numpy_f32()), replay
+        assert np.array_equal(e_out.numpy_f32(), w_out.numpy_f32()), replay
+    host = dict(case)
+    host.update(q=ora.Tensor(q.to_host(), ora.F32, case["q"].ne, case["q"].nb))
+    assert_parity(g_out.numpy_f32(), run_oracle(host), "after the replays")
+
+
 def test_graph_replays_of_the_relpos_attention_call_match_eager_calls():
     # a FastConformer block's attention (F32 K/V views, F32 table, pad mask) recorded with a caller's workspace:
     # table copy, mask kernel, K/V conversion and the tile kernel are all kernel nodes
