@@ -174,7 +174,10 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
  * MI355X_ERR_WORKSPACE and launches nothing (mi355x_fattn_workspace_size tells beforehand).
  * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race -
  * serialise them, or give the overlapping ones their own workspace through mi355x_flash_attn_ext.  Nothing in the array
- * has to start at zero: every byte a call reads has been written by that call's own kernels before.
+ * has to start at zero: every byte a call reads has been written by that call's own kernels before.  (Split-KV decode
+ * calls that merge inside the kernel count their workgroups in a second static array, 128 KiB of counters per GPU that
+ * starts at zero when the library is loaded and that every launch leaves at zero; this entry point and the calls on the
+ * library's scratch block use separate halves of it.)
  * The array's address is looked up once per device, on the first call there (or in mi355x_set_device).
  */
 #define MI355X_NOALLOC_SCRATCH_BYTES (32u << 20)
