@@ -691,6 +691,8 @@ def bench_configs(args, ca, ora, torch):
     run("decoder_cross_attn_f16", dict(seed=9, D=128, Nq=1, Nkv=375, Hq=8, q_layout="thd"),
         note="core_cross_attn::cross_attn_step (src/core/cross_attn.h:119-153): one decoder token against 375 encoder "
              "frames of f16 K/V, 8 heads x 128, no mask")
+    run("moonshine_cross_attn_d36_f32", dict(seed=10, D=36, Nq=1, Nkv=375, Hq=8, q_layout="thd", ktype=ora.F32),
+        note="the same call at Moonshine tiny's shape (8 heads x 36: a head size that is a multiple of 4 only), F32 K/V: vector kernel")
     return res
 
 

@@ -344,8 +344,11 @@ int check(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor 
     if (v->ne[1] != Nkv || v->ne[2] != Hkv || v->ne[3] != Bk) return fail(MI355X_ERR_INVALID, "k and v shapes differ");
     if (Hkv <= 0 || Bk <= 0 || Hq % Hkv || B % Bk) return fail(MI355X_ERR_INVALID, "q heads/batch not a multiple of kv heads/batch");
     if (v->ne[0] != D) return fail(MI355X_ERR_UNSUPPORTED, "DV %lld != DK %lld", (long long)v->ne[0], (long long)D);
-    if (D <= 0 || D % 8 || D > 256) return fail(MI355X_ERR_UNSUPPORTED, "head size %lld (need a multiple of 8, <= 256)", (long long)D);
+    // (multiples of 8 everywhere; 36 and 52 - the decoder cross-attention of src/core/cross_attn.h:119-153 in the smaller
+    //  Moonshine models - and the like run on the vector kernel)
+    if (D <= 0 || D % 4 || D > 256) return fail(MI355X_ERR_UNSUPPORTED, "head size %lld (need a multiple of 4, <= 256)", (long long)D);
     if ((FATTN_IS_BLOCK_TYPE(k->type) || FATTN_IS_BLOCK_TYPE(v->type)) && D % FATTN_QK8_0) return fail(MI355X_ERR_INVALID, "quantised rows need D %% 32 == 0");
+    if (D % 8 && k->type != v->type) return fail(MI355X_ERR_UNSUPPORTED, "head size %lld with K and V of different types", (long long)D);
     if (Nq < 0 || Nkv < 0 || Hq <= 0 || B <= 0) return fail(MI355X_ERR_INVALID, "negative or zero extent");
     if (q->nb[0] != 4) return fail(MI355X_ERR_UNSUPPORTED, "q rows must be contiguous (nb0 = %zu)", q->nb[0]);
     if (k->nb[0] != type_size(k->type) || v->nb[0] != type_size(v->type))

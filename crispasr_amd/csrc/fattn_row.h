@@ -11,9 +11,10 @@
 
 #include "fattn_common.h"
 
-// 8 consecutive elements of a K/V row starting at element d0, as f32 (exact for all types)
+// 8 consecutive elements of a K/V row starting at element d0, as f32 (exact for all types); of a row that ends inside
+// them (head sizes that are multiples of 4 only: aligned16 is false then) the first nvalid, zeros behind
 template <int TYPE>
-static __device__ __forceinline__ void row_load8(const char * row, int d0, bool aligned16, float (&out)[8]) {
+static __device__ __forceinline__ void row_load8(const char * row, int d0, bool aligned16, int nvalid, float (&out)[8]) {
     if constexpr (TYPE == MI355X_TYPE_F16) {
         const char * p = row + (size_t)d0 * 2;
         if (aligned16) {
@@ -27,7 +28,7 @@ static __device__ __forceinline__ void row_load8(const char * row, int d0, bool 
         } else {
             const uint16_t * h = (const uint16_t *)p;
 #pragma unroll
-            for (int i = 0; i < 8; i++) out[i] = h2f_bits(h[i]);
+            for (int i = 0; i < 8; i++) out[i] = i < nvalid ? h2f_bits(h[i]) : 0.0f;
         }
     } else if constexpr (TYPE == MI355X_TYPE_F32) {
         const char * p = row + (size_t)d0 * 4;
@@ -39,7 +40,7 @@ static __device__ __forceinline__ void row_load8(const char * row, int d0, bool 
         } else {
             const float * f = (const float *)p;
 #pragma unroll
-            for (int i = 0; i < 8; i++) out[i] = f[i];
+            for (int i = 0; i < 8; i++) out[i] = i < nvalid ? f[i] : 0.0f;
         }
     } else {  // block-32 types: blocks are only 2-byte aligned
         dequant8<TYPE>(row + (size_t)(d0 / FATTN_QK8_0) * fattn_block_bytes(TYPE), d0 % FATTN_QK8_0, out);
@@ -74,7 +75,8 @@ struct RowScanArgs {
 };
 static __device__ __forceinline__ RowScanArgs row_scan_args(const FattnArgs & a) {
     RowScanArgs r;
-    r.D = a.D; r.scale = a.scale; r.softcap = a.softcap; r.nbk1 = a.nbk1; r.nbv1 = a.nbv1; r.aligned16 = a.aligned16 != 0;
+    r.D = a.D; r.scale = a.scale; r.softcap = a.softcap; r.nbk1 = a.nbk1; r.nbv1 = a.nbv1;
+    r.aligned16 = a.aligned16 != 0 && a.D % 8 == 0;       // (a 16-byte load of a row's last 4 elements would run past the row)
     return r;
 }
 
@@ -97,6 +99,7 @@ static __device__ __forceinline__ void row_scan(const RowScanArgs & a, const flo
     const int  grp    = lane / LPR;
     const int  d0     = (lane % LPR) * 8;
     const int  d0c    = d0 < a.D ? d0 : 0;
+    const int  nv     = a.D - d0c;               // 8 or more, but for the last lane of a head size that is 4 modulo 8
     const bool al     = a.aligned16;
     const int  stride = NWAVES * G * ROW_UNROLL;
     // every lane runs the same trip count so that the DPP reductions see full groups
@@ -110,12 +113,12 @@ static __device__ __forceinline__ void row_scan(const RowScanArgs & a, const flo
         for (int u = 0; u < ROW_UNROLL; u++) {
             jj[u] = j0 + (u * NWAVES + wave) * G + grp;
             const int jc = min(jj[u], k_end - 1);
-            row_load8<TYPE_K>(kbase + (size_t)jc * a.nbk1, d0c, al, kf[u]);
+            row_load8<TYPE_K>(kbase + (size_t)jc * a.nbk1, d0c, al, nv, kf[u]);
         }
 #pragma unroll
         for (int u = 0; u < ROW_UNROLL; u++) {
             const int jc = min(jj[u], k_end - 1);
-            row_load8<TYPE_V>(vbase + (size_t)jc * a.nbv1, d0c, al, vf[u]);
+            row_load8<TYPE_V>(vbase + (size_t)jc * a.nbv1, d0c, al, nv, vf[u]);
         }
         float mloc = -INFINITY;
 #pragma unroll
@@ -176,11 +179,13 @@ static __device__ __forceinline__ void row_store(const FattnArgs & a, const RowP
         const float inv = st.l > 0.0f ? 1.0f / st.l : (st.l == st.l ? 0.0f : st.l);      // a NaN sum stays NaN, as on the CPU
         float * out = a.dst + row * a.D + d0;
 #pragma unroll
-        for (int e = 0; e < 8; e++) out[e] = st.acc[e] * inv;
+        for (int e = 0; e < 8; e++)
+            if (e < 4 || d0 + e < a.D) out[e] = st.acc[e] * inv;        // (D is a multiple of 4)
     } else {
         float * pa = a.part_acc + (row * a.n_splits + split) * a.D + d0;
 #pragma unroll
-        for (int e = 0; e < 8; e++) pa[e] = st.acc[e];
+        for (int e = 0; e < 8; e++)
+            if (e < 4 || d0 + e < a.D) pa[e] = st.acc[e];
         if (lane == 0) {
             float * pm = a.part_ml + (row * a.n_splits + split) * 2;
             pm[0] = st.m;
@@ -233,7 +238,7 @@ struct RowMaskRelpos {
     __device__ __forceinline__ bool present() const { return true; }
     __device__ __forceinline__ float operator()(int j) const {
         float r[8];
-        row_load8<MI355X_TYPE_F16>(rrow0 + (int64_t)j * nbr1, d0, true, r);
+        row_load8<MI355X_TYPE_F16>(rrow0 + (int64_t)j * nbr1, d0, true, 8, r);
         float dot = 0.0f;
 #pragma unroll
         for (int e = 0; e < 8; e++) dot = fmaf(qv[e], r[e], dot);

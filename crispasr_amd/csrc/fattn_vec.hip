@@ -24,8 +24,7 @@ __global__ void __launch_bounds__(VEC_THREADS) fattn_vec_kernel(const FattnArgs 
     const int tid  = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
-    const int d0   = (lane % LPR) * 8;          // the lane's 8 elements of d
-    const bool dvalid = d0 < a.D;               // D is a multiple of 8
+    const int d0   = (lane % LPR) * 8;          // the lane's 8 elements of d (D is a multiple of 4: the last lane may hold 4)
 
     // blockIdx.x = row * n_splits + split, row = (b*Nq + iq1)*Hq + h  (the dst row order)
     const int split = blockIdx.x % a.n_splits;
@@ -43,7 +42,7 @@ __global__ void __launch_bounds__(VEC_THREADS) fattn_vec_kernel(const FattnArgs 
     {
         const float * qrow = (const float *)(a.q + iq1 * a.nbq1 + h * a.nbq2 + b * a.nbq3);
 #pragma unroll
-        for (int e = 0; e < 8; e++) q[e] = dvalid ? qrow[d0 + e] : 0.0f;
+        for (int e = 0; e < 8; e++) q[e] = d0 + e < a.D ? qrow[d0 + e] : 0.0f;
     }
     const char * kbase = a.k + hk * a.nbk2 + bk * a.nbk3;
     const char * vbase = a.v + hk * a.nbv2 + bk * a.nbv3;

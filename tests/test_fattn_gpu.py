@@ -31,6 +31,14 @@ SHAPES = [
     dict(seed=17, D=256, Nq=2, Nkv=70, Hq=2, ktype=ora.F16),
     dict(seed=18, D=64, Nq=3, Nkv=1000, Hq=2, ktype=ora.F32, kv_layout="gap"),
     dict(seed=19, D=128, Nq=2, Nkv=513, Hq=4, Hkv=1, ktype=ora.F16, kv_layout="gap", mask="random_inf"),
+    # head sizes that are multiples of 4 only: core_cross_attn::cross_attn_step (src/core/cross_attn.h:119-153) at Moonshine
+    # tiny (8 heads x 36) and base (8 x 52): one decoder token, or a few, against the encoder's frames; and other odd ones
+    dict(seed=20, D=36, Nq=1, Nkv=375, Hq=8, q_layout="thd", ktype=ora.F32),
+    dict(seed=21, D=52, Nq=3, Nkv=200, Hq=8, q_layout="thd", ktype=ora.F16),
+    dict(seed=22, D=36, Nq=5, Nkv=61, Hq=4, Hkv=2, B=2, ktype=ora.F16, kv_layout="thd", mask="random_inf"),
+    dict(seed=23, D=12, Nq=2, Nkv=33, Hq=2, ktype=ora.F32, mask="bias", max_bias=2.0),
+    dict(seed=24, D=100, Nq=4, Nkv=50, Hq=2, ktype=ora.F16, kv_layout="gap", softcap=10.0),
+    dict(seed=25, D=252, Nq=2, Nkv=40, Hq=2, ktype=ora.F32, mask="causal"),
 ]
 
 

@@ -82,8 +82,14 @@ def test_supports_rejects_contract_violations_and_uncovered_ops():
     k12 = ca.Tensor.__new__(ca.Tensor); k12.__dict__.update(_t(ca.F16, (64, 16, 8, 1)).__dict__); k12.type = 12   # a k-quant
     assert ggml.flash_attn_supports(q, k12, k12, None) == ggml.ERR_UNSUPPORTED
     assert ggml.flash_attn_supports(q, k, k, _t(ca.F32, (16, 4, 1, 1))) == ggml.ERR_UNSUPPORTED          # F32 mask
-    q72 = _t(ca.F32, (36, 4, 8, 1))
-    assert ggml.flash_attn_supports(q72, _t(ca.F16, (36, 16, 8, 1)), _t(ca.F16, (36, 16, 8, 1)), None) == ggml.ERR_UNSUPPORTED
+    # head sizes: multiples of 4 (Moonshine's 36 and 52, src/core/cross_attn.h:119-153) with K and V of one plain type
+    q36 = _t(ca.F32, (36, 4, 8, 1))
+    assert ggml.flash_attn_supports(q36, _t(ca.F16, (36, 16, 8, 1)), _t(ca.F16, (36, 16, 8, 1)), None) == ggml.OK
+    assert ggml.flash_attn_supports(q36, _t(ca.F32, (36, 16, 8, 1)), _t(ca.F32, (36, 16, 8, 1)), None) == ggml.OK
+    assert ggml.flash_attn_supports(q36, _t(ca.F16, (36, 16, 8, 1)), _t(ca.F32, (36, 16, 8, 1)), None) == ggml.ERR_UNSUPPORTED
+    assert ggml.flash_attn_plan(q36, _t(ca.F16, (36, 16, 8, 1)), _t(ca.F16, (36, 16, 8, 1)), None, 1.0)[0] == ggml.KERNEL_VEC
+    q38 = _t(ca.F32, (38, 4, 8, 1))
+    assert ggml.flash_attn_supports(q38, _t(ca.F16, (38, 16, 8, 1)), _t(ca.F16, (38, 16, 8, 1)), None) == ggml.ERR_UNSUPPORTED
     assert ggml.flash_attn_supports(q, k, _t(ca.F16, (32, 16, 8, 1)), None) == ggml.ERR_UNSUPPORTED      # DV != DK
     assert ggml.lib().mi355x_last_error() != b""
 
