@@ -497,7 +497,11 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
     // touching registers) read the result: same values, same rounding.
     plan.ws_partials = 0;
     const bool convertible = (ktype == MI355X_TYPE_F32 && a.kv_aligned16) || (ktype == MI355X_TYPE_Q8_0 && a.kv_aligned2);
-    if (mixed || (kernel == MI355X_FATTN_MMA && ((convertible && a.Nq >= 128) || narrow_quant(ktype)))) {
+    // (F32 rows of 128-wide heads are the costliest to stage through registers - that form still spills - so they are
+    //  converted from 0.4 GFLOP of work on, whatever the number of queries: 100 queries x 700 keys x 32 heads 30.9 -> 20.8 us,
+    //  127 x 127 x 64 heads 16.6 -> 15.2 us, 100 x 100 x 64 heads 13.5 us either way, 48 x 48 x 64 heads 8.3 against 11.6)
+    const bool heavy_f32 = ktype == MI355X_TYPE_F32 && a.D == 128 && (int64_t)a.Nq * a.Nkv * a.Hq * a.B >= 800000;
+    if (mixed || (kernel == MI355X_FATTN_MMA && ((convertible && (a.Nq >= 128 || heavy_f32)) || narrow_quant(ktype)))) {
         plan.kv_to_f16 = true;
         plan.workspace = ((size_t)2 * a.D * a.Nkv * a.Hkv * a.Bk * sizeof(uint16_t) + 255) / 256 * 256;
         plan.ws_partials = plan.workspace;
