@@ -189,6 +189,7 @@ struct HostBuf {
     char * base   = nullptr;
     size_t size   = 0;
     char * mirror = nullptr;
+    int    dev    = -1;                // the device that holds the mirror: calls made with another device current use the host copy
     std::vector<uint8_t> valid;        // per page
     size_t uploaded = 0;               // bytes brought up to date so far (statistics)
 };
@@ -255,17 +256,21 @@ int mirror_for_write(const mi355x_tensor * dst, hipStream_t st, int64_t * delta)
     const size_t off = (size_t)((const char *)dst->data - b->base);
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &cs) != hipSuccess) (void)hipGetLastError();
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) (void)hipGetLastError();
     if (!b->mirror) {
         void * m = nullptr;
-        if (cs != hipStreamCaptureStatusNone || hipMalloc(&m, b->size) != hipSuccess) {
+        if (cs != hipStreamCaptureStatusNone || dev < 0 || hipMalloc(&m, b->size) != hipSuccess) {
             (void)hipGetLastError();
             return MI355X_OK;                        // no mirror: the buffer stays a plain host buffer
         }
         b->mirror = (char *)m;
+        b->dev    = dev;
         b->valid.assign((b->size + MIRROR_PAGE - 1) / MIRROR_PAGE, 0);
     }
-    if (cs != hipStreamCaptureStatusNone) {
-        // a captured write would be replayed without this bookkeeping: keep it to the host copy, pages become stale
+    if (cs != hipStreamCaptureStatusNone || dev != b->dev) {
+        // a captured write would be replayed without this bookkeeping, and another GPU cannot store into this one's
+        // memory: keep the write to the host copy, the pages become stale
         const size_t p0 = off / MIRROR_PAGE, p1 = (off + n + MIRROR_PAGE - 1) / MIRROR_PAGE;
         for (size_t p = p0; p < p1; p++) b->valid[p] = 0;
         return MI355X_OK;
@@ -286,6 +291,9 @@ int mirror_for_read(const mi355x_tensor * t, hipStream_t st, void ** data) {
     std::lock_guard<std::mutex> lk(g_mu);
     HostBuf * b = hostbuf_of(t->data, n);
     if (!b || !b->mirror) return MI355X_OK;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) (void)hipGetLastError();
+    if (dev != b->dev) return MI355X_OK;             // the mirror lives on another GPU
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &cs) != hipSuccess) (void)hipGetLastError();
     const size_t off = (size_t)((const char *)t->data - b->base);
@@ -1417,7 +1425,11 @@ static int mirror_of_range(void * ptr, size_t size, hipStream_t st, HostBuf ** b
     hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(st, &cs) != hipSuccess) (void)hipGetLastError();
     const size_t off = (size_t)((char *)ptr - b->base);
-    if (cs != hipStreamCaptureStatusNone) {           // replays would bypass the bookkeeping: host copy only, pages stale
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) (void)hipGetLastError();
+    // replays would bypass the bookkeeping, and a call made with another GPU current must not touch this one's memory:
+    // host copy only, pages stale
+    if (cs != hipStreamCaptureStatusNone || dev != b->dev) {
         for (size_t p = off / MIRROR_PAGE; p < (off + size + MIRROR_PAGE - 1) / MIRROR_PAGE; p++) b->valid[p] = 0;
         return MI355X_OK;
     }

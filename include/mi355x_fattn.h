@@ -324,7 +324,9 @@ int mi355x_buffer_free(void * ptr);                                /* free_buffe
  *     into it directly (or another device) says so with mi355x_host_buffer_invalidate before the next call;
  *   - all calls that touch one buffer belong on one stream at a time (the bookkeeping is done when a call is enqueued).
  *     While a stream is being captured into a HIP graph, writes go to the host copy alone (their pages turn stale) and
- *     reads take the mirror only where it is up to date already: replays bypass the bookkeeping.
+ *     reads take the mirror only where it is up to date already: replays bypass the bookkeeping.  The mirror lives on the
+ *     GPU that was current at the buffer's first KV write; a call made with another GPU current treats the buffer the
+ *     same way (host copy only).
  * MI355X_NO_MIRROR=1 in the environment switches mirrors off (comparison runs). */
 int mi355x_host_buffer_alloc(size_t size, void ** ptr);
 int mi355x_host_buffer_free(void * ptr);
