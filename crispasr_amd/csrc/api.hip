@@ -583,7 +583,7 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         plan.n_splits = ns;
         plan.keys_per_split = a.Nkv > 0 ? kps : 0;
         if (ns > 1) plan.workspace += (size_t)rows * ns * (a.D + 2) * sizeof(float);
-        if (ns > 1 && kernel == MI355X_FATTN_DECODE_MMA && groups <= MERGE_COUNTERS) plan.merge_sets = groups;
+        if (ns > 1 && groups <= MERGE_COUNTERS) plan.merge_sets = groups;      // (vector kernel: one set per row)
     }
 }
 

@@ -170,8 +170,9 @@ static __device__ __forceinline__ void row_scan(const RowScanArgs & a, const flo
     }
 }
 
-// lanes 0 .. LPR-1 hold the row's final state: write dst, or this split's partial for fattn_merge_kernel (natural-log units)
-template <int LPR>
+// lanes 0 .. LPR-1 hold the row's final state: write dst, or this split's partial for the merge (natural-log units).
+// COHERENT: the partial goes out by device-coherent stores, for a merge by another workgroup of the same launch.
+template <int LPR, bool COHERENT = false>
 static __device__ __forceinline__ void row_store(const FattnArgs & a, const RowPartial & st, int64_t row, int split, int lane) {
     const int d0 = lane * 8;
     if (lane >= LPR || d0 >= a.D) return;
@@ -185,11 +186,19 @@ static __device__ __forceinline__ void row_store(const FattnArgs & a, const RowP
         float * pa = a.part_acc + (row * a.n_splits + split) * a.D + d0;
 #pragma unroll
         for (int e = 0; e < 8; e++)
-            if (e < 4 || d0 + e < a.D) pa[e] = st.acc[e];
+            if (e < 4 || d0 + e < a.D) {
+                if (COHERENT) device_store(pa + e, st.acc[e]);
+                else          pa[e] = st.acc[e];
+            }
         if (lane == 0) {
             float * pm = a.part_ml + (row * a.n_splits + split) * 2;
-            pm[0] = st.m;
-            pm[1] = st.l;
+            if (COHERENT) {
+                device_store(pm, st.m);
+                device_store(pm + 1, st.l);
+            } else {
+                pm[0] = st.m;
+                pm[1] = st.l;
+            }
         }
     }
 }

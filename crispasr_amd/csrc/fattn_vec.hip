@@ -76,7 +76,13 @@ __global__ void __launch_bounds__(VEC_THREADS) fattn_vec_kernel(const FattnArgs 
             for (int e = 0; e < 8; e++) o.acc[e] = sh[w][lane][2 + e];
             row_partial_merge(st, o);
         }
-        row_store<LPR>(a, st, row, split, lane);
+        if (a.counters) row_store<LPR, true>(a, st, row, split, lane);
+        else            row_store<LPR>(a, st, row, split, lane);
+    }
+    // the last of the row's n_splits workgroups merges them: no launch for the merge
+    if (a.n_splits > 1 && a.counters) {
+        __shared__ int last;
+        if (fattn_last_of_set(a, row, a.n_splits, &last, false) && tid < a.D / 4) fattn_merge_row<true>(a, row, tid);
     }
 }
 

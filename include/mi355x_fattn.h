@@ -88,7 +88,7 @@ typedef struct mi355x_fattn_params {
                               * shared by every call that passes NULL, so such calls (and replays of graphs that recorded
                               * them) belong on one stream at a time; while its stream is capturing, a call that would
                               * have to grow the block is refused with MI355X_ERR_WORKSPACE instead.  (Such a call of the
-                              * split-KV decode kernel also merges its partial results inside the kernel - the last workgroup
+                              * split-KV decode or vector kernel also merges its partial results inside the kernel - the last workgroup
                               * to finish a set of key ranges does it - where a call on a caller's workspace, which may overlap
                               * others, uses a second launch: same arithmetic, same bits.)
                               * Else 16-byte aligned.  With a caller's workspace of mi355x_fattn_workspace_size bytes the call allocates nothing
@@ -176,7 +176,7 @@ int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
  * MI355X_ERR_WORKSPACE and launches nothing (mi355x_fattn_workspace_size tells beforehand).
  * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race -
  * serialise them, or give the overlapping ones their own workspace through mi355x_flash_attn_ext.  Nothing in the array
- * has to start at zero: every byte a call reads has been written by that call's own kernels before.  (Split-KV decode
+ * has to start at zero: every byte a call reads has been written by that call's own kernels before.  (Split-KV
  * calls that merge inside the kernel count their workgroups in a second static array, 128 KiB of counters per GPU that
  * starts at zero when the library is loaded and that every launch leaves at zero; this entry point and the calls on the
  * library's scratch block use separate halves of it.)

@@ -169,3 +169,26 @@ def test_alibi_slope_applied_by_each_kernel_is_the_published_one(kernel, n_head)
     slopes = np.log(out[0, :, :, 0] / out[0, :, :, 1])
     want = np.array(_published_alibi_slopes(n_head))
     assert np.allclose(slopes, want[None, :], rtol=2e-3, atol=2e-3), (n_head, slopes[0], want)   # p is an f16 ratio in the MFMA kernels
+
+
+@pytest.mark.parametrize("spec", [
+    dict(seed=31, D=128, Nq=1, Nkv=663, Hq=32, ktype=ora.F32),                                   # Voxtral's step with K/V repeated to 32 heads, F32
+    dict(seed=32, D=80, Nq=3, Nkv=500, Hq=4, Hkv=2, B=2, ktype=ora.F16, mask="random_inf"),
+    dict(seed=33, D=36, Nq=2, Nkv=900, Hq=8, ktype=ora.F32, q_layout="thd"),
+], ids=lambda s: "seed%d" % s["seed"])
+def test_vec_kernel_merges_its_key_ranges_in_the_kernel_on_the_librarys_scratch(spec):
+    """As the decode kernel does: the last workgroup of a row's key ranges merges them when the call runs on the library's
+    scratch, a second launch does when the workspace is the caller's.  Same bits, call after call."""
+    import numpy as np
+    import torch
+    case = make_case(**spec)
+    q, k, v = upload(case["q"]), upload(case["k"]), upload(case["v"])
+    m = upload(case["mask"]) if case["mask"] is not None else None
+    kw = dict(kernel=ggml.KERNEL_VEC, n_splits=5)
+    info = ggml.flash_attn_plan_details(q, k, v, m, case["scale"], **kw)
+    assert info["n_splits"] == 5 and info["merge_in_kernel"] == 1, info
+    ws = torch.empty(info["workspace"], dtype=torch.uint8, device="cuda")
+    launch = ggml.flash_attn_ext(q, k, v, m, case["scale"], workspace=ws, **kw).numpy_f32()
+    assert_parity(launch, run_oracle(case), "merge launch %s" % spec)
+    for rep in range(3):
+        assert np.array_equal(ggml.flash_attn_ext(q, k, v, m, case["scale"], **kw).numpy_f32(), launch), rep
