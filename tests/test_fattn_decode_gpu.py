@@ -156,3 +156,18 @@ def test_merge_in_the_kernel_equals_the_merge_launch(spec):
     for rep in range(3):
         fused = ggml.flash_attn_ext(q, k, v, m, case["scale"], kernel=ggml.KERNEL_DECODE_MMA).numpy_f32()
         assert np.array_equal(fused, launch), rep
+
+
+def test_more_sets_of_key_ranges_than_counters_fall_back_to_the_merge_launch():
+    """The in-kernel merge counts workgroups in 16384 counters per GPU; a call with more sets than that keeps the merge
+    launch and says so in its plan."""
+    case = make_case(seed=245, D=64, Nq=1, Nkv=70, Hq=8, B=2100, mask="random_inf_batched")      # 16800 (head, batch) pairs
+    q, k, v, m = (upload(case[n]) for n in ("q", "k", "v", "mask"))
+    kw = dict(kernel=ggml.KERNEL_DECODE_MMA, n_splits=2)
+    info = ggml.flash_attn_plan_details(q, k, v, m, case["scale"], **kw)
+    assert info["n_splits"] == 2 and info["merge_in_kernel"] == 0, info
+    assert_parity(ggml.flash_attn_ext(q, k, v, m, case["scale"], **kw).numpy_f32(), run_oracle(case), "merge launch beyond the counters")
+    few = make_case(seed=246, D=64, Nq=1, Nkv=70, Hq=8, B=2000, mask="random_inf_batched")       # 16000: within
+    q, k, v, m = (upload(few[n]) for n in ("q", "k", "v", "mask"))
+    assert ggml.flash_attn_plan_details(q, k, v, m, few["scale"], **kw)["merge_in_kernel"] == 1
+    assert_parity(ggml.flash_attn_ext(q, k, v, m, few["scale"], **kw).numpy_f32(), run_oracle(few), "merge in the kernel at 16000 sets")
