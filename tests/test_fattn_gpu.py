@@ -1,5 +1,7 @@
 """GPU parity: the HIP kernels, called through the C-ABI, against the CPU oracle (exact mode)
 on the same seeded inputs.  Tolerance as stated for this path: max-abs 2e-3, rel-L2 1e-3."""
+import os
+
 import numpy as np
 import pytest
 
@@ -171,6 +173,7 @@ def test_alibi_slope_applied_by_each_kernel_is_the_published_one(kernel, n_head)
     assert np.allclose(slopes, want[None, :], rtol=2e-3, atol=2e-3), (n_head, slopes[0], want)   # p is an f16 ratio in the MFMA kernels
 
 
+@pytest.mark.skipif(os.environ.get("MI355X_NO_FUSED_MERGE") is not None, reason="the in-kernel merge is switched off in this environment")
 @pytest.mark.parametrize("spec", [
     dict(seed=31, D=128, Nq=1, Nkv=663, Hq=32, ktype=ora.F32),                                   # Voxtral's step with K/V repeated to 32 heads, F32
     dict(seed=32, D=80, Nq=3, Nkv=500, Hq=4, Hkv=2, B=2, ktype=ora.F16, mask="random_inf"),

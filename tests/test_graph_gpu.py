@@ -1,6 +1,8 @@
 """The entry points recorded into a HIP graph: replays must give what eager calls give, replay after replay, with
 eager work and synchronisations in between and with new input contents each time.  Callers that capture pass their
 own workspaces (the library's scratch may have to grow, which a capture cannot do)."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -85,6 +87,7 @@ def test_graph_replays_match_eager_calls():
     assert_parity(e_dec.numpy_f32(), run_oracle(host_case), "decode step after the replays")
 
 
+@pytest.mark.skipif(os.environ.get("MI355X_NO_FUSED_MERGE") is not None, reason="the in-kernel merge is switched off in this environment")
 def test_graph_replays_of_a_call_that_merges_its_key_ranges_in_the_kernel():
     """A split decode call on the library's scratch (sized by an eager call first) merges inside the kernel through counters
     that every launch must leave at zero: recorded once and replayed with new contents, eager calls of the same kind in

@@ -14,7 +14,10 @@ import crispasr_amd as ca
 import oracle as ora
 from cases import errors, MAX_ABS_TOL, REL_L2_TOL
 
-pytestmark = pytest.mark.gpu
+import os
+
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skipif(os.environ.get("MI355X_NO_MIRROR") is not None, reason="mirrors are switched off in this environment")]
 
 K = ca.ggml
 PAGE = 64 * 1024

@@ -7,6 +7,8 @@ kernel family is held to the exact oracle - which skips such keys - on caches wh
 and inf bit patterns (f16 / f32 values, block scales and minima)."""
 import math
 
+import os
+
 import numpy as np
 import pytest
 
@@ -99,6 +101,7 @@ TILE = [
 ]
 
 
+@pytest.mark.skipif(os.environ.get("MI355X_NO_FUSED_MERGE") is not None, reason="the in-kernel merge is switched off in this environment")
 def test_rows_computed_again_reach_the_merge_in_the_kernel():
     """A row of a split launch that is computed a second time stores its partial with ordinary stores; the workgroup that
     merges the set (possibly on another die) must still see it: the same bits as with the merge as a launch of its own."""
