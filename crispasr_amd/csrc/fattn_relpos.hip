@@ -36,6 +36,8 @@ namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float    float2v __attribute__((ext_vector_type(2)));
 typedef float    float16v __attribute__((ext_vector_type(16)));
 typedef float    float4v __attribute__((ext_vector_type(4)));
 typedef short    short4v __attribute__((ext_vector_type(4)));
@@ -45,7 +47,7 @@ typedef _Float16 half4_a2 __attribute__((ext_vector_type(4), aligned(2)));
 
 constexpr int   FR_SQP   = 36;                      // pitch of the un-skew square in floats
 constexpr float FR_LOG2E = 1.4426950408889634f;
-constexpr float FR_SLACK = 8.0f;                    // log2 of the largest probability kept before the reference is raised
+constexpr float FR_SUM_LIMIT = 4096.0f;               // a tile's 16 probabilities of a lane sum to at most this before the reference is raised
 
 template <int D> constexpr int fr_kp() { return 2 * D; }          // bytes per K / table row in LDS (chunks swizzled, no padding)
 template <int D> __device__ __forceinline__ int fr_swz(int r) { return D == 64 ? (r >> 1) & 7 : r & 15; }
@@ -303,10 +305,16 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
         for (int g = 0; g < 4; g++) {
             const float4v bd = *(const float4v *)&sq[il * FR_SQP + 8 * g + 4 * hh];
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const float mk = ADD ? mul_then_add(bd[c], a.scale, (float)araw[g][c]) : bd[c] * a.scale;   // as the graph: scale, then add
-                const _Float16 mh = (_Float16)mk;
-                s2[4 * g + c] = fmaf((float)mh, FR_LOG2E, s[4 * g + c]);
+            for (int c = 0; c < 4; c += 2) {
+                float2v mk;
+#pragma unroll
+                for (int e = 0; e < 2; e++)                    // as the graph: scale, then add
+                    mk[e] = ADD ? mul_then_add(bd[c + e], a.scale, (float)araw[g][c + e]) : bd[c + e] * a.scale;
+                uint32_t pk;                                   // rounded two at a time (the compiler converts one at a time)
+                asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(pk) : "v"(mk[0]), "v"(mk[1]));
+                const half2v mh = __builtin_bit_cast(half2v, pk);
+#pragma unroll
+                for (int e = 0; e < 2; e++) s2[4 * g + c + e] = fmaf((float)mh[e], FR_LOG2E, s[4 * g + c + e]);
             }
         }
         if (tail) {                                        // keys past the end of the last tile
@@ -317,31 +325,42 @@ __global__ void __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2,
         __builtin_amdgcn_wave_barrier();
 
         // ---- online softmax ----------------------------------------------------------------------------------------------
-        // The reference m of a row is raised only when the tile's maximum exceeds it by more than FR_SLACK (a factor 256):
-        // probabilities stay below 2^8 in f16, sums and accumulators are f32, and the accumulators are rescaled on a
-        // handful of steps instead of on most.
-        float tmax = s2[0];
+        // P = 2^(s2 - m) in f16 against the row's reference m as it stands; the row sum is taken over the rounded values
+        // the MFMA will use.  No maximum is computed on this path: a reference that has fallen too far behind shows up as
+        // a large (or infinite, or NaN) tile sum, and only then - and on a row's first step - is the tile done again
+        // with the reference raised to the tile's maximum.  Sums and accumulators are f32; a probability stays below
+        // FR_SUM_LIMIT in f16.
+        half8 p[2];
+        float lsum;
+        auto exp_tile = [&](float ref) __attribute__((always_inline)) {
+            const half2v ones = {(_Float16)1.0f, (_Float16)1.0f};
+            float dsum = 0.0f;
 #pragma unroll
-        for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, s2[r]);
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        if (__builtin_amdgcn_ballot_w64(tmax > m + FR_SLACK) != 0) {
-            const float mn = tmax > m + FR_SLACK ? tmax : m;
+            for (int r = 0; r < 16; r += 2) {
+                half2v p2;
+                p2[0] = (_Float16)__builtin_amdgcn_exp2f(s2[r] - ref);
+                p2[1] = (_Float16)__builtin_amdgcn_exp2f(s2[r + 1] - ref);
+                dsum = __builtin_amdgcn_fdot2(p2, ones, dsum, false);
+                p[r >> 3][r & 7]       = p2[0];
+                p[r >> 3][(r & 7) + 1] = p2[1];
+            }
+            lsum = dsum;
+        };
+        exp_tile(m == -INFINITY ? 0.0f : m);
+        if (__builtin_amdgcn_ballot_w64(!(lsum <= FR_SUM_LIMIT) || m == -INFINITY) != 0) {     // wave-uniform; rare after the first step
+            float tmax = s2[0];
+#pragma unroll
+            for (int r = 1; r < 16; r++) tmax = fmaxf(tmax, s2[r]);
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));      // both halves of a query must agree
+            const float mn = tmax > m ? tmax : m;
             const float f  = mn == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m - mn);     // m = -inf: nothing accumulated yet, f = 0
             l *= f;
 #pragma unroll
             for (int db = 0; db < DBO; db++) oacc[db] *= f;
             m = mn;
+            exp_tile(m == -INFINITY ? 0.0f : m);
         }
-        const float ms = m == -INFINITY ? 0.0f : m;
-        half8 p[2];
-        float ls[4] = {0.0f, 0.0f, 0.0f, 0.0f};           // four chains instead of one of sixteen dependent additions
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const float e = __builtin_amdgcn_exp2f(s2[r] - ms);
-            ls[r & 3] += e;
-            p[r >> 3][r & 7] = (_Float16)e;
-        }
-        l += (ls[0] + ls[1]) + (ls[2] + ls[3]);
+        l += lsum;
 
         // ---- O^T += V^T . P^T -------------------------------------------------------------------------------------------
         {
