@@ -229,6 +229,32 @@ def test_relpos_attention_random_shapes(seed):
     assert_parity(got, ref, str(spec), max_abs_tol=5e-3, rel_l2_tol=2e-3 if few else 1e-3)
 
 
+@pytest.mark.parametrize("D,add", [(128, "pad"), (64, None)])
+def test_relpos_attention_with_scores_that_grow_along_the_keys(D, add):
+    """K rows scaled up along the key axis: the softmax reference of the one-kernel form, set on a row's first tile, is
+    overtaken by far more than an f16 probability can hold and has to be raised again and again on the way"""
+    spec = dict(seed=341, D=D, Nq=100, Nkv=333, H=2, B=2, add=add)
+    c = make(qgain=0.7, **spec)
+    Nq, Nkv, H, B = c["Nq"], c["Nkv"], c["H"], c["B"]
+    quf = np.float32(0.7) * ora.randn(351, (B, H, Nq, D))
+    qu = strided(quf, "cont")
+    gain = np.linspace(0.2, 10.0, Nkv, dtype=np.float32)[None, None, :, None]
+    kf = ora.randn(352, (B, H, Nkv, D)) * gain
+    k, v = ora.from_f32(kf, ora.F16), ora.from_f32(ora.randn(353, (B, H, Nkv, D)), ora.F16)
+    mask = ora.relpos_bias(c["qv"], c["r"], c["add"], c["scale"], Nkv)
+    ref = ora.flash_attn_ext(qu, k, v, mask, c["scale"])
+    scores = np.einsum("bhqd,bhkd->bhqk", quf, kf) * c["scale"]
+    # the largest score of a row's later tiles exceeds that of its first 32 keys by more than 16 / log2(e) in most rows
+    lead = scores[..., 32:].max(-1) - scores[..., :32].max(-1)
+    assert np.median(lead) > 16 / 1.4427
+    print("relpos attention, growing scores", spec, "median lead %.1f" % np.median(lead), flush=True)
+    got = ggml.flash_attn_relpos(upload(qu), upload(c["qv"]), upload(k), upload(v), upload(c["r"]),
+                                 upload(c["add"]) if c["add"] is not None else None, c["scale"]).numpy_f32()
+    # a row's weight sits on a few keys with scores near 15 here: the f16 rounding of Q and of the mask moves those by a few
+    # 1e-3, the output by as much (3.2e-3 / 3.6e-3 measured, 3.3e-3 / 3.8e-3 for the two-launch form; rel. L2 5e-4)
+    assert_parity(got, ref, "growing scores %s" % spec, max_abs_tol=8e-3, rel_l2_tol=1.5e-3)
+
+
 @pytest.mark.skipif(ora.ref_lib() is None, reason="oracle/_ref not built (needs the reference tree)")
 @pytest.mark.parametrize("T,n_heads,hd", [(150, 2, 128), (97, 3, 64)])
 def test_fused_relpos_attention_matches_the_reference_relpos_attention(T, n_heads, hd):
