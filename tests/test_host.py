@@ -273,3 +273,63 @@ def test_public_header_is_plain_c(tmp_path):
         res = subprocess.run([cc, std, "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc, *extra, "-c", str(src), "-o", str(tmp_path / "chk.o")],
                              capture_output=True, text=True)
         assert res.returncode == 0, res.stderr
+
+
+def _split_top_level(args: str):
+    """the comma-separated pieces of an argument or parameter list, commas inside brackets left alone"""
+    parts, depth, cur = [], 0, ""
+    for ch in args:
+        if ch in "([{":
+            depth += 1
+        elif ch in ")]}":
+            depth -= 1
+        if ch == "," and depth == 0:
+            parts.append(cur.strip())
+            cur = ""
+        else:
+            cur += ch
+    if cur.strip() and cur.strip() != "void":
+        parts.append(cur.strip())
+    return parts
+
+
+def _balanced(text: str, open_at: int) -> str:
+    depth = 0
+    for i in range(open_at, len(text)):
+        depth += text[i] == "("
+        depth -= text[i] == ")"
+        if depth == 0:
+            return text[open_at + 1:i]
+    raise AssertionError("unbalanced parentheses")
+
+
+def test_backend_glue_source_calls_the_library_as_the_header_declares_it():
+    """crispasr_amd/ggml-mi355x/ggml-mi355x.cpp needs ggml's headers and is not compiled here: what can be held in step
+    without them is that every library name it uses is declared by the public header and that every call passes as many
+    arguments as the prototype has parameters"""
+    strip = lambda s: re.sub(r"//[^\n]*", "", re.sub(r"/\*.*?\*/", "", s, flags=re.S))
+    header = strip(open(os.path.join(ROOT, "include", "mi355x_fattn.h")).read())
+    glue = strip(open(os.path.join(ROOT, "crispasr_amd", "ggml-mi355x", "ggml-mi355x.cpp")).read())
+    glue = re.sub(r'"(?:\\.|[^"\\])*"', '""', glue)                        # string literals may hold commas and brackets
+    protos = {}
+    for m in re.finditer(r"\b(mi355x_[a-z0-9_]+)\s*\(", header):
+        protos[m.group(1)] = len(_split_top_level(_balanced(header, m.end() - 1)))
+    assert set(protos) == set(_declared_symbols())
+    declared = set(re.findall(r"\b(?:mi355x|MI355X)_\w+\b", header))
+    own = set(re.findall(r"\b(?:static|struct)\s+(?:[\w:<>\*&]+\s+)*?((?:mi355x|MI355X)_\w+)\b", glue))
+    used = set(re.findall(r"\b(?:mi355x|MI355X)_\w+\b", glue))
+    unknown = sorted(n for n in used - declared - own)
+    assert not unknown, f"the glue uses names that the header does not declare: {unknown}"
+    calls = 0
+    for m in re.finditer(r"\b(mi355x_[a-z0-9_]+)\s*\(", glue):
+        name = m.group(1)
+        if name not in protos:
+            continue                                                       # one of the glue's own functions
+        n = len(_split_top_level(_balanced(glue, m.end() - 1)))
+        assert n == protos[name], f"{name}: called with {n} arguments, declared with {protos[name]}"
+        calls += 1
+    assert calls >= 15
+    # the entry points a backend cannot do without are all bound
+    for name in ("mi355x_api_version", "mi355x_fattn_supports", "mi355x_flash_attn_ext", "mi355x_cpy", "mi355x_set_rows",
+                 "mi355x_host_buffer_alloc", "mi355x_buffer_alloc"):
+        assert name in used, name
