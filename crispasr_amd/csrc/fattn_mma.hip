@@ -955,7 +955,7 @@ int launch_type(const FattnArgs & a, const FattnMmaVariant & v, hipStream_t stre
 // Which instantiation a call takes (also what mi355x_fattn_plan_info reports):
 //  - two query blocks per wave (256 queries per workgroup) halve the LDS operand traffic per MFMA; one block keeps
 //    more workgroups in flight when there are few queries;
-//  - the key-split form (64 queries per workgroup) when even 128-query workgroups number no more than the CUs;
+//  - the key-split form (64 queries per workgroup) when 128-query workgroups leave CUs empty or alone;
 //  - f16 rows go straight to LDS when a tile's row offsets fit 32 bits;
 //  - the mask follows K/V through LDS when its rows start on dwords, Nkv is even (the tail tile's dword-aligned
 //    stand-in chunk) and a wave's row offsets fit 32 bits.
@@ -970,14 +970,30 @@ void fattn_mma_variant(const FattnArgs & a, int ktype, FattnMmaVariant & v) {
     const int     cus = a.n_cus > 0 ? a.n_cus : 256;
     const int want_nqb = a.tile_variant ? (a.tile_variant & 15) : force_nqb ? atoi(force_nqb) : 0;
     const int want_ksp = a.tile_variant ? (a.tile_variant >> 4) : force_ksp ? atoi(force_ksp) : 0;
-    const bool two  = a.D == 64 && (want_nqb ? want_nqb == 2 : wg2 >= 128);
-    const bool ksp2 = !two && ktype == MI355X_TYPE_F16 && a.softcap == 0.0f && (want_ksp ? want_ksp == 2 : wg1 <= cus);
+    // Measured over square shapes of 128 .. 2500 tokens x 8 .. 160 heads, with and without a mask: two query blocks pay
+    // from one workgroup per CU on, and only where 256-query workgroups cover the queries about as tightly as 128-query
+    // ones (300 queries: 512 slots against 384); the key split pays up to about half a workgroup per CU, and up to a
+    // whole one when the key loop is long enough to carry its merge.
+    const int64_t slots1 = (int64_t)(a.Nq + 127) / 128 * 128, slots2 = (int64_t)(a.Nq + 255) / 256 * 256;
+    const bool two_auto = wg2 >= cus && slots2 * 10 <= slots1 * 11;
+    // (With a mask the split form, which skips excluded blocks, carries its merge from 512 keys on; and a mask whose rows
+    // cannot go through LDS costs the unsplit forms a quarter of their speed: there the split form wins up to 1.6
+    // workgroups per CU.)
+    const bool direct = ktype == MI355X_TYPE_F16 && !no_direct && a.nbk1 < (1u << 24) && a.nbv1 < (1u << 24);
+    const bool mdma_ok = a.mask != nullptr && a.softcap == 0.0f && direct && !no_mdma && a.mask_al4 && a.Nkv >= 64 && !(a.Nkv & 1) &&
+                         (uint64_t)a.Nq * a.nbm1 < (1ull << 31);
+    bool ksp_auto;
+    if (a.D == 128)           ksp_auto = wg1 * 2 <= cus || (wg1 <= cus && a.Nkv >= 2048);
+    else if (!a.mask)         ksp_auto = wg1 <= cus && (wg1 * 5 <= (int64_t)cus * 3 || a.Nkv >= 1024) && a.Nkv > 128;
+    else if (!mdma_ok && a.Nkv >= 256) ksp_auto = wg1 * 5 <= (int64_t)cus * 8;
+    else                      ksp_auto = wg1 <= cus && (wg1 * 5 <= (int64_t)cus * 3 || a.Nkv >= 512);
+    const bool two  = a.D == 64 && (want_nqb ? want_nqb == 2 : two_auto);
+    const bool ksp2 = !two && ktype == MI355X_TYPE_F16 && a.softcap == 0.0f && (want_ksp ? want_ksp == 2 : ksp_auto);
     v.query_blocks = two ? 2 : 1;
     v.key_split    = ksp2 ? 2 : 1;
     v.queries_per_workgroup = 32 * v.query_blocks * MMA_WAVES / v.key_split;
-    v.direct   = ktype == MI355X_TYPE_F16 && !no_direct && a.nbk1 < (1u << 24) && a.nbv1 < (1u << 24);
-    v.mask_dma = a.mask != nullptr && a.softcap == 0.0f && v.direct && !ksp2 && !no_mdma && a.mask_al4 && a.Nkv >= 64 &&
-                 !(a.Nkv & 1) && (uint64_t)a.Nq * a.nbm1 < (1ull << 31);
+    v.direct   = direct;
+    v.mask_dma = mdma_ok && !ksp2;
 }
 
 bool fattn_mma_supported(const FattnArgs & a, int ktype) {

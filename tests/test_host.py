@@ -333,3 +333,25 @@ def test_backend_glue_source_calls_the_library_as_the_header_declares_it():
     for name in ("mi355x_api_version", "mi355x_fattn_supports", "mi355x_flash_attn_ext", "mi355x_cpy", "mi355x_set_rows",
                  "mi355x_host_buffer_alloc", "mi355x_buffer_alloc"):
         assert name in used, name
+
+
+def test_tile_kernel_instantiation_follows_the_grid_and_the_query_padding():
+    """which form of the tile kernel a shape takes (planning needs no GPU; 256 CUs are assumed without one): two query blocks
+    per wave from one workgroup per CU on and only where 256-query workgroups pad the queries no worse than 128-query
+    ones; the key split where 128-query workgroups would leave CUs empty or alone"""
+    def form(D, N, H, B=1, Hkv=None, kernel=ggml.KERNEL_MMA):
+        q = _t(ca.F32, (D, N, H, B))
+        k = _t(ca.F16, (D, N, Hkv or H, B))
+        info = ggml.flash_attn_plan_details(q, k, k, None, kernel=kernel)
+        return info["query_blocks"], info["key_split"], info["queries_per_workgroup"]
+    assert form(64, 1500, 20, 4) == (2, 1, 256)          # Whisper large-v3 encoder, four windows: 480 workgroups
+    assert form(64, 1500, 20, 1) == (1, 2, 64)           # one window: 240 workgroups of 128 queries, long key loop
+    assert form(64, 1500, 8, 1) == (1, 2, 64)            # Whisper base
+    assert form(64, 300, 64) == (1, 1, 128)              # 256-query workgroups would carry 512 slots for 300 queries
+    assert form(64, 128, 160) == (1, 1, 128)
+    assert form(64, 448, 64) == (1, 1, 128)              # one workgroup per CU and 7 key tiles: the split's merge does not pay
+    assert form(64, 750, 20) == (1, 2, 64)
+    assert form(128, 407, 32, Hkv=8) == (1, 2, 64)       # Voxtral prefill: 128 workgroups of 128 queries
+    assert form(128, 300, 64) == (1, 1, 128)             # 192 workgroups of 128 queries: more than half the CUs
+    assert form(128, 2500, 8) == (1, 2, 64)              # ... unless the key loop is long
+    assert form(128, 750, 8, 8) == (1, 1, 128)           # FastConformer block
