@@ -477,7 +477,29 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         // 18.0 -> 14.3 us; 24 x 300, 8 heads: 14.2 -> 10.9 us; at 407 x 407, 816 chunks, the tile kernel wins 29 to 31).
         // With f16 K/V the two are within a microsecond of each other and the tile kernel keeps the shape.
         const int64_t chunk_wgs = (int64_t)a.q_chunks * a.Hkv * a.B;
-        const bool    chunked   = ktype == MI355X_TYPE_Q8_0 && chunk_wgs <= 2 * (int64_t)device_cus() && a.Nkv <= 1024;
+        bool          chunked   = ktype == MI355X_TYPE_Q8_0 && chunk_wgs <= 2 * (int64_t)device_cus() && a.Nkv <= 1024;
+        // A longer Q8_0 cache under fewer than 128 queries: the tile kernel would dequantise every tile in its loop, once per
+        // query head (1.7 us per 64-key tile at 64-wide heads, 2.1 at 128-wide; 5 sequences x 32 q / 8 kv heads x 16 queries
+        // against 4096 keys: 111 us, the decode kernel 29), so the two are priced - the tile kernel's tiles per workgroup
+        // after its own key split, the decode kernel's chunks x keys at its measured rate - and the decode kernel has to
+        // win by 1.4 (its rate drops with a mask row per query row).
+        if (!chunked && ktype == MI355X_TYPE_Q8_0 && a.q_chunks > 1 && a.Nq < 128 && a.Nkv > 1024) {
+            const int     cus     = device_cus();
+            const int     n_tiles = (a.Nkv + 63) / 64;
+            const int64_t wgs     = (int64_t)a.Hq * a.B;
+            int ns = 1;
+            if (wgs * 4 <= cus) {
+                ns = (int)(cus / wgs);
+                if (ns > n_tiles / 4) ns = n_tiles / 4;
+                if (ns < 1) ns = 1;
+            } else if (wgs * 2 <= cus && n_tiles >= 16) {
+                ns = 2;
+            }
+            const double rounds = (double)wgs * ns > 2.0 * cus ? (double)wgs * ns / (2.0 * cus) : 1.0;
+            const double tile   = (double)((n_tiles + ns - 1) / ns) * (a.D == 64 ? 1.73 : 2.1) * rounds + (ns > 1 ? 5.0 : 0.0);
+            const double decode = (double)chunk_wgs * a.Nkv * (a.D == 64 ? 20.7e-6 : 39.0e-6) + 12.0;
+            chunked = decode * 1.4 < tile;
+        }
         // The MFMA kernels round F32 and Q8_0 K/V to f16 (2^-12 relative per element).  Over many keys that averages out;
         // a row that sees a handful of keys keeps it (up to 1e-3 on |v| = 4, measured 2.01e-3 in all at 7 keys), so
         // such calls go to the vector kernel, which works on the exact values - and has nothing to gain from MFMA there.
@@ -572,6 +594,37 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
             //  than in 6 of 128, by 2-3%)
             const int max_by_keys = kernel == MI355X_FATTN_VEC ? (a.Nkv + min_keys - 1) / min_keys : (a.Nkv + min_keys / 2) / min_keys;
             if (ns > max_by_keys) ns = max_by_keys;
+            // Decode kernel, long caches under few heads: those bounds alone give 40 to 64 ranges, and every range costs the
+            // set's merge (0.2 us each for one row, 0.45 us for sixteen: 4096 f16 keys x 8 heads of 128 took 16 us in
+            // 43 ranges and 12 us in 16).  Of the counts up to that bound, take the one a small model likes best -
+            // the longer of the cache's pass through HBM (at 5 TB/s) and a wave's chain of 32-key steps (1.3 us each, more
+            // where workgroups share a CU), plus the merge - and the larger count among near-equals (663 keys stay at 7
+            // ranges, 1500 at 8).  Against the best of ten forced counts on 192 shapes (1024 .. 8192 keys, 8 .. 40 KV
+            // heads x sequences, 1 .. 64 rows each, f16 and Q8_0) this is 5% off in the geometric mean, 35% at worst;
+            // the bounds alone were 20% and 2x.
+            if (kernel == MI355X_FATTN_DECODE_MMA && ns > 2) {
+                const double rows   = (double)(a.Nq * a.gqa < 16 ? a.Nq * a.gqa : 16);
+                const double per    = 0.2 + 0.017 * rows;
+                double t_hbm = ((double)a.Hkv * a.B * a.Nkv *
+                                (double)(a.D / block_size(ktype) * type_size(ktype) + a.D / block_size(vtype) * type_size(vtype)) - 8.0e6) / 5.0e6;
+                if (t_hbm < 0.0) t_hbm = 0.0;       // (the first megabytes are a matter of latency, which the chain prices)
+                double best = 1e30;
+                int    pick = ns;
+                for (int pass = 0; pass < 2; pass++)
+                    for (int n = 1; n <= ns; n++) {
+                        const int kps_n = ((a.Nkv + n - 1) / n + 31) / 32 * 32;
+                        if ((a.Nkv + kps_n - 1) / kps_n != n) continue;             // not a count that whole steps give
+                        double chain = kps_n / 128.0;
+                        if (chain < 1.0) chain = 1.0;
+                        chain *= 1.3;
+                        const double per_cu = (double)groups * n / device_cus();     // workgroups sharing a CU share its steps
+                        if (per_cu > 1.0) chain *= per_cu;
+                        const double est = (chain > t_hbm ? chain : t_hbm) + (n > 1 ? n * per : 0.0);
+                        if (pass == 0) { if (est < best) best = est; }
+                        else if (est <= best * 1.10) pick = n;
+                    }
+                ns = pick;
+            }
         }
         if (ns > a.Nkv) ns = a.Nkv;
         if (ns < 1) ns = 1;

@@ -147,35 +147,38 @@ static __device__ __forceinline__ float4 device_load4(const float4 * p) {
 }
 
 // out[row] = sum_s acc_s * exp(m_s - M) / sum_s l_s * exp(m_s - M), for the four values d4*4 .. d4*4+3 of the row.
-// The (m, l) pairs and the accumulators of the first FATTN_MERGE_BATCH splits are requested together, so a row costs
-// one memory round trip, not one per split.  DEVICE: the partials come from other workgroups of this launch.
+// The (m, l) pairs and the accumulators of FATTN_MERGE_BATCH splits are requested together, and the next batch is
+// requested before the current one is folded in: a row costs about one memory round trip however many splits it has
+// (folded in split order, one batch after the other, whatever is in flight).  DEVICE: the partials come from other
+// workgroups of this launch.
 constexpr int FATTN_MERGE_BATCH = 8;
 template <bool DEVICE>
 static __device__ __forceinline__ void fattn_merge_row(const FattnArgs & a, int64_t row, int d4) {
+    constexpr int NB = FATTN_MERGE_BATCH;
     const int lpr = a.D / 4;
     const float2 * pm = (const float2 *)(a.part_ml + (size_t)row * a.n_splits * 2);
     const float4 * pa = (const float4 *)(a.part_acc + (size_t)row * a.n_splits * a.D) + d4;
     float4 out = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     float  M = -INFINITY, L = 0.0f;
-    for (int s0 = 0; s0 < a.n_splits; s0 += FATTN_MERGE_BATCH) {
-        float2 ml[FATTN_MERGE_BATCH];
-        float4 v[FATTN_MERGE_BATCH];
+    auto request = [&](int s0, float2 (&ml)[NB], float4 (&v)[NB]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < FATTN_MERGE_BATCH; i++) {
+        for (int i = 0; i < NB; i++) {
             const int s = min(s0 + i, a.n_splits - 1);          // (past the end: a second look at the last one, not used)
             ml[i] = DEVICE ? device_load2(pm + s) : pm[s];
             v[i]  = DEVICE ? device_load4(pa + (size_t)s * lpr) : pa[(size_t)s * lpr];
             if (s0 + i >= a.n_splits) ml[i] = make_float2(-INFINITY, 0.0f);
         }
+    };
+    auto fold = [&](const float2 (&ml)[NB], const float4 (&v)[NB]) __attribute__((always_inline)) {
         float Mb = M;
 #pragma unroll
-        for (int i = 0; i < FATTN_MERGE_BATCH; i++) Mb = fmaxf(Mb, ml[i].x);
-        if (Mb == -INFINITY) continue;              // nothing visible so far
+        for (int i = 0; i < NB; i++) Mb = fmaxf(Mb, ml[i].x);
+        if (Mb == -INFINITY) return;                // nothing visible so far
         const float f = __expf(M - Mb);             // M = -inf gives 0
         L *= f; out.x *= f; out.y *= f; out.z *= f; out.w *= f;
         M = Mb;
 #pragma unroll
-        for (int i = 0; i < FATTN_MERGE_BATCH; i++) {
+        for (int i = 0; i < NB; i++) {
             // a split that saw no key carries m = -inf and an accumulator that must not be touched (select, not multiply)
             const bool  seen = ml[i].x != -INFINITY;
             const float w    = seen ? __expf(ml[i].x - M) : 0.0f;
@@ -185,6 +188,17 @@ static __device__ __forceinline__ void fattn_merge_row(const FattnArgs & a, int6
             out.z += seen ? v[i].z * w : 0.0f;
             out.w += seen ? v[i].w * w : 0.0f;
         }
+    };
+    float2 ml0[NB], ml1[NB];
+    float4 v0[NB], v1[NB];
+    request(0, ml0, v0);
+    for (int s0 = 0; s0 < a.n_splits; s0 += 2 * NB) {
+        const bool more1 = s0 + NB < a.n_splits, more2 = s0 + 2 * NB < a.n_splits;
+        if (more1) request(s0 + NB, ml1, v1);
+        fold(ml0, v0);
+        if (!more1) break;
+        if (more2) request(s0 + 2 * NB, ml0, v0);
+        fold(ml1, v1);
     }
     const float inv = L > 0.0f ? 1.0f / L : 0.0f;
     out.x *= inv; out.y *= inv; out.z *= inv; out.w *= inv;

@@ -336,11 +336,28 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     const int j    = lane & 15;                    // query column
     const int g4   = lane >> 4;
 
-    // workgroup = (split, 16-row chunk, KV head, batch), splits fastest
-    const int split = blockIdx.x % a.n_splits;
-    const int chunk = (blockIdx.x / a.n_splits) % a.q_chunks;
-    const int hk    = (blockIdx.x / (a.n_splits * a.q_chunks)) % a.Hkv;
-    const int b     = blockIdx.x / (a.n_splits * a.q_chunks * a.Hkv);
+    // workgroup = (split, 16-row chunk, KV head, batch), splits fastest.  With more than one chunk of rows per KV head the
+    // chunks of one (split, KV head, batch) read the same keys: workgroups go to the 8 XCDs round-robin, each with its own
+    // L2, so those chunks are numbered to follow each other on ONE XCD (the grid is rounded up to whole rounds of 8;
+    // the spare workgroups leave here, before any barrier, and belong to no set of the merge).
+    int     split, chunk, hk, b;
+    int64_t set;                                   // index of (chunk, KV head, batch): the merge's counter
+    if (a.q_chunks == 1) {
+        split = blockIdx.x % a.n_splits;
+        chunk = 0;
+        hk    = (blockIdx.x / a.n_splits) % a.Hkv;
+        b     = blockIdx.x / (a.n_splits * a.Hkv);
+        set   = blockIdx.x / a.n_splits;
+    } else {
+        const int64_t w = blockIdx.x >> 3;
+        const int64_t p = (w / a.q_chunks) * 8 + (blockIdx.x & 7);
+        if (p >= (int64_t)a.n_splits * a.Hkv * a.B) return;
+        chunk = (int)(w % a.q_chunks);
+        split = (int)(p % a.n_splits);
+        hk    = (int)((p / a.n_splits) % a.Hkv);
+        b     = (int)(p / ((int64_t)a.n_splits * a.Hkv));
+        set   = ((int64_t)b * a.Hkv + hk) * a.q_chunks + chunk;
+    }
     const int bk    = b / a.bq;
 
     // row r = iq1 * gqa + gg of this KV head  <->  query iq1 of q head hk*gqa + gg; column j is row chunk*16 + j
@@ -689,7 +706,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     }
     // the last of the n_splits workgroups of this (chunk, KV head, batch) merges its rows: no launch for the merge
     if (a.n_splits > 1 && a.counters) {
-        if (!fattn_last_of_set(a, blockIdx.x / a.n_splits, a.n_splits, (int *)smem, redone)) return;
+        if (!fattn_last_of_set(a, set, a.n_splits, (int *)smem, redone)) return;
         constexpr int LPR = D / 4;                  // lanes per row: 8 or 4 rows per pass
         for (int c = tid / LPR; c < 16 && row0 + c < R; c += DEC_THREADS / LPR) {
             const int r = row0 + c;
@@ -700,7 +717,8 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
 
 template <int D, int TYPE, bool MASK, bool RAW, bool V8 = false>
 int launch_one(const FattnArgs & a, hipStream_t stream) {
-    const int64_t wgs = (int64_t)a.n_splits * a.q_chunks * a.Hkv * a.B;
+    const int64_t pairs = (int64_t)a.n_splits * a.Hkv * a.B;
+    const int64_t wgs   = a.q_chunks == 1 ? pairs : (pairs + 7) / 8 * 8 * a.q_chunks;      // as the kernel numbers them
     if (wgs > 0x7fffffff || a.q_chunks != (a.Nq * a.gqa + 15) / 16) return (int)hipErrorInvalidValue;
     const dim3 grid((unsigned)wgs);
     constexpr int lds = decode_lds_bytes<D, TYPE, RAW, V8>();

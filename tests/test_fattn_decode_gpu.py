@@ -175,3 +175,26 @@ def test_more_sets_of_key_ranges_than_counters_fall_back_to_the_merge_launch():
     q, k, v, m = (upload(few[n]) for n in ("q", "k", "v", "mask"))
     assert ggml.flash_attn_plan_details(q, k, v, m, few["scale"], **kw)["merge_in_kernel"] == 1
     assert_parity(ggml.flash_attn_ext(q, k, v, m, few["scale"], **kw).numpy_f32(), run_oracle(few), "merge in the kernel at 16000 sets")
+
+
+@pytest.mark.parametrize("spec", [
+    # 64 rows per KV head (four 16-row chunks) x 40 (KV head, sequence) pairs against 1100 Q8_0 keys: chosen by price
+    dict(seed=251, D=64, Nq=16, Nkv=1100, Hq=32, Hkv=8, B=5, ktype=ora.Q8_0, mask="causal"),
+    dict(seed=252, D=128, Nq=20, Nkv=1300, Hq=16, Hkv=4, B=6, ktype=ora.Q8_0, mask="random_inf_batched"),    # 80 rows: five chunks
+    # chunks of one (key range, KV head, sequence) follow each other on one XCD; 3 x 2 x 3 = 18 such triples, not a multiple of 8
+    dict(seed=253, D=64, Nq=9, Nkv=600, Hq=8, Hkv=2, B=3, ktype=ora.F16, mask="causal", n_splits=3, kernel=3),
+], ids=lambda s: "seed%d" % s["seed"])
+def test_several_row_chunks_per_kv_head_in_the_decode_kernel(spec):
+    """more than 16 query rows per KV head in the decode kernel: a short prompt against a long Q8_0 cache goes there of its
+    own accord (the tile kernel would dequantise the cache once per query head), and the workgroup numbering that keeps a
+    key range's chunks on one XCD must cover every (chunk, key range, KV head, sequence) exactly once"""
+    spec = dict(spec)
+    kw = {k: spec.pop(k) for k in ("n_splits", "kernel") if k in spec}
+    case = make_case(**spec)
+    q, k, v, m = (upload(case[n]) for n in ("q", "k", "v", "mask"))
+    info = ggml.flash_attn_plan_details(q, k, v, m, case["scale"], **kw)
+    assert info["kernel"] == ggml.KERNEL_DECODE_MMA, info
+    print("decode kernel, several chunks", spec, info["n_splits"], flush=True)
+    ref = run_oracle(case)
+    for rep in range(2):
+        assert_parity(ggml.flash_attn_ext(q, k, v, m, case["scale"], **kw).numpy_f32(), ref, "%s call %d" % (spec, rep))

@@ -355,3 +355,29 @@ def test_tile_kernel_instantiation_follows_the_grid_and_the_query_padding():
     assert form(128, 300, 64) == (1, 1, 128)             # 192 workgroups of 128 queries: more than half the CUs
     assert form(128, 2500, 8) == (1, 2, 64)              # ... unless the key loop is long
     assert form(128, 750, 8, 8) == (1, 1, 128)           # FastConformer block
+
+
+def test_decode_kernel_key_ranges_follow_the_priced_plan():
+    """how many key ranges a decode call is cut into (planning needs no GPU; 256 CUs assumed without one): the measured
+    optima of the BASELINE shapes, and no more than the merge is worth on long caches under few heads"""
+    def plan(D, Nq, Hq, Hkv, B, Nkv, kt=ca.F16):
+        q = _t(ca.F32, (D, Nq, Hq, B))
+        k = _t(kt, (D, Nkv, Hkv, B))
+        info = ggml.flash_attn_plan_details(q, k, k, None)
+        return info["kernel"], info["n_splits"]
+    dec = ggml.KERNEL_DECODE_MMA
+    assert plan(64, 5, 20, 20, 1, 1500) == (dec, 8)                 # Whisper cross-attention, 5 beams: 8 ranges of 192
+    assert plan(64, 1, 20, 20, 5, 224) == (dec, 1)                  # ... self-attention: unsplit
+    assert plan(128, 1, 32, 8, 1, 663, ca.Q8_0) == (dec, 7)         # Voxtral step at the end of the 256: 7 of 96
+    assert plan(128, 1, 32, 32, 1, 663) == (dec, 7)                 # the same with the heads expanded, f16
+    assert plan(128, 1, 32, 8, 64, 4096, ca.Q8_0) == (dec, 1)       # 64 sequences fill the chip unsplit
+    k, n = plan(128, 1, 8, 8, 1, 4096)                              # 8 heads alone: bounded by the merge (43 before)
+    assert k == dec and 12 <= n <= 20, n
+    k, n = plan(128, 16, 8, 8, 1, 8192)
+    assert k == dec and 12 <= n <= 24, n
+    # a short prompt against a long Q8_0 cache, several 16-row chunks per KV head: the decode kernel where the tile kernel
+    # would dequantise the cache once per query head, the tile kernel where its own key split makes it cheap
+    assert plan(64, 16, 32, 8, 5, 4096, ca.Q8_0)[0] == dec
+    assert plan(128, 32, 32, 8, 5, 4096, ca.Q8_0)[0] == dec
+    assert plan(128, 64, 8, 8, 1, 4096, ca.Q8_0)[0] == ggml.KERNEL_MMA
+    assert plan(64, 100, 20, 20, 5, 4096, ca.Q8_0)[0] == ggml.KERNEL_MMA
