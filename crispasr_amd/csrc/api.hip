@@ -511,6 +511,12 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
                                                                                 : MI355X_FATTN_VEC;
         else if (fattn_decode_supported(a, ktype) && (a.q_chunks <= 1 || chunked)) kernel = MI355X_FATTN_DECODE_MMA;
         else if (a.Nq >= 16 && fattn_mma_supported(a, ktype)) kernel = MI355X_FATTN_MMA;
+        // F32 K/V under 2 .. 15 queries (the decode kernel does not read F32): the vector kernel streams the keys once per
+        // query row, the tile kernel once per head - worth its padding from about 40k (row, key) pairs on at 64-wide heads
+        // and 100k at 128-wide ones (4 queries x 32 heads x 5 sequences against 256 keys: 20.1 -> 10.0 us and 30.7 -> 17.8)
+        else if (ktype == MI355X_TYPE_F32 && a.Nq >= 2 && fattn_mma_supported(a, ktype) &&
+                 (int64_t)a.Nq * a.Hq * a.B * a.Nkv >= (a.D == 64 ? 40000 : 100000))
+                                                              kernel = MI355X_FATTN_MMA;
         else                                                  kernel = MI355X_FATTN_VEC;
     }
     plan.kernel = kernel;
