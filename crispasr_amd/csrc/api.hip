@@ -589,10 +589,15 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         // decode kernel: a split must be worth the merge launch (about 2.5 us): measured on Whisper cross-attention
         // (64-wide heads, 1500 keys: best at 8 splits) and a Q8_0 LLM cache (128-wide, 663 keys: best at 6 to 8),
         // while 224 keys are fastest unsplit
-        const int     min_keys = kernel == MI355X_FATTN_VEC ? 128 : (a.D <= 64 ? 192 : 96);
+        // vector kernel (one workgroup per row and range; sweep of 1 and 2 queries x 8 .. 128 heads x sequences against 224 ..
+        // 4096 F32 keys, twelve forced counts each): 1.5 workgroups per CU in all, ranges of at least 56 keys for heads wider
+        // than 64 and 128 keys otherwise, at most 8 ranges (16 from 4096 keys on: every range costs its row's merge
+        // 0.5 us), and a power of two - with 6 or 12 ranges the ranges of one KV head's rows do not meet on an XCD
+        // (32 heads of 128 against 4096 keys: 29.0 us in 32 ranges, 21.9 in 16; 2 x 128 rows against 1024 keys: 32.8 us in 4, 29.5 in 2)
+        const int     min_keys = kernel == MI355X_FATTN_VEC ? (a.D > 64 ? 56 : 128) : (a.D <= 64 ? 192 : 96);
         int ns = p->n_splits;
         if (ns <= 0) {
-            const int64_t target = (int64_t)device_cus() * (kernel == MI355X_FATTN_VEC ? 4 : 2);
+            const int64_t target = kernel == MI355X_FATTN_VEC ? (int64_t)device_cus() * 3 / 2 : (int64_t)device_cus() * 2;
             // whole splits only while they still fit the target: past it a split doubles the grid and adds the merge
             ns = kernel == MI355X_FATTN_VEC ? (int)((target + groups - 1) / (groups > 0 ? groups : 1))
                                             : (int)(target / (groups > 0 ? groups : 1));
@@ -600,6 +605,16 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
             //  than in 6 of 128, by 2-3%)
             const int max_by_keys = kernel == MI355X_FATTN_VEC ? (a.Nkv + min_keys - 1) / min_keys : (a.Nkv + min_keys / 2) / min_keys;
             if (ns > max_by_keys) ns = max_by_keys;
+            if (kernel == MI355X_FATTN_VEC) {
+                // the workgroup budget rounds down to a power of two, the key bound to the nearest one
+                int by_wgs = 1, by_keys = 1;
+                while (by_wgs * 2 <= (int)((target + groups - 1) / (groups > 0 ? groups : 1))) by_wgs *= 2;
+                while (by_keys * 2 <= max_by_keys) by_keys *= 2;
+                if (max_by_keys * 10 >= by_keys * 14) by_keys *= 2;
+                ns = by_wgs < by_keys ? by_wgs : by_keys;
+                const int cap = a.Nkv >= 4096 ? 16 : 8;
+                if (ns > cap) ns = cap;
+            }
             // Decode kernel, long caches under few heads: those bounds alone give 40 to 64 ranges, and every range costs the
             // set's merge (0.2 us each for one row, 0.45 us for sixteen: 4096 f16 keys x 8 heads of 128 took 16 us in
             // 43 ranges and 12 us in 16).  Of the counts up to that bound, take the one a small model likes best -
