@@ -563,14 +563,26 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         const int     n_tiles = (a.Nkv + 63) / 64;
         int ns = p->n_splits;
         if (ns <= 0) {
+            // (revised after a sweep of 32 .. 256 queries x 1 .. 40 heads against 1024 .. 8192 keys, ten forced counts each:
+            //  tiny grids, one workgroup per CU as before, go down to two tiles per range - 32 queries x 8 heads against 1024
+            //  keys under a causal mask 10.7 -> 9.4 us in 8 ranges instead of 4 - but not past 16 ranges, whose merge then
+            //  costs more than the shorter loop gains; grids of a quarter of the CUs to two per CU, which were left whole or
+            //  cut in two, are cut towards two workgroups per CU in ranges of at least 16 tiles: 256 queries x 40 heads of
+            //  128 against 8192 keys, 160 workgroups, 146 -> 81 us in 3 ranges; the Whisper-base encoder's 24 tiles stay whole.)
             ns = 1;
             const int cus = device_cus();
+            // (the key-split form of 64-wide heads without a mask walks tiles of 128 keys and more)
+            const int nt = var.key_split == 2 && a.D == 64 && !a.mask ? (a.Nkv + 127) / 128 : n_tiles;
             if (wgs * 4 <= cus) {
                 int want = (int)(cus / wgs);
-                if (want > n_tiles / 4) want = n_tiles / 4;
+                const int by_tiles = nt >= 16 ? nt / 2 : nt / 4;      // (short loops: as before the sweep, which began at 16 tiles)
+                if (want > by_tiles) want = by_tiles;
+                if (want > 16) want = 16;
                 if (want >= 2) ns = want;
-            } else if (wgs * 2 <= cus && n_tiles >= 16) {
-                ns = 2;
+            } else if (wgs < 2 * (int64_t)cus) {
+                int want = (int)((4 * (int64_t)cus / wgs + 1) / 2);          // 2 * cus / wgs, rounded
+                if (want > nt / 16) want = nt / 16;
+                if (want >= 2) ns = want;
             }
         }
         if (ns > n_tiles) ns = n_tiles;
