@@ -566,7 +566,7 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
             // (revised after a sweep of 32 .. 256 queries x 1 .. 40 heads against 1024 .. 8192 keys, ten forced counts each:
             //  tiny grids, one workgroup per CU as before, go down to two tiles per range - 32 queries x 8 heads against 1024
             //  keys under a causal mask 10.7 -> 9.4 us in 8 ranges instead of 4 - but not past 16 ranges, whose merge then
-            //  costs more than the shorter loop gains; grids of a quarter of the CUs to two per CU, which were left whole or
+            //  costs more than the shorter loop gains; grids of a quarter to three quarters of the CUs, which were left whole or
             //  cut in two, are cut towards two workgroups per CU in ranges of at least 16 tiles: 256 queries x 40 heads of
             //  128 against 8192 keys, 160 workgroups, 146 -> 81 us in 3 ranges; the Whisper-base encoder's 24 tiles stay whole.)
             ns = 1;
@@ -579,7 +579,7 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
                 if (want > by_tiles) want = by_tiles;
                 if (want > 16) want = 16;
                 if (want >= 2) ns = want;
-            } else if (wgs < 2 * (int64_t)cus) {
+            } else if (wgs * 4 <= 3 * (int64_t)cus) {                        // (measured up to 160 workgroups; 320 lose 20% cut in two)
                 int want = (int)((4 * (int64_t)cus / wgs + 1) / 2);          // 2 * cus / wgs, rounded
                 if (want > nt / 16) want = nt / 16;
                 if (want >= 2) ns = want;
