@@ -381,3 +381,26 @@ def test_decode_kernel_key_ranges_follow_the_priced_plan():
     assert plan(128, 32, 32, 8, 5, 4096, ca.Q8_0)[0] == dec
     assert plan(128, 64, 8, 8, 1, 4096, ca.Q8_0)[0] == ggml.KERNEL_MMA
     assert plan(64, 100, 20, 20, 5, 4096, ca.Q8_0)[0] == ggml.KERNEL_MMA
+
+
+def test_key_ranges_of_the_vector_and_tile_kernels():
+    """the other two split plans (256 CUs assumed without a GPU): the vector kernel keeps to few, power-of-two ranges; the
+    tile kernel cuts long caches under small grids"""
+    def plan(D, Nq, H, B, Nkv, kt, **kw):
+        q = _t(ca.F32, (D, Nq, H, B))
+        k = _t(kt, (D, Nkv, H, B))
+        info = ggml.flash_attn_plan_details(q, k, k, None, **kw)
+        return info["kernel"], info["n_splits"]
+    vec, mma = ggml.KERNEL_VEC, ggml.KERNEL_MMA
+    assert plan(128, 1, 32, 1, 663, ca.F32) == (vec, 8)              # Voxtral's step with F32 K/V repeated to 32 heads
+    assert plan(128, 1, 32, 1, 224, ca.F32) == (vec, 4)              # 56 keys a range for wide heads
+    assert plan(64, 1, 20, 1, 224, ca.F32) == (vec, 2)               # 128 keys a range for 64-wide ones
+    assert plan(128, 1, 32, 1, 4096, ca.F32) == (vec, 8)             # 32 before
+    assert plan(64, 1, 20, 1, 4096, ca.F32) == (vec, 16)             # fewer rows: up to 16 from 4096 keys on
+    assert plan(128, 2, 32, 4, 1024, ca.F32, kernel=vec) == (vec, 2) # 256 rows: 4 before
+    assert plan(128, 1, 32, 4, 1024, ca.F32) == (vec, 2)
+    assert plan(128, 256, 40, 1, 8192, ca.F16) == (mma, 3)           # 160 workgroups of 64 queries: towards two per CU
+    assert plan(128, 256, 40, 1, 1024, ca.F16) == (mma, 1)           # ... but no range under 16 tiles there
+    assert plan(128, 32, 8, 1, 1024, ca.F16, kernel=mma) == (mma, 8) # 8 workgroups: ranges of two tiles
+    assert plan(64, 1500, 8, 1, 1500, ca.F16) == (mma, 1)            # Whisper base: 192 key-split workgroups x 24 tiles, whole
+    assert plan(128, 407, 32, 1, 407, ca.F16) == (mma, 1)            # the 407-token prefill
