@@ -504,13 +504,20 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         // a row that sees a handful of keys keeps it (up to 1e-3 on |v| = 4, measured 2.01e-3 in all at 7 keys), so
         // such calls go to the vector kernel, which works on the exact values - and has nothing to gain from MFMA there.
         const bool few_keys = a.Nkv <= 16 && ktype != MI355X_TYPE_F16;
+        // 9 to 16 rows per KV head over an f16 cache: the decode kernel's waves merge their rows 8 at a time at 128-wide
+        // heads, and its partial rows and merge grow with the rows, while the tile kernel (cut into key ranges of its own)
+        // does not care: 128-wide 16 rows x 8 heads against 256 keys 12.2 against 9.7 us, against 4096 keys 17.9 against
+        // 13.6; 64-wide from 2048 keys on (20 heads x 16 rows against 4096: 17.1 against 12.8).  Up to 8 rows, and over Q8_0
+        // caches, the decode kernel stays ahead or level.
+        const bool tile_rows = ktype == MI355X_TYPE_F16 && (int64_t)a.Nq * a.gqa > 8 && (a.D == 128 || a.Nkv >= 2048) &&
+                               fattn_mma_supported(a, ktype);
         if (few_keys)                                                              kernel = MI355X_FATTN_VEC;
         else if (narrow_quant(ktype))     // up to 16 rows per KV head read the blocks in the decode kernel; more rows share one conversion to f16
             kernel = fattn_decode_supported(a, ktype) && a.q_chunks <= 1                  ? MI355X_FATTN_DECODE_MMA
                      : a.Nq >= 16 && (a.D == 64 || a.D == 128) && a.q_aligned16 ? MI355X_FATTN_MMA
                                                                                 : MI355X_FATTN_VEC;
-        else if (fattn_decode_supported(a, ktype) && (a.q_chunks <= 1 || chunked)) kernel = MI355X_FATTN_DECODE_MMA;
-        else if (a.Nq >= 16 && fattn_mma_supported(a, ktype)) kernel = MI355X_FATTN_MMA;
+        else if (fattn_decode_supported(a, ktype) && ((a.q_chunks <= 1 && !tile_rows) || chunked)) kernel = MI355X_FATTN_DECODE_MMA;
+        else if ((a.Nq >= 16 || tile_rows) && fattn_mma_supported(a, ktype)) kernel = MI355X_FATTN_MMA;
         // F32 K/V under 2 .. 15 queries (the decode kernel does not read F32): the vector kernel streams the keys once per
         // query row, the tile kernel once per head - worth its padding from about 40k (row, key) pairs on at 64-wide heads
         // and 100k at 128-wide ones (4 queries x 32 heads x 5 sequences against 256 keys: 20.1 -> 10.0 us and 30.7 -> 17.8)

@@ -373,8 +373,14 @@ def test_decode_kernel_key_ranges_follow_the_priced_plan():
     assert plan(128, 1, 32, 8, 64, 4096, ca.Q8_0) == (dec, 1)       # 64 sequences fill the chip unsplit
     k, n = plan(128, 1, 8, 8, 1, 4096)                              # 8 heads alone: bounded by the merge (43 before)
     assert k == dec and 12 <= n <= 20, n
-    k, n = plan(128, 16, 8, 8, 1, 8192)
+    k, n = plan(128, 16, 8, 8, 1, 8192, ca.Q8_0)
     assert k == dec and 12 <= n <= 24, n
+    # 9 .. 16 rows per KV head over an f16 cache: the tile kernel at 128-wide heads, and at 64-wide ones from 2048 keys on
+    assert plan(128, 16, 8, 8, 1, 8192)[0] == ggml.KERNEL_MMA
+    assert plan(128, 4, 32, 8, 1, 256)[0] == ggml.KERNEL_MMA            # 4 queries x 4 query heads per KV head
+    assert plan(128, 8, 8, 8, 1, 256)[0] == dec
+    assert plan(64, 16, 20, 20, 1, 4096)[0] == ggml.KERNEL_MMA
+    assert plan(64, 16, 20, 20, 1, 1024)[0] == dec
     # a short prompt against a long Q8_0 cache, several 16-row chunks per KV head: the decode kernel where the tile kernel
     # would dequantise the cache once per query head, the tile kernel where its own key split makes it cheap
     assert plan(64, 16, 32, 8, 5, 4096, ca.Q8_0)[0] == dec
