@@ -509,7 +509,9 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         // does not care: 128-wide 16 rows x 8 heads against 256 keys 12.2 against 9.7 us, against 4096 keys 17.9 against
         // 13.6; 64-wide from 2048 keys on (20 heads x 16 rows against 4096: 17.1 against 12.8).  Up to 8 rows, and over Q8_0
         // caches, the decode kernel stays ahead or level.
-        const bool tile_rows = ktype == MI355X_TYPE_F16 && (int64_t)a.Nq * a.gqa > 8 && (a.D == 128 || a.Nkv >= 2048) &&
+        // (Rows that are several query heads of few queries stay: the tile kernel would walk the keys once per query head -
+        //  4 queries x 32 q / 8 kv heads x 5 sequences against 1024 keys 26.8 us there, 14.2 here.)
+        const bool tile_rows = ktype == MI355X_TYPE_F16 && a.gqa == 1 && a.Nq > 8 && (a.D == 128 || a.Nkv >= 2048) &&
                                fattn_mma_supported(a, ktype);
         if (few_keys)                                                              kernel = MI355X_FATTN_VEC;
         else if (narrow_quant(ktype))     // up to 16 rows per KV head read the blocks in the decode kernel; more rows share one conversion to f16

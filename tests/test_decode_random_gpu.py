@@ -32,10 +32,9 @@ def test_random_decode_shape_matches_oracle(seed):
     case = make_case(**spec)
     ref = run_oracle(case)
     plan = plan_details(case)
-    # <= 16 rows per KV head, more than 16 keys: the decode kernel - except 9 .. 16 rows over an f16 cache of 128-wide heads
-    # or of 2048 keys and more, which the tile kernel takes
-    rows = spec["Nq"] * spec["Hq"] // spec["Hkv"]
-    to_tile = spec["ktype"] == ora.F16 and rows > 8 and (spec["D"] == 128 or spec["Nkv"] >= 2048)
+    # <= 16 rows per KV head, more than 16 keys: the decode kernel - except 9 .. 16 queries (no GQA) over an f16 cache of
+    # 128-wide heads or of 2048 keys and more, which the tile kernel takes
+    to_tile = spec["ktype"] == ora.F16 and spec["Hq"] == spec["Hkv"] and spec["Nq"] > 8 and (spec["D"] == 128 or spec["Nkv"] >= 2048)
     assert plan["kernel"] == (ggml.KERNEL_MMA if to_tile else ggml.KERNEL_DECODE_MMA), plan
     # (a causal mask over more keys than queries leaves every row at least Nkv - Nq + 1 keys)
     got = run_gpu(case)

@@ -377,7 +377,7 @@ def test_decode_kernel_key_ranges_follow_the_priced_plan():
     assert k == dec and 12 <= n <= 24, n
     # 9 .. 16 rows per KV head over an f16 cache: the tile kernel at 128-wide heads, and at 64-wide ones from 2048 keys on
     assert plan(128, 16, 8, 8, 1, 8192)[0] == ggml.KERNEL_MMA
-    assert plan(128, 4, 32, 8, 1, 256)[0] == ggml.KERNEL_MMA            # 4 queries x 4 query heads per KV head
+    assert plan(128, 4, 32, 8, 1, 256)[0] == dec                        # 4 queries x 4 query heads per KV head: not these
     assert plan(128, 8, 8, 8, 1, 256)[0] == dec
     assert plan(64, 16, 20, 20, 1, 4096)[0] == ggml.KERNEL_MMA
     assert plan(64, 16, 20, 20, 1, 1024)[0] == dec
