@@ -478,6 +478,11 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         // With f16 K/V the two are within a microsecond of each other and the tile kernel keeps the shape.
         const int64_t chunk_wgs = (int64_t)a.q_chunks * a.Hkv * a.B;
         bool          chunked   = ktype == MI355X_TYPE_Q8_0 && chunk_wgs <= 2 * (int64_t)device_cus() && a.Nkv <= 1024;
+        // (f16: only the smallest calls - up to one chunk per CU against 64 keys, or 256 keys at 64-wide heads - where the
+        //  decode kernel's single round is 1 to 2 us shorter than the tile kernel's 6 to 9: 64 queries x 32 q / 8 kv heads
+        //  against 256 keys 8.8 -> 6.9 us)
+        if (ktype == MI355X_TYPE_F16 && a.q_chunks > 1 && chunk_wgs <= device_cus() && (a.Nkv <= 64 || (a.D == 64 && a.Nkv <= 256)))
+            chunked = true;
         // A longer Q8_0 cache under fewer than 128 queries: the tile kernel would dequantise every tile in its loop, once per
         // query head (1.7 us per 64-key tile at 64-wide heads, 2.1 at 128-wide; 5 sequences x 32 q / 8 kv heads x 16 queries
         // against 4096 keys: 111 us, the decode kernel 29), so the two are priced - the tile kernel's tiles per workgroup
