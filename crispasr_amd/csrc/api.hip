@@ -629,12 +629,14 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
                                             : (int)(target / (groups > 0 ? groups : 1));
             // (decode kernel: to the nearest count - 1500 keys are faster in 8 ranges of 192 than in 7 of 224, 663 in 7 of 96
             //  than in 6 of 128, by 2-3%)
-            const int max_by_keys = kernel == MI355X_FATTN_VEC ? (a.Nkv + min_keys - 1) / min_keys : (a.Nkv + min_keys / 2) / min_keys;
+            const int max_by_keys = kernel == MI355X_FATTN_VEC ? (a.Nkv < 2 * min_keys ? 1 : (a.Nkv + min_keys - 1) / min_keys)
+                                                               : (a.Nkv + min_keys / 2) / min_keys;
             if (ns > max_by_keys) ns = max_by_keys;
             if (kernel == MI355X_FATTN_VEC) {
                 // the workgroup budget rounds down to a power of two, the key bound to the nearest one
                 int by_wgs = 1, by_keys = 1;
-                while (by_wgs * 2 <= (int)((target + groups - 1) / (groups > 0 ? groups : 1))) by_wgs *= 2;
+                const int64_t streams = groups / a.gqa > 0 ? groups / a.gqa : 1;      // the rows of a GQA group read the same keys
+                while (by_wgs * 2 <= (int)((target + streams - 1) / streams)) by_wgs *= 2;
                 while (by_keys * 2 <= max_by_keys) by_keys *= 2;
                 if (max_by_keys * 10 >= by_keys * 14) by_keys *= 2;
                 ns = by_wgs < by_keys ? by_wgs : by_keys;
