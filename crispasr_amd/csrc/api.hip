@@ -616,11 +616,11 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         // (64-wide heads, 1500 keys: best at 8 splits) and a Q8_0 LLM cache (128-wide, 663 keys: best at 6 to 8),
         // while 224 keys are fastest unsplit
         // vector kernel (one workgroup per row and range; sweep of 1 and 2 queries x 8 .. 128 heads x sequences against 224 ..
-        // 4096 F32 keys, twelve forced counts each): 1.5 workgroups per CU in all, ranges of at least 56 keys for heads wider
-        // than 64 and 128 keys otherwise, at most 8 ranges (16 from 4096 keys on: every range costs its row's merge
-        // 0.5 us), and a power of two - with 6 or 12 ranges the ranges of one KV head's rows do not meet on an XCD
+        // 4096 F32 keys, twelve forced counts each, also with K/V that no cache holds): 1.5 workgroups per CU in all, a power
+        // of two per row; ranges of at least 128 keys, for heads wider than 64 of 56 keys up to 448 keys and 112 beyond;
+        // at most 8 ranges (16 from 4096 keys on: every range costs its row's merge 0.5 us)
         // (32 heads of 128 against 4096 keys: 29.0 us in 32 ranges, 21.9 in 16; 2 x 128 rows against 1024 keys: 32.8 us in 4, 29.5 in 2)
-        const int     min_keys = kernel == MI355X_FATTN_VEC ? (a.D > 64 ? 56 : 128) : (a.D <= 64 ? 192 : 96);
+        const int     min_keys = kernel == MI355X_FATTN_VEC ? (a.D > 64 ? (a.Nkv > 448 ? 112 : 56) : 128) : (a.D <= 64 ? 192 : 96);
         int ns = p->n_splits;
         if (ns <= 0) {
             const int64_t target = kernel == MI355X_FATTN_VEC ? (int64_t)device_cus() * 3 / 2 : (int64_t)device_cus() * 2;
@@ -633,13 +633,11 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
                                                                : (a.Nkv + min_keys / 2) / min_keys;
             if (ns > max_by_keys) ns = max_by_keys;
             if (kernel == MI355X_FATTN_VEC) {
-                // the workgroup budget rounds down to a power of two, the key bound to the nearest one
-                int by_wgs = 1, by_keys = 1;
+                // the workgroup budget rounds down to a power of two
+                int by_wgs = 1;
                 const int64_t streams = groups / a.gqa > 0 ? groups / a.gqa : 1;      // the rows of a GQA group read the same keys
                 while (by_wgs * 2 <= (int)((target + streams - 1) / streams)) by_wgs *= 2;
-                while (by_keys * 2 <= max_by_keys) by_keys *= 2;
-                if (max_by_keys * 10 >= by_keys * 14) by_keys *= 2;
-                ns = by_wgs < by_keys ? by_wgs : by_keys;
+                ns = by_wgs < max_by_keys ? by_wgs : max_by_keys;
                 const int cap = a.Nkv >= 4096 ? 16 : 8;
                 if (ns > cap) ns = cap;
             }
@@ -653,7 +651,7 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
             // the bounds alone were 20% and 2x.
             if (kernel == MI355X_FATTN_DECODE_MMA && ns > 2) {
                 const double rows   = (double)(a.Nq * a.gqa < 16 ? a.Nq * a.gqa : 16);
-                const double per    = 0.2 + 0.017 * rows;
+                const double per    = 0.25 + 0.017 * rows;
                 double t_hbm = ((double)a.Hkv * a.B * a.Nkv *
                                 (double)(a.D / block_size(ktype) * type_size(ktype) + a.D / block_size(vtype) * type_size(vtype)) - 8.0e6) / 5.0e6;
                 if (t_hbm < 0.0) t_hbm = 0.0;       // (the first megabytes are a matter of latency, which the chain prices)

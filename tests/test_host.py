@@ -398,10 +398,11 @@ def test_key_ranges_of_the_vector_and_tile_kernels():
         info = ggml.flash_attn_plan_details(q, k, k, None, **kw)
         return info["kernel"], info["n_splits"]
     vec, mma = ggml.KERNEL_VEC, ggml.KERNEL_MMA
-    assert plan(128, 1, 32, 1, 663, ca.F32) == (vec, 8)              # Voxtral's step with F32 K/V repeated to 32 heads
-    assert plan(128, 1, 32, 1, 224, ca.F32) == (vec, 4)              # 56 keys a range for wide heads
+    assert plan(128, 1, 32, 1, 663, ca.F32) == (vec, 6)              # Voxtral's step with F32 K/V repeated to 32 heads
+    assert plan(128, 1, 32, 1, 224, ca.F32) == (vec, 4)              # 56 keys a range for wide heads, 112 beyond 448 keys
+    assert plan(128, 1, 32, 1, 408, ca.F32) == (vec, 8)
     assert plan(64, 1, 20, 1, 224, ca.F32) == (vec, 1)               # 128 keys a range for 64-wide ones, and no cut under two ranges' worth
-    assert plan(64, 1, 20, 1, 663, ca.F32) == (vec, 8)
+    assert plan(64, 1, 20, 1, 663, ca.F32) == (vec, 6)
     assert plan(64, 1, 20, 1, 408, ca.F32) == (vec, 4)
     assert plan(128, 1, 32, 1, 64, ca.F32) == (vec, 1)
     assert plan(128, 1, 32, 1, 4096, ca.F32) == (vec, 8)             # 32 before
