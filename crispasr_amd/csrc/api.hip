@@ -420,7 +420,8 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
     for (int i = 1; i < 4; i++) kv2 = kv2 && !(k->nb[i] % 2) && !(v->nb[i] % 2);
     a.kv_aligned2 = kv2 ? 1 : 0;
     const bool al16 = q16 && kv16;
-    if (a.mask) {
+    a.masked = has_mask(mask) ? 1 : 0;
+    if (a.masked) {
         a.Hm = (int)mask->ne[2]; a.Bm = (int)mask->ne[3];
         a.nbm1 = mask->nb[1]; a.nbm2 = mask->nb[2]; a.nbm3 = mask->nb[3];
         bool m8 = !((uintptr_t)mask->data % 8);
@@ -586,7 +587,7 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
             ns = 1;
             const int cus = device_cus();
             // (the key-split form of 64-wide heads without a mask walks tiles of 128 keys and more)
-            const int nt = var.key_split == 2 && a.D == 64 && !a.mask ? (a.Nkv + 127) / 128 : n_tiles;
+            const int nt = var.key_split == 2 && a.D == 64 && !a.masked ? (a.Nkv + 127) / 128 : n_tiles;
             if (wgs * 4 <= cus) {
                 int want = (int)(cus / wgs);
                 const int by_tiles = nt >= 16 ? nt / 2 : nt / 4;      // (short loops: as before the sweep, which began at 16 tiles)

@@ -24,6 +24,7 @@ struct FattnArgs {
     int32_t bq;          // B / Bk
     int32_t q_chunks;    // decode kernel: 16-row chunks of the Nq * gqa query rows that share a KV head
     int32_t Hm, Bm;      // mask broadcast extents
+    int32_t masked;      // the call has a mask (planning looks here: `mask` may still be null when a call is only being sized)
 
     int64_t nbq1, nbq2, nbq3;
     int64_t nbk1, nbk2, nbk3;

@@ -980,11 +980,11 @@ void fattn_mma_variant(const FattnArgs & a, int ktype, FattnMmaVariant & v) {
     // cannot go through LDS costs the unsplit forms a quarter of their speed: there the split form wins up to 1.6
     // workgroups per CU.)
     const bool direct = ktype == MI355X_TYPE_F16 && !no_direct && a.nbk1 < (1u << 24) && a.nbv1 < (1u << 24);
-    const bool mdma_ok = a.mask != nullptr && a.softcap == 0.0f && direct && !no_mdma && a.mask_al4 && a.Nkv >= 64 && !(a.Nkv & 1) &&
+    const bool mdma_ok = a.masked && a.softcap == 0.0f && direct && !no_mdma && a.mask_al4 && a.Nkv >= 64 && !(a.Nkv & 1) &&
                          (uint64_t)a.Nq * a.nbm1 < (1ull << 31);
     bool ksp_auto;
     if (a.D == 128)           ksp_auto = wg1 * 2 <= cus || (wg1 <= cus && a.Nkv >= 2048);
-    else if (!a.mask)         ksp_auto = wg1 <= cus && (wg1 * 5 <= (int64_t)cus * 3 || a.Nkv >= 1024) && a.Nkv > 128;
+    else if (!a.masked)       ksp_auto = wg1 <= cus && (wg1 * 5 <= (int64_t)cus * 3 || a.Nkv >= 1024) && a.Nkv > 128;
     else if (!mdma_ok && a.Nkv >= 256) ksp_auto = wg1 * 5 <= (int64_t)cus * 8;
     else                      ksp_auto = wg1 <= cus && (wg1 * 5 <= (int64_t)cus * 3 || a.Nkv >= 512);
     const bool two  = a.D == 64 && (want_nqb ? want_nqb == 2 : two_auto);

@@ -414,3 +414,24 @@ def test_key_ranges_of_the_vector_and_tile_kernels():
     assert plan(128, 32, 8, 1, 1024, ca.F16, kernel=mma) == (mma, 8) # 8 workgroups: ranges of two tiles
     assert plan(64, 1500, 8, 1, 1500, ca.F16) == (mma, 1)            # Whisper base: 192 key-split workgroups x 24 tiles, whole
     assert plan(128, 407, 32, 1, 407, ca.F16) == (mma, 1)            # the 407-token prefill
+
+
+def test_a_call_is_sized_the_same_with_and_without_its_data_pointers():
+    """graph planning asks for a call's workspace before its tensors have addresses (data NULL): the plan - kernel, form,
+    key ranges, bytes - must not depend on whether the mask's pointer is there yet, only on whether the call has a mask"""
+    for D, N, H in ((64, 900, 32), (64, 600, 40), (64, 2048, 4), (128, 256, 40), (64, 128, 64)):
+        q = _t(ca.F32, (D, N, H, 1))
+        k = _t(ca.F16, (D, N if D == 64 else 8192, H, 1))
+        nkv = k.ne[1]
+        pitch = (2 * nkv + 31) // 32 * 32
+        for off in (0, 32):                         # no address yet / an address with the alignment the buffer will give
+            m = ca.Tensor(None, ca.F16, (nkv, N, 1, 1), (2, pitch, pitch * N, pitch * N), offset=off)
+            info = ggml.flash_attn_plan_details(q, k, k, m)
+            size = ggml.flash_attn_workspace_size(q, k, k, m)
+            if off == 0:
+                first = (info["kernel"], info["n_splits"], info["key_split"], info["query_blocks"], size)
+            else:
+                assert (info["kernel"], info["n_splits"], info["key_split"], info["query_blocks"], size) == first, (D, N, H)
+        unmasked = ggml.flash_attn_plan_details(q, k, k, None)
+        if (D, N, H) == (64, 900, 32):
+            assert first[2] == 2 and unmasked["key_split"] == 1          # the mask is what decides the form here
