@@ -1227,6 +1227,14 @@ static RelposFused relpos_fused_plan(const mi355x_tensor * q_u, const mi355x_ten
     const uint64_t kpitch = f.kv_copy ? (uint64_t)a.D * 2 : (uint64_t)k->nb[1], vpitch = f.kv_copy ? (uint64_t)a.D * 2 : (uint64_t)v->nb[1];
     const uint64_t rpitch = f.table_bytes ? (uint64_t)a.D * 2 : (uint64_t)r->nb[1];
     if ((uint64_t)a.Nkv * kpitch >= lim || (uint64_t)a.Nkv * vpitch >= lim || (uint64_t)r->ne[1] * rpitch >= lim) return f;
+    // A workgroup of the one-kernel form walks all keys of its head by itself.  A single long utterance leaves most CUs
+    // without one, and then the mask kernel + the tile kernel - which cuts the keys of a small grid into ranges - is
+    // ahead: 8 heads x 128, one sequence of 750 frames (48 workgroups) 54.4 against 45.8 us, 4 heads 51.9 against 38.1,
+    // 1500 frames 90 against 80; up to 375 frames and from 8 sequences on the one kernel wins everywhere (60 against 67 us
+    // at 4 heads x 750 frames x 8, 21 against 26 at 100 frames).
+    static const bool one_kernel = getenv("MI355X_RELPOS_ONE_KERNEL") != nullptr;     // comparison runs
+    const int64_t wgs = (int64_t)((a.Nq + 127) / 128) * a.Hq * a.B;
+    if (!one_kernel && wgs * 8 <= 3 * (int64_t)device_cus() && a.Nkv >= 512) return f;
     f.ok = true;
     return f;
 }

@@ -315,3 +315,33 @@ def test_relpos_mask_with_a_caller_workspace_for_the_f32_table():
         graph.replay()
         torch.cuda.synchronize()
         assert np.array_equal(out.to_host()[: plain.size], plain)
+
+
+def test_a_single_long_utterance_takes_the_two_launch_form():
+    """the one-kernel form walks a head's keys with one workgroup per 128 queries: where that leaves most CUs without work
+    (one sequence of 600 frames, 2 heads: 10 workgroups) the call computes the mask and runs the tile kernel, which cuts
+    small grids into key ranges; a batch of such sequences goes through the one kernel.  Seen from outside: the workspace
+    the call asks of its caller (the one-kernel form needs only the f16 table here), and the same results."""
+    import torch
+    for B, fused in ((1, False), (12, True)):
+        spec = dict(seed=361, D=64, Nq=600, Nkv=600, H=2, B=B, add="pad", rtype=ora.F32)
+        c = make(qgain=0.7, **spec)
+        D, Nq, Nkv, H = c["D"], c["Nq"], c["Nkv"], c["H"]
+        qu = strided(np.float32(0.7) * ora.randn(371, (B, H, Nq, D)), "cont")
+        k = ora.from_f32(ora.randn(372, (B, H, Nkv, D)), ora.F16)
+        v = ora.from_f32(ora.randn(373, (B, H, Nkv, D)), ora.F16)
+        args = [upload(t) for t in (qu, c["qv"], k, v, c["r"], c["add"])]
+        print("relpos attention, %d sequence(s) of 600 frames" % B, flush=True)
+        got = ggml.flash_attn_relpos(*args, c["scale"]).numpy_f32()
+        mask = ora.relpos_bias(c["qv"], c["r"], c["add"], c["scale"], Nkv)
+        assert_parity(got, ora.flash_attn_ext(qu, k, v, mask, c["scale"]), "B=%d" % B, max_abs_tol=5e-3, rel_l2_tol=1e-3)
+        one = ggml.relpos_bias_workspace_size(args[4])                      # f16 K/V: the one-kernel form's whole need
+        ws = torch.empty(one, dtype=torch.uint8, device="cuda")
+        if fused:
+            assert np.array_equal(ggml.flash_attn_relpos(*args, c["scale"], workspace=ws).numpy_f32(), got)
+        else:
+            with pytest.raises(ggml.Mi355xError, match="workspace"):
+                ggml.flash_attn_relpos(*args, c["scale"], workspace=ws)
+            need = ggml.flash_attn_relpos_workspace_size(*args, c["scale"])
+            big = torch.empty(need, dtype=torch.uint8, device="cuda")
+            assert np.array_equal(ggml.flash_attn_relpos(*args, c["scale"], workspace=big).numpy_f32(), got)
