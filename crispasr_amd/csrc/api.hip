@@ -621,7 +621,7 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         // of two per row; ranges of at least 128 keys, for heads wider than 64 of 56 keys up to 448 keys and 112 beyond;
         // at most 8 ranges (16 from 4096 keys on: every range costs its row's merge 0.5 us)
         // (32 heads of 128 against 4096 keys: 29.0 us in 32 ranges, 21.9 in 16; 2 x 128 rows against 1024 keys: 32.8 us in 4, 29.5 in 2)
-        const int     min_keys = kernel == MI355X_FATTN_VEC ? (a.D > 64 ? (a.Nkv > 448 ? 112 : 56) : 128) : (a.D <= 64 ? 192 : 96);
+        const int     min_keys = kernel == MI355X_FATTN_VEC ? (a.D > 64 ? (a.Nkv > 448 ? 112 : 56) : 128) : (a.D <= 64 ? 128 : 64);
         int ns = p->n_splits;
         if (ns <= 0) {
             const int64_t target = kernel == MI355X_FATTN_VEC ? (int64_t)device_cus() * 3 / 2 : (int64_t)device_cus() * 2;
@@ -645,12 +645,14 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
             // Decode kernel, long caches under few heads: those bounds alone give 40 to 64 ranges, and every range costs the
             // set's merge (0.2 us each for one row, 0.45 us for sixteen: 4096 f16 keys x 8 heads of 128 took 16 us in
             // 43 ranges and 12 us in 16).  Of the counts up to that bound, take the one a small model likes best -
-            // the longer of the cache's pass through HBM (at 5 TB/s) and a wave's chain of 32-key steps (1.3 us each, more
-            // where workgroups share a CU), plus the merge - and the larger count among near-equals (663 keys stay at 7
-            // ranges, 1500 at 8).  Against the best of ten forced counts on 192 shapes (1024 .. 8192 keys, 8 .. 40 KV
+            // the longer of the cache's pass through HBM (at 5 TB/s) and a wave's chain of 32-key steps (four of them 0.7 us
+            // on 64-wide heads, 1.3 us on wider ones, more where workgroups share a CU), plus 1 us for the merge and a
+            // share for every range - and the larger count among near-equals (663 keys stay at 7 ranges, 1500 at 8).
+            // With K/V that no cache holds, 2 ranges were almost never the best count and up to 384 keys (256 under
+            // 128-wide heads) no split was: the fixed microsecond is what keeps those whole.  Against the best of ten forced counts on 192 shapes (1024 .. 8192 keys, 8 .. 40 KV
             // heads x sequences, 1 .. 64 rows each, f16 and Q8_0) this is 5% off in the geometric mean, 35% at worst;
             // the bounds alone were 20% and 2x.
-            if (kernel == MI355X_FATTN_DECODE_MMA && ns > 2) {
+            if (kernel == MI355X_FATTN_DECODE_MMA && ns > 1) {
                 const double rows   = (double)(a.Nq * a.gqa < 16 ? a.Nq * a.gqa : 16);
                 const double per    = 0.25 + 0.017 * rows;
                 double t_hbm = ((double)a.Hkv * a.B * a.Nkv *
@@ -664,10 +666,10 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
                         if ((a.Nkv + kps_n - 1) / kps_n != n) continue;             // not a count that whole steps give
                         double chain = kps_n / 128.0;
                         if (chain < 1.0) chain = 1.0;
-                        chain *= 1.3;
+                        chain *= a.D <= 64 ? 0.7 : 1.3;
                         const double per_cu = (double)groups * n / device_cus();     // workgroups sharing a CU share its steps
                         if (per_cu > 1.0) chain *= per_cu;
-                        const double est = (chain > t_hbm ? chain : t_hbm) + (n > 1 ? n * per : 0.0);
+                        const double est = (chain > t_hbm ? chain : t_hbm) + (n > 1 ? 1.0 + n * per : 0.0);
                         if (pass == 0) { if (est < best) best = est; }
                         else if (est <= best * 1.10) pick = n;
                     }

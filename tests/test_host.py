@@ -371,6 +371,12 @@ def test_decode_kernel_key_ranges_follow_the_priced_plan():
     assert plan(128, 1, 32, 8, 1, 663, ca.Q8_0) == (dec, 7)         # Voxtral step at the end of the 256: 7 of 96
     assert plan(128, 1, 32, 32, 1, 663) == (dec, 7)                 # the same with the heads expanded, f16
     assert plan(128, 1, 32, 8, 64, 4096, ca.Q8_0) == (dec, 1)       # 64 sequences fill the chip unsplit
+    # short caches (timed with K/V that no cache holds): whole up to 384 keys at 64-wide heads and 256 at 128-wide ones,
+    # then 3 ranges or more - 2 were almost never the best count
+    assert plan(64, 1, 20, 20, 1, 384) == (dec, 1)
+    assert plan(64, 1, 20, 20, 1, 448) == (dec, 3)
+    assert plan(128, 1, 32, 8, 1, 256) == (dec, 1)
+    assert plan(128, 1, 32, 8, 1, 320) == (dec, 4)
     k, n = plan(128, 1, 8, 8, 1, 4096)                              # 8 heads alone: bounded by the merge (43 before)
     assert k == dec and 12 <= n <= 20, n
     k, n = plan(128, 16, 8, 8, 1, 8192, ca.Q8_0)

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 CALLS = [
     # larger first: Q8_0 K/V rounded to f16 copies in the scratch (tile kernel), then split-KV partials (decode kernel),
     # then the query rows staged as Q8_0 in front of the partials
-    (dict(seed=801, D=128, Nq=300, Nkv=400, Hq=8, Hkv=2, ktype=ora.Q8_0, mask="causal"), {}),
+    (dict(seed=801, D=128, Nq=300, Nkv=1100, Hq=8, Hkv=2, ktype=ora.Q8_0, mask="causal"), {}),
     (dict(seed=802, D=64, Nq=5, Nkv=1500, Hq=20, q_layout="thd", kv_layout="thd", scale=0.35355339), {}),
     (dict(seed=803, D=128, Nq=1, Nkv=663, Hq=32, Hkv=8, ktype=ora.Q8_0), dict(q_quant=ggml.Q8_0)),
 ]
