@@ -334,7 +334,16 @@ struct Plan {
     int64_t merge_sets;      // > 0: the kernel can merge its splits itself, given this many counters
     bool    kv_to_f16;       // K and V are rounded to f16 copies in the workspace first (F32 / quantised K/V before the tile kernel; a
                              // K and a V of different types before any kernel)
+    int     pad;             // 0, or the head size (64 / 128) the copies' rows are zero-padded to for the tile kernel
 };
+
+// the call as the kernels see it when the plan pads the head: D the padded size, Dv the real one
+void apply_pad(FattnArgs & a, const Plan & plan) {
+    if (plan.pad) {
+        a.Dv = a.D;
+        a.D  = plan.pad;
+    }
+}
 
 int check(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
           const mi355x_tensor * mask, const mi355x_tensor * dst, const mi355x_fattn_params * p) {
@@ -398,6 +407,7 @@ void fill_args(FattnArgs & a, const mi355x_tensor * q, const mi355x_tensor * k, 
     a.mask = has_mask(mask) ? (const char *)mask->data : nullptr;
     a.dst = dst;
     a.D = (int)q->ne[0]; a.Nq = (int)q->ne[1]; a.Hq = (int)q->ne[2]; a.B = (int)q->ne[3];
+    a.Dv = a.D;
     a.Nkv = (int)k->ne[1]; a.Hkv = (int)k->ne[2]; a.Bk = (int)k->ne[3];
     a.gqa = a.Hq / a.Hkv; a.bq = a.B / a.Bk;
     a.q_chunks = (int32_t)(((int64_t)a.Nq * a.gqa + 15) / 16);
@@ -462,9 +472,11 @@ void use_f16_copies(FattnArgs & a, void * ws) {
 
 // A K and a V of different storage types (CRISPASR_KV_QUANT_K / _V, src/core/attention.h:132-137) are both rounded to f16
 // copies first, whatever the kernel: the call is then planned and run as an F16 one.
-void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_params * p, Plan & plan) {
+
+// (padded: a0.D is the padded head size and the copies are needed whatever the types)
+void make_plan_core(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_params * p, bool padded, Plan & plan) {
     FattnArgs a = a0;
-    const bool mixed = ktype != vtype;
+    const bool mixed = ktype != vtype || padded;
     if (mixed) {
         use_f16_copies(a, nullptr);
         ktype = MI355X_TYPE_F16;
@@ -541,6 +553,7 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
     plan.kv_to_f16 = false;
     plan.ws_partials = 0;
     plan.merge_sets = 0;
+    plan.pad = 0;
     // nothing to launch (no query rows) or nothing to read (no keys: the result is zeros): one range, no workspace
     if ((int64_t)a.Nq * a.Hq * a.B == 0 || a.Nkv == 0) return;
     // The tile kernel rounds F32 and Q8_0 K/V to f16 on their way into LDS anyway.  With enough queries to share the work it
@@ -690,6 +703,43 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
     }
 }
 
+// Head sizes the tile kernel has no form for (multiples of 8 below 128 other than 64: 32 and 48, 80 and 96 of other
+// Whisper-like towers, ...) can still run on it: the launch that makes f16 copies of K and V pads their rows with zeros to
+// 64 or 128, the kernel reads Dv elements of every q row and writes Dv of every dst row.  The products over the padding
+// are exact zeros, so the result is what the head size itself would give; the cost is the padded share of the MFMA work
+// and the copy.  The vector kernel, which takes any head size, keeps the calls the padded plan would not give to the tile
+// kernel (few query rows) and those too small to pay for the copy launch.
+void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_params * p, Plan & plan) {
+    static const bool no_pad = getenv("MI355X_FATTN_NO_PAD") != nullptr;        // comparison runs
+    const int pad = a0.D >= 8 && a0.D < 128 && a0.D != 64 && a0.D % 8 == 0 ? (a0.D < 64 ? 64 : 128) : 0;
+    if (pad && !no_pad && (p->kernel == MI355X_FATTN_AUTO || p->kernel == MI355X_FATTN_MMA)) {
+        FattnArgs b = a0;
+        b.Dv = a0.D;
+        b.D  = pad;
+        make_plan_core(b, ktype, vtype, p, true, plan);
+        const int64_t pairs = (int64_t)a0.Nq * a0.Hq * a0.B * a0.Nkv;
+        // (vector against padded tile kernel over 2 .. 1500 queries x 4 .. 64 heads x 64 .. 1500 keys at head sizes 32, 48, 80
+        //  and 96, f16 and F32 K/V, the choice against the faster of the two: from 16 queries and 100k (query row, key)
+        //  pairs on the copy launch and the padding pay - 1 to 3% off in the geometric mean, where the vector kernel alone
+        //  is 27 to 71% off and 16 to 44 times slower at worst; above 64 also for 2 .. 15 queries from 150k pairs on, as
+        //  for F32 caches of the sizes the tile kernel has forms for)
+        bool tile = plan.kernel == MI355X_FATTN_MMA && (p->kernel == MI355X_FATTN_MMA || pairs >= 100000);
+        if (!tile && p->kernel == MI355X_FATTN_AUTO && pad == 128 && a0.Nq >= 2 && a0.Nq < 16 && pairs >= 150000) {
+            mi355x_fattn_params by_name = *p;
+            by_name.kernel = MI355X_FATTN_MMA;
+            make_plan_core(b, ktype, vtype, &by_name, true, plan);
+            FattnArgs c = b;
+            use_f16_copies(c, nullptr);
+            tile = fattn_mma_supported(c, MI355X_TYPE_F16);
+        }
+        if (tile) {
+            plan.pad = pad;
+            return;
+        }
+    }
+    make_plan_core(a0, ktype, vtype, p, false, plan);
+}
+
 // q_quant: the query rows rounded to Q8_0 and back, as contiguous F32 [D, Nq, Hq, B] at ws + q8_bytes
 size_t qq_q8_bytes(const mi355x_tensor * q) {
     return ((size_t)q->ne[0] / FATTN_QK8_0 * FATTN_Q8_0_BYTES * q->ne[1] * q->ne[2] * q->ne[3] + 255) / 256 * 256;
@@ -835,10 +885,12 @@ int mi355x_fattn_plan_details(const mi355x_tensor * q, const mi355x_tensor * k, 
     info->keys_per_split = plan.keys_per_split;
     info->kv_to_f16      = plan.kv_to_f16 ? 1 : 0;
     info->workspace      = plan.workspace;
+    info->head_pad       = plan.pad;
     info->merge_in_kernel = plan.merge_sets > 0 && !params->workspace && !g_no_fused_merge ? 1 : 0;
     if (plan.kernel == MI355X_FATTN_MMA) {
         // the order of the call itself: the f16 copies first, then the question whether the tile kernel takes the shape
         int ktype = k->type;
+        apply_pad(a, plan);
         if (plan.kv_to_f16) {
             use_f16_copies(a, nullptr);
             ktype = MI355X_TYPE_F16;
@@ -922,6 +974,7 @@ static int flash_attn_run(const mi355x_tensor * q, const mi355x_tensor * k, cons
 
     Plan plan;
     make_plan(a, k->type, v->type, params, plan);
+    apply_pad(a, plan);
     hipStream_t st = (hipStream_t)stream;
 
     int ktype = k->type;

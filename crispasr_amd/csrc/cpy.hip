@@ -256,6 +256,8 @@ __global__ void __launch_bounds__(256) kv_to_f16_kernel(const FattnArgs a, char 
 // The same for a K and a V of different storage types (CRISPASR_KV_QUANT_K / _V, src/core/attention.h:132-137; the
 // Canary decoder hands both cache views to the op as they are, src/canary.cpp:953-972): the type is looked up per
 // tensor at run time.  Scalar loads: such rows are only as aligned as their type.
+// It is also the launch that pads: the copies' rows are a.D elements long, the first a.Dv of them the source row's
+// (a multiple of 8), zeros behind - how the tile kernel, which has forms for 64- and 128-wide heads, gets the others.
 __global__ void __launch_bounds__(256) kv_to_f16_mixed_kernel(const FattnArgs a, const int ktype, const int vtype, char * dst) {
     const int     cpr  = a.D / 8;
     const int64_t half = (int64_t)cpr * a.Nkv * a.Hkv * a.Bk;
@@ -264,6 +266,10 @@ __global__ void __launch_bounds__(256) kv_to_f16_mixed_kernel(const FattnArgs a,
     const bool is_v = i >= half;
     if (is_v) i -= half;
     const int     c = (int)(i % cpr);
+    if (c * 8 >= a.Dv) {
+        *(uint4 *)(dst + ((is_v ? half : 0) + i) * 16) = uint4{0u, 0u, 0u, 0u};
+        return;
+    }
     int64_t       r = i / cpr;
     const int64_t j = r % a.Nkv;  r /= a.Nkv;
     const int64_t h = r % a.Hkv;
@@ -328,7 +334,7 @@ int kv_to_f16_launch(const FattnArgs & a, int ktype, int vtype, void * dst, hipS
     if (n == 0) return 0;
     if ((n + 255) / 256 > 0x7fffffff) return (int)hipErrorInvalidValue;
     const unsigned g = (unsigned)((n + 255) / 256);
-    if (ktype != vtype) {
+    if (ktype != vtype || a.Dv != a.D) {
         if (rider) return (int)hipErrorInvalidValue;
         hipLaunchKernelGGL(kv_to_f16_mixed_kernel, dim3(g), dim3(256), 0, stream, a, ktype, vtype, (char *)dst);
         return (int)hipGetLastError();

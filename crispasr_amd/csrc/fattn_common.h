@@ -20,6 +20,8 @@ struct FattnArgs {
     float *      dst;    // F32 [D, Hq, Nq, B] contiguous
 
     int32_t D, Nq, Hq, B, Nkv, Hkv, Bk;
+    int32_t Dv;          // elements of a q row and of a dst row; = D, except when the tile kernel runs a head size it has no
+                         // form for on f16 copies of K/V whose rows are zero-padded to D (64 or 128): then the real head size
     int32_t gqa;         // Hq / Hkv
     int32_t bq;          // B / Bk
     int32_t q_chunks;    // decode kernel: 16-row chunks of the Nq * gqa query rows that share a KV head
@@ -203,7 +205,8 @@ static __device__ __forceinline__ void fattn_merge_row(const FattnArgs & a, int6
     }
     const float inv = L > 0.0f ? 1.0f / L : 0.0f;
     out.x *= inv; out.y *= inv; out.z *= inv; out.w *= inv;
-    *((float4 *)(a.dst + (size_t)row * a.D) + d4) = out;
+    // (dst rows are Dv floats - the head size - also where the partial rows are those of a head zero-padded to D)
+    if (d4 * 4 < a.Dv) *((float4 *)(a.dst + (size_t)row * a.Dv) + d4) = out;
 }
 
 // The end of a workgroup that has stored its partials, when the launch merges in the kernel (a.counters): true for the

@@ -148,8 +148,13 @@ template <int D> __device__ __forceinline__ int swz_m(int r) { return (r >> 2) &
 // CUs, since four such tiles are 128 KB of LDS and leave room for one workgroup per CU only.
 // (two query blocks per wave with 128-key tiles: 240 bytes of scratch per lane in the loop, 110 us instead of 60 on the
 //  large-v3 encoder layer)
-template <int D, int NQB, int KSP, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA, int TK = BC>
+// PAD: the head is one of a.Dv elements (a multiple of 8 below D) on K/V copies whose rows are zero-padded to D: a.Dv
+// elements of every q row are read and a.Dv of every dst row written.  An instantiation of its own, so that the others
+// stay the code they were (the guards cost the one-block forms 2% as a run-time branch).
+template <int D, int NQB, int KSP, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA, int TK = BC, bool PAD = false>
 __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnArgs a, const int n_qtiles) {
+    static_assert(!PAD || (DIRECT && NQB == 1), "zero-padded heads: f16 copies, one query block per wave");
+    constexpr bool whole_head = !PAD;
     static_assert(!DIRECT || TYPE == MI355X_TYPE_F16, "only f16 rows can go to LDS unconverted");
     static_assert(!MDMA || (DIRECT && MASK), "the mask goes through LDS only beside directly loaded K/V");
     static_assert(KSP == 1 || (KSP == 2 && NQB == 1 && !MDMA), "key-split form: one query block per wave, mask through registers");
@@ -222,8 +227,11 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         const float * qrow = (const float *)(a.q + (int64_t)qi * a.nbq1 + (int64_t)h * a.nbq2 + (int64_t)b * a.nbq3);
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-            const float4 x0 = *(const float4 *)(qrow + ks * 16 + hh * 8);
-            const float4 x1 = *(const float4 *)(qrow + ks * 16 + hh * 8 + 4);
+            float4 x0 = {0.0f, 0.0f, 0.0f, 0.0f}, x1 = x0;
+            if (whole_head || ks * 16 + hh * 8 < a.Dv) {   // (a head zero-padded to D: nothing to read behind Dv, a multiple of 8)
+                x0 = *(const float4 *)(qrow + ks * 16 + hh * 8);
+                x1 = *(const float4 *)(qrow + ks * 16 + hh * 8 + 4);
+            }
             half8 v;
             v[0] = (_Float16)(x0.x * qscale); v[1] = (_Float16)(x0.y * qscale);
             v[2] = (_Float16)(x0.z * qscale); v[3] = (_Float16)(x0.w * qscale);
@@ -846,7 +854,8 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
             const int   qi   = q0 + qb * 32 + l32;
             if (qi < a.Nq) {
                 const int64_t row = ((int64_t)b * a.Nq + qi) * a.Hq + h;
-                float * out = a.n_splits > 1 ? a.part_acc + (row * a.n_splits + split) * D : a.dst + row * D;
+                // (a zero-padded head, Dv < D: dst rows are Dv floats apart and end there; partial rows are D apart)
+                float * out = a.n_splits > 1 ? a.part_acc + (row * a.n_splits + split) * D : a.dst + row * (PAD ? a.Dv : D);
 #pragma unroll
                 for (int db = 0; db < DB; db++)
 #pragma unroll
@@ -856,7 +865,7 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
                         o.y = oacc[qb][db][g * 4 + 1] * inv;
                         o.z = oacc[qb][db][g * 4 + 2] * inv;
                         o.w = oacc[qb][db][g * 4 + 3] * inv;
-                        *(float4 *)(out + db * 32 + g * 8 + hh * 4) = o;
+                        if (whole_head || db * 32 + g * 8 + hh * 4 < a.Dv) *(float4 *)(out + db * 32 + g * 8 + hh * 4) = o;
                     }
                 if (a.n_splits > 1 && hh == 0) {
                     // (reference, sum) in natural-log units; a range with no visible key contributes nothing
@@ -888,8 +897,8 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
     }
 }
 
-template <int D, int NQB, int KSP, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA, int TK = BC>
-int launch(const FattnArgs & a, hipStream_t stream) {
+template <int D, int NQB, int KSP, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA, int TK, bool PAD>
+int launch_kernel(const FattnArgs & a, hipStream_t stream) {
     const int bmg = 32 * NQB * MMA_WAVES / KSP;
     const int n_qtiles = (a.Nq + bmg - 1) / bmg;
     if ((int64_t)n_qtiles * a.Hq * a.B * a.n_splits > 0x7fffffff) return (int)hipErrorInvalidValue;
@@ -897,17 +906,26 @@ int launch(const FattnArgs & a, hipStream_t stream) {
     const size_t lds = DIRECT ? (size_t)4 * TK * D * sizeof(_Float16) + (MDMA ? (size_t)MMA_WAVES * NQB * 4096 : 0)
                               : (size_t)2 * BC * (Pitch<D>::K + Pitch<D>::V) * sizeof(_Float16);
     static std::atomic<uint64_t> lds_allowed{0};     // per instantiation
-    const hipError_t ea = fattn_allow_lds((const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA, TK>, (int)lds, lds_allowed);
+    const hipError_t ea = fattn_allow_lds((const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA, TK, PAD>, (int)lds, lds_allowed);
     if (ea != hipSuccess) return (int)ea;
     static const bool debug = getenv("MI355X_FATTN_DEBUG") != nullptr;
     if (debug) {
         int nb = -1;
-        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA, TK>, MMA_THREADS, lds);
+        (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void *)fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA, TK, PAD>, MMA_THREADS, lds);
         fprintf(stderr, "[mi355x] fattn_mma<%d,%d,%d,%d,%d,%d,%d,%d> grid %u lds %zu B, resident workgroups per CU: %d\n",
                 D, NQB, KSP, TYPE, (int)MASK, (int)SOFTCAP, (int)DIRECT, (int)MDMA, grid.x, lds, nb);
     }
-    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA, TK>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
+    hipLaunchKernelGGL((fattn_mma_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA, TK, PAD>), grid, dim3(MMA_THREADS), lds, stream, a, n_qtiles);
     return (int)hipGetLastError();
+}
+
+template <int D, int NQB, int KSP, int TYPE, bool MASK, bool SOFTCAP, bool DIRECT, bool MDMA, int TK = BC>
+int launch(const FattnArgs & a, hipStream_t stream) {
+    if (a.Dv != a.D) {              // a zero-padded head: the forms that exist for it, or none
+        if constexpr (DIRECT && NQB == 1) return launch_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA, TK, true>(a, stream);
+        return (int)hipErrorInvalidValue;
+    }
+    return launch_kernel<D, NQB, KSP, TYPE, MASK, SOFTCAP, DIRECT, MDMA, TK, false>(a, stream);
 }
 
 template <int D, int NQB, int KSP, int TYPE, bool DIRECT>
@@ -979,7 +997,8 @@ void fattn_mma_variant(const FattnArgs & a, int ktype, FattnMmaVariant & v) {
     // (With a mask the split form, which skips excluded blocks, carries its merge from 512 keys on; and a mask whose rows
     // cannot go through LDS costs the unsplit forms a quarter of their speed: there the split form wins up to 1.6
     // workgroups per CU.)
-    const bool direct = ktype == MI355X_TYPE_F16 && !no_direct && a.nbk1 < (1u << 24) && a.nbv1 < (1u << 24);
+    // (a zero-padded head exists in the direct forms only: its K/V are the call's own f16 copies)
+    const bool direct = ktype == MI355X_TYPE_F16 && (!no_direct || a.Dv != a.D) && a.nbk1 < (1u << 24) && a.nbv1 < (1u << 24);
     const bool mdma_ok = a.masked && a.softcap == 0.0f && direct && !no_mdma && a.mask_al4 && a.Nkv >= 64 && !(a.Nkv & 1) &&
                          (uint64_t)a.Nq * a.nbm1 < (1ull << 31);
     bool ksp_auto;
@@ -987,7 +1006,8 @@ void fattn_mma_variant(const FattnArgs & a, int ktype, FattnMmaVariant & v) {
     else if (!a.masked)       ksp_auto = wg1 <= cus && (wg1 * 5 <= (int64_t)cus * 3 || a.Nkv >= 1024) && a.Nkv > 128;
     else if (!mdma_ok && a.Nkv >= 256) ksp_auto = wg1 * 5 <= (int64_t)cus * 8;
     else                      ksp_auto = wg1 <= cus && (wg1 * 5 <= (int64_t)cus * 3 || a.Nkv >= 512);
-    const bool two  = a.D == 64 && (want_nqb ? want_nqb == 2 : two_auto);
+    // (a head zero-padded to 64 keeps to one query block: the two-block form stores whole rows of D floats)
+    const bool two  = a.D == 64 && a.Dv == a.D && (want_nqb ? want_nqb == 2 : two_auto);
     const bool ksp2 = !two && ktype == MI355X_TYPE_F16 && a.softcap == 0.0f && (want_ksp ? want_ksp == 2 : ksp_auto);
     v.query_blocks = two ? 2 : 1;
     v.key_split    = ksp2 ? 2 : 1;
@@ -998,6 +1018,7 @@ void fattn_mma_variant(const FattnArgs & a, int ktype, FattnMmaVariant & v) {
 
 bool fattn_mma_supported(const FattnArgs & a, int ktype) {
     if (a.D != 64 && a.D != 128) return false;
+    if (a.Dv != a.D && (a.Dv % 8 || a.Dv > a.D || ktype != MI355X_TYPE_F16)) return false;     // zero-padded heads
     if (a.Nq < 1 || a.Nkv < 1) return false;
     if (ktype != MI355X_TYPE_Q8_0 && !a.aligned16) return false;   // 128-bit K/V loads
     if (ktype == MI355X_TYPE_Q8_0 && !a.q_aligned16) return false;

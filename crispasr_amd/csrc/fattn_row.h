@@ -175,13 +175,13 @@ static __device__ __forceinline__ void row_scan(const RowScanArgs & a, const flo
 template <int LPR, bool COHERENT = false>
 static __device__ __forceinline__ void row_store(const FattnArgs & a, const RowPartial & st, int64_t row, int split, int lane) {
     const int d0 = lane * 8;
-    if (lane >= LPR || d0 >= a.D) return;
+    if (lane >= LPR || d0 >= a.Dv) return;           // (Dv < D: a head zero-padded to D; partial rows are D apart, dst rows Dv)
     if (a.n_splits == 1) {
         const float inv = st.l > 0.0f ? 1.0f / st.l : (st.l == st.l ? 0.0f : st.l);      // a NaN sum stays NaN, as on the CPU
-        float * out = a.dst + row * a.D + d0;
+        float * out = a.dst + row * a.Dv + d0;
 #pragma unroll
         for (int e = 0; e < 8; e++)
-            if (e < 4 || d0 + e < a.D) out[e] = st.acc[e] * inv;        // (D is a multiple of 4)
+            if (e < 4 || d0 + e < a.Dv) out[e] = st.acc[e] * inv;       // (the head size is a multiple of 4)
     } else {
         float * pa = a.part_acc + (row * a.n_splits + split) * a.D + d0;
 #pragma unroll
@@ -214,7 +214,7 @@ static __device__ __forceinline__ void attn_row_redo(const FattnArgs & a, int iq
     {
         const float * qrow = (const float *)(a.q + (int64_t)iq1 * a.nbq1 + (int64_t)h * a.nbq2 + (int64_t)b * a.nbq3);
 #pragma unroll
-        for (int e = 0; e < 8; e++) q[e] = qrow[d0 + e];
+        for (int e = 0; e < 8; e++) q[e] = d0 + e < a.Dv ? qrow[d0 + e] : 0.0f;      // (zero-padded head: Dv < D)
     }
     const int hk = h / a.gqa, bk = b / a.bq;
     RowMaskTensor mask;

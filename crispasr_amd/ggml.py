@@ -66,7 +66,8 @@ class CPlanInfo(ctypes.Structure):
     _fields_ = [("kernel", ctypes.c_int32), ("n_splits", ctypes.c_int32), ("keys_per_split", ctypes.c_int32),
                 ("kv_to_f16", ctypes.c_int32), ("workspace", ctypes.c_size_t),
                 ("queries_per_workgroup", ctypes.c_int32), ("query_blocks", ctypes.c_int32), ("key_split", ctypes.c_int32),
-                ("direct", ctypes.c_int32), ("mask_dma", ctypes.c_int32), ("merge_in_kernel", ctypes.c_int32)]
+                ("direct", ctypes.c_int32), ("mask_dma", ctypes.c_int32), ("merge_in_kernel", ctypes.c_int32),
+                ("head_pad", ctypes.c_int32)]
 
 
 class CDeviceInfo(ctypes.Structure):

@@ -215,6 +215,8 @@ typedef struct mi355x_fattn_plan_info {
     int32_t merge_in_kernel;         /* 1: the split-KV partials are merged by the last workgroup to finish each set of ranges (no
                                       * merge launch): calls on the library's scratch (params->workspace == NULL); the
                                       * allocation-free entry point does the same for the same shapes */
+    int32_t head_pad;                /* 0, or 64 / 128: the head size is neither, and the tile kernel runs on f16 copies of K and V
+                                      * whose rows are zero-padded to this size (kv_to_f16 is 1 then) */
 } mi355x_fattn_plan_info;
 int mi355x_fattn_plan_details(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
                               const mi355x_tensor * mask, const mi355x_fattn_params * params,

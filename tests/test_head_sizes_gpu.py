@@ -1,0 +1,115 @@
+"""Head sizes the tile kernel has no form of its own for (multiples of 8 below 128 other than 64) on the tile kernel:
+the launch that makes f16 copies of K and V pads their rows with zeros to 64 or 128, the kernel reads and writes the real
+head size.  Against the exact oracle at the head size itself, and against the vector kernel, which takes any head size.
+
+(The reference's runtimes with such heads: 32 in src/beat_this.cpp:41 and src/lfm2_audio.cpp:282, 48 in
+src/gigaam.cpp:166, 96 in src/piper_tts.cpp:471 and src/melotts.cpp:779; 80 is the 1280 / 16 of wider Whisper-like
+towers.  None of them is a BASELINE configuration; the op's contract covers them.)"""
+import numpy as np
+import pytest
+
+import oracle as ora
+from cases import make_case
+from crispasr_amd import ggml
+from gpu_util import assert_parity, plan_details, run_gpu, run_oracle
+from test_masked_nonfinite_gpu import dead_key_case
+
+pytestmark = pytest.mark.gpu
+
+VEC, MMA = ggml.KERNEL_VEC, ggml.KERNEL_MMA
+
+SHAPES = [
+    dict(seed=1201, D=80, Nq=300, Nkv=300, Hq=16, ktype=ora.F16),
+    dict(seed=1202, D=96, Nq=200, Nkv=333, Hq=8, Hkv=2, ktype=ora.F16, mask="causal"),
+    dict(seed=1203, D=32, Nq=130, Nkv=257, Hq=8, B=2, ktype=ora.F16, mask="bias_perhead"),
+    dict(seed=1204, D=48, Nq=64, Nkv=500, Hq=4, ktype=ora.F32),
+    dict(seed=1205, D=96, Nq=77, Nkv=190, Hq=8, Hkv=4, ktype=ora.Q8_0, mask="random_inf"),
+    dict(seed=1206, D=112, Nq=33, Nkv=65, Hq=6, B=2, Bk=1, ktype=ora.F16),
+    dict(seed=1207, D=72, Nq=100, Nkv=100, Hq=4, ktype=ora.F32, mask="causal", q_layout="thd", kv_layout="thd"),
+    dict(seed=1208, D=8, Nq=40, Nkv=70, Hq=4, ktype=ora.F16),
+    dict(seed=1209, D=32, Nq=48, Nkv=96, Hq=8, Hkv=2, ktype=ora.Q4_0, vtype=ora.Q8_0, mask="causal"),
+    dict(seed=1210, D=80, Nq=1500, Nkv=1500, Hq=16, ktype=ora.F16),                 # a Whisper-like tower of 16 heads of 80
+    dict(seed=1211, D=120, Nq=50, Nkv=2100, Hq=2, ktype=ora.F16, kv_layout="gap"),  # few query tiles, many keys: key ranges
+]
+
+
+@pytest.mark.parametrize("spec", SHAPES, ids=lambda s: "seed%d" % s["seed"])
+def test_tile_kernel_on_zero_padded_heads(spec):
+    case = make_case(**spec)
+    D = spec["D"]
+    plan = plan_details(case, kernel=MMA)
+    print("padded head", spec, plan, flush=True)
+    assert plan["kernel"] == MMA and plan["head_pad"] == (64 if D < 64 else 128) and plan["kv_to_f16"] == 1, plan
+    assert plan["query_blocks"] == 1, plan
+    ref = run_oracle(case)
+    got = run_gpu(case, kernel=MMA)
+    assert got.shape[-1] == D
+    assert_parity(got, ref, "tile kernel, head size %d padded to %d" % (D, plan["head_pad"]))
+    # in key ranges: partial rows of the padded size, merged into rows of the head size
+    if spec["Nkv"] >= 256:
+        assert plan_details(case, kernel=MMA, n_splits=3)["n_splits"] == 3
+    assert_parity(run_gpu(case, kernel=MMA, n_splits=3), ref, "... in 3 key ranges")
+    # what AUTO takes for the shape, and the vector kernel
+    auto = plan_details(case)
+    assert auto["kernel"] in (VEC, MMA), auto
+    assert_parity(run_gpu(case), ref, "AUTO (%s)" % ("tile" if auto["kernel"] == MMA else "vector"))
+    if spec["Nq"] * spec["Nkv"] <= 100000:
+        assert_parity(run_gpu(case, kernel=VEC), ref, "vector kernel")
+
+
+@pytest.mark.parametrize("variant", [17, 33])
+def test_both_one_block_forms_take_a_padded_head(variant):
+    """128-query workgroups and the key-split form (64 queries, the waves of a pair merging through LDS); the two-block
+    form, which stores whole rows of the padded size, is never taken"""
+    case = make_case(seed=1220, D=48, Nq=200, Nkv=300, Hq=6, ktype=ora.F16, mask="causal")
+    plan = plan_details(case, kernel=MMA, tile_variant=variant)
+    assert plan["head_pad"] == 64 and plan["query_blocks"] == 1 and plan["key_split"] == variant >> 4, plan
+    assert_parity(run_gpu(case, kernel=MMA, tile_variant=variant), run_oracle(case), "variant %d" % variant)
+    two = plan_details(case, kernel=MMA, tile_variant=18)
+    assert two["query_blocks"] == 1, two
+    assert_parity(run_gpu(case, kernel=MMA, tile_variant=18), run_oracle(case), "two blocks asked for")
+
+
+def test_padded_head_leaves_the_neighbouring_rows_alone():
+    """every dst row is Dv floats: a write of the padded width would land in the next (head, query)'s row - seen here as a
+    difference, since all rows are compared - and behind the last row in memory the call does not own"""
+    case = make_case(seed=1221, D=40, Nq=70, Nkv=90, Hq=3, B=2, ktype=ora.F16)
+    from gpu_util import upload
+    q, k, v = upload(case["q"]), upload(case["k"]), upload(case["v"])
+    import torch
+    n = 40 * 3 * 70 * 2
+    buf = torch.full((n + 256,), 7.0, device="cuda")
+    out = ggml.Tensor(buf.view(torch.uint8), ggml.F32, (40, 3, 70, 2))
+    ggml.flash_attn_ext(q, k, v, None, case["scale"], kernel=MMA, out=out)
+    torch.cuda.synchronize()
+    assert bool((buf[n:] == 7.0).all())
+    got = buf[:n].cpu().numpy().reshape(2, 70, 3, 40)
+    assert_parity(got, run_oracle(case), "rows of 40 floats")
+
+
+def test_padded_head_with_excluded_keys_that_hold_nan():
+    """the rows the tile kernel computes again (a non-finite K/V cell under a -inf mask value) read Dv elements of q and
+    write Dv of dst"""
+    n = 150
+    for pattern in (0, 1):
+        case = dead_key_case(range(n - 40, n), pattern, None, seed=1230 + pattern, D=96, Nq=40, Nkv=n, Hq=4, Hkv=2, ktype=ora.F16)
+        ref = run_oracle(case)
+        assert np.isfinite(ref).all()
+        assert plan_details(case, kernel=MMA)["head_pad"] == 128
+        assert_parity(run_gpu(case, kernel=MMA), ref, "pattern %d" % pattern)
+        assert_parity(run_gpu(case, kernel=MMA, n_splits=2), ref, "pattern %d, 2 key ranges" % pattern)
+
+
+def test_automatic_choice_for_other_head_sizes():
+    """few query rows stay on the vector kernel (the padded plan would not give them to the tile kernel); a prompt or an
+    encoder window goes to the tile kernel"""
+    small = make_case(seed=1240, D=80, Nq=1, Nkv=300, Hq=16, ktype=ora.F16)
+    assert plan_details(small)["kernel"] == VEC
+    big = make_case(seed=1241, D=80, Nq=256, Nkv=256, Hq=16, ktype=ora.F16)
+    p = plan_details(big)
+    assert p["kernel"] == MMA and p["head_pad"] == 128, p
+    # head sizes that are not multiples of 8, and those above 128, stay where they were
+    for D in (36, 52, 160, 256):
+        c = make_case(seed=1242, D=D, Nq=64, Nkv=64, Hq=2, ktype=ora.F16)
+        p = plan_details(c)
+        assert p["kernel"] == VEC and p["head_pad"] == 0, (D, p)
