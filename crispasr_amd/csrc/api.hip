@@ -723,11 +723,20 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         //  pairs on the copy launch and the padding pay - 1 to 3% off in the geometric mean, where the vector kernel alone
         //  is 27 to 71% off and 16 to 44 times slower at worst; above 64 also for 2 .. 15 queries from 150k pairs on, as
         //  for F32 caches of the sizes the tile kernel has forms for)
-        bool tile = plan.kernel == MI355X_FATTN_MMA && (p->kernel == MI355X_FATTN_MMA || pairs >= 100000);
-        if (!tile && p->kernel == MI355X_FATTN_AUTO && pad == 128 && a0.Nq >= 2 && a0.Nq < 16 && pairs >= 150000) {
-            mi355x_fattn_params by_name = *p;
-            by_name.kernel = MI355X_FATTN_MMA;
-            make_plan_core(b, ktype, vtype, &by_name, true, plan);
+        // (where the padded plan would take the decode kernel - 16 queries or more in 16-row chunks - the tile kernel stands
+        //  in: there is no padded decode kernel, and the vector kernel is 2 to 4 times slower on those shapes)
+        bool want = p->kernel == MI355X_FATTN_MMA;
+        if (!want) {
+            want = (pairs >= 100000 && (plan.kernel == MI355X_FATTN_MMA || (plan.kernel == MI355X_FATTN_DECODE_MMA && a0.Nq >= 16))) ||
+                   (pad == 128 && a0.Nq >= 2 && a0.Nq < 16 && pairs >= 150000);
+        }
+        bool tile = want;
+        if (want && p->kernel == MI355X_FATTN_AUTO) {
+            if (plan.kernel != MI355X_FATTN_MMA) {
+                mi355x_fattn_params by_name = *p;
+                by_name.kernel = MI355X_FATTN_MMA;
+                make_plan_core(b, ktype, vtype, &by_name, true, plan);
+            }
             FattnArgs c = b;
             use_f16_copies(c, nullptr);
             tile = fattn_mma_supported(c, MI355X_TYPE_F16);

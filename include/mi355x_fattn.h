@@ -143,8 +143,11 @@ int mi355x_stream_synchronize(void * stream);
  *   mask NULL, or F16 [>=Nkv, >=Nq, Hm, Bm], rows contiguous; head h reads h % Hm,
  *        batch b reads b % Bm; -inf entries exclude the key
  *   Hq % Hkv == 0 (query head h reads KV head h / (Hq/Hkv)), B % Bk == 0.
- *   D: a multiple of 4 up to 256.  64 and 128 run on the MFMA kernels; other multiples of 8 and - with F16 or F32 K/V of
- *   one type - multiples of 4 such as the 36 and 52 of src/core/cross_attn.h:119-153's smaller callers on the vector kernel.
+ *   D: a multiple of 4 up to 256.  64 and 128 run on the MFMA kernels.  Other multiples of 8 below 128 (32, 48, 80, 96 ...)
+ *   with 16 queries or more and 100000 (query row, key) pairs or more also run on the tile kernel, on f16 copies of K and V
+ *   in the workspace whose rows are zero-padded to 64 or 128 (mi355x_fattn_plan_info.head_pad; the result is that of the
+ *   head size itself); smaller calls of those sizes, larger multiples of 8 and - with F16 or F32 K/V of one type -
+ *   multiples of 4 such as the 36 and 52 of src/core/cross_attn.h:119-153's smaller callers run on the vector kernel.
  *   A row whose keys are all excluded (or Nkv == 0) yields zeros.
  *   An excluded key contributes nothing whatever its K/V bytes are - NaN, inf, a Q8_0 block whose scale is NaN - as in
  *   ggml-cpu, which skips it: cache slots that were never written may be masked out instead of cleared
