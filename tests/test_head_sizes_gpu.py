@@ -113,3 +113,37 @@ def test_automatic_choice_for_other_head_sizes():
         c = make_case(seed=1242, D=D, Nq=64, Nkv=64, Hq=2, ktype=ora.F16)
         p = plan_details(c)
         assert p["kernel"] == VEC and p["head_pad"] == 0, (D, p)
+
+
+def draw_padded(seed: int) -> dict:
+    """a draw of tests/test_fattn_random_gpu.py with the head size replaced by one that is padded (the block types where
+    the head is whole blocks, F16 / F32 elsewhere)"""
+    from test_fattn_random_gpu import draw
+    spec = draw(40000 + seed)
+    r = np.random.default_rng(77000 + seed)
+    spec["D"] = int(r.choice([8, 16, 24, 32, 40, 48, 56, 72, 80, 88, 96, 104, 112, 120]))
+    if spec["D"] % 32 and spec["ktype"] not in (ora.F16, ora.F32):
+        spec["ktype"] = int(r.choice([ora.F16, ora.F32]))
+    if "scale" in spec:
+        spec["scale"] = float(r.choice([0.5, 1.5])) * spec["D"] ** -0.5
+    spec["n_splits"] = int(r.choice([0, 1, 2, 3]))
+    return spec
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_shapes_on_zero_padded_heads(seed):
+    from test_fattn_random_gpu import assert_parity_by_rows
+    spec = draw_padded(seed)
+    variant, ns = spec.pop("variant"), spec.pop("n_splits")
+    print("padded case", spec, "variant", variant, "splits", ns, flush=True)
+    case = make_case(**spec)
+    ref = run_oracle(case)
+    hot = spec.get("scale", 0.0) * spec["D"] ** 0.5 > 1.2
+    tol = dict(max_abs_tol=3e-3) if hot else {}
+    f16_kv = spec["ktype"] == ora.F16
+    plan = plan_details(case, kernel=MMA, n_splits=ns)
+    assert plan["head_pad"] == (64 if spec["D"] < 64 else 128), plan
+    assert_parity_by_rows(run_gpu(case, kernel=MMA, n_splits=ns), ref, case, "padded tile kernel %s" % spec, f16_kv, **tol)
+    assert_parity_by_rows(run_gpu(case, kernel=MMA, n_splits=ns, tile_variant=variant), ref, case, "variant %d %s" % (variant, spec), f16_kv, **tol)
+    auto = plan_details(case)["kernel"]
+    assert_parity_by_rows(run_gpu(case), ref, case, "auto %s" % spec, f16_kv or auto == VEC, **tol)
