@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import oracle as ora
-from cases import make_case
+from cases import make_case, sweep_seeds
 from crispasr_amd import ggml
 from gpu_util import assert_parity, plan_details, run_gpu, run_oracle
 from test_masked_nonfinite_gpu import dead_key_case
@@ -130,7 +130,7 @@ def draw_padded(seed: int) -> dict:
     return spec
 
 
-@pytest.mark.parametrize("seed", range(60))
+@pytest.mark.parametrize("seed", sweep_seeds("PADDED_RANDOM_CASES", 60))
 def test_random_shapes_on_zero_padded_heads(seed):
     from test_fattn_random_gpu import assert_parity_by_rows
     spec = draw_padded(seed)
