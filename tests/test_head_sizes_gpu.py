@@ -147,3 +147,40 @@ def test_random_shapes_on_zero_padded_heads(seed):
     assert_parity_by_rows(run_gpu(case, kernel=MMA, n_splits=ns, tile_variant=variant), ref, case, "variant %d %s" % (variant, spec), f16_kv, **tol)
     auto = plan_details(case)["kernel"]
     assert_parity_by_rows(run_gpu(case), ref, case, "auto %s" % spec, f16_kv or auto == VEC, **tol)
+
+
+def test_graph_replays_of_a_padded_call_match_eager_calls():
+    """copy launch + tile kernel in key ranges + merge launch, recorded once and replayed with new contents in the same
+    buffers (a caller that captures passes its own workspace)"""
+    import torch
+    from gpu_util import upload
+    case = make_case(seed=1250, D=80, Nq=48, Nkv=900, Hq=6, Hkv=2, ktype=ora.F32, mask="causal")
+    q, k, v, m = upload(case["q"]), upload(case["k"]), upload(case["v"]), upload(case["mask"])
+    kw = dict(kernel=MMA, n_splits=3)
+    n = ggml.flash_attn_workspace_size(q, k, v, m, case["scale"], **kw)
+    assert n > 0
+    ws = torch.empty(n, dtype=torch.uint8, device="cuda")
+    got, want = ggml.Tensor.empty(ggml.F32, (80, 6, 48, 1)), ggml.Tensor.empty(ggml.F32, (80, 6, 48, 1))
+    ggml.flash_attn_ext(q, k, v, m, case["scale"], out=want, workspace=ws, **kw)          # modules loaded before the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            ggml.flash_attn_ext(q, k, v, m, case["scale"], out=got, workspace=ws, stream=side, **kw)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(11)
+    for replay in range(3):
+        for t in (q, k, v):
+            t.buf.copy_(torch.from_numpy(rng.standard_normal(t.buf.numel() // 4, dtype=np.float32).view(np.uint8)).cuda())
+        got.buf.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ggml.flash_attn_ext(q, k, v, m, case["scale"], out=want, workspace=ws, **kw)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.numpy_f32(), want.numpy_f32()), replay
+    host = dict(case)
+    host.update(q=ora.Tensor(q.to_host(), ora.F32, case["q"].ne, case["q"].nb), k=ora.Tensor(k.to_host(), ora.F32, case["k"].ne, case["k"].nb),
+                v=ora.Tensor(v.to_host(), ora.F32, case["v"].ne, case["v"].nb))
+    assert_parity(want.numpy_f32(), run_oracle(host), "after the replays")
