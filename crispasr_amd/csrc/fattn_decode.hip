@@ -295,8 +295,11 @@ template <int D> __device__ const V8Places<D> v8_places_table = v8_places<D>();
 // coalesced stream as K, and each 2-byte piece of a unit is written to its place - a pair of quants to [key][column],
 // a scale to [block][key] - by one ds_write_b16 whose address depends on the lane alone (read from a table behind the
 // first K/V request: computing the 36 of them costs more instructions than a 32-key step).
-template <int D, int TYPE, bool MASK, bool RAW, bool V8>
+// PAD: f16 rows of a.Dv elements (a multiple of 8 below D) read in place: the chunks of a row behind Dv are zeros in the
+// registers, q is read and dst written up to Dv.  An instantiation of its own: the others stay the code they were.
+template <int D, int TYPE, bool MASK, bool RAW, bool V8, bool PAD = false>
 __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const FattnArgs a) {
+    static_assert(!PAD || (TYPE == MI355X_TYPE_F16 && !RAW && !V8), "other head sizes: f16 rows, read per lane");
     static_assert(!V8 || RAW, "the int8 V stage belongs to the streamed Q8_0 path");
     constexpr int KS  = D / 32;                    // reduction steps of Q.K^T (one Q8_0 block each)
     constexpr int DBK = D / 16;                    // 16-wide blocks of the output's d
@@ -416,13 +419,17 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
             const int key = min(j0 + kb * 16 + j, k_end - 1);
             const char * row = kbase + (int64_t)key * a.nbk1;
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) kraw[s][kb][ks] = load_chunk<TYPE>(row, ks * 4 + g4);
+            for (int ks = 0; ks < KS; ks++) {
+                if (!PAD || (ks * 4 + g4) * 8 < a.Dv) kraw[s][kb][ks] = load_chunk<TYPE>(row, ks * 4 + g4);
+                else                                  kraw[s][kb][ks].v = make_uint4(0u, 0u, 0u, 0u);
+            }
         }
 #pragma unroll
         for (int i = 0; i < NV; i++) {
             const int flat = i * 64 + lane;
             const int key  = min(j0 + flat / CH, k_end - 1);
-            vraw[s][i] = load_chunk<TYPE>(vbase + (int64_t)key * a.nbv1, flat % CH);
+            if (!PAD || (flat % CH) * 8 < a.Dv) vraw[s][i] = load_chunk<TYPE>(vbase + (int64_t)key * a.nbv1, flat % CH);
+            else                                vraw[s][i].v = make_uint4(0u, 0u, 0u, 0u);
         }
     };
 
@@ -616,7 +623,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
         for (int ks = 0; ks < KS; ks++) {
             half8 v;
 #pragma unroll
-            for (int e = 0; e < 8; e++) v[e] = (_Float16)(qrow[ks * 32 + g4 * 8 + e] * qs);
+            for (int e = 0; e < 8; e++) v[e] = !PAD || ks * 32 + g4 * 8 < a.Dv ? (_Float16)(qrow[ks * 32 + g4 * 8 + e] * qs) : (_Float16)0.0f;
             qreg[ks] = v;
         }
     }
@@ -659,13 +666,14 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
         const int     ciq1 = (row0 + col) / a.gqa;
         const int     ch   = hk * a.gqa + (row0 + col) % a.gqa;
         const int64_t row  = ((int64_t)b * a.Nq + ciq1) * a.Hq + ch;
-        for (int d = tid & 15; d < D; d += 16) {
+        const int dv = PAD ? a.Dv : D;              // dst rows are dv floats; partial rows stay D apart
+        for (int d = tid & 15; d < dv; d += 16) {
             float acc = 0.0f;
 #pragma unroll
             for (int w = 0; w < DEC_WAVES; w++) acc += red_o[w][col][d] * f[w];
             bad = bad || not_finite(acc);
             if (a.n_splits == 1) {
-                a.dst[row * D + d] = L > 0.0f ? acc / L : 0.0f;
+                a.dst[row * dv + d] = L > 0.0f ? acc / L : 0.0f;
             } else if (a.counters) {
                 device_store(a.part_acc + (row * a.n_splits + split) * D + d, acc);
             } else {
@@ -715,7 +723,7 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
     }
 }
 
-template <int D, int TYPE, bool MASK, bool RAW, bool V8 = false>
+template <int D, int TYPE, bool MASK, bool RAW, bool V8 = false, bool PAD = false>
 int launch_one(const FattnArgs & a, hipStream_t stream) {
     const int64_t pairs = (int64_t)a.n_splits * a.Hkv * a.B;
     const int64_t wgs   = a.q_chunks == 1 ? pairs : (pairs + 7) / 8 * 8 * a.q_chunks;      // as the kernel numbers them
@@ -723,14 +731,19 @@ int launch_one(const FattnArgs & a, hipStream_t stream) {
     const dim3 grid((unsigned)wgs);
     constexpr int lds = decode_lds_bytes<D, TYPE, RAW, V8>();
     static std::atomic<uint64_t> lds_allowed{0};
-    const hipError_t e = fattn_allow_lds((const void *)fattn_decode_kernel<D, TYPE, MASK, RAW, V8>, lds, lds_allowed);
+    const hipError_t e = fattn_allow_lds((const void *)fattn_decode_kernel<D, TYPE, MASK, RAW, V8, PAD>, lds, lds_allowed);
     if (e != hipSuccess) return (int)e;
-    hipLaunchKernelGGL((fattn_decode_kernel<D, TYPE, MASK, RAW, V8>), grid, dim3(DEC_THREADS), lds, stream, a);
+    hipLaunchKernelGGL((fattn_decode_kernel<D, TYPE, MASK, RAW, V8, PAD>), grid, dim3(DEC_THREADS), lds, stream, a);
     return (int)hipGetLastError();
 }
 
 template <int D, int TYPE>
 int launch(const FattnArgs & a, hipStream_t stream) {
+    if (a.Dv != a.D) {              // another head size on f16 rows, or nothing
+        if constexpr (TYPE == MI355X_TYPE_F16)
+            return a.mask ? launch_one<D, TYPE, true, false, false, true>(a, stream) : launch_one<D, TYPE, false, false, false, true>(a, stream);
+        return (int)hipErrorInvalidValue;
+    }
     if constexpr (FATTN_IS_BLOCK_TYPE(TYPE)) {
         // contiguous rows, and every step of every (head, batch, split) starts on a unit boundary
         constexpr int RS   = D / 32 * raw_block_bytes<TYPE>();
@@ -754,6 +767,7 @@ int launch(const FattnArgs & a, hipStream_t stream) {
 
 bool fattn_decode_supported(const FattnArgs & a, int ktype) {
     if (a.D != 64 && a.D != 128) return false;
+    if (a.Dv != a.D && (a.Dv % 8 || a.Dv > a.D || ktype != MI355X_TYPE_F16)) return false;       // other head sizes: f16 rows read in place
     if (a.Nq < 1 || a.Nkv < 1) return false;
     if ((int64_t)a.Nq * a.gqa > ((int64_t)1 << 20)) return false;      // 16-row chunks of the rows that share a KV head
     if (a.softcap != 0.0f) return false;

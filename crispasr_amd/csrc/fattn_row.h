@@ -75,8 +75,8 @@ struct RowScanArgs {
 };
 static __device__ __forceinline__ RowScanArgs row_scan_args(const FattnArgs & a) {
     RowScanArgs r;
-    r.D = a.D; r.scale = a.scale; r.softcap = a.softcap; r.nbk1 = a.nbk1; r.nbv1 = a.nbv1;
-    r.aligned16 = a.aligned16 != 0 && a.D % 8 == 0;       // (a 16-byte load of a row's last 4 elements would run past the row)
+    r.D = a.Dv; r.scale = a.scale; r.softcap = a.softcap; r.nbk1 = a.nbk1; r.nbv1 = a.nbv1;
+    r.aligned16 = a.aligned16 != 0 && a.Dv % 8 == 0;       // (a 16-byte load of a row's last 4 elements would run past the row)
     return r;
 }
 

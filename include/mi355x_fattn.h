@@ -143,11 +143,13 @@ int mi355x_stream_synchronize(void * stream);
  *   mask NULL, or F16 [>=Nkv, >=Nq, Hm, Bm], rows contiguous; head h reads h % Hm,
  *        batch b reads b % Bm; -inf entries exclude the key
  *   Hq % Hkv == 0 (query head h reads KV head h / (Hq/Hkv)), B % Bk == 0.
- *   D: a multiple of 4 up to 256.  64 and 128 run on the MFMA kernels.  Other multiples of 8 below 128 (32, 48, 80, 96 ...)
- *   with 16 queries or more and 100000 (query row, key) pairs or more also run on the tile kernel, on f16 copies of K and V
- *   in the workspace whose rows are zero-padded to 64 or 128 (mi355x_fattn_plan_info.head_pad; the result is that of the
- *   head size itself); smaller calls of those sizes, larger multiples of 8 and - with F16 or F32 K/V of one type -
- *   multiples of 4 such as the 36 and 52 of src/core/cross_attn.h:119-153's smaller callers run on the vector kernel.
+ *   D: a multiple of 4 up to 256.  64 and 128 run on the MFMA kernels.  So do the other multiples of 8 below 128 (32, 48,
+ *   80, 96 ...; mi355x_fattn_plan_info.head_pad; the result is that of the head size itself): decode-shaped calls over
+ *   F16 caches on the decode kernel, which reads the rows where they lie and fills a row's registers behind the head's
+ *   own elements with zeros; calls with 16 queries or more and 100000 (query row, key) pairs or more on the tile kernel, on
+ *   f16 copies of K and V in the workspace whose rows are zero-padded to 64 or 128.  Smaller calls of those sizes, few
+ *   query rows over F32 or quantised caches, larger multiples of 8 and - with F16 or F32 K/V of one type - multiples of 4
+ *   such as the 36 and 52 of src/core/cross_attn.h:119-153's smaller callers run on the vector kernel.
  *   A row whose keys are all excluded (or Nkv == 0) yields zeros.
  *   An excluded key contributes nothing whatever its K/V bytes are - NaN, inf, a Q8_0 block whose scale is NaN - as in
  *   ggml-cpu, which skips it: cache slots that were never written may be masked out instead of cleared
@@ -218,8 +220,9 @@ typedef struct mi355x_fattn_plan_info {
     int32_t merge_in_kernel;         /* 1: the split-KV partials are merged by the last workgroup to finish each set of ranges (no
                                       * merge launch): calls on the library's scratch (params->workspace == NULL); the
                                       * allocation-free entry point does the same for the same shapes */
-    int32_t head_pad;                /* 0, or 64 / 128: the head size is neither, and the tile kernel runs on f16 copies of K and V
-                                      * whose rows are zero-padded to this size (kv_to_f16 is 1 then) */
+    int32_t head_pad;                /* 0, or 64 / 128: the head size is neither, and the kernel runs the form for this size - the
+                                      * tile kernel on f16 copies of K and V whose rows are zero-padded to it (kv_to_f16 is 1), the
+                                      * decode kernel on the F16 rows themselves (kv_to_f16 is 0) */
 } mi355x_fattn_plan_info;
 int mi355x_fattn_plan_details(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
                               const mi355x_tensor * mask, const mi355x_fattn_params * params,

@@ -1,6 +1,7 @@
-"""Head sizes the tile kernel has no form of its own for (multiples of 8 below 128 other than 64) on the tile kernel:
-the launch that makes f16 copies of K and V pads their rows with zeros to 64 or 128, the kernel reads and writes the real
-head size.  Against the exact oracle at the head size itself, and against the vector kernel, which takes any head size.
+"""Head sizes the MFMA kernels have no form of their own for (multiples of 8 below 128 other than 64).  On the tile
+kernel: the launch that makes f16 copies of K and V pads their rows with zeros to 64 or 128, the kernel reads and writes
+the real head size.  On the decode kernel: f16 rows are read where they lie, the chunks behind the head's own are zeros
+in registers.  Against the exact oracle at the head size itself, and against the vector kernel, which takes any head size.
 
 (The reference's runtimes with such heads: 32 in src/beat_this.cpp:41 and src/lfm2_audio.cpp:282, 48 in
 src/gigaam.cpp:166, 96 in src/piper_tts.cpp:471 and src/melotts.cpp:779; 80 is the 1280 / 16 of wider Whisper-like
@@ -16,7 +17,7 @@ from test_masked_nonfinite_gpu import dead_key_case
 
 pytestmark = pytest.mark.gpu
 
-VEC, MMA = ggml.KERNEL_VEC, ggml.KERNEL_MMA
+VEC, MMA, DEC = ggml.KERNEL_VEC, ggml.KERNEL_MMA, ggml.KERNEL_DECODE_MMA
 
 SHAPES = [
     dict(seed=1201, D=80, Nq=300, Nkv=300, Hq=16, ktype=ora.F16),
@@ -51,8 +52,7 @@ def test_tile_kernel_on_zero_padded_heads(spec):
     assert_parity(run_gpu(case, kernel=MMA, n_splits=3), ref, "... in 3 key ranges")
     # what AUTO takes for the shape, and the vector kernel
     auto = plan_details(case)
-    assert auto["kernel"] in (VEC, MMA), auto
-    assert_parity(run_gpu(case), ref, "AUTO (%s)" % ("tile" if auto["kernel"] == MMA else "vector"))
+    assert_parity(run_gpu(case), ref, "AUTO (kernel %d)" % auto["kernel"])
     if spec["Nq"] * spec["Nkv"] <= 100000:
         assert_parity(run_gpu(case, kernel=VEC), ref, "vector kernel")
 
@@ -100,11 +100,69 @@ def test_padded_head_with_excluded_keys_that_hold_nan():
         assert_parity(run_gpu(case, kernel=MMA, n_splits=2), ref, "pattern %d, 2 key ranges" % pattern)
 
 
+DECODE_SHAPES = [
+    dict(seed=1301, D=80, Nq=1, Nkv=300, Hq=16),                                          # one token, unsplit or split
+    dict(seed=1302, D=80, Nq=5, Nkv=1500, Hq=16, q_layout="thd", kv_layout="thd"),        # 5 beams against an encoder memory
+    dict(seed=1303, D=96, Nq=1, Nkv=663, Hq=32, Hkv=8),                                   # a GQA step
+    dict(seed=1304, D=48, Nq=1, Nkv=224, Hq=12, B=5, mask="random_inf"),                  # beams in a unified cache, masked
+    dict(seed=1305, D=32, Nq=3, Nkv=77, Hq=8, Hkv=2, B=2, Bk=1, mask="causal"),
+    dict(seed=1306, D=112, Nq=2, Nkv=1031, Hq=4, kv_layout="gap", mask="bias_perhead"),
+    dict(seed=1307, D=8, Nq=1, Nkv=40, Hq=4),
+    dict(seed=1308, D=120, Nq=40, Nkv=50, Hq=4, Hkv=2, mask="causal"),                    # five 16-row chunks per KV head
+    dict(seed=1309, D=72, Nq=1, Nkv=4100, Hq=8, kv_pad_rows=28),
+]
+
+
+@pytest.mark.parametrize("ns", [0, 1, 3])
+@pytest.mark.parametrize("spec", DECODE_SHAPES, ids=lambda s: "seed%d" % s["seed"])
+def test_decode_kernel_reads_other_head_sizes_in_place(spec, ns):
+    case = make_case(ktype=ora.F16, **spec)
+    D = spec["D"]
+    plan = plan_details(case, kernel=DEC, n_splits=ns)
+    print("decode kernel, head size", D, spec, plan, flush=True)
+    assert plan["kernel"] == DEC and plan["head_pad"] == (64 if D < 64 else 128) and plan["kv_to_f16"] == 0, plan
+    ref = run_oracle(case)
+    got = run_gpu(case, kernel=DEC, n_splits=ns)
+    assert got.shape[-1] == D
+    assert_parity(got, ref, "decode kernel, head size %d, %d key ranges" % (D, plan["n_splits"]))
+    if ns == 0:
+        auto = plan_details(case)
+        assert_parity(run_gpu(case), ref, "AUTO (kernel %d)" % auto["kernel"])
+
+
+def test_decode_kernel_at_another_head_size_with_excluded_keys_that_hold_nan():
+    n = 300
+    for pattern in (0, 1):
+        case = dead_key_case(range(n - 50, n), pattern, None, seed=1320 + pattern, D=80, Nq=2, Nkv=n, Hq=8, Hkv=4, ktype=ora.F16)
+        ref = run_oracle(case)
+        assert np.isfinite(ref).all()
+        for ns in (1, 4):
+            assert plan_details(case, kernel=DEC, n_splits=ns)["head_pad"] == 128
+            assert_parity(run_gpu(case, kernel=DEC, n_splits=ns), ref, "pattern %d, %d key ranges" % (pattern, ns))
+
+
+def test_decode_kernel_at_another_head_size_leaves_the_neighbouring_rows_alone():
+    import torch
+    from gpu_util import upload
+    case = make_case(seed=1330, D=40, Nq=3, Nkv=200, Hq=6, B=2, ktype=ora.F16)
+    q, k, v = upload(case["q"]), upload(case["k"]), upload(case["v"])
+    n = 40 * 6 * 3 * 2
+    for ns in (1, 3):
+        buf = torch.full((n + 256,), 7.0, device="cuda")
+        out = ggml.Tensor(buf.view(torch.uint8), ggml.F32, (40, 6, 3, 2))
+        ggml.flash_attn_ext(q, k, v, None, case["scale"], kernel=DEC, n_splits=ns, out=out)
+        torch.cuda.synchronize()
+        assert bool((buf[n:] == 7.0).all())
+        assert_parity(buf[:n].cpu().numpy().reshape(2, 3, 6, 40), run_oracle(case), "rows of 40 floats, %d ranges" % ns)
+
+
 def test_automatic_choice_for_other_head_sizes():
-    """few query rows stay on the vector kernel (the padded plan would not give them to the tile kernel); a prompt or an
-    encoder window goes to the tile kernel"""
+    """decode-shaped calls over f16 caches go to the decode kernel, over F32 caches they stay on the vector kernel; a
+    prompt or an encoder window goes to the tile kernel"""
     small = make_case(seed=1240, D=80, Nq=1, Nkv=300, Hq=16, ktype=ora.F16)
-    assert plan_details(small)["kernel"] == VEC
+    p = plan_details(small)
+    assert p["kernel"] == DEC and p["head_pad"] == 128 and p["kv_to_f16"] == 0, p
+    assert plan_details(make_case(seed=1240, D=80, Nq=1, Nkv=300, Hq=16, ktype=ora.F32))["kernel"] == VEC
     big = make_case(seed=1241, D=80, Nq=256, Nkv=256, Hq=16, ktype=ora.F16)
     p = plan_details(big)
     assert p["kernel"] == MMA and p["head_pad"] == 128, p
@@ -147,6 +205,13 @@ def test_random_shapes_on_zero_padded_heads(seed):
     assert_parity_by_rows(run_gpu(case, kernel=MMA, n_splits=ns, tile_variant=variant), ref, case, "variant %d %s" % (variant, spec), f16_kv, **tol)
     auto = plan_details(case)["kernel"]
     assert_parity_by_rows(run_gpu(case), ref, case, "auto %s" % spec, f16_kv or auto == VEC, **tol)
+    if f16_kv:                                                  # the decode kernel reads such rows in place (no soft cap)
+        try:
+            got = run_gpu(case, kernel=DEC, n_splits=ns)
+        except ggml.UnsupportedError:
+            assert spec.get("softcap", 0.0) != 0.0, spec
+        else:
+            assert_parity_by_rows(got, ref, case, "decode kernel %s" % spec, True, **tol)
 
 
 def test_graph_replays_of_a_padded_call_match_eager_calls():

@@ -422,32 +422,41 @@ def test_key_ranges_of_the_vector_and_tile_kernels():
     assert plan(128, 407, 32, 1, 407, ca.F16) == (mma, 1)            # the 407-token prefill
 
 
-def test_other_head_sizes_are_planned_onto_zero_padded_copies():
-    """multiples of 8 below 128 other than 64: the tile kernel on f16 copies of K/V padded to 64 or 128 - one query
-    block per wave, the copies in the workspace; few query rows, other head sizes and MI355X_FATTN_VEC by name keep the
-    vector kernel"""
+def test_other_head_sizes_are_planned_onto_zero_padded_forms():
+    """multiples of 8 below 128 other than 64.  Prompts and encoder windows: the tile kernel on f16 copies of K/V padded to
+    64 or 128 - one query block per wave, the copies in the workspace.  Decode-shaped calls over f16 caches: the decode
+    kernel, which reads the rows where they lie.  F32 and quantised caches under few query rows, small calls, other head
+    sizes and MI355X_FATTN_VEC by name keep the vector kernel."""
+    mma, dec, vec = ggml.KERNEL_MMA, ggml.KERNEL_DECODE_MMA, ggml.KERNEL_VEC
     def details(D, Nq, H, Nkv, kt=ca.F16, **kw):
         q = _t(ca.F32, (D, Nq, H, 1))
         k = _t(kt, (D, Nkv, H, 1))
         return ggml.flash_attn_plan_details(q, k, k, None, **kw)
     for D, pad in ((32, 64), (48, 64), (80, 128), (96, 128), (120, 128)):
         p = details(D, 300, 16, 300)
-        assert (p["kernel"], p["head_pad"], p["kv_to_f16"], p["n_splits"], p["query_blocks"]) == (ggml.KERNEL_MMA, pad, 1, 1, 1), (D, p)
+        assert (p["kernel"], p["head_pad"], p["kv_to_f16"], p["n_splits"], p["query_blocks"]) == (mma, pad, 1, 1, 1), (D, p)
         assert p["workspace"] == 2 * pad * 300 * 16 * 2, (D, p)
-        assert details(D, 300, 16, 300, kernel=ggml.KERNEL_VEC)["head_pad"] == 0
+        assert details(D, 300, 16, 300, kernel=vec)["head_pad"] == 0
+        # one query row per head: the decode kernel in place (no copies; partial rows of the padded size when it splits)
+        p = details(D, 1, 16, 1500)
+        assert (p["kernel"], p["head_pad"], p["kv_to_f16"]) == (dec, pad, 0), (D, p)
+        assert p["n_splits"] > 1 and p["workspace"] == 16 * p["n_splits"] * (pad + 2) * 4, (D, p)
+        assert details(D, 1, 16, 1500, ca.F32)["kernel"] == vec                    # (the decode kernel does not read F32)
     assert details(96, 300, 16, 300, ca.Q8_0)["head_pad"] == 128
-    p = details(80, 32, 4, 8192, kernel=ggml.KERNEL_MMA)             # a small grid against a long cache: key ranges, partial rows of 128
+    assert details(96, 1, 16, 300, ca.Q8_0)["kernel"] == vec
+    p = details(80, 32, 4, 8192, kernel=mma)                         # a small grid against a long cache: key ranges, partial rows of 128
     assert p["n_splits"] > 1 and p["workspace"] == 2 * 128 * 8192 * 4 * 2 + 32 * 4 * p["n_splits"] * (128 + 2) * 4, p
     for D in (36, 52, 64, 128, 160):
         assert details(D, 300, 16, 300)["head_pad"] == 0, D
-    p = details(80, 1, 16, 300)
-    assert (p["kernel"], p["head_pad"]) == (ggml.KERNEL_VEC, 0), p
-    # too small to pay for the copy launch (100k query-key pairs); 2 .. 15 queries only above 64, from 150k pairs on
-    assert details(48, 300, 1, 200)["kernel"] == ggml.KERNEL_VEC
-    assert details(48, 300, 1, 400)["kernel"] == ggml.KERNEL_MMA
-    assert (details(80, 8, 16, 4096)["kernel"], details(80, 8, 16, 4096)["head_pad"]) == (ggml.KERNEL_MMA, 128)
-    assert details(80, 8, 16, 1024)["kernel"] == ggml.KERNEL_VEC
-    assert details(32, 8, 16, 4096)["kernel"] == ggml.KERNEL_VEC
+    # a small f16 call in 16-row chunks: the decode kernel, as at 64
+    assert details(48, 300, 1, 200)["kernel"] == dec
+    assert details(48, 300, 1, 400)["kernel"] == mma
+    # F32 caches: too small to pay for the copy launch (100k query-key pairs); 2 .. 15 queries only above 64, from 150k pairs on
+    assert details(48, 300, 1, 200, ca.F32)["kernel"] == vec
+    assert (details(80, 8, 16, 4096, ca.F32)["kernel"], details(80, 8, 16, 4096, ca.F32)["head_pad"]) == (mma, 128)
+    assert details(80, 8, 16, 1024, ca.F32)["kernel"] == vec
+    assert details(32, 8, 16, 4096, ca.F32)["kernel"] == vec
+    assert details(80, 8, 16, 4096)["kernel"] == dec
 
 
 def test_a_call_is_sized_the_same_with_and_without_its_data_pointers():
