@@ -18,6 +18,8 @@ CALLS = [
     (dict(seed=801, D=128, Nq=300, Nkv=1100, Hq=8, Hkv=2, ktype=ora.Q8_0, mask="causal"), {}),
     (dict(seed=802, D=64, Nq=5, Nkv=1500, Hq=20, q_layout="thd", kv_layout="thd", scale=0.35355339), {}),
     (dict(seed=803, D=128, Nq=1, Nkv=663, Hq=32, Hkv=8, ktype=ora.Q8_0), dict(q_quant=ggml.Q8_0)),
+    # a head size the tile kernel takes on zero-padded f16 copies, which go to the scratch as well
+    (dict(seed=804, D=80, Nq=200, Nkv=300, Hq=8, ktype=ora.F32, mask="causal"), {}),
 ]
 
 
