@@ -703,12 +703,14 @@ void make_plan_core(const FattnArgs & a0, int ktype, int vtype, const mi355x_fat
     }
 }
 
-// Head sizes the tile kernel has no form for (multiples of 8 below 128 other than 64: 32 and 48, 80 and 96 of other
-// Whisper-like towers, ...) can still run on it: the launch that makes f16 copies of K and V pads their rows with zeros to
-// 64 or 128, the kernel reads Dv elements of every q row and writes Dv of every dst row.  The products over the padding
-// are exact zeros, so the result is what the head size itself would give; the cost is the padded share of the MFMA work
-// and the copy.  The vector kernel, which takes any head size, keeps the calls the padded plan would not give to the tile
-// kernel (few query rows) and those too small to pay for the copy launch.
+// Head sizes the MFMA kernels have no form for (multiples of 8 below 128 other than 64: 32 and 48, 80 and 96 of other
+// Whisper-like towers, ...) can still run on them, as the next larger of 64 and 128 with zeros behind the head's own
+// elements: the products over the padding are exact zeros, so the result is what the head size itself would give.
+//  - The tile kernel: the launch that makes f16 copies of K and V pads their rows, the kernel reads Dv elements of every q
+//    row and writes Dv of every dst row.  The cost is the padded share of the MFMA work and the copy.
+//  - The decode kernel, over F16 caches: it reads the rows where they lie and pads in its registers.  No copy.
+// The vector kernel, which takes any head size, keeps what neither takes: few query rows over F32 and quantised caches,
+// and calls too small to pay for the copy launch.
 void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_params * p, Plan & plan) {
     static const bool no_pad = getenv("MI355X_FATTN_NO_PAD") != nullptr;        // comparison runs
     const int pad = a0.D >= 8 && a0.D < 128 && a0.D != 64 && a0.D % 8 == 0 ? (a0.D < 64 ? 64 : 128) : 0;
@@ -767,8 +769,8 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         //  pairs on the copy launch and the padding pay - 1 to 3% off in the geometric mean, where the vector kernel alone
         //  is 27 to 71% off and 16 to 44 times slower at worst; above 64 also for 2 .. 15 queries from 150k pairs on, as
         //  for F32 caches of the sizes the tile kernel has forms for)
-        // (where the padded plan would take the decode kernel - 16 queries or more in 16-row chunks - the tile kernel stands
-        //  in: there is no padded decode kernel, and the vector kernel is 2 to 4 times slower on those shapes)
+        // (where the padded plan would take the decode kernel - 16 queries or more in 16-row chunks over F32 or quantised
+        //  K/V, which that kernel does not pad - the tile kernel stands in: the vector kernel is 2 to 4 times slower there)
         bool want = p->kernel == MI355X_FATTN_MMA;
         if (!want) {
             want = (pairs >= 100000 && (plan.kernel == MI355X_FATTN_MMA || (plan.kernel == MI355X_FATTN_DECODE_MMA && a0.Nq >= 16))) ||
