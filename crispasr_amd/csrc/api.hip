@@ -727,24 +727,19 @@ void make_plan(const FattnArgs & a0, int ktype, int vtype, const mi355x_fattn_pa
         // (decode against vector and padded tile kernel over 1 .. 1024 queries x 4 .. 64 heads x 64 .. 4096 keys at head
         // sizes 32, 48, 80, 96; 864 shapes):
         //  - up to 16 rows per KV head: always, whatever the plan at the padded size says of 9 .. 16 rows (the tile kernel
-        //    would need the copies) - but for small calls above 64, where the vector kernel's 5.6 - 6.4 us beat its 7.2 - 9;
-        //  - more rows: while the 16-row chunks fit two rounds of workgroups, there are at most 32 of them per KV head (each
-        //    streams the head's K/V again) and, above 64, up to 1024 keys or 64k chunk-keys.
-        // These rules are 1-3% off the fastest of the three in the geometric mean; the tile kernel alone is 11-19% off on
-        // the shapes of more than 16 rows, the vector kernel 2 to 10 times slower from 1024 keys on.
+        //    would need the copies; the vector kernel is level at 64 keys and 1 - 2 us behind from 256 on);
+        //  - more rows: up to 64 chunks of 16 per KV head, each of which streams the head's K/V again, in up to three rounds
+        //    of workgroups, while a head's chunks see no more than 64k keys between them and all chunks 512k.
+        // These rules are 1% off the fastest of the three in the geometric mean (1.5x at worst); the tile kernel alone is
+        // 11-19% off on the shapes of more than 16 rows, the vector kernel 2 to 10 times slower from 1024 keys on.
         if (p->kernel == MI355X_FATTN_AUTO && fattn_decode_supported(b, ktype)) {
             bool dec = plan.kernel == MI355X_FATTN_DECODE_MMA;
-            // (small calls above 64: up to 1024 rows against up to 64 keys, up to 128 rows against up to 256 keys)
-            const int64_t rows      = (int64_t)a0.Nq * a0.Hq * a0.B;
-            const bool    vec_small = pad == 128 && ((a0.Nkv <= 64 && rows <= 1024) || (a0.Nkv <= 256 && rows <= 128));
-            if (vec_small) {
-                dec = false;
-            } else if (a0.q_chunks <= 1) {
+            if (a0.q_chunks <= 1) {
                 dec = true;
-            } else if (!dec && a0.q_chunks <= 32) {
+            } else if (!dec) {
                 const int64_t chunk_wgs = (int64_t)a0.q_chunks * a0.Hkv * a0.B;
-                dec = chunk_wgs <= 2 * (int64_t)device_cus() &&
-                      (pad == 64 ? chunk_wgs * a0.Nkv <= (1 << 20) : a0.Nkv <= 1024 || chunk_wgs * a0.Nkv <= (1 << 16));
+                dec = a0.q_chunks <= 64 && chunk_wgs <= 3 * (int64_t)device_cus() &&
+                      (int64_t)a0.q_chunks * a0.Nkv <= (1 << 16) && chunk_wgs * a0.Nkv <= (1 << 19);
             }
             if (dec && plan.kernel != MI355X_FATTN_DECODE_MMA) {
                 mi355x_fattn_params by_name = *p;

@@ -622,8 +622,19 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             half8 v;
+            if constexpr (PAD) {
+                // every lane reads 8 elements that exist (its own, or the row's first 8 where it has none) and the lanes
+                // without scale them by zero: under a guard each, the 8 * KS loads waited for one another - 2 us per call.
+                // (A q row with inf or NaN in it gives NaN either way.)
+                const bool    own = ks * 32 + g4 * 8 < a.Dv;
+                const float * q8  = qrow + (own ? ks * 32 + g4 * 8 : 0);
+                const float   qsl = own ? qs : 0.0f;
 #pragma unroll
-            for (int e = 0; e < 8; e++) v[e] = !PAD || ks * 32 + g4 * 8 < a.Dv ? (_Float16)(qrow[ks * 32 + g4 * 8 + e] * qs) : (_Float16)0.0f;
+                for (int e = 0; e < 8; e++) v[e] = (_Float16)(q8[e] * qsl);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) v[e] = (_Float16)(qrow[ks * 32 + g4 * 8 + e] * qs);
+            }
             qreg[ks] = v;
         }
     }

@@ -227,16 +227,19 @@ __global__ void __launch_bounds__(MMA_THREADS, 2) fattn_mma_kernel(const FattnAr
         const float * qrow = (const float *)(a.q + (int64_t)qi * a.nbq1 + (int64_t)h * a.nbq2 + (int64_t)b * a.nbq3);
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-            float4 x0 = {0.0f, 0.0f, 0.0f, 0.0f}, x1 = x0;
-            if (whole_head || ks * 16 + hh * 8 < a.Dv) {   // (a head zero-padded to D: nothing to read behind Dv, a multiple of 8)
-                x0 = *(const float4 *)(qrow + ks * 16 + hh * 8);
-                x1 = *(const float4 *)(qrow + ks * 16 + hh * 8 + 4);
-            }
+            // (a head zero-padded to D: a lane with nothing to read behind Dv, a multiple of 8, reads the row's first 8
+            //  elements instead and scales them by zero - loads under a guard each wait for one another.  A q row with inf
+            //  or NaN in it gives NaN either way.)
+            const bool    own = whole_head || ks * 16 + hh * 8 < a.Dv;
+            const float * q8  = qrow + (own ? ks * 16 + hh * 8 : 0);
+            const float   qs  = own ? qscale : 0.0f;
+            const float4  x0  = *(const float4 *)q8;
+            const float4  x1  = *(const float4 *)(q8 + 4);
             half8 v;
-            v[0] = (_Float16)(x0.x * qscale); v[1] = (_Float16)(x0.y * qscale);
-            v[2] = (_Float16)(x0.z * qscale); v[3] = (_Float16)(x0.w * qscale);
-            v[4] = (_Float16)(x1.x * qscale); v[5] = (_Float16)(x1.y * qscale);
-            v[6] = (_Float16)(x1.z * qscale); v[7] = (_Float16)(x1.w * qscale);
+            v[0] = (_Float16)(x0.x * qs); v[1] = (_Float16)(x0.y * qs);
+            v[2] = (_Float16)(x0.z * qs); v[3] = (_Float16)(x0.w * qs);
+            v[4] = (_Float16)(x1.x * qs); v[5] = (_Float16)(x1.y * qs);
+            v[6] = (_Float16)(x1.z * qs); v[7] = (_Float16)(x1.w * qs);
             qreg[qb][ks] = v;
         }
     }

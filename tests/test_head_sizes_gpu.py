@@ -163,10 +163,10 @@ def test_automatic_choice_for_other_head_sizes():
     p = plan_details(small)
     assert p["kernel"] == DEC and p["head_pad"] == 128 and p["kv_to_f16"] == 0, p
     assert plan_details(make_case(seed=1240, D=80, Nq=1, Nkv=300, Hq=16, ktype=ora.F32))["kernel"] == VEC
-    big = make_case(seed=1241, D=80, Nq=600, Nkv=600, Hq=16, ktype=ora.F16)
+    big = make_case(seed=1241, D=80, Nq=1100, Nkv=1100, Hq=16, ktype=ora.F16)
     p = plan_details(big)
     assert p["kernel"] == MMA and p["head_pad"] == 128, p
-    assert_parity(run_gpu(big), run_oracle(big), "600 x 600 x 16 heads of 80")
+    assert_parity(run_gpu(big), run_oracle(big), "1100 x 1100 x 16 heads of 80")
     mid = make_case(seed=1243, D=80, Nq=256, Nkv=256, Hq=16, ktype=ora.F16, mask="causal")       # 16 chunks per head, 256 in all
     p = plan_details(mid)
     assert p["kernel"] == DEC and p["head_pad"] == 128 and p["kv_to_f16"] == 0, p

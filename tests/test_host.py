@@ -433,11 +433,11 @@ def test_other_head_sizes_are_planned_onto_zero_padded_forms():
         k = _t(kt, (D, Nkv, H, 1))
         return ggml.flash_attn_plan_details(q, k, k, None, **kw)
     for D, pad in ((32, 64), (48, 64), (80, 128), (96, 128), (120, 128)):
-        p = details(D, 600, 16, 600)
+        p = details(D, 1100, 16, 1100)
         assert (p["kernel"], p["head_pad"], p["kv_to_f16"], p["n_splits"], p["query_blocks"]) == (mma, pad, 1, 1, 1), (D, p)
-        assert p["workspace"] == 2 * pad * 600 * 16 * 2, (D, p)
-        assert details(D, 600, 16, 600, kernel=vec)["head_pad"] == 0
-        # up to 32 chunks of 16 rows per KV head in two rounds of workgroups: the decode kernel in place, no copy launch
+        assert p["workspace"] == 2 * pad * 1100 * 16 * 2, (D, p)
+        assert details(D, 1100, 16, 1100, kernel=vec)["head_pad"] == 0
+        # up to 64 chunks of 16 rows per KV head in three rounds of workgroups: the decode kernel in place, no copy launch
         p = details(D, 300, 16, 300)
         assert (p["kernel"], p["head_pad"], p["kv_to_f16"]) == (dec, pad, 0), (D, p)
         assert details(D, 300, 16, 300, ca.F32)["kernel"] == mma
@@ -452,14 +452,14 @@ def test_other_head_sizes_are_planned_onto_zero_padded_forms():
     assert p["n_splits"] > 1 and p["workspace"] == 2 * 128 * 8192 * 4 * 2 + 32 * 4 * p["n_splits"] * (128 + 2) * 4, p
     for D in (36, 52, 64, 128, 160):
         assert details(D, 300, 16, 300)["head_pad"] == 0, D
-    # a small f16 call in 16-row chunks: the decode kernel, as at 64; above 64 up to 1024 keys
+    # f16 calls in 16-row chunks: the decode kernel while a head's chunks see no more than 64k keys between them
     assert details(48, 300, 1, 200)["kernel"] == dec
-    assert details(48, 300, 1, 4000)["kernel"] == dec
-    assert details(80, 300, 1, 1000)["kernel"] == dec
-    assert details(80, 300, 1, 2000)["kernel"] == dec                # 19 chunks x 2000 keys: under 64k chunk-keys
+    assert details(48, 300, 1, 3000)["kernel"] == dec                # 19 chunks x 3000 keys
+    assert details(80, 300, 1, 2000)["kernel"] == dec
     assert details(80, 300, 1, 4000)["kernel"] == mma
+    assert details(80, 600, 16, 600)["kernel"] == dec                # 38 chunks per head, 608 in all: three rounds
     assert details(80, 16, 16, 4096)["kernel"] == dec                # 16 rows per head: never the tile kernel, which would need the copies
-    assert details(80, 1, 16, 64)["kernel"] == vec                   # a handful of keys above 64: the vector kernel
+    assert details(80, 1, 16, 64)["kernel"] == dec
     assert details(48, 1, 16, 64)["kernel"] == dec
     assert details(48, 3000, 1, 400)["kernel"] == mma                # 188 chunks on one KV head
     # F32 caches: too small to pay for the copy launch (100k query-key pairs); 2 .. 15 queries only above 64, from 150k pairs on
