@@ -352,13 +352,16 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) fattn_decode_kernel(const Fatt
         b     = blockIdx.x / (a.n_splits * a.Hkv);
         set   = blockIdx.x / a.n_splits;
     } else {
-        const int64_t w = blockIdx.x >> 3;
-        const int64_t p = (w / a.q_chunks) * 8 + (blockIdx.x & 7);
-        if (p >= (int64_t)a.n_splits * a.Hkv * a.B) return;
-        chunk = (int)(w % a.q_chunks);
-        split = (int)(p % a.n_splits);
-        hk    = (int)((p / a.n_splits) % a.Hkv);
-        b     = (int)(p / ((int64_t)a.n_splits * a.Hkv));
+        // (32-bit arithmetic: the grid has fewer than 2^31 workgroups, and 64-bit divisions are loops of a hundred
+        //  instructions each - 1 us before the first request leaves)
+        const uint32_t w  = blockIdx.x >> 3;
+        const uint32_t p  = (w / (uint32_t)a.q_chunks) * 8u + (blockIdx.x & 7u);
+        const uint32_t sh = (uint32_t)a.n_splits * (uint32_t)a.Hkv;           // (<= pairs <= the grid)
+        if (p >= sh * (uint32_t)a.B) return;
+        chunk = (int)(w % (uint32_t)a.q_chunks);
+        split = (int)(p % (uint32_t)a.n_splits);
+        hk    = (int)((p / (uint32_t)a.n_splits) % (uint32_t)a.Hkv);
+        b     = (int)(p / sh);
         set   = ((int64_t)b * a.Hkv + hk) * a.q_chunks + chunk;
     }
     const int bk    = b / a.bq;
